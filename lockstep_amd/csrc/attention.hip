@@ -1,0 +1,369 @@
+// Causal attention over the paged cache, one kernel family for prompt
+// portions and for decoded tokens, compiled for one head size (LS_HEAD_DIM).
+//
+// Rows.  For one sequence and one kv head the queries of the step are laid
+// out as rows r = i * G + g (i: query index in the step, g: head inside the
+// group of G query heads that share the kv head).  A wave owns 16 rows; a
+// lane owns one row (lane % 16) and a quarter of its columns.  With one
+// decoded token the G heads share one wave and each key is read once.
+//
+// Keys.  Positions are tiled in tiles of kTileKeys anchored at multiples of
+// kTileKeys, and in splits of kSplitKeys anchored at multiples of kSplitKeys,
+// whatever the step's first position is.  Inside a split the tiles are walked
+// in ascending order with the online softmax
+//     m' = max(m, rowmax(s)); a = exp(m - m'); p = exp(s - m') (0 if masked);
+//     l = l*a + sum(p); acc = acc*a + round(p) . V
+// and the splits are folded in ascending order with
+//     m' = max(M, m); A = exp(M - m'); B = exp(m - m');
+//     ACC = ACC*A + acc*B; L = L*A + l*B
+// starting from (0, -1e30, 0); out = ACC / L.  A split that holds no visible
+// key for a row (l == 0) is skipped for that row.  A workgroup either walks
+// all splits itself and writes the output ("direct"), or handles one split
+// and writes (acc, m, l) for the combine kernel, which runs the same fold.
+// Both give the same bits, so the choice is free; it is made on the host.
+//
+// A row's result therefore depends on its own query, its own position and
+// the cached keys and values below it, and on nothing else in the launch.
+//
+// Operands come straight from global memory in the MFMA layouts:
+//   S^T = K . Q^T      first operand: 16 keys x one chunk of d (key pages
+//                      [page][kv head][slot][d]), second: the wave's 16 rows;
+//                      a lane ends with keys 4*(lane/16)+{0..3} of its row.
+//   O^T = V^T . P^T    first operand: 16 columns of d x keys (value pages are
+//                      stored transposed, [page][kv head][d][slot], so four
+//                      consecutive keys of one column are one load), second:
+//                      the probabilities exactly as S^T left them in the lane.
+
+#include "common.h"
+
+#ifndef LS_HEAD_DIM
+#error "compile with -DLS_HEAD_DIM=<head size, a multiple of 16>"
+#endif
+
+namespace ls {
+
+constexpr int D = LS_HEAD_DIM;
+static_assert(D % 16 == 0 && D >= 16 && D <= 256, "head size must be a multiple of 16 up to 256");
+constexpr int kTileKeys = 128;
+constexpr int kSplitKeys = 256;
+constexpr int NB = kTileKeys / 16;  // 16-key blocks per tile
+constexpr int DB = D / 16;          // 16-column blocks of the head
+
+struct SeqMeta {
+  int q_off, q_len, q_start, kv_len, table_row, reserved[3];
+};
+struct AttnItem {  // one workgroup column of the attention launch
+  int seq;         // index into SeqMeta
+  int row_block;   // 64-row block of the sequence's rows
+  int split_begin, split_end;
+  int part_base;   // first partial row of the sequence, or -1: direct
+  int n_splits;    // splits of the sequence that have a partial
+  int split_lo;    // first of them (splits below lie behind the window)
+  int reserved;
+};
+
+template <typename T> __device__ __forceinline__ float softmax_exp(float x);
+template <> __device__ __forceinline__ float softmax_exp<float>(float x) { return expf(x); }
+template <> __device__ __forceinline__ float softmax_exp<bf16_t>(float x) { return __expf(x); }
+
+struct RowState {
+  f32x4 acc[DB];
+  float m, l;
+  __device__ __forceinline__ void reset() {
+#pragma unroll
+    for (int b = 0; b < DB; ++b) acc[b] = f32x4{0.f, 0.f, 0.f, 0.f};
+    m = kNegSentinel;
+    l = 0.f;
+  }
+};
+
+// Fold one split's (acc, m, l) into the running state; the same code runs in
+// the attention kernel and in the combine kernel.
+template <typename T>
+__device__ __forceinline__ void fold_split(RowState& run, const f32x4 (&acc)[DB], float m, float l) {
+  if (!(l > 0.f)) return;
+  const float m_new = fmaxf(run.m, m);
+  const float a = softmax_exp<T>(run.m - m_new);
+  const float b = softmax_exp<T>(m - m_new);
+#pragma unroll
+  for (int blk = 0; blk < DB; ++blk)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) run.acc[blk][e] = run.acc[blk][e] * a + acc[blk][e] * b;
+  run.l = run.l * a + l * b;
+  run.m = m_new;
+}
+
+template <typename T>
+__device__ __forceinline__ void store_output(const RowState& run, T* __restrict__ dst, int g) {
+  // dst: start of this row's head in the output; lane writes columns blk*16 + 4g + {0..3}
+#pragma unroll
+  for (int blk = 0; blk < DB; ++blk) {
+    float o[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) o[e] = run.l > 0.f ? run.acc[blk][e] / run.l : 0.f;
+    T* p = dst + blk * 16 + 4 * g;
+    if (sizeof(T) == 2) {
+      bf16x4 v;
+      v[0] = (bf16_t)o[0]; v[1] = (bf16_t)o[1]; v[2] = (bf16_t)o[2]; v[3] = (bf16_t)o[3];
+      *reinterpret_cast<bf16x4*>(p) = v;
+    } else {
+      *reinterpret_cast<f32x4*>(p) = f32x4{o[0], o[1], o[2], o[3]};
+    }
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void attention_kernel(
+    const T* __restrict__ q, long ldq, const T* __restrict__ k_pages, const T* __restrict__ v_pages, int nkv,
+    int page_size, const int* __restrict__ table, int table_stride, const SeqMeta* __restrict__ seqs,
+    const AttnItem* __restrict__ items, T* __restrict__ out, long ldo, float* __restrict__ part_acc,
+    float* __restrict__ part_ml, int G, float scale, int window) {
+  typedef Atom<T> A;
+  typedef typename A::vec_t vec_t;
+  constexpr int NC = (D + A::KCHUNK - 1) / A::KCHUNK;  // chunks over the head
+
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const AttnItem item = items[blockIdx.x];
+  const SeqMeta sm = seqs[item.seq];
+  const int kvh = blockIdx.y;
+  const int rows_total = sm.q_len * G;
+  const int r0 = item.row_block * 64 + wave * 16;
+  if (r0 >= rows_total) return;
+
+  const int row16 = lane & 15;
+  const int g = lane >> 4;
+  const int r = r0 + row16;
+  const bool row_ok = r < rows_total;
+  const int qi = row_ok ? r / G : 0;
+  const int head = kvh * G + (row_ok ? r % G : 0);
+  const int q_pos = sm.q_start + qi;
+  const int wave_first_pos = sm.q_start + r0 / G;
+  const int wave_last_pos = sm.q_start + min(r0 + 15, rows_total - 1) / G;
+  const int lo_valid = window > 0 ? max(0, sm.q_start - window + 1) : 0;
+  const int* __restrict__ tbl = table + (long)sm.table_row * table_stride;
+  const bool direct = item.part_base < 0;
+
+  vec_t qv[NC];
+#pragma unroll
+  for (int c = 0; c < NC; ++c)
+    qv[c] = load_vec<T>(q + (long)head * D, sm.q_off + qi, c * A::KCHUNK + g * A::VEC, D, ldq, row_ok, true);
+
+  RowState run;
+  run.reset();
+
+  for (int split = item.split_begin; split < item.split_end; ++split) {
+    const int s_begin = split * kSplitKeys;
+    const int s_end = min(s_begin + kSplitKeys, sm.kv_len);
+    RowState cur;
+    cur.reset();
+
+    for (int t0 = s_begin; t0 < s_end && t0 <= wave_last_pos; t0 += kTileKeys) {
+      if (window > 0 && t0 + kTileKeys <= wave_first_pos - window + 1) continue;  // behind every row's window
+
+      // ---- S^T = K . Q^T ---------------------------------------------------
+      f32x4 s[NB];
+#pragma unroll
+      for (int kb = 0; kb < NB; ++kb) {
+        s[kb] = f32x4{0.f, 0.f, 0.f, 0.f};
+        const int key = t0 + kb * 16 + row16;
+        bool key_ok = key < sm.kv_len && key >= lo_valid && key <= wave_last_pos;
+        long page = key_ok ? tbl[key / page_size] : -1;
+        key_ok = key_ok && page >= 0;
+        const T* krow = k_pages + ((page * nkv + kvh) * page_size + key % page_size) * D;
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+          vec_t kv = load_vec<T>(krow, 0, c * A::KCHUNK + g * A::VEC, D, 0, key_ok, true);
+          A::mma(s[kb], kv, qv[c]);
+        }
+      }
+
+      // ---- scale, mask, online softmax --------------------------------------
+      // lane holds keys t0 + kb*16 + 4g + e of its row
+      float tile_max = kNegSentinel;
+#pragma unroll
+      for (int kb = 0; kb < NB; ++kb)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int key = t0 + kb * 16 + 4 * g + e;
+          const bool keep = row_ok && key <= q_pos && (window <= 0 || q_pos - key < window);
+          const float v = keep ? s[kb][e] * scale : kNegSentinel;
+          s[kb][e] = v;
+          tile_max = fmaxf(tile_max, v);
+        }
+      tile_max = quad16_max(tile_max);
+      const float m_new = fmaxf(cur.m, tile_max);
+      const float alpha = softmax_exp<T>(cur.m - m_new);
+      float p_sum = 0.f;
+#pragma unroll
+      for (int kb = 0; kb < NB; ++kb)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int key = t0 + kb * 16 + 4 * g + e;
+          const bool keep = row_ok && key <= q_pos && (window <= 0 || q_pos - key < window);
+          const float p = keep ? softmax_exp<T>(s[kb][e] - m_new) : 0.f;
+          s[kb][e] = p;
+          p_sum = p_sum + p;
+        }
+      p_sum = quad16_sum(p_sum);
+      cur.l = cur.l * alpha + p_sum;
+      cur.m = m_new;
+#pragma unroll
+      for (int blk = 0; blk < DB; ++blk)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) cur.acc[blk][e] = cur.acc[blk][e] * alpha;
+
+      // ---- O^T += V^T . P^T --------------------------------------------------
+      // one atom covers KB16 blocks of 16 keys: bf16 two (8 keys per lane), f32 one (4 keys per lane)
+      constexpr int KB16 = A::VEC / 4;
+#pragma unroll
+      for (int kb = 0; kb < NB; kb += KB16) {
+        vec_t pv;
+        long vbase[KB16];
+        int vkey[KB16];
+#pragma unroll
+        for (int h = 0; h < KB16; ++h) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) pv[h * 4 + e] = from_f32<T>(s[kb + h][e]);
+          const int key = t0 + (kb + h) * 16 + 4 * g;
+          vkey[h] = key;
+          const bool any = key < sm.kv_len && key + 3 >= lo_valid;
+          const long page = any ? tbl[key / page_size] : -1;
+          vbase[h] = page >= 0 ? ((page * nkv + kvh) * D) * (long)page_size + key % page_size : -1;
+        }
+#pragma unroll
+        for (int blk = 0; blk < DB; ++blk) {
+          vec_t vv = A::zero();
+#pragma unroll
+          for (int h = 0; h < KB16; ++h) {
+            if (vbase[h] >= 0) {
+              const T* vp = v_pages + vbase[h] + (long)(blk * 16 + row16) * page_size;
+              if (sizeof(T) == 2) {
+                bf16x4 four = *reinterpret_cast<const bf16x4*>(vp);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) vv[h * 4 + e] = four[e];
+              } else {
+                f32x4 four = *reinterpret_cast<const f32x4*>(vp);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) vv[h * 4 + e] = four[e];
+              }
+#pragma unroll
+              for (int e = 0; e < 4; ++e)
+                if (vkey[h] + e >= sm.kv_len || vkey[h] + e < lo_valid) vv[h * 4 + e] = 0;
+            }
+          }
+          A::mma(cur.acc[blk], vv, pv);
+        }
+      }
+    }
+
+    if (direct) {
+      fold_split<T>(run, cur.acc, cur.m, cur.l);
+    } else if (row_ok) {
+      const long pr = item.part_base + ((long)kvh * rows_total + r) * item.n_splits + (split - item.split_lo);
+      float* pa = part_acc + pr * D;
+#pragma unroll
+      for (int blk = 0; blk < DB; ++blk) *reinterpret_cast<f32x4*>(pa + blk * 16 + 4 * g) = cur.acc[blk];
+      if (g == 0) {
+        part_ml[pr * 2] = cur.m;
+        part_ml[pr * 2 + 1] = cur.l;
+      }
+    }
+  }
+
+  if (direct && row_ok) store_output<T>(run, out + (long)(sm.q_off + qi) * ldo + (long)head * D, g);
+}
+
+struct CombineItem {
+  int seq, row_block, part_base, n_splits;
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void combine_kernel(const SeqMeta* __restrict__ seqs,
+                                                      const CombineItem* __restrict__ items,
+                                                      const float* __restrict__ part_acc,
+                                                      const float* __restrict__ part_ml, T* __restrict__ out,
+                                                      long ldo, int G) {
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const CombineItem item = items[blockIdx.x];
+  const SeqMeta sm = seqs[item.seq];
+  const int kvh = blockIdx.y;
+  const int rows_total = sm.q_len * G;
+  const int r = item.row_block * 64 + wave * 16 + (lane & 15);
+  if (r >= rows_total) return;
+  const int g = lane >> 4;
+  const int qi = r / G;
+  const int head = kvh * G + r % G;
+
+  RowState run;
+  run.reset();
+  const long pr0 = item.part_base + ((long)kvh * rows_total + r) * item.n_splits;
+  for (int s = 0; s < item.n_splits; ++s) {
+    const long pr = pr0 + s;
+    f32x4 acc[DB];
+#pragma unroll
+    for (int blk = 0; blk < DB; ++blk) acc[blk] = *reinterpret_cast<const f32x4*>(part_acc + pr * D + blk * 16 + 4 * g);
+    fold_split<T>(run, acc, part_ml[pr * 2], part_ml[pr * 2 + 1]);
+  }
+  store_output<T>(run, out + (long)(sm.q_off + qi) * ldo + (long)head * D, g);
+}
+
+}  // namespace ls
+
+LS_DEFINE_ERROR_API
+
+using namespace ls;
+
+extern "C" int ls_attn_head_dim() { return D; }
+extern "C" int ls_attn_tile_keys() { return kTileKeys; }
+extern "C" int ls_attn_split_keys() { return kSplitKeys; }
+
+// q [tokens, ldq]: head h of a token at columns [h*D, (h+1)*D).  out likewise
+// with ldo.  k_pages [pages][nkv][page_size][D], v_pages [pages][nkv][D][page_size].
+// table [rows][table_stride] int32 (page id or -1).  items: n_items AttnItem.
+extern "C" int ls_attention(int dtype, const void* q, long ldq, const void* k_pages, const void* v_pages, int nkv,
+                            int page_size, const int* table, int table_stride, const void* seqs, const void* items,
+                            int n_items, void* out, long ldo, float* part_acc, float* part_ml, int G, float scale,
+                            int window, void* stream) {
+  LS_REQUIRE(n_items > 0 && nkv > 0 && G > 0, "attention: bad sizes (items %d, kv heads %d, group %d)", n_items, nkv, G);
+  LS_REQUIRE(page_size >= 4 && page_size % 4 == 0 && kTileKeys % page_size == 0,
+             "attention: page size %d must be a multiple of 4 that divides the key tile %d", page_size, kTileKeys);
+  LS_REQUIRE(ldq % 8 == 0 && ldo % 4 == 0, "attention: row strides ldq=%ld ldo=%ld are not vector aligned", ldq, ldo);
+  LS_REQUIRE(ldq >= (long)nkv * G * D && ldo >= (long)nkv * G * D, "attention: row strides shorter than the heads");
+  LS_REQUIRE(reinterpret_cast<uintptr_t>(q) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0 &&
+                 reinterpret_cast<uintptr_t>(k_pages) % 16 == 0 && reinterpret_cast<uintptr_t>(v_pages) % 16 == 0,
+             "attention: operands must be 16-byte aligned");
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  dim3 grid(n_items, nkv);
+  if (dtype == kF32)
+    hipLaunchKernelGGL(attention_kernel<float>, grid, dim3(256), 0, s, (const float*)q, ldq, (const float*)k_pages,
+                       (const float*)v_pages, nkv, page_size, table, table_stride, (const SeqMeta*)seqs,
+                       (const AttnItem*)items, (float*)out, ldo, part_acc, part_ml, G, scale, window);
+  else if (dtype == kBF16)
+    hipLaunchKernelGGL(attention_kernel<bf16_t>, grid, dim3(256), 0, s, (const bf16_t*)q, ldq,
+                       (const bf16_t*)k_pages, (const bf16_t*)v_pages, nkv, page_size, table, table_stride,
+                       (const SeqMeta*)seqs, (const AttnItem*)items, (bf16_t*)out, ldo, part_acc, part_ml, G, scale,
+                       window);
+  else
+    return fail("attention: unknown dtype %d", dtype);
+  return check_launch("attention");
+}
+
+extern "C" int ls_attention_combine(int dtype, const void* seqs, const void* items, int n_items, int nkv,
+                                    const float* part_acc, const float* part_ml, void* out, long ldo, int G,
+                                    void* stream) {
+  LS_REQUIRE(n_items > 0 && nkv > 0 && G > 0, "combine: bad sizes");
+  LS_REQUIRE(ldo % 4 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0, "combine: output not vector aligned");
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  dim3 grid(n_items, nkv);
+  if (dtype == kF32)
+    hipLaunchKernelGGL(combine_kernel<float>, grid, dim3(256), 0, s, (const SeqMeta*)seqs, (const CombineItem*)items,
+                       part_acc, part_ml, (float*)out, ldo, G);
+  else if (dtype == kBF16)
+    hipLaunchKernelGGL(combine_kernel<bf16_t>, grid, dim3(256), 0, s, (const SeqMeta*)seqs,
+                       (const CombineItem*)items, part_acc, part_ml, (bf16_t*)out, ldo, G);
+  else
+    return fail("combine: unknown dtype %d", dtype);
+  return check_launch("combine");
+}

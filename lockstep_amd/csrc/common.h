@@ -1,0 +1,146 @@
+// Shared device helpers for the gfx950 kernels: element types, the MFMA
+// "atom" that every contraction is built from, cross-lane reductions with a
+// fixed order, and launch checking.
+//
+// Numerics contract shared by all kernels: a value that belongs to one row
+// (one token, one query) is reduced in an order that depends on compile-time
+// constants and the row's own sizes only -- never on the number of rows in
+// the launch or on where the row sits in a tile.  There are no atomics on
+// results and no split of a reduction across workgroups other than the
+// fixed, position-anchored splits that a separate kernel folds in ascending
+// order.  Floating-point contraction is switched off for the whole library
+// (-ffp-contract=off): a fused multiply-add appears only where fmaf is
+// written, so the same expression gives the same bits in every kernel.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace ls {
+
+typedef __bf16 bf16_t;
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+constexpr int kWave = 64;
+constexpr float kNegSentinel = -1e30f;  // finite "minus infinity" of the softmax
+
+enum DType : int { kF32 = 0, kBF16 = 1 };
+
+__device__ __forceinline__ float to_f32(float x) { return x; }
+__device__ __forceinline__ float to_f32(bf16_t x) { return static_cast<float>(x); }
+
+template <typename T> __device__ __forceinline__ T from_f32(float x);
+template <> __device__ __forceinline__ float from_f32<float>(float x) { return x; }
+// float -> bfloat16 is round-to-nearest-even (LLVM fptrunc semantics).
+template <> __device__ __forceinline__ bf16_t from_f32<bf16_t>(float x) { return static_cast<bf16_t>(x); }
+
+// ---------------------------------------------------------------------------
+// The contraction atom.  One "chunk" is 64 bytes of K per row: a lane holds
+// 16 bytes of it (VEC elements) at element offset VEC * (lane / 16), for row
+// (lane % 16) of its operand.  mma() adds the 16x16 product of two such
+// operands to a 16x16 float accumulator of which a lane holds four entries:
+// column (lane % 16) of the second operand, rows 4 * (lane / 16) + {0,1,2,3}
+// of the first.
+//   bf16:  one v_mfma_f32_16x16x32_bf16 (32 K per chunk).
+//   f32:   four v_mfma_f32_16x16x4_f32 (16 K per chunk) -- full 32-bit
+//          products and sums, no reduced-precision matrix mode.
+// ---------------------------------------------------------------------------
+template <typename T> struct Atom;
+
+template <> struct Atom<bf16_t> {
+  static constexpr int VEC = 8;
+  static constexpr int KCHUNK = 32;
+  typedef bf16x8 vec_t;
+  static __device__ __forceinline__ vec_t zero() { return vec_t{0, 0, 0, 0, 0, 0, 0, 0}; }
+  static __device__ __forceinline__ void mma(f32x4& acc, const vec_t& a, const vec_t& b) {
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc, 0, 0, 0);
+  }
+};
+
+template <> struct Atom<float> {
+  static constexpr int VEC = 4;
+  static constexpr int KCHUNK = 16;
+  typedef f32x4 vec_t;
+  static __device__ __forceinline__ vec_t zero() { return vec_t{0.f, 0.f, 0.f, 0.f}; }
+  static __device__ __forceinline__ void mma(f32x4& acc, const vec_t& a, const vec_t& b) {
+    acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[0], b[0], acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[1], b[1], acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[2], b[2], acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[3], b[3], acc, 0, 0, 0);
+  }
+};
+
+// Load VEC elements of row `row` at element offset `k` of a row-major matrix
+// with `ld` elements per row, zero where the row is not `ok` or k >= limit.
+// `aligned` (uniform) says every row start and k are 16-byte aligned.
+template <typename T>
+__device__ __forceinline__ typename Atom<T>::vec_t load_vec(const T* __restrict__ base, long row, int k,
+                                                            int limit, long ld, bool ok, bool aligned) {
+  typedef typename Atom<T>::vec_t vec_t;
+  constexpr int VEC = Atom<T>::VEC;
+  vec_t v = Atom<T>::zero();
+  if (!ok || k >= limit) return v;
+  const T* p = base + row * ld + k;
+  if (aligned && k + VEC <= limit) {
+    v = *reinterpret_cast<const vec_t*>(p);
+  } else {
+#pragma unroll
+    for (int e = 0; e < VEC; ++e)
+      if (k + e < limit) v[e] = p[e];
+  }
+  return v;
+}
+
+// Sum / max over the four lanes {l, l^16, l^32, l^48}; every lane of the
+// four ends with the same bits because each step adds a pair commutatively.
+__device__ __forceinline__ float quad16_sum(float v) {
+  v = v + __shfl_xor(v, 16, kWave);
+  v = v + __shfl_xor(v, 32, kWave);
+  return v;
+}
+__device__ __forceinline__ float quad16_max(float v) {
+  v = fmaxf(v, __shfl_xor(v, 16, kWave));
+  v = fmaxf(v, __shfl_xor(v, 32, kWave));
+  return v;
+}
+
+// Butterfly sum over all 64 lanes, same bits in every lane.
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int m = 1; m < kWave; m <<= 1) v = v + __shfl_xor(v, m, kWave);
+  return v;
+}
+
+}  // namespace ls
+
+// Error reporting across the C interface: every entry point returns 0 or a
+// negative code and leaves a message that ls_last_error() of the same library
+// returns.  Each shared library defines ls_last_error() once through
+// LS_DEFINE_ERROR_API.
+#include <stdarg.h>
+#include <stdio.h>
+namespace ls {
+inline char g_error[1024] = {0};
+inline int fail(const char* fmt, ...) {
+  va_list args;
+  va_start(args, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, args);
+  va_end(args);
+  return -1;
+}
+inline int check_launch(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail("%s: %s", what, hipGetErrorString(e));
+  return 0;
+}
+}  // namespace ls
+
+#define LS_DEFINE_ERROR_API \
+  extern "C" const char* ls_last_error() { return ls::g_error; }
+
+#define LS_REQUIRE(cond, ...)                   \
+  do {                                          \
+    if (!(cond)) return ls::fail(__VA_ARGS__);  \
+  } while (0)

@@ -1,0 +1,285 @@
+// Row-wise kernels of the step: embedding gather, RMSNorm of the residual
+// stream, per-head norm + rotation + cache write, SwiGLU, arg-max.
+//
+// The residual stream is float in both precisions; everything that goes into
+// a matrix product is in the compute dtype T (float or bfloat16).  All
+// reductions are per row with an order fixed by the row's width alone.
+
+#include "common.h"
+
+namespace ls {
+
+// ---------------------------------------------------------------------------
+// Embedding: h[t, :] = float(E[token[t], :]).  A token id outside the table
+// writes zeros (the host rejects such ids before the launch; the kernel must
+// not fault on them).
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void embed_kernel(const int* __restrict__ tokens, const T* __restrict__ table,
+                                                    float* __restrict__ out, int vocab, int width, long ld_out) {
+  const int t = blockIdx.x;
+  const int id = tokens[t];
+  const bool ok = id >= 0 && id < vocab;
+  const T* row = table + (long)(ok ? id : 0) * width;
+  float* dst = out + (long)t * ld_out;
+  for (int e = threadIdx.x; e < width; e += blockDim.x) dst[e] = ok ? to_f32(row[e]) : 0.f;
+}
+
+// ---------------------------------------------------------------------------
+// RMSNorm over rows of the float residual stream:
+//   y = (x * 1/sqrt(sum(x^2)/N + eps)) * w      (all in float), stored as T.
+// One workgroup per output row.  Thread i sums x[i]^2, x[i+256]^2, ... in
+// ascending order; a wave adds its lanes by butterfly; the four wave sums are
+// added in wave order.  `rows` (optional) picks the input row of each output.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ x, const float* __restrict__ weight,
+                                                      T* __restrict__ out, const int* __restrict__ rows, int width,
+                                                      long ldx, long ld_out, float eps) {
+  __shared__ float wave_part[4];
+  const int r_out = blockIdx.x;
+  const long r_in = rows ? rows[r_out] : r_out;
+  const float* src = x + r_in * ldx;
+  float part = 0.f;
+  for (int e = threadIdx.x; e < width; e += 256) {
+    const float v = src[e];
+    part = part + v * v;
+  }
+  part = wave_sum(part);
+  if ((threadIdx.x & 63) == 0) wave_part[threadIdx.x >> 6] = part;
+  __syncthreads();
+  const float total = ((wave_part[0] + wave_part[1]) + wave_part[2]) + wave_part[3];
+  const float scale = 1.0f / sqrtf(total / (float)width + eps);
+  T* dst = out + (long)r_out * ld_out;
+  for (int e = threadIdx.x; e < width; e += 256) dst[e] = from_f32<T>((src[e] * scale) * weight[e]);
+}
+
+// ---------------------------------------------------------------------------
+// Per (token, head) of the fused q|k|v projection output:
+//   q, k heads: optional RMSNorm over the head (one [d] weight for all
+//   heads), then optional half rotation of the first `rot` dims with the
+//   pair (i, i + rot/2):  lo' = lo*c - hi*s,  hi' = hi*c + lo*s  at the
+//   token's absolute position; q is written back in place, k goes to the
+//   key pages [page][kv head][slot][d];
+//   v heads: copied to the transposed value pages [page][kv head][d][slot].
+// One wave per (token, head); sums of squares: lane i adds x[i]^2,
+// x[i+64]^2, ... ascending, then a butterfly over the wave.
+// ---------------------------------------------------------------------------
+constexpr int kMaxHeadDim = 256;
+
+struct SeqMeta {  // one per sequence of the step (all int32)
+  int q_off;      // first packed row
+  int q_len;      // rows in this step
+  int q_start;    // absolute position of the first row
+  int kv_len;     // q_start + q_len
+  int table_row;  // row of the block table
+  int reserved[3];
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void qk_rope_kv_kernel(
+    T* __restrict__ qkv, long ld, int nq, int nkv, int d, const float* __restrict__ q_weight,
+    const float* __restrict__ k_weight, float eps, const float* __restrict__ cos_table,
+    const float* __restrict__ sin_table, int rot, const int* __restrict__ tok_seq, const int* __restrict__ tok_pos,
+    const SeqMeta* __restrict__ seqs, const int* __restrict__ table, int table_stride, T* __restrict__ k_pages,
+    T* __restrict__ v_pages, int page_size, int write_kv) {
+  __shared__ float stage[4][kMaxHeadDim];
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int t = blockIdx.x;
+  const int head = blockIdx.y * 4 + wave;
+  const int heads = write_kv ? nq + 2 * nkv : nq;
+  if (head >= heads) return;
+
+  T* src = qkv + (long)t * ld + (long)head * d;
+  const int pos = tok_pos[t];
+  const bool is_q = head < nq;
+  const bool is_k = !is_q && head < nq + nkv;
+
+  long page = 0;
+  int slot = 0;
+  if (!is_q) {
+    const SeqMeta sm = seqs[tok_seq[t]];
+    page = table[(long)sm.table_row * table_stride + pos / page_size];
+    slot = pos % page_size;
+    if (page < 0) return;  // the host never schedules a write to a page it does not hold
+  }
+
+  if (!is_q && !is_k) {
+    const int kvh = head - nq - nkv;
+    T* dst = v_pages + ((page * nkv + kvh) * d) * page_size + slot;
+    for (int e = lane; e < d; e += 64) dst[(long)e * page_size] = src[e];
+    return;
+  }
+
+  const float* weight = is_q ? q_weight : k_weight;
+  float* y = stage[wave];
+  float part = 0.f;
+  for (int e = lane; e < d; e += 64) {
+    const float v = to_f32(src[e]);
+    y[e] = v;
+    part = part + v * v;
+  }
+  if (weight) {
+    const float total = wave_sum(part);
+    const float scale = 1.0f / sqrtf(total / (float)d + eps);
+    for (int e = lane; e < d; e += 64) y[e] = (y[e] * scale) * weight[e];
+  }
+  // The staging row is private to this wave: order its writes before the
+  // reads of other lanes without a workgroup barrier (waves of other heads
+  // may have left already).
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+  T* dst = is_q ? src : k_pages + ((page * nkv + (head - nq)) * page_size + slot) * d;
+  const int half = rot / 2;
+  for (int e = lane; e < d; e += 64) {
+    float v = y[e];
+    if (cos_table && e < rot) {
+      const int i = e < half ? e : e - half;
+      const float c = cos_table[(long)pos * half + i];
+      const float s = sin_table[(long)pos * half + i];
+      const float lo = y[i];
+      const float hi = y[i + half];
+      v = e < half ? lo * c - hi * s : hi * c + lo * s;
+    }
+    dst[e] = from_f32<T>(v);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// SwiGLU: act = (g * 1/(1 + exp(-g))) * u in float; gu [rows, 2*I] holds the
+// gates in columns [0, I) and the ups in [I, 2I).
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int rows,
+                                                     int inter, long ld_in, long ld_out) {
+  const long idx = (long)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (long)rows * inter) return;
+  const long r = idx / inter;
+  const int c = (int)(idx % inter);
+  const float g = to_f32(gu[r * ld_in + c]);
+  const float u = to_f32(gu[r * ld_in + inter + c]);
+  const float sig = 1.0f / (1.0f + expf(-g));
+  out[r * ld_out + c] = from_f32<T>((g * sig) * u);
+}
+
+// ---------------------------------------------------------------------------
+// Arg-max of float rows with the lowest index among equal maxima.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(1024) void argmax_kernel(const float* __restrict__ x, int* __restrict__ out, int width,
+                                                      long ld) {
+  __shared__ float best_v[1024];
+  __shared__ int best_i[1024];
+  const float* row = x + (long)blockIdx.x * ld;
+  float bv = -INFINITY;
+  int bi = 0x7fffffff;
+  for (int e = threadIdx.x; e < width; e += 1024) {
+    const float v = row[e];
+    if (v > bv || (v == bv && e < bi)) { bv = v; bi = e; }
+  }
+  best_v[threadIdx.x] = bv;
+  best_i[threadIdx.x] = bi;
+  __syncthreads();
+  for (int stride = 512; stride > 0; stride >>= 1) {
+    if (threadIdx.x < stride) {
+      const float ov = best_v[threadIdx.x + stride];
+      const int oi = best_i[threadIdx.x + stride];
+      if (ov > best_v[threadIdx.x] || (ov == best_v[threadIdx.x] && oi < best_i[threadIdx.x])) {
+        best_v[threadIdx.x] = ov;
+        best_i[threadIdx.x] = oi;
+      }
+    }
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) out[blockIdx.x] = best_i[0] == 0x7fffffff ? 0 : best_i[0];
+}
+
+}  // namespace ls
+
+LS_DEFINE_ERROR_API
+
+using namespace ls;
+
+extern "C" int ls_embed(int dtype, const int* tokens, const void* table, float* out, int n_tokens, int vocab,
+                        int width, long ld_out, void* stream) {
+  LS_REQUIRE(n_tokens > 0 && vocab > 0 && width > 0 && ld_out >= width, "embed: bad sizes");
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  if (dtype == kF32)
+    hipLaunchKernelGGL(embed_kernel<float>, dim3(n_tokens), dim3(256), 0, s, tokens, (const float*)table, out, vocab,
+                       width, ld_out);
+  else if (dtype == kBF16)
+    hipLaunchKernelGGL(embed_kernel<bf16_t>, dim3(n_tokens), dim3(256), 0, s, tokens, (const bf16_t*)table, out,
+                       vocab, width, ld_out);
+  else
+    return fail("embed: unknown dtype %d", dtype);
+  return check_launch("embed");
+}
+
+extern "C" int ls_rmsnorm(int dtype, const float* x, const float* weight, void* out, const int* rows, int n_rows,
+                          int width, long ldx, long ld_out, float eps, void* stream) {
+  LS_REQUIRE(n_rows > 0 && width > 0 && ldx >= width && ld_out >= width, "rmsnorm: bad sizes");
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  if (dtype == kF32)
+    hipLaunchKernelGGL(rmsnorm_kernel<float>, dim3(n_rows), dim3(256), 0, s, x, weight, (float*)out, rows, width, ldx,
+                       ld_out, eps);
+  else if (dtype == kBF16)
+    hipLaunchKernelGGL(rmsnorm_kernel<bf16_t>, dim3(n_rows), dim3(256), 0, s, x, weight, (bf16_t*)out, rows, width,
+                       ldx, ld_out, eps);
+  else
+    return fail("rmsnorm: unknown dtype %d", dtype);
+  return check_launch("rmsnorm");
+}
+
+extern "C" int ls_qk_rope_kv(int dtype, void* qkv, long ld, int n_tokens, int nq, int nkv, int d,
+                             const float* q_weight, const float* k_weight, float eps, const float* cos_table,
+                             const float* sin_table, int rot, int table_positions, const int* tok_seq,
+                             const int* tok_pos, const void* seqs, const int* table, int table_stride, void* k_pages,
+                             void* v_pages, int page_size, int write_kv, void* stream) {
+  LS_REQUIRE(n_tokens > 0 && nq >= 0 && nkv >= 0 && d > 0, "qk_rope_kv: bad sizes");
+  LS_REQUIRE(d <= kMaxHeadDim, "qk_rope_kv: head_dim %d exceeds the supported maximum %d", d, kMaxHeadDim);
+  LS_REQUIRE(rot >= 0 && rot <= d && rot % 2 == 0, "qk_rope_kv: rotary_dim %d must be even and at most head_dim %d",
+             rot, d);
+  LS_REQUIRE(!cos_table || (sin_table && table_positions > 0), "qk_rope_kv: rotation tables incomplete");
+  const int heads = write_kv ? nq + 2 * nkv : nq;
+  LS_REQUIRE(ld >= (long)heads * d, "qk_rope_kv: row stride %ld shorter than %d heads of %d", ld, heads, d);
+  LS_REQUIRE(!write_kv || (k_pages && v_pages && table && page_size > 0), "qk_rope_kv: cache operands missing");
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  dim3 grid(n_tokens, (heads + 3) / 4);
+  if (dtype == kF32)
+    hipLaunchKernelGGL(qk_rope_kv_kernel<float>, grid, dim3(256), 0, s, (float*)qkv, ld, nq, nkv, d, q_weight,
+                       k_weight, eps, cos_table, sin_table, rot, tok_seq, tok_pos, (const SeqMeta*)seqs, table,
+                       table_stride, (float*)k_pages, (float*)v_pages, page_size, write_kv);
+  else if (dtype == kBF16)
+    hipLaunchKernelGGL(qk_rope_kv_kernel<bf16_t>, grid, dim3(256), 0, s, (bf16_t*)qkv, ld, nq, nkv, d, q_weight,
+                       k_weight, eps, cos_table, sin_table, rot, tok_seq, tok_pos, (const SeqMeta*)seqs, table,
+                       table_stride, (bf16_t*)k_pages, (bf16_t*)v_pages, page_size, write_kv);
+  else
+    return fail("qk_rope_kv: unknown dtype %d", dtype);
+  return check_launch("qk_rope_kv");
+}
+
+extern "C" int ls_swiglu(int dtype, const void* gu, void* out, int rows, int inter, long ld_in, long ld_out,
+                         void* stream) {
+  LS_REQUIRE(rows > 0 && inter > 0 && ld_in >= 2L * inter && ld_out >= inter, "swiglu: bad sizes");
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  const long total = (long)rows * inter;
+  dim3 grid((unsigned)((total + 255) / 256));
+  if (dtype == kF32)
+    hipLaunchKernelGGL(swiglu_kernel<float>, grid, dim3(256), 0, s, (const float*)gu, (float*)out, rows, inter, ld_in,
+                       ld_out);
+  else if (dtype == kBF16)
+    hipLaunchKernelGGL(swiglu_kernel<bf16_t>, grid, dim3(256), 0, s, (const bf16_t*)gu, (bf16_t*)out, rows, inter,
+                       ld_in, ld_out);
+  else
+    return fail("swiglu: unknown dtype %d", dtype);
+  return check_launch("swiglu");
+}
+
+extern "C" int ls_argmax(const float* x, int* out, int rows, int width, long ld, void* stream) {
+  LS_REQUIRE(rows > 0 && width > 0 && ld >= width, "argmax: bad sizes");
+  hipLaunchKernelGGL(argmax_kernel, dim3(rows), dim3(1024), 0, reinterpret_cast<hipStream_t>(stream), x, out, width,
+                     ld);
+  return check_launch("argmax");
+}

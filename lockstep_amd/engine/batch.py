@@ -1,0 +1,168 @@
+"""One step's batch: packed tokens, per-request metadata and the attention
+work lists, built on the host and uploaded in one copy.
+
+A step holds, for each request in it, one run of consecutive tokens that
+starts at the request's current length: a whole prompt, a portion of one, or
+a single decoded token.  All runs are packed into one ``[T, ...]`` batch.
+Device-side layout of the metadata (int32):
+
+    token ids [T] | request index of each token [T] | position of each token [T]
+    | per request 8 ints: first row, rows, first position, length after the
+      step, block-table row (the request's slot), 0, 0, 0
+    | rows whose logits are wanted [W]
+    | attention items (8 ints each) and combine items (4 ints each) per plan
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Hashable, Sequence
+
+import numpy as np
+import torch
+
+
+@dataclass
+class StepEntry:
+    """A request's next tokens and the places among them whose logits are wanted."""
+
+    request: Hashable
+    tokens: Sequence[int]
+    want: Sequence[int] = ()
+
+
+@dataclass
+class AttentionPlan:
+    items: torch.Tensor
+    n_items: int
+    combine_items: torch.Tensor | None
+    n_combine: int
+    part_acc: torch.Tensor | None
+    part_ml: torch.Tensor | None
+
+
+class Workspace:
+    """Named device buffers that grow on demand and persist between steps."""
+
+    def __init__(self, device):
+        self.device = device
+        self._buffers: dict[tuple, torch.Tensor] = {}
+
+    def get(self, name: str, shape, dtype) -> torch.Tensor:
+        shape = tuple(int(s) for s in shape)
+        rows, inner = shape[0], shape[1:]
+        key = (name, inner, dtype)
+        have = self._buffers.get(key)
+        if have is None or have.shape[0] < rows:
+            grow = max(rows, 2 * have.shape[0] if have is not None else rows)
+            have = torch.empty((grow, *inner), dtype=dtype, device=self.device)
+            self._buffers[key] = have
+        return have[:rows]
+
+
+class StepContext:
+    """Everything a part may read about the step (see module docstring)."""
+
+    def __init__(self, rt, cache, workspace: Workspace, entries: Sequence[StepEntry]):
+        self.rt = rt
+        self.cache = cache
+        self.workspace = workspace
+        self.entries = list(entries)
+        lengths = [len(e.tokens) for e in self.entries]
+        self.n_seqs = len(self.entries)
+        self.n_tokens = int(sum(lengths))
+        # host-side views, also for parts written in plain torch (tests)
+        self.q_len = np.asarray(lengths, dtype=np.int64)
+        self.q_off = np.concatenate([[0], np.cumsum(self.q_len)[:-1]]).astype(np.int64)
+        self.q_start = np.asarray([cache.length(e.request) for e in self.entries], dtype=np.int64)
+        self.kv_len = self.q_start + self.q_len
+        self.slots = np.asarray([cache.slot(e.request) for e in self.entries], dtype=np.int64)
+        self.max_position = int(self.kv_len.max()) - 1
+
+        tokens = np.concatenate([np.asarray(e.tokens, dtype=np.int64) for e in self.entries])
+        tok_seq = np.repeat(np.arange(self.n_seqs), self.q_len)
+        tok_pos = np.concatenate([np.arange(s, s + n) for s, n in zip(self.q_start, self.q_len)])
+        seqs = np.zeros((self.n_seqs, 8), dtype=np.int64)
+        seqs[:, 0], seqs[:, 1], seqs[:, 2], seqs[:, 3], seqs[:, 4] = (
+            self.q_off, self.q_len, self.q_start, self.kv_len, self.slots)
+        want = [int(self.q_off[i]) + int(w) for i, e in enumerate(self.entries) for w in e.want]
+        self.n_want = len(want)
+        self._host_parts: list[np.ndarray] = [tokens, tok_seq, tok_pos, seqs.reshape(-1),
+                                              np.asarray(want, dtype=np.int64)]
+        self._plans: dict[tuple, tuple] = {}
+        self._plan_specs: list[tuple] = []
+        self._uploaded = False
+        self.token_ids = self.tok_seq = self.tok_pos = self.seqs = self.want_rows = None
+        self.host_tokens = tokens
+
+    # -- attention work lists -----------------------------------------------------
+    def plan_attention(self, group_size: int, nkv: int, head_dim: int, window: int) -> None:
+        """Declare that a mixer with these constants runs in this step (before upload)."""
+        key = (group_size, nkv, head_dim, window)
+        if key in self._plans:
+            return
+        tile, split = self.rt.kernels.attention_geometry(head_dim)
+        items, combine = [], []
+        part_rows = 0
+        for i in range(self.n_seqs):
+            q_len, q_start, kv_len = int(self.q_len[i]), int(self.q_start[i]), int(self.kv_len[i])
+            rows = q_len * group_size
+            lo_valid = max(0, q_start - window + 1) if window > 0 else 0
+            split_lo = lo_valid // split
+            n_splits = (kv_len - 1) // split + 1 - split_lo
+            if rows <= 64 and n_splits > 1:
+                base = part_rows
+                part_rows += nkv * rows * n_splits
+                for s in range(split_lo, split_lo + n_splits):
+                    items.append((i, 0, s, s + 1, base, n_splits, split_lo, 0))
+                combine.append((i, 0, base, n_splits))
+            else:
+                for block in range(-(-rows // 64)):
+                    first_pos = q_start + (block * 64) // group_size
+                    last_pos = q_start + min(block * 64 + 63, rows - 1) // group_size
+                    begin = (max(0, first_pos - window + 1) // split) if window > 0 else 0
+                    items.append((i, block, begin, last_pos // split + 1, -1, 0, 0, 0))
+        self._plans[key] = (np.asarray(items, dtype=np.int64).reshape(-1),
+                            np.asarray(combine, dtype=np.int64).reshape(-1), len(items), len(combine), part_rows)
+        self._plan_specs.append(key)
+
+    def upload(self) -> None:
+        """Copy all metadata to the device in one transfer."""
+        parts = list(self._host_parts)
+        for key in self._plan_specs:
+            items, combine, *_ = self._plans[key]
+            parts += [items, combine]
+        flat = np.concatenate(parts).astype(np.int32)
+        host = torch.from_numpy(flat)
+        dev = self.workspace.get("step.meta", (flat.shape[0],), torch.int32)
+        dev.copy_(host, non_blocking=False)
+        offset = 0
+
+        def take(n):
+            nonlocal offset
+            out = dev[offset:offset + n]
+            offset += n
+            return out
+
+        t, s = self.n_tokens, self.n_seqs
+        self.token_ids, self.tok_seq, self.tok_pos = take(t), take(t), take(t)
+        self.seqs = take(8 * s)
+        self.want_rows = take(self.n_want)
+        self._device_plans: dict[tuple, AttentionPlan] = {}
+        for key in self._plan_specs:
+            items, combine, n_items, n_combine, part_rows = self._plans[key]
+            head_dim = key[2]
+            d_items, d_combine = take(items.shape[0]), take(combine.shape[0])
+            part_acc = part_ml = None
+            if part_rows:
+                part_acc = self.workspace.get(f"attention.part_acc.{head_dim}", (part_rows, head_dim), torch.float32)
+                part_ml = self.workspace.get("attention.part_ml", (part_rows, 2), torch.float32)
+            self._device_plans[key] = AttentionPlan(d_items, n_items, d_combine if n_combine else None,
+                                                    n_combine, part_acc, part_ml)
+        self._uploaded = True
+
+    def attention_plan(self, group_size: int, nkv: int, head_dim: int, window: int) -> AttentionPlan:
+        return self._device_plans[(group_size, nkv, head_dim, window)]
+
+    def buf(self, name: str, shape, dtype) -> torch.Tensor:
+        return self.workspace.get(name, shape, dtype)

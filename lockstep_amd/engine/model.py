@@ -1,0 +1,149 @@
+"""The model: parts assembled from a ``ModelSpec``, and the step function.
+
+``Model.step`` is the one way tokens go through the network: a batch of
+(request, its next tokens), prompt portions beside single decoded tokens, cut
+anywhere.  It runs only the tokens it is given, as one packed batch, on top
+of what earlier steps left in the cache, and returns float32 logits at the
+wanted places (reference engine/model/qwen3.py:294-378, which computes every
+row; here the final norm and the head run on the wanted rows only).
+"""
+
+from __future__ import annotations
+
+from pathlib import Path
+from typing import Sequence
+
+import numpy as np
+import torch
+
+from ..cache import CacheManager
+from ..config import ModelConfig, ModelSpec, config_from_dir
+from ..parts import WeightSpec, build_part, part_class
+from ..weights.store import load_weights, weights_from_dict
+from .batch import StepContext, StepEntry, Workspace
+from .runtime import Runtime
+
+
+def collect_weight_specs(spec: ModelSpec) -> list[WeightSpec]:
+    """Every tensor the model expects, in checkpoint order."""
+    out = list(part_class(spec.embedding.kind).weight_specs(spec.embedding, ""))
+    for layer in spec.layers:
+        out += part_class(layer.arrangement.kind).weight_specs(layer)
+    out += part_class(spec.final_norm.kind).weight_specs(spec.final_norm, "")
+    out += part_class(spec.head.kind).weight_specs(spec.head, "")
+    seen, unique = set(), []
+    for w in out:
+        if w.name not in seen:
+            seen.add(w.name)
+            unique.append(w)
+    return unique
+
+
+def collect_ties(spec: ModelSpec) -> dict[str, str]:
+    head = part_class(spec.head.kind)
+    return dict(head.ties(spec.head)) if hasattr(head, "ties") else {}
+
+
+class Model:
+    def __init__(self, config: ModelConfig, rt: Runtime):
+        self.config = config
+        self.rt = rt
+        self.spec = config.model_spec()
+        self.embedding = build_part(self.spec.embedding)
+        self.layers = [part_class(layer.arrangement.kind)(layer) for layer in self.spec.layers]
+        self.final_norm = build_part(self.spec.final_norm, "")
+        self.head = build_part(self.spec.head)
+        self.schedule = self.spec.schedule
+        for run in self.schedule:
+            if not 0 <= run.layer < len(self.layers):
+                raise ValueError(f"the schedule names layer {run.layer}, the model has {len(self.layers)}")
+        self.workspace = Workspace(rt.device)
+
+    # -- weights --------------------------------------------------------------
+    def load(self, weights) -> "Model":
+        self.embedding.load(weights, self.rt)
+        for layer in self.layers:
+            layer.load(weights, self.rt)
+        self.final_norm.load(weights, self.rt)
+        self.head.load(weights, self.rt)
+        return self
+
+    # -- cache ------------------------------------------------------------------
+    def cache_unit_specs(self) -> list:
+        units = [None] * self.spec.cache_units()
+        for run in self.schedule:
+            if run.writes_cache:
+                units[run.cache] = self.layers[run.layer].mixer.cache_spec()
+        return units
+
+    def make_cache(self, num_pages: int, page_size: int = 16, max_requests: int = 64,
+                   max_tokens_per_request: int | None = None, poison_on_free: bool = False) -> CacheManager:
+        if max_tokens_per_request is None:
+            max_tokens_per_request = num_pages * page_size
+        return CacheManager(self.cache_unit_specs(), page_size, num_pages, max_requests, max_tokens_per_request,
+                            torch_dtype=self.rt.dtype, device=self.rt.device, poison_on_free=poison_on_free)
+
+    # -- the step ------------------------------------------------------------------
+    def step(self, cache: CacheManager, entries: Sequence[StepEntry]):
+        """Run one batch.  Returns float32 logits ``[wanted, vocab]`` on the
+        device in the order of the entries and of their ``want``, or None."""
+        entries = [e for e in entries if len(e.tokens)]
+        if not entries:
+            return None
+        vocab = self.spec.vocab_size
+        seen = set()
+        for e in entries:
+            if e.request in seen:
+                raise ValueError(f"request {e.request!r} appears twice in one step")
+            seen.add(e.request)
+            ids = np.asarray(e.tokens)
+            if ids.min() < 0 or ids.max() >= vocab:
+                raise ValueError(f"request {e.request!r} brings a token id outside [0, {vocab})")
+            for w in e.want:
+                if not 0 <= w < len(e.tokens):
+                    raise ValueError(f"request {e.request!r} wants logits at {w}, it brings {len(e.tokens)} tokens")
+        for e in entries:
+            start = cache.length(e.request)
+            cache.reserve(e.request, start + len(e.tokens))
+            for gi, group in enumerate(cache.groups):
+                if group.pinned or max(group.pool.holders, default=0) > 1:
+                    for logical in range(start // cache.page_size, -(-(start + len(e.tokens)) // cache.page_size)):
+                        cache.assert_exclusive(e.request, gi, logical)
+        cache.sync_tables()
+
+        ctx = StepContext(self.rt, cache, self.workspace, entries)
+        for layer in self.layers:
+            layer.mixer.prepare(ctx)
+        ctx.upload()
+
+        h = ctx.buf("residual", (ctx.n_tokens, self.spec.hidden_size), torch.float32)
+        self.embedding.forward(ctx, ctx.token_ids, h)
+        for run in self.schedule:
+            self.layers[run.layer].forward(ctx, run, h)
+
+        logits = None
+        if ctx.n_want:
+            x = ctx.buf("final.normed", (ctx.n_want, self.spec.hidden_size), self.rt.dtype)
+            self.final_norm.forward(ctx, h, x, rows=ctx.want_rows)
+            logits = torch.empty((ctx.n_want, vocab), dtype=torch.float32, device=self.rt.device)
+            self.head.forward(ctx, x, logits)
+        for e, end in zip(entries, ctx.kv_len):
+            cache.commit(e.request, int(end))
+        return logits
+
+
+def load_model(model_dir, dtype="bfloat16", device="cuda:0") -> Model:
+    """Open a folder with config.json and model.safetensors; the class of the
+    configuration, and with it the architecture, is chosen by config.json."""
+    config = config_from_dir(model_dir)
+    rt = Runtime(device, dtype)
+    model = Model(config, rt)
+    weights = load_weights(model_dir, collect_weight_specs(model.spec), collect_ties(model.spec))
+    return model.load(weights)
+
+
+def model_from_tensors(config: ModelConfig, tensors, dtype="bfloat16", device="cuda:0") -> Model:
+    rt = Runtime(device, dtype)
+    model = Model(config, rt)
+    weights = weights_from_dict(tensors, collect_weight_specs(model.spec), collect_ties(model.spec))
+    return model.load(weights)

@@ -1,0 +1,5 @@
+"""Hand-written gfx950 kernels and the code that builds and loads them."""
+
+from .kernels import ADD_F32, STORE, STORE_F32, KernelError, Kernels, kernels
+
+__all__ = ["ADD_F32", "STORE", "STORE_F32", "KernelError", "Kernels", "kernels"]

@@ -1,0 +1,175 @@
+"""Compile the HIP sources under ``lockstep_amd/csrc`` into shared libraries.
+
+Two kinds of library exist:
+
+``core``            every kernel whose code does not depend on a model size
+                    (matrix products, norms, rotation and cache write, SwiGLU,
+                    embedding, arg-max);
+``attention<D>``    the attention kernels for one head size ``D``; a model
+                    needs only its own.
+
+A library's file name carries a hash of its sources and flags, so a stale
+build is never loaded.  Libraries are written next to the package
+(``lockstep_amd/_lib``) when that folder can be written, otherwise to a
+per-user folder under the system's temporary directory.  ``load`` compiles at
+the first call what is not there yet and says so on stderr while it works.
+There is no fallback: without the library (and without ``hipcc`` to make it)
+the import of the kernels fails.
+"""
+
+from __future__ import annotations
+
+import hashlib
+import os
+import shutil
+import subprocess
+import sys
+import tempfile
+import threading
+import time
+from pathlib import Path
+
+CSRC = Path(__file__).resolve().parent.parent / "csrc"
+ARCH = "gfx950"
+FLAGS = [
+    f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-ffp-contract=off", "-Wno-pass-failed",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-shared", "-fPIC",
+]
+CORE_SOURCES = ("core.hip", "gemm.hip")
+ATTENTION_SOURCES = ("attention.hip",)
+HEADERS = ("common.h",)
+
+
+class BuildError(RuntimeError):
+    pass
+
+
+def _hash(sources, defines) -> str:
+    digest = hashlib.sha256()
+    for name in tuple(sources) + HEADERS:
+        digest.update(name.encode())
+        digest.update((CSRC / name).read_bytes())
+    digest.update(" ".join(FLAGS + list(defines)).encode())
+    return digest.hexdigest()[:12]
+
+
+def _writable(folder: Path) -> bool:
+    try:
+        folder.mkdir(parents=True, exist_ok=True)
+        handle, probe = tempfile.mkstemp(prefix=".probe-", dir=folder)
+        os.close(handle)
+        os.unlink(probe)
+        return True
+    except OSError:
+        return False
+
+
+def lib_dirs() -> list[Path]:
+    """Folders searched for built libraries, the first writable one is built into."""
+    in_tree = Path(__file__).resolve().parent.parent / "_lib"
+    user = Path(tempfile.gettempdir()) / f"lockstep_amd-{os.getuid()}" / "_lib"
+    return [in_tree, user]
+
+
+def _target(kind: str, sources, defines) -> str:
+    return f"liblockstep_{kind}-{_hash(sources, defines)}.so"
+
+
+def find_hipcc() -> str:
+    for candidate in (os.environ.get("HIPCC"), shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
+        if candidate and Path(candidate).is_file():
+            return candidate
+    raise BuildError("hipcc was not found (looked at $HIPCC, PATH and /opt/rocm/bin); the kernels cannot be built")
+
+
+def _compile(kind: str, sources, defines, out: Path) -> None:
+    cmd = [find_hipcc(), *FLAGS, *defines, "-o", str(out), *[str(CSRC / s) for s in sources]]
+    started = time.time()
+    print(f"[lockstep_amd] compiling {kind} kernels for {ARCH} -> {out.name}", file=sys.stderr, flush=True)
+    done = threading.Event()
+
+    def ticker():
+        while not done.wait(15.0):
+            print(f"[lockstep_amd] ... still compiling {kind} ({time.time() - started:.0f} s)",
+                  file=sys.stderr, flush=True)
+
+    thread = threading.Thread(target=ticker, daemon=True)
+    thread.start()
+    try:
+        env = dict(os.environ)
+        env.setdefault("TMPDIR", tempfile.gettempdir())
+        if not env.get("HOME") or not os.access(env["HOME"], os.W_OK):
+            env["HOME"] = tempfile.gettempdir()
+        proc = subprocess.run(cmd, capture_output=True, text=True, env=env)
+    finally:
+        done.set()
+    if proc.returncode != 0:
+        raise BuildError(f"hipcc failed for {kind}:\n{' '.join(cmd)}\n{proc.stderr[-4000:]}")
+    print(f"[lockstep_amd] compiled {kind} in {time.time() - started:.1f} s", file=sys.stderr, flush=True)
+
+
+def build(kind: str, sources, defines=(), force: bool = False) -> Path:
+    """Return the path of the library, compiling it if it is missing (or ``force``)."""
+    name = _target(kind, sources, defines)
+    if not force:
+        for folder in lib_dirs():
+            if (folder / name).is_file():
+                return folder / name
+    for folder in lib_dirs():
+        if not _writable(folder):
+            continue
+        for stale in folder.glob(f"liblockstep_{kind}-*.so"):
+            if stale.name != name:
+                try:
+                    stale.unlink()
+                except OSError:
+                    pass
+        tmp = folder / f".{name}.{os.getpid()}.{threading.get_ident()}.tmp"
+        try:
+            _compile(kind, sources, list(defines), tmp)
+            os.replace(tmp, folder / name)
+        finally:
+            if tmp.exists():
+                tmp.unlink()
+        return folder / name
+    raise BuildError(f"no writable folder for built kernels among {[str(d) for d in lib_dirs()]}")
+
+
+def build_core(force: bool = False) -> Path:
+    return build("core", CORE_SOURCES, (), force)
+
+
+def build_attention(head_dim: int, force: bool = False) -> Path:
+    if head_dim % 16 or not 16 <= head_dim <= 256:
+        raise BuildError(
+            f"head size {head_dim} is not supported: the attention kernels take multiples of 16 from 16 to 256")
+    return build(f"attention{head_dim}", ATTENTION_SOURCES, (f"-DLS_HEAD_DIM={head_dim}",), force)
+
+
+DEFAULT_HEAD_DIMS = (16, 32, 48, 64, 80, 128, 256)
+
+
+def build_all(head_dims=DEFAULT_HEAD_DIMS, force: bool = True) -> list[Path]:
+    """Compile the core library and the attention library of each head size,
+    a few at a time."""
+    jobs = [lambda: build_core(force)] + [lambda d=d: build_attention(d, force) for d in head_dims]
+    results: list = [None] * len(jobs)
+    errors: list = []
+
+    def run(i):
+        try:
+            results[i] = jobs[i]()
+        except Exception as exc:  # noqa: BLE001 - reported below
+            errors.append(exc)
+
+    width = max(1, min(4, (os.cpu_count() or 2) // 2))
+    for lo in range(0, len(jobs), width):
+        threads = [threading.Thread(target=run, args=(i,)) for i in range(lo, min(lo + width, len(jobs)))]
+        for t in threads:
+            t.start()
+        for t in threads:
+            t.join()
+    if errors:
+        raise errors[0]
+    return results

@@ -1,0 +1,251 @@
+"""Python face of the HIP kernels: shape checks on the host, then the launch.
+
+Every wrapper verifies what the kernel and its grid assume (device, dtype,
+contiguity of rows, matching sizes) before it launches, because a kernel that
+reads out of bounds can take the whole GPU down.  Launches go to torch's
+current stream, so they order with torch's own copies and can be captured in
+a HIP graph.  There is no fallback path: if the library cannot be loaded the
+constructor raises.
+"""
+
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_float, c_int, c_long, c_void_p
+
+import torch
+
+from . import build as _build
+
+DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1}
+STORE, STORE_F32, ADD_F32 = 0, 1, 2
+MAX_HEAD_DIM = 256
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def _ptr(t) -> c_void_p:
+    return c_void_p(t.data_ptr()) if t is not None else c_void_p(0)
+
+
+def _stream() -> c_void_p:
+    return c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _need(cond: bool, message: str) -> None:
+    if not cond:
+        raise KernelError(message)
+
+
+def _rows_ok(t: torch.Tensor, name: str) -> None:
+    _need(t.is_cuda, f"{name} must live on the GPU")
+    _need(t.dim() == 2 and t.stride(1) == 1, f"{name} must be 2-D with contiguous rows, got shape "
+          f"{tuple(t.shape)} strides {t.stride()}")
+
+
+class Kernels:
+    """The loaded libraries.  One instance per process (see ``kernels()``)."""
+
+    def __init__(self):
+        self.core_path = _build.build_core()
+        self.core = ctypes.CDLL(str(self.core_path))
+        self.core.ls_last_error.restype = ctypes.c_char_p
+        self._attention: dict[int, ctypes.CDLL] = {}
+        self.attention_paths: dict[int, str] = {}
+
+    # -- helpers ------------------------------------------------------------
+    @staticmethod
+    def _check(lib, code: int) -> None:
+        if code != 0:
+            raise KernelError(lib.ls_last_error().decode())
+
+    def attention_lib(self, head_dim: int):
+        lib = self._attention.get(head_dim)
+        if lib is None:
+            path = _build.build_attention(head_dim)
+            lib = ctypes.CDLL(str(path))
+            lib.ls_last_error.restype = ctypes.c_char_p
+            _need(lib.ls_attn_head_dim() == head_dim, f"{path} was built for another head size")
+            self._attention[head_dim] = lib
+            self.attention_paths[head_dim] = str(path)
+        return lib
+
+    def attention_geometry(self, head_dim: int) -> tuple[int, int]:
+        """(keys per tile, keys per split) of the attention kernels."""
+        lib = self.attention_lib(head_dim)
+        return lib.ls_attn_tile_keys(), lib.ls_attn_split_keys()
+
+    # -- matrix product -------------------------------------------------------
+    def gemm(self, x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, epilogue: int = STORE) -> None:
+        """``out (+)= x @ w.T``; ``x [M,K]``, ``w [N,K]`` contiguous, ``out [M,N]``."""
+        _rows_ok(x, "gemm x"); _rows_ok(w, "gemm w"); _rows_ok(out, "gemm out")
+        _need(x.dtype in DTYPE_CODE and w.dtype == x.dtype, f"gemm operands must share float32 or bfloat16, got "
+              f"{x.dtype} and {w.dtype}")
+        m, k = x.shape
+        n = w.shape[0]
+        _need(w.shape[1] == k and w.is_contiguous(), f"gemm w must be contiguous [N,{k}], got {tuple(w.shape)}")
+        _need(tuple(out.shape) == (m, n), f"gemm out must be [{m},{n}], got {tuple(out.shape)}")
+        want = x.dtype if epilogue == STORE else torch.float32
+        _need(out.dtype == want, f"gemm out dtype {out.dtype} does not fit epilogue {epilogue}")
+        if m == 0:
+            return
+        code = self.core.ls_gemm(c_int(DTYPE_CODE[x.dtype]), c_int(epilogue), _ptr(x), _ptr(w), _ptr(out),
+                                 c_int(m), c_int(n), c_int(k), c_long(x.stride(0)), c_long(out.stride(0)), _stream())
+        self._check(self.core, code)
+
+    # -- rows -------------------------------------------------------------------
+    def embed(self, tokens: torch.Tensor, table: torch.Tensor, out: torch.Tensor) -> None:
+        _need(tokens.is_cuda and tokens.dtype == torch.int32 and tokens.dim() == 1 and tokens.is_contiguous(),
+              "embed tokens must be a contiguous int32 vector on the GPU")
+        _rows_ok(table, "embed table"); _rows_ok(out, "embed out")
+        _need(table.is_contiguous() and table.dtype in DTYPE_CODE, "embed table must be contiguous float32/bfloat16")
+        _need(out.dtype == torch.float32 and out.shape == (tokens.shape[0], table.shape[1]),
+              f"embed out must be float32 [{tokens.shape[0]},{table.shape[1]}]")
+        if tokens.shape[0] == 0:
+            return
+        code = self.core.ls_embed(c_int(DTYPE_CODE[table.dtype]), _ptr(tokens), _ptr(table), _ptr(out),
+                                  c_int(tokens.shape[0]), c_int(table.shape[0]), c_int(table.shape[1]),
+                                  c_long(out.stride(0)), _stream())
+        self._check(self.core, code)
+
+    def rmsnorm(self, x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, eps: float,
+                rows: torch.Tensor | None = None) -> None:
+        """Rows of float ``x`` (all, or those listed in ``rows``) normalised into ``out``."""
+        _rows_ok(x, "rmsnorm x"); _rows_ok(out, "rmsnorm out")
+        _need(x.dtype == torch.float32, "rmsnorm reads the float32 residual stream")
+        _need(weight.is_cuda and weight.dtype == torch.float32 and weight.is_contiguous()
+              and weight.shape == (x.shape[1],), f"rmsnorm weight must be float32 [{x.shape[1]}]")
+        _need(out.dtype in DTYPE_CODE and out.shape[1] == x.shape[1], "rmsnorm out has the wrong width or dtype")
+        n = out.shape[0]
+        if rows is not None:
+            _need(rows.is_cuda and rows.dtype == torch.int32 and rows.is_contiguous() and rows.shape == (n,),
+                  f"rmsnorm rows must be int32 [{n}]")
+        else:
+            _need(x.shape[0] == n, "rmsnorm out must have as many rows as x")
+        if n == 0:
+            return
+        code = self.core.ls_rmsnorm(c_int(DTYPE_CODE[out.dtype]), _ptr(x), _ptr(weight), _ptr(out), _ptr(rows),
+                                    c_int(n), c_int(x.shape[1]), c_long(x.stride(0)), c_long(out.stride(0)),
+                                    c_float(eps), _stream())
+        self._check(self.core, code)
+
+    def swiglu(self, gate_up: torch.Tensor, out: torch.Tensor) -> None:
+        _rows_ok(gate_up, "swiglu input"); _rows_ok(out, "swiglu out")
+        rows, inter = out.shape
+        _need(gate_up.shape == (rows, 2 * inter) and gate_up.dtype == out.dtype and out.dtype in DTYPE_CODE,
+              f"swiglu input must be [{rows},{2 * inter}] of the output's dtype")
+        if rows == 0:
+            return
+        code = self.core.ls_swiglu(c_int(DTYPE_CODE[out.dtype]), _ptr(gate_up), _ptr(out), c_int(rows), c_int(inter),
+                                   c_long(gate_up.stride(0)), c_long(out.stride(0)), _stream())
+        self._check(self.core, code)
+
+    def argmax(self, logits: torch.Tensor, out: torch.Tensor) -> None:
+        _rows_ok(logits, "argmax logits")
+        _need(logits.dtype == torch.float32, "argmax reads float32 logits")
+        _need(out.is_cuda and out.dtype == torch.int32 and out.is_contiguous() and out.shape == (logits.shape[0],),
+              f"argmax out must be int32 [{logits.shape[0]}]")
+        if logits.shape[0] == 0:
+            return
+        code = self.core.ls_argmax(_ptr(logits), _ptr(out), c_int(logits.shape[0]), c_int(logits.shape[1]),
+                                   c_long(logits.stride(0)), _stream())
+        self._check(self.core, code)
+
+    # -- attention ----------------------------------------------------------------
+    def qk_rope_kv(self, qkv: torch.Tensor, n_tokens: int, nq: int, nkv: int, d: int, q_weight, k_weight,
+                   eps: float, cos, sin, rot: int, tok_seq, tok_pos, seqs, max_pos: int, table, k_pages,
+                   v_pages, page_size: int, write_kv: bool) -> None:
+        """Per-head norm, rotation and cache write on the fused projection ``qkv``.
+
+        ``max_pos`` is the largest position in the step (checked against the
+        tables); ``table`` is the group's block table ``[rows, stride]``.
+        """
+        _rows_ok(qkv, "qkv")
+        _need(qkv.dtype in DTYPE_CODE and qkv.shape[0] >= n_tokens, "qkv has too few rows or a wrong dtype")
+        heads = nq + 2 * nkv if write_kv else nq
+        _need(qkv.shape[1] >= heads * d, f"qkv rows hold {qkv.shape[1]} values, {heads} heads of {d} are needed")
+        _need(d <= MAX_HEAD_DIM, f"head size {d} exceeds the supported maximum {MAX_HEAD_DIM}")
+        for name, w in (("q norm weight", q_weight), ("k norm weight", k_weight)):
+            if w is not None:
+                _need(w.is_cuda and w.dtype == torch.float32 and w.is_contiguous() and w.shape == (d,),
+                      f"{name} must be float32 [{d}]")
+        positions = 0
+        if cos is not None:
+            _need(sin is not None and cos.shape == sin.shape and cos.dim() == 2 and cos.shape[1] * 2 == rot
+                  and cos.dtype == torch.float32 and cos.is_contiguous() and sin.is_contiguous() and cos.is_cuda,
+                  "rotation tables must be float32 [positions, rotary_dim/2]")
+            positions = cos.shape[0]
+            _need(max_pos < positions, f"position {max_pos} is beyond the rotation tables ({positions})")
+        for name, t in (("tok_seq", tok_seq), ("tok_pos", tok_pos)):
+            _need(t.is_cuda and t.dtype == torch.int32 and t.is_contiguous() and t.numel() >= n_tokens,
+                  f"{name} must be int32 with at least {n_tokens} entries")
+        if write_kv:
+            _need(table is not None and table.is_cuda and table.dtype == torch.int32 and table.dim() == 2
+                  and table.is_contiguous(), "block table must be a contiguous int32 matrix")
+            _need(max_pos // page_size < table.shape[1],
+                  f"position {max_pos} needs page {max_pos // page_size}, the block table has {table.shape[1]} columns")
+            for name, pages in (("key pages", k_pages), ("value pages", v_pages)):
+                _need(pages.is_cuda and pages.dtype == qkv.dtype and pages.is_contiguous() and pages.dim() == 4,
+                      f"{name} must be contiguous 4-D of the compute dtype")
+            _need(k_pages.shape[1:] == (nkv, page_size, d) and v_pages.shape[1:] == (nkv, d, page_size)
+                  and k_pages.shape[0] == v_pages.shape[0],
+                  f"cache pages do not have the layout [pages,{nkv},{page_size},{d}] / [pages,{nkv},{d},{page_size}]")
+        if n_tokens == 0:
+            return
+        code = self.core.ls_qk_rope_kv(
+            c_int(DTYPE_CODE[qkv.dtype]), _ptr(qkv), c_long(qkv.stride(0)), c_int(n_tokens), c_int(nq), c_int(nkv),
+            c_int(d), _ptr(q_weight), _ptr(k_weight), c_float(eps), _ptr(cos), _ptr(sin), c_int(rot),
+            c_int(positions), _ptr(tok_seq), _ptr(tok_pos), _ptr(seqs), _ptr(table),
+            c_int(table.shape[1] if table is not None else 0), _ptr(k_pages), _ptr(v_pages), c_int(page_size),
+            c_int(1 if write_kv else 0), _stream())
+        self._check(self.core, code)
+
+    def attention(self, q: torch.Tensor, nq: int, nkv: int, d: int, k_pages, v_pages, page_size: int, table,
+                  seqs, items, n_items: int, out: torch.Tensor, part_acc, part_ml, scale: float,
+                  window: int) -> None:
+        """Launch the attention kernel over ``n_items`` work items (see attention.hip)."""
+        lib = self.attention_lib(d)
+        _rows_ok(q, "attention q"); _rows_ok(out, "attention out")
+        _need(q.dtype in DTYPE_CODE and out.dtype == q.dtype, "attention q/out dtype")
+        _need(nq % nkv == 0, f"{nq} query heads are not a multiple of {nkv} kv heads")
+        _need(q.shape[1] >= nq * d and out.shape[1] >= nq * d, "attention q/out rows are too short")
+        _need(k_pages.dtype == q.dtype and v_pages.dtype == q.dtype and k_pages.is_contiguous()
+              and v_pages.is_contiguous() and k_pages.shape[1:] == (nkv, page_size, d)
+              and v_pages.shape[1:] == (nkv, d, page_size), "attention cache pages have the wrong layout or dtype")
+        _need(table.dtype == torch.int32 and table.dim() == 2 and table.is_contiguous(), "attention block table")
+        _need(items.dtype == torch.int32 and items.is_contiguous() and items.numel() >= 8 * n_items,
+              "attention items must hold 8 int32 each")
+        if n_items == 0:
+            return
+        code = lib.ls_attention(
+            c_int(DTYPE_CODE[q.dtype]), _ptr(q), c_long(q.stride(0)), _ptr(k_pages), _ptr(v_pages), c_int(nkv),
+            c_int(page_size), _ptr(table), c_int(table.shape[1]), _ptr(seqs), _ptr(items), c_int(n_items),
+            _ptr(out), c_long(out.stride(0)), _ptr(part_acc), _ptr(part_ml), c_int(nq // nkv), c_float(scale),
+            c_int(window), _stream())
+        self._check(lib, code)
+
+    def attention_combine(self, d: int, seqs, items, n_items: int, nq: int, nkv: int, part_acc, part_ml,
+                          out: torch.Tensor) -> None:
+        lib = self.attention_lib(d)
+        _rows_ok(out, "combine out")
+        _need(out.dtype in DTYPE_CODE and out.shape[1] >= nq * d, "combine out rows are too short")
+        _need(items.dtype == torch.int32 and items.is_contiguous() and items.numel() >= 4 * n_items,
+              "combine items must hold 4 int32 each")
+        if n_items == 0:
+            return
+        code = lib.ls_attention_combine(c_int(DTYPE_CODE[out.dtype]), _ptr(seqs), _ptr(items), c_int(n_items),
+                                        c_int(nkv), _ptr(part_acc), _ptr(part_ml), _ptr(out),
+                                        c_long(out.stride(0)), c_int(nq // nkv), _stream())
+        self._check(lib, code)
+
+
+_INSTANCE: Kernels | None = None
+
+
+def kernels() -> Kernels:
+    global _INSTANCE
+    if _INSTANCE is None:
+        _INSTANCE = Kernels()
+    return _INSTANCE

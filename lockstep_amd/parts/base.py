@@ -1,0 +1,173 @@
+"""Interfaces of the parts a layer is put together from.
+
+A *part* is built from a ``PartSpec`` (its kind and constants) and a tensor
+name prefix.  It states which tensors it needs (``weight_specs``), takes them
+(``load``) and runs on a packed batch (``forward``).  Parts never look at the
+model configuration and never know which model they are in; every size and
+constant arrives through the spec.
+
+Kinds of part and what each must provide:
+
+``Norm``            ``forward(ctx, x, out, rows=None)``: normalise rows of the
+                    32-bit residual stream ``x [T, H]`` into ``out`` in the
+                    compute dtype; ``rows`` optionally selects input rows.
+``PositionEncoding`` tables or constants a mixer applies at absolute
+                    positions; ``ensure(max_position)`` grows them.
+``Mixer``           ``cache_spec()`` says what it keeps between steps (paged
+                    keys/values, a fixed-size state, or nothing) and
+                    ``forward(ctx, run, x, out, accumulate)`` mixes tokens of
+                    the same request: it reads what earlier steps left in the
+                    cache, writes this step's part of it, and writes (or adds)
+                    ``[T, H]`` into the 32-bit ``out``.
+``FeedForward``     ``forward(ctx, x, out, accumulate)``: token-wise.
+``Arrangement``     owns one layer's parts and the order they run in.
+
+Rule for every ``forward``: a row's result depends on rows of the same
+request at earlier positions only, and not on how the request's tokens were
+cut into steps or on what else is in the batch.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Any, Callable, Optional, Sequence
+
+from ..config.base import PartSpec
+
+
+@dataclass(frozen=True)
+class WeightSpec:
+    """A tensor a part expects in the checkpoint.
+
+    ``kind``: ``matrix`` tensors are operands of matrix products and live in
+    the compute dtype; ``vector`` tensors (norm weights, biases) are used in
+    32-bit arithmetic and are kept in float32; ``int`` tensors are integer
+    tables kept as int32.  ``init`` steers the random-weights mode: ``normal``
+    is N(0, std), ``norm`` is 1 + N(0, norm_std), ``zeros`` is 0.
+    """
+
+    name: str
+    shape: tuple[int, ...]
+    kind: str = "matrix"
+    init: str = "normal"
+    optional: bool = False
+
+
+@dataclass(frozen=True)
+class PagedKVSpec:
+    """Keys and values of every token, or of the last ``window`` tokens."""
+
+    num_kv_heads: int
+    head_dim: int
+    window: Optional[int] = None
+
+
+@dataclass(frozen=True)
+class StateSpec:
+    """A state of fixed size per request (``shape`` elements of float32)."""
+
+    shape: tuple[int, ...]
+
+
+class Part:
+    """Base of all parts."""
+
+    kind: str = ""
+
+    def __init__(self, spec: PartSpec, prefix: str = ""):
+        self.spec = spec
+        self.prefix = prefix
+
+    @classmethod
+    def weight_specs(cls, spec: PartSpec, prefix: str) -> list[WeightSpec]:
+        return []
+
+    def load(self, weights, rt) -> None:
+        """Take tensors from ``weights`` (name -> CPU tensor) onto ``rt.device``."""
+
+    @staticmethod
+    def join(prefix: str, name: str) -> str:
+        return f"{prefix}.{name}" if prefix else name
+
+
+class Norm(Part):
+    def forward(self, ctx, x, out, rows=None) -> None:
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    def ensure(self, max_position: int, rt) -> None:
+        """Make tables cover positions ``< max_position``."""
+
+
+class Mixer(Part):
+    def cache_spec(self):
+        """``PagedKVSpec``, ``StateSpec`` or ``None``."""
+        return None
+
+    def prepare(self, ctx) -> None:
+        """Declare per-step needs (work lists) before the step's metadata is uploaded."""
+
+    def forward(self, ctx, run, x, out, accumulate: bool) -> None:
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, ctx, x, out, accumulate: bool) -> None:
+        raise NotImplementedError
+
+
+class Arrangement(Part):
+    """One layer: builds its parts from a ``LayerSpec`` and runs them."""
+
+    def __init__(self, layer_spec, build_part: Callable[..., Part]):
+        super().__init__(layer_spec.arrangement, layer_spec.prefix)
+        self.layer_spec = layer_spec
+
+    def parts(self) -> Sequence[Part]:
+        raise NotImplementedError
+
+    @property
+    def mixer(self) -> Mixer:
+        raise NotImplementedError
+
+    def forward(self, ctx, run, h) -> None:
+        raise NotImplementedError
+
+
+# --------------------------------------------------------------------------
+# registry of part kinds
+# --------------------------------------------------------------------------
+
+_PARTS: dict[str, type] = {}
+
+
+def register_part(kind: str):
+    """Class decorator: make a part class buildable from ``PartSpec(kind, ...)``."""
+
+    def decorate(cls):
+        known = _PARTS.get(kind)
+        if known is not None and known is not cls:
+            raise ValueError(f"part kind {kind!r} is already registered by {known.__name__}")
+        cls.kind = kind
+        _PARTS[kind] = cls
+        return cls
+
+    return decorate
+
+
+def unregister_part(kind: str) -> None:
+    _PARTS.pop(kind, None)
+
+
+def part_class(kind: str) -> type:
+    try:
+        return _PARTS[kind]
+    except KeyError:
+        raise KeyError(
+            f"no part of kind {kind!r} is registered; known: {', '.join(sorted(_PARTS))}"
+        ) from None
+
+
+def build_part(spec: PartSpec, prefix: str = "", **extra: Any) -> Part:
+    return part_class(spec.kind)(spec, prefix, **extra)

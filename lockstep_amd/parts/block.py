@@ -1,0 +1,59 @@
+"""Arrangements: how a layer's parts are wired around the residual stream."""
+
+from __future__ import annotations
+
+from .base import Arrangement, build_part, register_part
+
+
+@register_part("prenorm_residual")
+class PreNormResidual(Arrangement):
+    """``h += mixer(norm_1(h)); h += feed_forward(norm_2(h))``
+    (reference engine/model/qwen3.py:324-370).
+
+    Parameters name the parts' tensor prefixes below the layer's prefix:
+    ``mixer_prefix``, ``feed_forward_prefix``, ``mixer_norm_name``,
+    ``feed_forward_norm_name``.
+    """
+
+    def __init__(self, layer_spec, prefix: str = ""):
+        super().__init__(layer_spec, build_part)
+        p = layer_spec.arrangement.params
+        base = layer_spec.prefix
+        self.mixer_norm = build_part(layer_spec.mixer_norm, self.join(base, p["mixer_norm_name"]))
+        self._mixer = build_part(layer_spec.mixer, self.join(base, p["mixer_prefix"]))
+        self.feed_forward_norm = build_part(layer_spec.feed_forward_norm,
+                                            self.join(base, p["feed_forward_norm_name"]))
+        self.feed_forward = build_part(layer_spec.feed_forward, self.join(base, p["feed_forward_prefix"]))
+
+    @classmethod
+    def weight_specs(cls, layer_spec, prefix: str = ""):
+        from .base import part_class
+
+        p = layer_spec.arrangement.params
+        base = layer_spec.prefix
+        out = []
+        for spec, name in ((layer_spec.mixer_norm, p["mixer_norm_name"]),
+                           (layer_spec.mixer, p["mixer_prefix"]),
+                           (layer_spec.feed_forward_norm, p["feed_forward_norm_name"]),
+                           (layer_spec.feed_forward, p["feed_forward_prefix"])):
+            out += part_class(spec.kind).weight_specs(spec, cls.join(base, name))
+        return out
+
+    def parts(self):
+        return (self.mixer_norm, self._mixer, self.feed_forward_norm, self.feed_forward)
+
+    @property
+    def mixer(self):
+        return self._mixer
+
+    def load(self, weights, rt) -> None:
+        for part in self.parts():
+            part.load(weights, rt)
+
+    def forward(self, ctx, run, h) -> None:
+        rt = ctx.rt
+        x = ctx.buf("block.normed", (ctx.n_tokens, h.shape[1]), rt.dtype)
+        self.mixer_norm.forward(ctx, h, x)
+        self._mixer.forward(ctx, run, x, h, accumulate=True)
+        self.feed_forward_norm.forward(ctx, h, x)
+        self.feed_forward.forward(ctx, x, h, accumulate=True)

@@ -1,0 +1,364 @@
+"""Each HIP kernel alone against a plain PyTorch reference of the same
+operation, at sizes other than the engine's, in float32 and in bfloat16."""
+
+from __future__ import annotations
+
+import math
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+def K():
+    from lockstep_amd.ops import kernels
+
+    return kernels()
+
+
+def rel_err(got: torch.Tensor, want: torch.Tensor) -> float:
+    got, want = got.double().cpu(), want.double().cpu()
+    return float((got - want).abs().max() / want.abs().max().clamp_min(1e-30))
+
+
+TOL = {torch.float32: 2e-5, torch.bfloat16: 1.5e-2}
+
+
+# -- matrix product ------------------------------------------------------------
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("m,n,k", [(1, 16, 32), (1, 1000, 96), (5, 48, 200), (16, 100, 64), (17, 33, 72),
+                                   (64, 256, 1024), (65, 130, 260), (37, 3072, 1024), (200, 96, 4100),
+                                   (130, 1000, 8), (3, 40, 12)])
+def test_gemm_matches_linear(dtype, m, n, k):
+    from lockstep_amd.ops import STORE, STORE_F32, ADD_F32
+
+    g = torch.Generator().manual_seed(m * 1000 + n + k)
+    x = torch.randn(m, k, generator=g).to(dtype)
+    w = torch.randn(n, k, generator=g).to(dtype)
+    want = x.double() @ w.double().T
+    xd, wd = x.cuda(), w.cuda()
+    out = torch.empty(m, n, dtype=dtype, device="cuda")
+    K().gemm(xd, wd, out, STORE)
+    assert rel_err(out, want) < TOL[dtype]
+    out32 = torch.empty(m, n, dtype=torch.float32, device="cuda")
+    K().gemm(xd, wd, out32, STORE_F32)
+    assert rel_err(out32, want) < (2e-5 if dtype is torch.float32 else 2e-5 + 0)  # float accumulate: tight in both
+    base = torch.randn(m, n, generator=g)
+    acc = base.cuda()
+    K().gemm(xd, wd, acc, ADD_F32)
+    assert rel_err(acc, base.double() + want) < 2e-5
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_gemm_row_does_not_depend_on_the_batch(dtype):
+    """Row i alone, in a 16-row batch, in a 64-row batch and in a 300-row batch:
+    same bits (the skinny and the tiled kernel share one summation order)."""
+    from lockstep_amd.ops import STORE_F32
+
+    g = torch.Generator().manual_seed(7)
+    for k, n in ((1024, 272), (3072, 96), (200, 130), (5000, 64)):
+        x = torch.randn(300, k, generator=g).to(dtype).cuda()
+        w = torch.randn(n, k, generator=g).to(dtype).cuda()
+        full = torch.empty(300, n, dtype=torch.float32, device="cuda")
+        K().gemm(x, w, full, STORE_F32)
+        for rows in (1, 16, 17, 64, 65, 128):
+            part = torch.empty(rows, n, dtype=torch.float32, device="cuda")
+            K().gemm(x[:rows], w, part, STORE_F32)
+            assert torch.equal(part, full[:rows]), f"rows={rows} k={k} n={n}"
+        for i in (0, 1, 17, 63, 64, 299):
+            one = torch.empty(1, n, dtype=torch.float32, device="cuda")
+            K().gemm(x[i:i + 1], w, one, STORE_F32)
+            assert torch.equal(one[0], full[i]), f"row {i} k={k} n={n}"
+
+
+def test_gemm_refuses_mismatched_operands():
+    from lockstep_amd.ops import KernelError
+
+    x = torch.zeros(4, 32, device="cuda")
+    w = torch.zeros(8, 48, device="cuda")
+    with pytest.raises(KernelError):
+        K().gemm(x, w, torch.zeros(4, 8, device="cuda"))
+
+
+# -- norm --------------------------------------------------------------------------
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("rows,width,eps", [(1, 64, 1e-6), (7, 96, 1e-5), (48, 1024, 1e-6), (3, 5120, 1e-6),
+                                            (5, 100, 1e-3)])
+def test_rmsnorm_matches_formula(dtype, rows, width, eps):
+    g = torch.Generator().manual_seed(width)
+    x = torch.randn(rows, width, generator=g) * 3
+    w = 1 + 0.1 * torch.randn(width, generator=g)
+    want = x.double() * torch.rsqrt(x.double().pow(2).mean(-1, keepdim=True) + eps) * w.double()
+    out = torch.empty(rows, width, dtype=dtype, device="cuda")
+    K().rmsnorm(x.cuda(), w.cuda(), out, eps)
+    assert rel_err(out, want) < (1e-6 if dtype is torch.float32 else 5e-3)
+    lib = torch.nn.functional.rms_norm(x, (width,), w, eps)
+    assert rel_err(out, lib) < (1e-6 if dtype is torch.float32 else 5e-3)
+    # selected rows, and a row alone gives the same bits as in the batch
+    idx = torch.tensor([rows - 1, 0], dtype=torch.int32, device="cuda")
+    sel = torch.empty(2, width, dtype=dtype, device="cuda")
+    K().rmsnorm(x.cuda(), w.cuda(), sel, eps, idx)
+    assert torch.equal(sel[0], out[rows - 1]) and torch.equal(sel[1], out[0])
+
+
+# -- SwiGLU, embedding, arg-max --------------------------------------------------------
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_swiglu_matches_silu_times_up(dtype):
+    g = torch.Generator().manual_seed(1)
+    gu = (torch.randn(7, 2 * 300, generator=g) * 2).to(dtype)
+    want = torch.nn.functional.silu(gu[:, :300].double()) * gu[:, 300:].double()
+    out = torch.empty(7, 300, dtype=dtype, device="cuda")
+    K().swiglu(gu.cuda(), out)
+    assert rel_err(out, want) < (1e-6 if dtype is torch.float32 else 5e-3)
+    zero = torch.zeros(2, 64, dtype=dtype, device="cuda")
+    out0 = torch.ones(2, 32, dtype=dtype, device="cuda")
+    K().swiglu(zero, out0)
+    assert torch.count_nonzero(out0) == 0
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_embedding_gathers_rows(dtype):
+    table = torch.randn(1000, 96).to(dtype)
+    ids = torch.tensor([0, 999, 5, 5, 731], dtype=torch.int32)
+    out = torch.empty(5, 96, dtype=torch.float32, device="cuda")
+    K().embed(ids.cuda(), table.cuda(), out)
+    assert torch.equal(out.cpu(), table[ids.long()].float())
+
+
+def test_argmax_takes_the_lowest_index_among_maxima():
+    x = torch.randn(6, 151936)
+    x[1, 77] = x[1, 150000] = 50.0
+    x[2, :] = 1.0
+    x[3, 151935] = 60.0
+    out = torch.empty(6, dtype=torch.int32, device="cuda")
+    K().argmax(x.cuda(), out)
+    want = [int(torch.nonzero(r == r.max())[0]) for r in x]
+    assert out.cpu().tolist() == want
+    assert want[1] == 77 and want[2] == 0 and want[3] == 151935
+    small = torch.tensor([[1.0, 5.0, 5.0, 5.0, 2.0]]).cuda()
+    one = torch.empty(1, dtype=torch.int32, device="cuda")
+    K().argmax(small, one)
+    assert one.item() == 1
+
+
+# -- norm + rotation + cache write, attention ---------------------------------------------
+
+def naive_attention(q, k, v, q_start, scale, window=None):
+    """q [Tq,nq,d], k,v [Tk,nkv,d] in float64; explicit max-subtract softmax."""
+    tq, nq, d = q.shape
+    tk, nkv, _ = k.shape
+    g = nq // nkv
+    k = k.repeat_interleave(g, dim=1)
+    v = v.repeat_interleave(g, dim=1)
+    s = torch.einsum("qhd,khd->hqk", q, k) * scale
+    qp = torch.arange(q_start, q_start + tq)[:, None]
+    kp = torch.arange(tk)[None, :]
+    hidden = kp > qp
+    if window:
+        hidden = hidden | (qp - kp >= window)
+    s = s.masked_fill(hidden[None], float("-inf"))
+    m = s.max(-1, keepdim=True).values
+    e = (s - m).exp()
+    return torch.einsum("hqk,khd->qhd", e / e.sum(-1, keepdim=True), v)
+
+
+class PagedCase:
+    """Lay keys and values into pages through the engine's own write kernel."""
+
+    def __init__(self, dtype, nq, nkv, d, page_size, n_tokens, shuffle_seed=None, extra_pages=3):
+        self.dtype, self.nq, self.nkv, self.d, self.ps = dtype, nq, nkv, d, page_size
+        n_pages = -(-n_tokens // page_size)
+        order = list(range(n_pages + extra_pages))
+        if shuffle_seed is not None:
+            g = torch.Generator().manual_seed(shuffle_seed)
+            order = torch.randperm(n_pages + extra_pages, generator=g).tolist()
+        self.table = torch.full((2, n_pages + 1), -1, dtype=torch.int32)
+        self.table[1, :n_pages] = torch.tensor(order[:n_pages], dtype=torch.int32)
+        self.table = self.table.cuda()
+        total = n_pages + extra_pages
+        self.k_pages = torch.full((total, nkv, page_size, d), float("nan"), dtype=dtype, device="cuda")
+        self.v_pages = torch.full((total, nkv, d, page_size), float("nan"), dtype=dtype, device="cuda")
+
+    def seqs(self, q_start, q_len):
+        return torch.tensor([0, q_len, q_start, q_start + q_len, 1, 0, 0, 0], dtype=torch.int32).cuda()
+
+    def write(self, qkv, q_start, q_norm=None, k_norm=None, eps=1e-6, cos=None, sin=None, rot=0):
+        t = qkv.shape[0]
+        tok_seq = torch.zeros(t, dtype=torch.int32, device="cuda")
+        tok_pos = torch.arange(q_start, q_start + t, dtype=torch.int32, device="cuda")
+        K().qk_rope_kv(qkv, t, self.nq, self.nkv, self.d, q_norm, k_norm, eps, cos, sin, rot, tok_seq, tok_pos,
+                       self.seqs(q_start, t), q_start + t - 1, self.table, self.k_pages, self.v_pages, self.ps, True)
+
+    def attend(self, qkv, q_start, scale, window=0, force_split=None):
+        from lockstep_amd.ops import kernels
+
+        t = qkv.shape[0]
+        tile, split = kernels().attention_geometry(self.d)
+        g = self.nq // self.nkv
+        rows = t * g
+        kv_len = q_start + t
+        lo = max(0, q_start - window + 1) if window else 0
+        split_lo = lo // split
+        n_splits = (kv_len - 1) // split + 1 - split_lo
+        use_split = (rows <= 64 and n_splits > 1) if force_split is None else force_split
+        items, combine, part_rows = [], [], 0
+        if use_split:
+            part_rows = self.nkv * rows * n_splits
+            for b in range(-(-rows // 64)):
+                for s in range(split_lo, split_lo + n_splits):
+                    items += [0, b, s, s + 1, 0, n_splits, split_lo, 0]
+                combine += [0, b, 0, n_splits]
+        else:
+            for b in range(-(-rows // 64)):
+                first = q_start + (b * 64) // g
+                last = q_start + min(b * 64 + 63, rows - 1) // g
+                begin = (max(0, first - window + 1) // split) if window else 0
+                items += [0, b, begin, last // split + 1, -1, 0, 0, 0]
+        items_t = torch.tensor(items, dtype=torch.int32).cuda()
+        out = torch.full((t, self.nq * self.d), float("nan"), dtype=self.dtype, device="cuda")
+        part_acc = torch.full((max(part_rows, 1), self.d), float("nan"), dtype=torch.float32, device="cuda")
+        part_ml = torch.full((max(part_rows, 1), 2), float("nan"), dtype=torch.float32, device="cuda")
+        K().attention(qkv, self.nq, self.nkv, self.d, self.k_pages, self.v_pages, self.ps, self.table,
+                      self.seqs(q_start, t), items_t, len(items) // 8, out, part_acc, part_ml, scale, window)
+        if combine:
+            comb = torch.tensor(combine, dtype=torch.int32).cuda()
+            K().attention_combine(self.d, self.seqs(q_start, t), comb, len(combine) // 4, self.nq, self.nkv,
+                                  part_acc, part_ml, out)
+        return out.view(t, self.nq, self.d)
+
+
+def rand_qkv(t, nq, nkv, d, dtype, seed, sharp=None):
+    g = torch.Generator().manual_seed(seed)
+    qkv = torch.randn(t, (nq + 2 * nkv) * d, generator=g)
+    if sharp is not None:
+        # make one far key stand out for the last query: a fault that drops it shows
+        key_pos, = sharp
+        q = qkv[:, : nq * d].view(t, nq, d)
+        k = qkv[:, nq * d:(nq + nkv) * d].view(t, nkv, d)
+        k[key_pos] = q[-1].view(nkv, nq // nkv, d)[:, 0] * 2.0
+    return qkv.to(dtype)
+
+
+def split_qkv(qkv, nq, nkv, d):
+    t = qkv.shape[0]
+    q = qkv[:, : nq * d].reshape(t, nq, d)
+    k = qkv[:, nq * d:(nq + nkv) * d].reshape(t, nkv, d)
+    v = qkv[:, (nq + nkv) * d:].reshape(t, nkv, d)
+    return q, k, v
+
+
+ATT_TOL = {torch.float32: 2e-5, torch.bfloat16: 2e-2}
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nq,nkv,d,ps", [(16, 8, 128, 16), (4, 4, 16, 8), (8, 1, 64, 32), (6, 2, 48, 16),
+                                         (32, 4, 80, 64), (2, 2, 256, 128)])
+@pytest.mark.parametrize("kv_len", [1, 5, 64, 129, 257, 600])
+def test_prefill_attention_matches_naive(dtype, nq, nkv, d, ps, kv_len):
+    qkv = rand_qkv(kv_len, nq, nkv, d, dtype, seed=kv_len + d)
+    case = PagedCase(dtype, nq, nkv, d, ps, kv_len, shuffle_seed=3)
+    dev = qkv.cuda()
+    case.write(dev, 0)
+    out = case.attend(dev, 0, d ** -0.5)
+    q, k, v = split_qkv(qkv.double(), nq, nkv, d)
+    want = naive_attention(q, k, v, 0, d ** -0.5)
+    assert not torch.isnan(out).any()
+    assert rel_err(out, want) < ATT_TOL[dtype]
+    if kv_len == 1:
+        assert torch.equal(out.cpu().float()[0], v.float()[0].repeat_interleave(nq // nkv, dim=0))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nq,nkv,d,ps", [(16, 8, 128, 16), (6, 3, 32, 8), (8, 1, 64, 16)])
+def test_attention_row_is_the_same_alone_in_a_portion_and_in_the_whole_prompt(dtype, nq, nkv, d, ps):
+    """A query row alone (decode, split mode), in a portion, and in a whole prefill: same bits;
+    also under a shuffled block table."""
+    kv_len = 700
+    qkv = rand_qkv(kv_len, nq, nkv, d, dtype, seed=11, sharp=(3,)).cuda()
+    whole = PagedCase(dtype, nq, nkv, d, ps, kv_len)
+    whole.write(qkv, 0)
+    full = whole.attend(qkv, 0, d ** -0.5)
+    shuffled = PagedCase(dtype, nq, nkv, d, ps, kv_len, shuffle_seed=99)
+    shuffled.write(qkv, 0)
+    assert torch.equal(shuffled.attend(qkv, 0, d ** -0.5), full)
+    for p in (0, 1, 15, 16, 17, 127, 128, 255, 256, 257, 511, 512, 699):
+        alone = whole.attend(qkv[p:p + 1], p, d ** -0.5)
+        assert torch.equal(alone[0], full[p]), f"row {p} alone"
+        both = whole.attend(qkv[p:p + 1], p, d ** -0.5, force_split=False)
+        assert torch.equal(both[0], full[p]), f"row {p} alone, direct"
+    for lo, hi in ((250, 262), (0, 3), (500, 700), (255, 257), (690, 700)):
+        part = whole.attend(qkv[lo:hi], lo, d ** -0.5)
+        assert torch.equal(part, full[lo:hi]), f"portion {lo}:{hi}"
+        part = whole.attend(qkv[lo:hi], lo, d ** -0.5, force_split=True)
+        assert torch.equal(part, full[lo:hi]), f"portion {lo}:{hi} split"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("window", [1, 7, 128, 300])
+def test_attention_window(dtype, window):
+    nq, nkv, d, ps, kv_len = 4, 2, 32, 16, 520
+    qkv = rand_qkv(kv_len, nq, nkv, d, dtype, seed=window, sharp=(kv_len - window,))
+    case = PagedCase(dtype, nq, nkv, d, ps, kv_len)
+    dev = qkv.cuda()
+    case.write(dev, 0)
+    out = case.attend(dev, 0, d ** -0.5, window=window)
+    q, k, v = split_qkv(qkv.double(), nq, nkv, d)
+    want = naive_attention(q, k, v, 0, d ** -0.5, window=window)
+    assert rel_err(out, want) < ATT_TOL[dtype]
+    # pages behind the window may be gone: mark them released and decode the last rows
+    for p in (kv_len - 1, 300, 130):
+        first_needed = max(0, p - window + 1) // ps
+        saved = case.table.clone()
+        case.table[1, :first_needed] = -1
+        alone = case.attend(dev[p:p + 1], p, d ** -0.5, window=window)
+        case.table.copy_(saved)
+        assert torch.equal(alone[0], out[p]), f"row {p}"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_norm_rotation_and_cache_write(dtype):
+    nq, nkv, d, ps, t, start = 6, 3, 32, 8, 21, 5
+    rot = 32
+    g = torch.Generator().manual_seed(5)
+    qkv = torch.randn(t, (nq + 2 * nkv) * d, generator=g).to(dtype)
+    qw = 1 + 0.2 * torch.randn(d, generator=g)
+    kw = 1 + 0.2 * torch.randn(d, generator=g)
+    eps, theta = 1e-5, 1e4
+    pos = torch.arange(64, dtype=torch.float64)
+    inv = 1.0 / (theta ** (torch.arange(0, rot // 2, dtype=torch.float64) * 2 / rot))
+    ang = pos[:, None] * inv[None, :]
+    cos, sin = ang.cos().float(), ang.sin().float()
+    case = PagedCase(dtype, nq, nkv, d, ps, start + t, shuffle_seed=1)
+    dev = qkv.clone().cuda()
+    case.write(dev, start, qw.cuda(), kw.cuda(), eps, cos.cuda(), sin.cuda(), rot)
+
+    q, k, v = split_qkv(qkv.double(), nq, nkv, d)
+
+    def norm_rope(x, w):
+        x = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * w.double()
+        c = cos[start:start + t].double()[:, None, :]
+        s = sin[start:start + t].double()[:, None, :]
+        lo, hi = x[..., : rot // 2], x[..., rot // 2:rot]
+        return torch.cat([lo * c - hi * s, hi * c + lo * s, x[..., rot:]], dim=-1)
+
+    tol = 1e-6 if dtype is torch.float32 else 8e-3
+    got_q = dev[:, : nq * d].view(t, nq, d)
+    assert rel_err(got_q, norm_rope(q, qw)) < tol
+    table = case.table[1].cpu()
+    want_k = norm_rope(k, kw)
+    for i in range(t):
+        p = start + i
+        page, slot = int(table[p // ps]), p % ps
+        assert rel_err(case.k_pages[page, :, slot, :], want_k[i]) < tol
+        assert torch.equal(case.v_pages[page, :, :, slot].cpu().double(), v[i])
+    # position 0 leaves a head untouched by the rotation (cos 1, sin 0)
+    case0 = PagedCase(dtype, nq, nkv, d, ps, 1)
+    one = qkv[:1].clone().cuda()
+    case0.write(one, 0, None, None, eps, cos.cuda(), sin.cuda(), rot)
+    assert torch.equal(one.cpu(), qkv[:1])
