@@ -176,6 +176,7 @@ class CacheManager:
             for unit, spec in self.state_units.items():
                 self.state[unit] = torch.zeros((max_requests, *spec.shape), dtype=torch.float32, device=device)
 
+        self.ever_shared = False     # set once a page got a second holder (prefix sharing)
         self._free_slots = list(range(max_requests))
         heapq.heapify(self._free_slots)
         self.requests: dict[Hashable, _Request] = {}
@@ -302,6 +303,7 @@ class CacheManager:
         group, mine = self.groups[0], request.groups[0]
         if mine.pages:
             raise CacheAuditError("adopt expects a request without pages")
+        self.ever_shared = True
         for logical, page in enumerate(pages):
             group.pool.retain(page)
             mine.pages.append(page)
@@ -310,6 +312,7 @@ class CacheManager:
             group.dirty_rows.add(request.slot)
 
     def pin(self, page: int) -> None:
+        self.ever_shared = True
         group = self.groups[0]
         group.pool.retain(page)
         group.pinned[page] = group.pinned.get(page, 0) + 1

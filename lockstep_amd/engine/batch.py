@@ -42,11 +42,14 @@ class AttentionPlan:
 
 
 class Workspace:
-    """Named device buffers that grow on demand and persist between steps."""
+    """Named device buffers that grow on demand and persist between steps.
+    ``version`` counts reallocations: a captured graph that points into these
+    buffers is stale once it changes."""
 
     def __init__(self, device):
         self.device = device
         self._buffers: dict[tuple, torch.Tensor] = {}
+        self.version = 0
 
     def get(self, name: str, shape, dtype) -> torch.Tensor:
         shape = tuple(int(s) for s in shape)
@@ -57,13 +60,21 @@ class Workspace:
             grow = max(rows, 2 * have.shape[0] if have is not None else rows)
             have = torch.empty((grow, *inner), dtype=dtype, device=self.device)
             self._buffers[key] = have
+            self.version += 1
         return have[:rows]
 
 
 class StepContext:
     """Everything a part may read about the step (see module docstring)."""
 
-    def __init__(self, rt, cache, workspace: Workspace, entries: Sequence[StepEntry]):
+    def __init__(self, rt, cache, workspace: Workspace, entries: Sequence[StepEntry], fixed_shape: bool = False):
+        """``fixed_shape`` lays the attention work out so that its size depends
+        only on the number of requests and on a bucket of the longest context:
+        every request gets one work item per split up to the bucket (items past a
+        request's own length produce empty partial results, which the combine
+        step skips, so the bits do not change).  A captured graph of the step
+        then stays valid from one decode step to the next."""
+        self.fixed_shape = fixed_shape
         self.rt = rt
         self.cache = cache
         self.workspace = workspace
@@ -104,13 +115,21 @@ class StepContext:
         tile, split = self.rt.kernels.attention_geometry(head_dim)
         items, combine = [], []
         part_rows = 0
+        bucket = 0
+        if self.fixed_shape:
+            longest = max((int(k) - 1) // split + 1 for k in self.kv_len)
+            bucket = 1
+            while bucket < longest:
+                bucket = bucket * 2 if bucket < 8 else bucket + 8
         for i in range(self.n_seqs):
             q_len, q_start, kv_len = int(self.q_len[i]), int(self.q_start[i]), int(self.kv_len[i])
             rows = q_len * group_size
             lo_valid = max(0, q_start - window + 1) if window > 0 else 0
             split_lo = lo_valid // split
             n_splits = (kv_len - 1) // split + 1 - split_lo
-            if rows <= 64 and n_splits > 1:
+            if self.fixed_shape:
+                split_lo, n_splits = 0, bucket
+            if rows <= 64 and (n_splits > 1 or self.fixed_shape):
                 base = part_rows
                 part_rows += nkv * rows * n_splits
                 for s in range(split_lo, split_lo + n_splits):
@@ -160,6 +179,11 @@ class StepContext:
             self._device_plans[key] = AttentionPlan(d_items, n_items, d_combine if n_combine else None,
                                                     n_combine, part_acc, part_ml)
         self._uploaded = True
+
+    def plan_signature(self) -> tuple:
+        """Sizes of the work lists: equal signatures mean an equal device layout."""
+        return tuple((key, self._plans[key][2], self._plans[key][3], self._plans[key][4])
+                     for key in self._plan_specs) + (self.n_tokens, self.n_want)
 
     def attention_plan(self, group_size: int, nkv: int, head_dim: int, window: int) -> AttentionPlan:
         return self._device_plans[(group_size, nkv, head_dim, window)]

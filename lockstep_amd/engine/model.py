@@ -10,6 +10,7 @@ row; here the final norm and the head run on the wanted rows only).
 
 from __future__ import annotations
 
+import os
 from pathlib import Path
 from typing import Sequence
 
@@ -58,6 +59,10 @@ class Model:
             if not 0 <= run.layer < len(self.layers):
                 raise ValueError(f"the schedule names layer {run.layer}, the model has {len(self.layers)}")
         self.workspace = Workspace(rt.device)
+        self.use_graphs = os.environ.get("LOCKSTEP_NO_GRAPHS", "") in ("", "0")
+        self._graphs: dict[tuple, tuple] = {}
+        self._graph_safe = all(layer.mixer.graph_safe for layer in self.layers)
+        self.graph_replays = 0
 
     # -- weights --------------------------------------------------------------
     def load(self, weights) -> "Model":
@@ -106,30 +111,71 @@ class Model:
             start = cache.length(e.request)
             cache.reserve(e.request, start + len(e.tokens))
             for gi, group in enumerate(cache.groups):
-                if group.pinned or max(group.pool.holders, default=0) > 1:
+                if cache.ever_shared:
                     for logical in range(start // cache.page_size, -(-(start + len(e.tokens)) // cache.page_size)):
                         cache.assert_exclusive(e.request, gi, logical)
         cache.sync_tables()
 
-        ctx = StepContext(self.rt, cache, self.workspace, entries)
+        # A step of single decoded tokens has a shape that repeats from step to
+        # step: run it from a captured HIP graph.
+        graphed = (self.use_graphs and self._graph_safe
+                   and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries))
+        ctx = StepContext(self.rt, cache, self.workspace, entries, fixed_shape=graphed)
         for layer in self.layers:
             layer.mixer.prepare(ctx)
+            position = getattr(layer.mixer, "position", None)
+            if position is not None:
+                position.ensure(ctx.max_position + 1, self.rt)
         ctx.upload()
+        logits = self._forward_graphed(ctx, cache) if graphed else self._forward(ctx)
+        for e, end in zip(entries, ctx.kv_len):
+            cache.commit(e.request, int(end))
+        return logits
 
+    def _forward(self, ctx: StepContext, logits=None):
+        """Launch the step's kernels on the current stream."""
         h = ctx.buf("residual", (ctx.n_tokens, self.spec.hidden_size), torch.float32)
         self.embedding.forward(ctx, ctx.token_ids, h)
         for run in self.schedule:
             self.layers[run.layer].forward(ctx, run, h)
-
-        logits = None
         if ctx.n_want:
             x = ctx.buf("final.normed", (ctx.n_want, self.spec.hidden_size), self.rt.dtype)
             self.final_norm.forward(ctx, h, x, rows=ctx.want_rows)
-            logits = torch.empty((ctx.n_want, vocab), dtype=torch.float32, device=self.rt.device)
+            if logits is None:
+                logits = torch.empty((ctx.n_want, self.spec.vocab_size), dtype=torch.float32, device=self.rt.device)
             self.head.forward(ctx, x, logits)
-        for e, end in zip(entries, ctx.kv_len):
-            cache.commit(e.request, int(end))
         return logits
+
+    def _graph_key(self, ctx: StepContext, cache) -> tuple:
+        tables = tuple(id(layer.mixer.position.cos) for layer in self.layers
+                       if getattr(layer.mixer, "position", None) is not None)
+        return (ctx.n_seqs, ctx.plan_signature(), self.workspace.version, id(cache), tables)
+
+    def _forward_graphed(self, ctx: StepContext, cache):
+        """Replay the captured graph of this step shape, capturing it first if
+        needed.  The graph reads the step's metadata, the block tables and the
+        cache through fixed addresses; only their contents change between
+        replays.  The first step of a shape runs eagerly (that also sizes the
+        workspace), then the same launches are recorded for the steps to come."""
+        key = self._graph_key(ctx, cache)
+        held = self._graphs.get(key)
+        if held is not None:
+            graph, logits = held
+            graph.replay()
+            self.graph_replays += 1
+            return logits.clone()
+        logits = torch.empty((ctx.n_want, self.spec.vocab_size), dtype=torch.float32, device=self.rt.device)
+        self._forward(ctx, logits)
+        key = self._graph_key(ctx, cache)          # the eager run may have grown the workspace
+        if len(self._graphs) >= 32:
+            self._graphs.clear()
+        result = logits.clone()
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            self._forward(ctx, logits)
+        self._graphs[key] = (graph, logits)
+        return result
 
 
 def load_model(model_dir, dtype="bfloat16", device="cuda:0") -> Model:

@@ -29,6 +29,8 @@ class Attention(Mixer):
     position-encoding ``PartSpec``), ``window`` (keys visible to a query,
     None for all), ``bias`` (must be False), ``scale`` (score multiplier)."""
 
+    graph_safe = True
+
     def __init__(self, spec: PartSpec, prefix: str = ""):
         super().__init__(spec, prefix)
         p = spec.params
@@ -97,7 +99,6 @@ class Attention(Mixer):
         t = ctx.n_tokens
         nq, nkv, d = self.nq, self.nkv, self.d
         group, key_pages, value_pages = ctx.cache.unit_pages(run.cache)
-        self.position.ensure(ctx.max_position + 1, rt)
         width = (nq + 2 * nkv) * d
         qkv = ctx.buf("attention.qkv", (t, width), rt.dtype)
         if run.writes_cache:

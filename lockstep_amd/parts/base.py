@@ -101,6 +101,12 @@ class PositionEncoding(Part):
 
 
 class Mixer(Part):
+    #: True if ``forward`` only launches kernels that read the step's metadata
+    #: from device memory, so a decode step may be captured in a HIP graph and
+    #: replayed with new metadata.  A mixer that reads sizes or slots on the
+    #: host while it runs must leave this False.
+    graph_safe = False
+
     def cache_spec(self):
         """``PagedKVSpec``, ``StateSpec`` or ``None``."""
         return None

@@ -76,3 +76,149 @@ def test_cuttings_give_the_same_bits(plain_logits, dtype, name, page_size):
             pytest.fail(f"{name} {dtype} {label}: first differing position {bad}, "
                         f"max diff {float((got - whole).abs().max()):.3e}")
     cache.audit()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name,page_size", [("A", 16), ("B", 8)])
+def test_mixed_batches_with_reused_pages(plain_logits, dtype, name, page_size):
+    """Up to four live requests, portions of some beside decoded tokens of
+    others, with so few pages that freed ones are used again (and poisoned in
+    between): every request's logits equal its whole run bit for bit and the
+    plain implementation within tolerance."""
+    from helpers import make_mixed_trace, max_live_tokens, replay_in_process
+    from plain.qwen3_plain import PlainModel
+
+    folder, _ = plain_logits[name]
+    plain = PlainModel(folder)
+    vocab = plain.cfg["vocab_size"]
+    lengths = [70, 45, 33, 90, 21, 64, 130, 17]
+    requests = {f"q{i}": random_tokens(n, vocab, seed=500 + i) for i, n in enumerate(lengths)}
+    steps = make_mixed_trace(requests, seed=3)
+    assert max(len(s["entries"]) for s in steps) == 4
+    assert any(len(e["tokens"]) == 2 for s in steps for e in s["entries"])
+    model = load(folder, dtype)
+    num_pages = max_live_tokens(steps, round_to=page_size) // page_size
+    cache = model.make_cache(num_pages=num_pages, page_size=page_size, max_requests=4,
+                             max_tokens_per_request=max(lengths), poison_on_free=True)
+    got = replay_in_process(model, cache, steps)
+    assert cache.groups[0].pool.taken_total > 2 * num_pages, "pages were not used again"
+    assert cache.free_pages == [num_pages]
+    roomy = model.make_cache(num_pages=64, page_size=page_size, poison_on_free=True)
+    for rid, tokens in requests.items():
+        whole = feed(model, roomy, rid, tokens, [])
+        roomy.close(rid)
+        assert torch.equal(got[rid], whole), f"{rid}: mixed run differs from the whole run"
+        assert rel_err(got[rid], plain.logits(tokens)) < TOL[dtype], rid
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_long_decoding_matches_plain(plain_logits, dtype):
+    """Forty tokens at once, then three hundred one by one (past two splits of the keys)."""
+    from plain.qwen3_plain import PlainModel
+
+    folder, _ = plain_logits["B"]
+    plain = PlainModel(folder)
+    tokens = random_tokens(340, plain.cfg["vocab_size"], seed=77)
+    model = load(folder, dtype)
+    cache = model.make_cache(num_pages=48, page_size=8, poison_on_free=True)
+    got = feed(model, cache, "long", tokens, [40] + [1] * 300)
+    err = rel_err(got, plain.logits(tokens))
+    print(f"long decode {dtype}: rel err {err:.3e}")
+    assert err < TOL[dtype]
+
+
+@pytest.mark.parametrize("name,page_size", [("A", 16), ("B", 8)])
+def test_greedy_generation_through_the_entry_points(plain_logits, name, page_size):
+    """Scheduler, LLM and generate_greedy against whole-sequence recomputation
+    by the plain implementation (float32 for token equality); in bfloat16 the
+    tokens do not depend on how the scheduler cuts the work."""
+    from lockstep_amd import LLM, FixedChunkPolicy, Request, generate_greedy
+    from plain.qwen3_plain import PlainModel
+
+    folder, _ = plain_logits[name]
+    plain = PlainModel(folder)
+    vocab = plain.cfg["vocab_size"]
+    prompts = [random_tokens(n, vocab, seed=900 + n) for n in ((7, 13, 32) if name == "A" else (1, 9, 17, 40, 64))]
+    new = 16 if name == "A" else 24
+    want = {f"r{i}": plain.generate_greedy(p, new) for i, p in enumerate(prompts)}
+
+    def requests():
+        return [Request(uid=f"r{i}", prompt=p, max_new_tokens=new) for i, p in enumerate(prompts)]
+
+    llm = LLM(folder, dtype="float32", num_pages=64, page_size=page_size, audit=True)
+    assert llm.generate(requests()) == want
+    assert llm.generate(requests(), policy=FixedChunkPolicy(12)) == want
+    ids, step_logits = generate_greedy(llm.model, prompts[-1], new)
+    assert ids == want[f"r{len(prompts) - 1}"] and len(step_logits) == new
+    assert rel_err(step_logits[0].cpu(), plain.logits(prompts[-1])[-1]) < FP32_TOL
+
+    half = LLM(folder, dtype="bfloat16", num_pages=64, page_size=page_size, audit=True)
+    base = half.generate(requests())
+    assert half.generate(requests(), policy=FixedChunkPolicy(12)) == base
+    half.options["max_batched_tokens"] = 20
+    assert half.generate(requests(), policy=FixedChunkPolicy(5)) == base
+    assert half.generate(requests()[1:2]) == {"r1": base["r1"]}
+
+
+def test_sampled_generation_follows_the_plain_sampler(plain_logits):
+    """Configuration B's workload: prompts of 1, 9, 17, 40 and 64 tokens as
+    mixed portions of 12 beside decoded tokens, temperature 0.8 with a seed per
+    request, 24 new tokens each; the sampled tokens equal what the plain
+    implementation's sampler draws from the plain logits (float32)."""
+    from lockstep_amd import LLM, FixedChunkPolicy, Request
+    from plain import qwen3_plain as P
+
+    folder, _ = plain_logits["B"]
+    plain = P.PlainModel(folder)
+    prompts = [random_tokens(n, plain.cfg["vocab_size"], seed=3000 + n) for n in (1, 9, 17, 40, 64)]
+    llm = LLM(folder, dtype="float32", num_pages=96, page_size=8, audit=True)
+    got = llm.generate([Request(uid=f"s{i}", prompt=p, seed=40 + i, max_new_tokens=24, temperature=0.8, top_p=0.95)
+                        for i, p in enumerate(prompts)], policy=FixedChunkPolicy(12))
+    for i, p in enumerate(prompts):
+        context, want = list(p), []
+        for _ in range(24):
+            token = P.top_p(plain.logits(context)[-1].float(), 40 + i, f"s{i}", len(context) - 1, 0.95, 0.8)
+            want.append(token); context.append(token)
+        assert got[f"s{i}"] == want, f"s{i}"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_decode_steps_from_a_captured_graph_equal_eager_steps(plain_logits, dtype):
+    """Decode steps are replayed from a HIP graph.  Replay it many times, with
+    eager work (another request's prompt, a step of another batch size) between
+    the replays, and compare every replay with the eager result."""
+    from lockstep_amd.engine.batch import StepEntry
+
+    folder, seqs = plain_logits["B"]
+    tokens, _ = seqs[333]
+    other = random_tokens(50, 1000, seed=4)
+    eager = load(folder, dtype)
+    eager.use_graphs = False
+    cache_e = eager.make_cache(num_pages=128, page_size=8)
+    want_a = feed(eager, cache_e, "a", tokens, [200] + [1] * 133)
+    want_b = feed(eager, cache_e, "b", other, [20] + [1] * 30)
+
+    model = load(folder, dtype)
+    assert model.use_graphs
+    cache = model.make_cache(num_pages=128, page_size=8)
+    cache.open("a"); cache.open("b")
+    got_a = [model.step(cache, [StepEntry("a", tokens[:200], list(range(200)))]).cpu()]
+    got_b = [model.step(cache, [StepEntry("b", other[:20], list(range(20)))]).cpu()]
+    pos_b = 20
+    for i in range(200, 333):
+        if i % 4 == 0 and pos_b < 50:                # a two-request decode step: another graph shape
+            both = model.step(cache, [StepEntry("a", tokens[i:i + 1], [0]), StepEntry("b", other[pos_b:pos_b + 1], [0])])
+            got_a.append(both[:1].cpu()); got_b.append(both[1:].cpu())
+            pos_b += 1
+        else:
+            got_a.append(model.step(cache, [StepEntry("a", tokens[i:i + 1], [0])]).cpu())
+        if i % 50 == 0:                                # eager work in between
+            cache.open(f"x{i}")
+            model.step(cache, [StepEntry(f"x{i}", other[:13], [12])])
+            cache.close(f"x{i}")
+    while pos_b < 50:
+        got_b.append(model.step(cache, [StepEntry("b", other[pos_b:pos_b + 1], [0])]).cpu())
+        pos_b += 1
+    assert model.graph_replays > 100
+    assert torch.equal(torch.cat(got_a), want_a)
+    assert torch.equal(torch.cat(got_b), want_b)

@@ -1,0 +1,342 @@
+"""Each part of a layer alone against the plain implementation, a toy mixer
+with state of its own registered from here, and schedules that name a layer
+twice or share a cache -- all without touching the framework's files."""
+
+from __future__ import annotations
+
+import json
+from dataclasses import dataclass
+
+import pytest
+import torch
+
+from helpers import FP32_TOL, feed, random_tokens, rel_err
+from plain import qwen3_plain as P
+
+pytestmark = pytest.mark.gpu
+
+
+class Harness:
+    """A runtime, a cache for one unit spec and a way to make step contexts."""
+
+    def __init__(self, dtype="float32", unit_specs=(None,), page_size=8, num_pages=32):
+        from lockstep_amd.cache import CacheManager
+        from lockstep_amd.engine.batch import Workspace
+        from lockstep_amd.engine.runtime import Runtime
+
+        self.rt = Runtime("cuda:0", dtype)
+        self.cache = CacheManager(list(unit_specs), page_size, num_pages, 4, num_pages * page_size,
+                                  torch_dtype=self.rt.dtype, device=self.rt.device, poison_on_free=True)
+        self.workspace = Workspace(self.rt.device)
+
+    def context(self, lengths: dict, mixers=()):
+        from lockstep_amd.engine.batch import StepContext, StepEntry
+
+        entries = []
+        for rid, n in lengths.items():
+            if rid not in self.cache.requests:
+                self.cache.open(rid)
+            self.cache.reserve(rid, self.cache.length(rid) + n)
+            entries.append(StepEntry(rid, [0] * n, []))
+        self.cache.sync_tables()
+        ctx = StepContext(self.rt, self.cache, self.workspace, entries)
+        for m in mixers:
+            m.prepare(ctx)
+        ctx.upload()
+        return ctx
+
+    def commit(self, ctx):
+        for e, end in zip(ctx.entries, ctx.kv_len):
+            self.cache.commit(e.request, int(end))
+
+
+def store(tensors):
+    from lockstep_amd.weights.store import DictWeightStore
+
+    return DictWeightStore(tensors)
+
+
+@dataclass
+class Run:
+    layer: int = 0
+    cache: int = 0
+    writes_cache: bool = True
+
+
+def test_norm_part_alone():
+    from lockstep_amd.config import PartSpec
+    from lockstep_amd.parts import build_part
+
+    h = Harness()
+    part = build_part(PartSpec("rmsnorm", {"size": 72, "eps": 1e-3}), "n")
+    w = 1 + 0.3 * torch.randn(72)
+    part.load(store({"n.weight": w}), h.rt)
+    x = torch.randn(5, 72) * 2
+    ctx = h.context({"a": 5})
+    out = torch.empty(5, 72, device="cuda")
+    part.forward(ctx, x.cuda(), out)
+    assert rel_err(out.cpu(), P.rmsnorm(x.double(), w.double(), 1e-3)) < 1e-6
+
+
+def test_position_part_alone_matches_the_plain_tables():
+    from lockstep_amd.config import PartSpec
+    from lockstep_amd.parts import build_part
+
+    h = Harness()
+    part = build_part(PartSpec("rope_half", {"rotary_dim": 48, "theta": 5e5}))
+    part.ensure(700, h.rt)
+    cos, sin = P.rope_tables(48, 5e5, torch.arange(700))
+    assert torch.equal(part.cos[:700].cpu(), cos.float()) and torch.equal(part.sin[:700].cpu(), sin.float())
+    part.ensure(5000, h.rt)                                     # grows on demand
+    assert part.cos.shape[0] >= 5000 and torch.equal(part.cos[:700].cpu(), cos.float())
+
+
+@pytest.mark.parametrize("dtype,tol", [("float32", 2e-5), ("bfloat16", 3e-2)])
+def test_attention_part_alone_in_portions(dtype, tol):
+    from lockstep_amd.config import PartSpec
+    from lockstep_amd.parts import build_part
+
+    hidden, nq, nkv, d = 40, 6, 2, 48
+    spec = PartSpec("attention", {
+        "hidden_size": hidden, "num_heads": nq, "num_kv_heads": nkv, "head_dim": d,
+        "qk_norm": PartSpec("rmsnorm", {"size": d, "eps": 1e-5}),
+        "position": PartSpec("rope_half", {"rotary_dim": d, "theta": 1e4}),
+        "window": None, "bias": False, "scale": d ** -0.5})
+    part = build_part(spec, "att")
+    g = torch.Generator().manual_seed(0)
+    w = {"att.q_proj.weight": torch.randn(nq * d, hidden, generator=g) * 0.3,
+         "att.k_proj.weight": torch.randn(nkv * d, hidden, generator=g) * 0.3,
+         "att.v_proj.weight": torch.randn(nkv * d, hidden, generator=g) * 0.3,
+         "att.o_proj.weight": torch.randn(hidden, nq * d, generator=g) * 0.3,
+         "att.q_norm.weight": 1 + 0.2 * torch.randn(d, generator=g),
+         "att.k_norm.weight": 1 + 0.2 * torch.randn(d, generator=g)}
+    w = {k: v.to(torch.bfloat16) for k, v in w.items()}
+    h = Harness(dtype, unit_specs=(part.cache_spec(),))
+    part.load(store(w), h.rt)
+    x = (torch.randn(29, hidden, generator=g)).to(torch.bfloat16)
+    cfg = {"num_attention_heads": nq, "num_key_value_heads": nkv, "head_dim": d, "rms_norm_eps": 1e-5,
+           "rope_theta": 1e4}
+    w64 = {k.replace("att.", "L."): v.double() for k, v in w.items()}
+    want = P.attention_block(cfg, w64, "L", x.double(), torch.arange(29))
+    got = []
+    pos = 0
+    for n in (11, 2, 15, 1):
+        ctx = h.context({"a": n}, mixers=[part])
+        out = torch.zeros(n, hidden, device="cuda")
+        part.forward(ctx, Run(), x[pos:pos + n].to(h.rt.dtype).cuda(), out, accumulate=False)
+        h.commit(ctx)
+        got.append(out.cpu())
+        pos += n
+    assert rel_err(torch.cat(got), want) < tol
+
+
+def test_feed_forward_part_and_block_alone():
+    from lockstep_amd.config import LayerSpec, PartSpec
+    from lockstep_amd.parts import build_part, part_class
+
+    hidden, inter = 56, 136
+    g = torch.Generator().manual_seed(1)
+    w = {"L.mlp.gate_proj.weight": torch.randn(inter, hidden, generator=g) * 0.3,
+         "L.mlp.up_proj.weight": torch.randn(inter, hidden, generator=g) * 0.3,
+         "L.mlp.down_proj.weight": torch.randn(hidden, inter, generator=g) * 0.3}
+    ff_spec = PartSpec("gated_mlp", {"hidden_size": hidden, "intermediate_size": inter, "activation": "silu"})
+    h = Harness()
+    part = build_part(ff_spec, "L.mlp")
+    part.load(store(w), h.rt)
+    x = torch.randn(9, hidden, generator=g)
+    ctx = h.context({"a": 9})
+    out = torch.ones(9, hidden, device="cuda")
+    part.forward(ctx, x.cuda(), out, accumulate=True)
+    want = 1 + P.mlp_block({k: v.double() for k, v in w.items()}, "L.mlp", x.double())
+    assert rel_err(out.cpu(), want) < 2e-5
+    with pytest.raises(ValueError):
+        build_part(PartSpec("gated_mlp", {"hidden_size": 8, "intermediate_size": 8, "activation": "gelu"}), "m")
+
+    # the whole arrangement: h += attn(norm(h)); h += mlp(norm(h))
+    nq, nkv, d = 4, 4, 16
+    norm = PartSpec("rmsnorm", {"size": hidden, "eps": 1e-6})
+    layer = LayerSpec(
+        prefix="L",
+        arrangement=PartSpec("prenorm_residual", {"mixer_prefix": "self_attn", "feed_forward_prefix": "mlp",
+                                                  "mixer_norm_name": "input_layernorm",
+                                                  "feed_forward_norm_name": "post_attention_layernorm"}),
+        mixer=PartSpec("attention", {"hidden_size": hidden, "num_heads": nq, "num_kv_heads": nkv, "head_dim": d,
+                                     "qk_norm": None, "position": PartSpec("no_position", {}), "window": None,
+                                     "bias": False, "scale": 0.2}),
+        feed_forward=ff_spec, mixer_norm=norm, feed_forward_norm=norm)
+    block = part_class("prenorm_residual")(layer)
+    w.update({"L.input_layernorm.weight": 1 + 0.1 * torch.randn(hidden, generator=g),
+              "L.post_attention_layernorm.weight": 1 + 0.1 * torch.randn(hidden, generator=g),
+              "L.self_attn.q_proj.weight": torch.randn(nq * d, hidden, generator=g) * 0.3,
+              "L.self_attn.k_proj.weight": torch.randn(nkv * d, hidden, generator=g) * 0.3,
+              "L.self_attn.v_proj.weight": torch.randn(nkv * d, hidden, generator=g) * 0.3,
+              "L.self_attn.o_proj.weight": torch.randn(hidden, nq * d, generator=g) * 0.3})
+    names = sorted(s.name for s in part_class("prenorm_residual").weight_specs(layer))
+    assert names == sorted(w)                                  # without q/k norm there are no norm tensors
+    h2 = Harness(unit_specs=(block.mixer.cache_spec(),))
+    block.load(store(w), h2.rt)
+    hs = torch.randn(13, hidden, generator=g)
+    ctx = h2.context({"a": 13}, mixers=[block.mixer])
+    dev = hs.clone().cuda()
+    block.forward(ctx, Run(), dev)
+    w64 = {k: v.double() for k, v in w.items()}
+    x64 = hs.double()
+    normed = P.rmsnorm(x64, w64["L.input_layernorm.weight"], 1e-6)
+    q = P.linear(normed, w64["L.self_attn.q_proj.weight"]).view(13, nq, d)
+    k = P.linear(normed, w64["L.self_attn.k_proj.weight"]).view(13, nkv, d)
+    v = P.linear(normed, w64["L.self_attn.v_proj.weight"]).view(13, nkv, d)
+    # plain attention without rotation; its score scale is 1/sqrt(d), the part's is 0.2: rescale q
+    attn = P.causal_attention(q * (0.2 * d ** 0.5), k, v)
+    x64 = x64 + P.linear(attn.reshape(13, nq * d), w64["L.self_attn.o_proj.weight"])
+    x64 = x64 + P.mlp_block(w64, "L.mlp", P.rmsnorm(x64, w64["L.post_attention_layernorm.weight"], 1e-6))
+    assert rel_err(dev.cpu(), x64) < 2e-5
+
+
+# ---------------------------------------------------------------------------
+# a toy architecture defined here: a mixer with a state of fixed size, a
+# layer that runs twice, and a layer that reads another layer's keys/values
+# ---------------------------------------------------------------------------
+
+def _register_toy():
+    from lockstep_amd.config import (LayerSpec, ModelConfig, ModelSpec, PartSpec, ScheduleEntry,
+                                     register_architecture)
+    from lockstep_amd.parts import Mixer, StateSpec, WeightSpec, register_part
+
+    @register_part("toy_decay")
+    class DecayMixer(Mixer):
+        """s_t = decay * s_{t-1} + x_t (one state vector per request); out_t = s_t @ W^T."""
+
+        def __init__(self, spec, prefix=""):
+            super().__init__(spec, prefix)
+            self.hidden, self.decay = int(spec["hidden_size"]), float(spec["decay"])
+
+        @classmethod
+        def weight_specs(cls, spec, prefix):
+            return [WeightSpec(f"{prefix}.mix.weight", (int(spec["hidden_size"]),) * 2)]
+
+        def cache_spec(self):
+            return StateSpec((self.hidden,))
+
+        def load(self, weights, rt):
+            self.w = rt.vector(weights.get(f"{self.prefix}.mix.weight"))
+
+        def forward(self, ctx, run, x, out, accumulate):
+            state = ctx.cache.unit_state(run.cache)
+            for i in range(ctx.n_seqs):
+                lo, n, slot = int(ctx.q_off[i]), int(ctx.q_len[i]), int(ctx.slots[i])
+                s = state[slot]
+                rows = []
+                for t in range(n):
+                    s = self.decay * s + x[lo + t].float()
+                    rows.append(s)
+                state[slot] = s
+                y = torch.stack(rows) @ self.w.T
+                out[lo:lo + n] = out[lo:lo + n] + y if accumulate else y
+
+    @register_architecture
+    @dataclass(frozen=True)
+    class ToyConfig(ModelConfig):
+        hidden_size: int
+        vocab_size: int
+        decay: float
+        schedule: list
+        architecture_names = ("toy-decay",)
+
+        def model_spec(self):
+            h = self.hidden_size
+            norm = PartSpec("rmsnorm", {"size": h, "eps": 1e-5})
+            ff = PartSpec("gated_mlp", {"hidden_size": h, "intermediate_size": 2 * h, "activation": "silu"})
+            arr = PartSpec("prenorm_residual", {"mixer_prefix": "mixer", "feed_forward_prefix": "ff",
+                                                "mixer_norm_name": "norm1", "feed_forward_norm_name": "norm2"})
+            attn = PartSpec("attention", {"hidden_size": h, "num_heads": 2, "num_kv_heads": 1, "head_dim": 16,
+                                          "qk_norm": None,
+                                          "position": PartSpec("rope_half", {"rotary_dim": 8, "theta": 100.0}),
+                                          "window": None, "bias": False, "scale": 0.25})
+            decay = PartSpec("toy_decay", {"hidden_size": h, "decay": self.decay})
+            layers = (LayerSpec("layers.0", arr, decay, ff, norm, norm),
+                      LayerSpec("layers.1", arr, attn, ff, norm, norm),
+                      LayerSpec("layers.2", arr, attn, ff, norm, norm))
+            return ModelSpec(
+                hidden_size=h, vocab_size=self.vocab_size,
+                embedding=PartSpec("token_embedding", {"name": "embed.weight", "vocab_size": self.vocab_size,
+                                                       "hidden_size": h}),
+                layers=layers,
+                schedule=tuple(ScheduleEntry(*e) for e in self.schedule),
+                final_norm=PartSpec("rmsnorm", {"size": h, "eps": 1e-5, "name": "final_norm.weight"}),
+                head=PartSpec("linear_head", {"name": "head.weight", "tied_to": None,
+                                              "vocab_size": self.vocab_size, "hidden_size": h}))
+
+    return ToyConfig
+
+
+def _toy_plain(cfg, w, tokens, schedule):
+    """Plain float64 forward of the toy architecture, whole sequence."""
+    t = len(tokens)
+    h = w["embed.weight"][torch.tensor(tokens)]
+    positions = torch.arange(t)
+    kv = {}
+    for layer, unit, writes in schedule:
+        p = f"layers.{layer}"
+        x = P.rmsnorm(h, w[f"{p}.norm1.weight"], 1e-5)
+        if layer == 0:
+            s = torch.zeros(cfg["hidden_size"], dtype=torch.float64)
+            rows = []
+            for i in range(t):
+                s = cfg["decay"] * s + x[i]
+                rows.append(s)
+            h = h + torch.stack(rows) @ w[f"{p}.mixer.mix.weight"].T
+        else:
+            q = P.linear(x, w[f"{p}.mixer.q_proj.weight"]).view(t, 2, 16)
+            if writes:
+                k = P.linear(x, w[f"{p}.mixer.k_proj.weight"]).view(t, 1, 16)
+                v = P.linear(x, w[f"{p}.mixer.v_proj.weight"]).view(t, 1, 16)
+                cos, sin = P.rope_tables(8, 100.0, positions)
+                k = torch.cat([P.apply_rope(k[..., :8], cos, sin), k[..., 8:]], -1)
+                kv[unit] = (k, v)
+            cos, sin = P.rope_tables(8, 100.0, positions)
+            q = torch.cat([P.apply_rope(q[..., :8], cos, sin), q[..., 8:]], -1)
+            k, v = kv[unit]
+            attn = P.causal_attention(q * (0.25 * 4.0), k, v)          # part scale 0.25, plain scale 1/sqrt(16)
+            h = h + P.linear(attn.reshape(t, 32), w[f"{p}.mixer.o_proj.weight"])
+        h = h + P.mlp_block({k_: v_ for k_, v_ in w.items()}, f"{p}.ff",
+                            P.rmsnorm(h, w[f"{p}.norm2.weight"], 1e-5))
+    return P.linear(P.rmsnorm(h, w["final_norm.weight"], 1e-5), w["head.weight"])
+
+
+@pytest.mark.parametrize("schedule", [
+    [(0, 0, True), (1, 1, True), (2, 2, True)],                      # state mixer, then two attention layers
+    [(0, 0, True), (1, 1, True), (1, 2, True), (2, 3, True)],        # layer 1 runs twice, each run with its own cache
+    [(0, 0, True), (1, 1, True), (2, 1, False)],                     # layer 2 reads the keys and values of layer 1
+])
+def test_toy_architecture_registers_builds_and_steps(tmp_path, schedule):
+    from lockstep_amd.config import unregister_architecture
+    from lockstep_amd.engine.model import load_model
+    from lockstep_amd.parts import unregister_part
+    from lockstep_amd.weights import write_random_model
+
+    ToyConfig = _register_toy()
+    try:
+        cfg = ToyConfig(hidden_size=48, vocab_size=90, decay=0.9, schedule=[list(e) for e in schedule])
+        folder = write_random_model(cfg, tmp_path / "toy", seed=5, std=0.2, norm_std=0.1)
+        assert json.loads((folder / "config.json").read_text())["model_type"] == "toy-decay"
+        model = load_model(folder, dtype="float32")
+        units = model.cache_unit_specs()
+        assert type(units[0]).__name__ == "StateSpec" and type(units[1]).__name__ == "PagedKVSpec"
+        from safetensors.torch import load_file
+
+        w = {k: v.double() for k, v in load_file(str(folder / "model.safetensors")).items()}
+        tokens = random_tokens(50, 90, seed=1)
+        want = _toy_plain({"hidden_size": 48, "decay": 0.9}, w, tokens, schedule)
+        cache = model.make_cache(num_pages=16, page_size=8, max_requests=3, poison_on_free=True)
+        whole = feed(model, cache, "w", tokens, [])
+        assert rel_err(whole, want) < 5e-5
+        other = feed(model, cache, "o", random_tokens(9, 90, seed=2), [])     # another request in between
+        cut = feed(model, cache, "c", tokens, [7, 2, 17, 1, 1, 13])
+        assert rel_err(cut, want) < 5e-5
+        cache.close("w"); cache.close("o")
+        again = feed(model, cache, "w2", tokens, [25])                          # a reused slot starts from zero state
+        assert rel_err(again, want) < 5e-5
+        cache.audit()
+    finally:
+        unregister_part("toy_decay")
+        unregister_architecture(ToyConfig)

@@ -1,0 +1,265 @@
+"""The scheduler's decisions, on the host with a stand-in model whose logits
+are a pure function of a request's context."""
+
+from __future__ import annotations
+
+import hashlib
+
+import pytest
+import torch
+
+from lockstep_amd.cache import CacheManager, OutOfPages
+from lockstep_amd.engine.policy import (DefaultPolicy, Event, FixedChunkPolicy, NoCacheHitPolicy,
+                                        PreemptAtStepsPolicy, ScriptedPolicy)
+from lockstep_amd.engine.scheduler import OversizedRequest, Request, Scheduler
+from lockstep_amd.parts import PagedKVSpec
+from lockstep_amd.sampling import Sampler, greedy, top_p
+
+VOCAB = 40
+
+
+def context_logits(context) -> torch.Tensor:
+    seed = int.from_bytes(hashlib.sha256(repr(list(context)).encode()).digest()[:7], "big")
+    return torch.randn(VOCAB, generator=torch.Generator().manual_seed(seed))
+
+
+class StandInModel:
+    """Keeps each request's tokens; logits at a place depend on the context up to it."""
+
+    def __init__(self):
+        self.history: dict[str, list[int]] = {}
+        self.prompts: dict[str, list[int]] = {}
+        self.batches: list[list[tuple]] = []
+
+    def make_cache(self, num_pages, page_size=16, max_requests=64, max_tokens_per_request=None, **_):
+        return CacheManager([PagedKVSpec(1, 16, None)], page_size, num_pages, max_requests,
+                            max_tokens_per_request or num_pages * page_size)
+
+    def step(self, cache, entries):
+        rows, batch = [], []
+        for e in entries:
+            start = cache.length(e.request)
+            if start == 0:
+                self.history[e.request] = []
+            hist = self.history.setdefault(e.request, [])
+            if len(hist) < start:                       # a prefix hit: those tokens were never fed
+                hist.extend(self.prompts[e.request][len(hist):start])
+            assert len(hist) == start, "the step must continue where the cache ends"
+            cache.reserve(e.request, start + len(e.tokens))
+            hist.extend(e.tokens)
+            batch.append((e.request, start, len(e.tokens)))
+            for w in e.want:
+                rows.append(context_logits(hist[: start + w + 1]))
+        for e in entries:
+            cache.commit(e.request, len(self.history[e.request]))
+        self.batches.append(batch)
+        return torch.stack(rows) if rows else None
+
+
+def expected_greedy(prompt, n, eos=()):
+    context, out = list(prompt), []
+    for _ in range(n):
+        token = greedy(context_logits(context))
+        out.append(token); context.append(token)
+        if token in eos:
+            break
+    return out
+
+
+def prompts(*lengths, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    return [torch.randint(0, VOCAB, (n,), generator=g).tolist() for n in lengths]
+
+
+def run(requests, **kw):
+    model = StandInModel()
+    for r in requests:
+        model.prompts[r.uid] = list(r.prompt)
+    kw.setdefault("num_blocks", 64)
+    s = Scheduler(model, **kw)
+    for r in requests:
+        s.submit(r)
+    return s.run(), s, model
+
+
+def reqs(ps, n=6, **kw):
+    return [Request(uid=f"r{i}", prompt=p, max_new_tokens=n, **kw) for i, p in enumerate(ps)]
+
+
+def test_outputs_do_not_depend_on_chunking_budget_or_company():
+    ps = prompts(1, 9, 17, 40, 64)
+    want = {f"r{i}": expected_greedy(p, 6) for i, p in enumerate(ps)}
+    assert run(reqs(ps))[0] == want
+    assert run(reqs(ps), policy=FixedChunkPolicy(12))[0] == want
+    assert run(reqs(ps), policy=FixedChunkPolicy(5), max_batched_tokens=16)[0] == want
+    assert run(reqs(ps), policy=ScriptedPolicy(chunk_plan=[7, 2, 17, 3, 2]))[0] == want
+    assert run(reqs(ps[2:3]))[0] == {"r0": want["r2"]}
+    assert run(list(reversed(reqs(ps))))[0] == want
+
+
+def test_token_budget_holds_and_decoded_tokens_go_first():
+    ps = prompts(30, 30, 30)
+    out, s, model = run(reqs(ps, n=4), policy=FixedChunkPolicy(8), max_batched_tokens=10)
+    assert all(sum(n for _, _, n in b) <= 10 for b in model.batches)
+    assert s.counters["budget_deferred"] > 0 and s.counters["prefill_chunk"] > 3
+    # once r0 decodes, its token is in every batch although the budget is short for the others
+    first_decode = next(i for i, b in enumerate(model.batches) if any(u == "r0" and n == 1 and st >= 30 for u, st, n in b))
+    later = model.batches[first_decode: first_decode + 3]
+    assert all(any(u == "r0" for u, _, _ in b) for b in later)
+    assert out == {f"r{i}": expected_greedy(p, 4) for i, p in enumerate(ps)}
+
+
+def test_admission_waits_for_pages_and_respects_max_running():
+    ps = prompts(20, 20, 20)
+    out, s, model = run(reqs(ps, n=4), num_blocks=4, block_size=8)        # each needs 3 of 4 pages
+    assert [len(b) for b in model.batches].count(1) == len(model.batches)  # never two at once
+    assert s.counters["admit_refused"] > 0 and s.counters["admit"] == 3
+    assert out == {f"r{i}": expected_greedy(p, 4) for i, p in enumerate(ps)}
+    out2, s2, model2 = run(reqs(ps, n=4), policy=DefaultPolicy(max_running=2))
+    assert max(len(b) for b in model2.batches) == 2 and out2 == out
+    s.cache.audit()
+    assert s.cache.free_pages == [4] and s.cache.free_slots == s.cache.max_requests
+
+
+def test_what_happens_when_pages_run_out():
+    model = StandInModel()
+    s = Scheduler(model, num_blocks=4, block_size=8)
+    with pytest.raises(OversizedRequest):
+        s.submit(Request(uid="big", prompt=[1] * 30, max_new_tokens=8))     # 5 pages > 4
+    with pytest.raises(ValueError):
+        s.submit(Request(uid="empty", prompt=[]))
+
+    class Never(DefaultPolicy):
+        def admit(self, state, uid, pages_needed):
+            return False
+
+    s = Scheduler(model, num_blocks=4, block_size=8, policy=Never())
+    s.submit(Request(uid="a", prompt=[1, 2, 3]))
+    with pytest.raises(OutOfPages, match="nothing running"):
+        s.step()
+    assert s.counters["out_of_pages"] == 1
+
+
+def test_lazy_reservation_preempts_the_newest_and_recomputes():
+    ps = prompts(20, 20, 20)
+    want = {f"r{i}": expected_greedy(p, 12) for i, p in enumerate(ps)}
+
+    class Eager(DefaultPolicy):                     # admit on the prompt alone; growth is found out later
+        def admit(self, state, uid, pages_needed):
+            return len(state.running) < self.max_running and state.free_pages >= 3
+
+    out, s, model = run(reqs(ps, n=12), num_blocks=8, block_size=8, reserve="lazy", policy=Eager())
+    assert out == want
+    assert s.counters["preempt_for_pages"] > 0 and s.counters["resume"] > 0
+    assert any(r.preempt_count for r in s.done)
+    s.cache.audit()
+    assert s.cache.free_pages == [8]
+
+
+def test_eos_stops_with_the_prefix_of_the_unbounded_run():
+    p = prompts(11)[0]
+    free = expected_greedy(p, 12)
+    eos = free[4]
+    cut = free[: free.index(eos) + 1]
+    out, s, _ = run([Request(uid="r", prompt=p, max_new_tokens=12)], eos_token_ids={eos})
+    assert out == {"r": cut} and s.counters["finish_eos"] == 1
+    out, s, _ = run([Request(uid="r", prompt=p, max_new_tokens=12)])
+    assert out == {"r": free} and s.counters["finish_limit"] == 1
+
+
+def test_scripted_preemption_leaves_tokens_unchanged():
+    ps = prompts(9, 23)
+    want = {f"r{i}": expected_greedy(p, 8) for i, p in enumerate(ps)}
+    for steps in ((2,), (2, 5), (2, 4, 6)):
+        out, s, _ = run(reqs(ps, n=8), policy=PreemptAtStepsPolicy("r0", steps, chunk=7))
+        assert out == want
+        assert s.counters["preempt_fired"] == len(steps) and s.counters["resume"] == len(steps)
+        assert [r.preempt_count for r in s.done if r.uid == "r0"] == [len(steps)]
+        assert Event.PREEMPT in s.lifecycle["r0"] and Event.RESUME in s.lifecycle["r0"]
+
+
+def test_prefix_index_hits_trims_a_whole_prompt_hit_and_evicts_under_pressure():
+    shared = prompts(32, seed=5)[0]
+    a = Request(uid="a", prompt=shared + [1, 2, 3], max_new_tokens=4)
+    model = StandInModel()
+    s = Scheduler(model, num_blocks=12, block_size=8, enable_prefix_cache=True)
+    for r in (a,):
+        model.prompts[r.uid] = list(r.prompt); s.submit(r)
+    s.run()
+    assert s.counters["cache_miss"] == 1 and s.counters["cache_insert"] >= 4
+    b = Request(uid="b", prompt=shared + [7, 8], max_new_tokens=4)
+    c = Request(uid="c", prompt=shared, max_new_tokens=4)                 # the whole prompt is indexed
+    for r in (b, c):
+        model.prompts[r.uid] = list(r.prompt); s.submit(r)
+    s.run()
+    done = {r.uid: r for r in s.done}
+    assert done["b"].cache_hit_tokens == 32 and done["c"].cache_hit_tokens == 24
+    assert s.counters["cache_hit"] == 2 and s.counters["cache_full_prompt_trimmed"] == 1
+    assert done["b"].generated == expected_greedy(b.prompt, 4)
+    assert done["c"].generated == expected_greedy(c.prompt, 4)
+    first_b = next(batch for batch in model.batches if any(u == "b" for u, _, _ in batch))
+    assert ("b", 32, 2) in first_b                                         # only the tail was computed
+    # pressure: a request that needs the indexed pages back
+    held = s.num_pages - s.cache.free_pages[0]
+    assert held > 0
+    d = Request(uid="d", prompt=prompts(80, seed=9)[0], max_new_tokens=8)
+    model.prompts["d"] = list(d.prompt); s.submit(d)
+    s.run()
+    assert s.counters["eviction_taken"] > 0 and s.evictions > 0
+    assert {r.uid: r for r in s.done}["d"].generated == expected_greedy(d.prompt, 8)
+    s.cache.audit()
+    # refusing hits gives the same tokens
+    s2 = Scheduler(model, num_blocks=12, block_size=8, enable_prefix_cache=True, policy=NoCacheHitPolicy())
+    out = {}
+    for uid, p in (("a2", a.prompt), ("b2", b.prompt)):      # one after the other: entries appear at finish
+        model.prompts[uid] = list(p); s2.submit(Request(uid=uid, prompt=list(p), max_new_tokens=4))
+        out.update(s2.run())
+    assert out["b2"] == done["b"].generated and s2.counters["cache_hit_refused"] == 1
+
+
+def test_sampled_tokens_depend_on_the_request_alone():
+    # reference harness/mr/relations.py:184-223: removing, adding or reordering requests leaves survivors unchanged
+    ps = prompts(5, 9, 14)
+
+    def sampled(subset, order=1):
+        rs = [Request(uid=f"r{i}", prompt=ps[i], seed=10 + i, max_new_tokens=10, temperature=0.8, top_p=0.95)
+              for i in subset][::order]
+        return run(rs)[0]
+
+    everyone = sampled([0, 1, 2])
+    assert sampled([1]) == {"r1": everyone["r1"]}
+    assert sampled([0, 2], order=-1) == {"r0": everyone["r0"], "r2": everyone["r2"]}
+    other_seed = run([Request(uid="r1", prompt=ps[1], seed=99, max_new_tokens=10, temperature=0.8, top_p=0.95)])[0]
+    assert other_seed["r1"] != everyone["r1"]
+    # position of the draw is the absolute index of the sampled row
+    context = list(ps[1])
+    want = []
+    for _ in range(10):
+        token = top_p(context_logits(context), 11, "r1", len(context) - 1, 0.95, 0.8)
+        want.append(token); context.append(token)
+    assert everyone["r1"] == want
+
+
+def test_lifecycle_follows_the_state_machine():
+    legal = {
+        ("waiting", Event.ADMIT): "admitted", ("admitted", Event.EVICT): "admitted",
+        ("admitted", Event.CACHE_HIT): "prefilling", ("admitted", Event.CHUNK): "prefilling",
+        ("admitted", Event.DECODE): "decoding", ("prefilling", Event.CHUNK): "prefilling",
+        ("prefilling", Event.DECODE): "decoding", ("prefilling", Event.PREEMPT): "preempted",
+        ("prefilling", Event.EVICT): "prefilling", ("decoding", Event.DECODE): "decoding",
+        ("decoding", Event.PREEMPT): "preempted", ("decoding", Event.FINISH): "done",
+        ("preempted", Event.RESUME): "admitted",
+    }   # reference engine/sched/lifecycle.py:26-40
+    ps = prompts(9, 23, 40)
+    _, s, _ = run(reqs(ps, n=8), policy=PreemptAtStepsPolicy("r1", (3, 6), chunk=7), max_batched_tokens=20)
+    for uid, events in s.lifecycle.items():
+        state = "waiting"
+        for event in events:
+            assert (state, event) in legal, f"{uid}: {event} in state {state}"
+            state = legal[(state, event)]
+        assert state == "done"
+    a = run(reqs(ps, n=8))[1].trajectory
+    b = run(reqs(ps, n=8))[1].trajectory
+    c = run(reqs(ps, n=8), policy=FixedChunkPolicy(7))[1].trajectory
+    assert a.hexdigest() == b.hexdigest() and a.first_divergence(b) is None
+    assert a.hexdigest() != c.hexdigest() and a.first_divergence(c) == 0
