@@ -10,6 +10,7 @@ row; here the final norm and the head run on the wanted rows only).
 
 from __future__ import annotations
 
+import itertools
 import os
 from pathlib import Path
 from typing import Sequence
@@ -45,8 +46,12 @@ def collect_ties(spec: ModelSpec) -> dict[str, str]:
     return dict(head.ties(spec.head)) if hasattr(head, "ties") else {}
 
 
+_MODEL_SERIAL = itertools.count()
+
+
 class Model:
     def __init__(self, config: ModelConfig, rt: Runtime):
+        self.serial = next(_MODEL_SERIAL)
         self.config = config
         self.rt = rt
         self.spec = config.model_spec()
@@ -60,7 +65,6 @@ class Model:
                 raise ValueError(f"the schedule names layer {run.layer}, the model has {len(self.layers)}")
         self.workspace = Workspace(rt.device)
         self.use_graphs = os.environ.get("LOCKSTEP_NO_GRAPHS", "") in ("", "0")
-        self._graphs: dict[tuple, tuple] = {}
         self._graph_safe = all(layer.mixer.graph_safe for layer in self.layers)
         self.graph_replays = 0
 
@@ -123,9 +127,6 @@ class Model:
         ctx = StepContext(self.rt, cache, self.workspace, entries, fixed_shape=graphed)
         for layer in self.layers:
             layer.mixer.prepare(ctx)
-            position = getattr(layer.mixer, "position", None)
-            if position is not None:
-                position.ensure(ctx.max_position + 1, self.rt)
         ctx.upload()
         logits = self._forward_graphed(ctx, cache) if graphed else self._forward(ctx)
         for e, end in zip(entries, ctx.kv_len):
@@ -146,19 +147,22 @@ class Model:
             self.head.forward(ctx, x, logits)
         return logits
 
-    def _graph_key(self, ctx: StepContext, cache) -> tuple:
-        tables = tuple(id(layer.mixer.position.cos) for layer in self.layers
-                       if getattr(layer.mixer, "position", None) is not None)
-        return (ctx.n_seqs, ctx.plan_signature(), self.workspace.version, id(cache), tables)
+    def _graph_key(self, ctx: StepContext) -> tuple:
+        tables = tuple((t.data_ptr(), t.shape[0]) for t in
+                       (getattr(getattr(layer.mixer, "position", None), "cos", None) for layer in self.layers)
+                       if t is not None)
+        return (self.serial, ctx.n_seqs, ctx.plan_signature(), self.workspace.version, tables)
 
     def _forward_graphed(self, ctx: StepContext, cache):
         """Replay the captured graph of this step shape, capturing it first if
         needed.  The graph reads the step's metadata, the block tables and the
         cache through fixed addresses; only their contents change between
         replays.  The first step of a shape runs eagerly (that also sizes the
-        workspace), then the same launches are recorded for the steps to come."""
-        key = self._graph_key(ctx, cache)
-        held = self._graphs.get(key)
+        workspace), then the same launches are recorded for the steps to come.
+        Graphs are kept on the cache manager they point into and die with it."""
+        graphs = cache.__dict__.setdefault("_step_graphs", {})
+        key = self._graph_key(ctx)
+        held = graphs.get(key)
         if held is not None:
             graph, logits = held
             graph.replay()
@@ -166,15 +170,15 @@ class Model:
             return logits.clone()
         logits = torch.empty((ctx.n_want, self.spec.vocab_size), dtype=torch.float32, device=self.rt.device)
         self._forward(ctx, logits)
-        key = self._graph_key(ctx, cache)          # the eager run may have grown the workspace
-        if len(self._graphs) >= 32:
-            self._graphs.clear()
+        key = self._graph_key(ctx)                 # the eager run may have grown the workspace
+        if len(graphs) >= 32:
+            graphs.clear()
         result = logits.clone()
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
             self._forward(ctx, logits)
-        self._graphs[key] = (graph, logits)
+        graphs[key] = (graph, logits)
         return result
 
 

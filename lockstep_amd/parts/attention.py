@@ -91,6 +91,7 @@ class Attention(Mixer):
         rt.kernels.attention_lib(self.d)
 
     def prepare(self, ctx) -> None:
+        self.position.ensure(ctx.max_position + 1, ctx.rt)
         ctx.plan_attention(self.nq // self.nkv, self.nkv, self.d, int(self.window) if self.window is not None else 0)
 
     def forward(self, ctx, run, x, out, accumulate: bool) -> None:

@@ -43,10 +43,15 @@ TINY_B_INIT = dict(seed=2, std=0.05, norm_std=0.1, page_size=8)
 TINY = {"A": (TINY_A, TINY_A_INIT), "B": (TINY_B, TINY_B_INIT)}
 
 
-def make_model_dir(tmp_path_factory, name: str, sharpen: float = 1.0) -> Path:
+def make_model_dir(tmp_path_factory, name: str, sharpen: float = 1.0, std: float | None = None) -> Path:
     """Write tiny configuration ``name`` with random weights.  ``sharpen``
     multiplies the per-head q/k norm weights so that attention is peaked and a
-    wrong key or a wrong position changes the logits visibly."""
+    wrong key or a wrong position changes the logits visibly (the float32 path
+    is compared on such weights; in bfloat16 the rounding of queries and keys
+    is amplified by the same factor squared, so the bfloat16 comparison with
+    the plain implementation uses the unsharpened weights and the sharpened
+    ones serve its bit-for-bit comparisons).  ``std`` overrides the spread of
+    the matrices (larger values separate the logits, for token comparisons)."""
     from lockstep_amd.config import Qwen3Config
     from lockstep_amd.weights import random_tensors, save_file
     import json
@@ -54,7 +59,7 @@ def make_model_dir(tmp_path_factory, name: str, sharpen: float = 1.0) -> Path:
     raw, init = TINY[name]
     config = Qwen3Config.from_dict(raw)
     out = tmp_path_factory.mktemp(f"tiny{name}")
-    tensors = random_tensors(config, init["seed"], init["std"], init["norm_std"], torch.bfloat16)
+    tensors = random_tensors(config, init["seed"], std or init["std"], init["norm_std"], torch.bfloat16)
     if sharpen != 1.0:
         for key in tensors:
             if key.endswith("q_norm.weight") or key.endswith("k_norm.weight"):
@@ -74,6 +79,13 @@ def tiny_b_dir(tmp_path_factory):
     return make_model_dir(tmp_path_factory, "B", sharpen=2.0)
 
 
-@pytest.fixture(scope="session", params=["A", "B"])
-def tiny_dir(request, tiny_a_dir, tiny_b_dir):
-    return {"A": tiny_a_dir, "B": tiny_b_dir}[request.param], TINY[request.param][1]["page_size"]
+@pytest.fixture(scope="session")
+def tiny_dirs(tmp_path_factory, tiny_a_dir, tiny_b_dir):
+    """(configuration, variant) -> model folder; variants: ``sharp`` (peaked
+    attention), ``soft`` (weights as drawn), ``gen`` (well separated logits)."""
+    return {
+        ("A", "sharp"): tiny_a_dir, ("B", "sharp"): tiny_b_dir,
+        ("A", "soft"): make_model_dir(tmp_path_factory, "A"), ("B", "soft"): make_model_dir(tmp_path_factory, "B"),
+        ("A", "gen"): make_model_dir(tmp_path_factory, "A", std=0.3),
+        ("B", "gen"): make_model_dir(tmp_path_factory, "B", std=0.3),
+    }

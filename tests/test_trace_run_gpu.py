@@ -90,10 +90,11 @@ def portions(requests, sizes=(7, 2, 17, 3, 37, 2, 16, 15, 64)):
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", ["A", "B"])
-def test_replay_under_four_cuttings(tiny_a_dir, tiny_b_dir, tmp_path, dtype, name):
+def test_replay_under_four_cuttings(tiny_dirs, tmp_path, dtype, name):
     from plain.qwen3_plain import PlainModel
 
-    folder = {"A": tiny_a_dir, "B": tiny_b_dir}[name]
+    # float32 on the sharpened weights; bfloat16 on the weights as drawn (see conftest.make_model_dir)
+    folder = tiny_dirs[(name, "sharp" if dtype == "float32" else "soft")]
     plain = PlainModel(folder)
     vocab = plain.cfg["vocab_size"]
     requests = {f"t{i}": random_tokens(n, vocab, seed=40 + i) for i, n in enumerate((150, 40, 3, 97, 300, 66))}
