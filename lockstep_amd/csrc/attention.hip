@@ -112,8 +112,11 @@ __device__ __forceinline__ void store_output(const RowState& run, T* __restrict_
   }
 }
 
+// Variant 1, "direct": every wave loads its operands straight from global
+// memory.  Needs no LDS, so it takes every head size in both precisions; it
+// is the fallback where the staged kernel's tiles do not fit into LDS.
 template <typename T>
-__global__ __launch_bounds__(256) void attention_kernel(
+__global__ __launch_bounds__(256) void attention_direct_kernel(
     const T* __restrict__ q, long ldq, const T* __restrict__ k_pages, const T* __restrict__ v_pages, int nkv,
     int page_size, const int* __restrict__ table, int table_stride, const SeqMeta* __restrict__ seqs,
     const AttnItem* __restrict__ items, T* __restrict__ out, long ldo, float* __restrict__ part_acc,
@@ -274,6 +277,264 @@ __global__ __launch_bounds__(256) void attention_kernel(
   if (direct && row_ok) store_output<T>(run, out + (long)(sm.q_off + qi) * ldo + (long)head * D, g);
 }
 
+
+// Variant 2, "staged": the four waves of a workgroup load each 128-key tile of
+// K and of V^T once, with wide coalesced loads, into LDS; every wave then
+// takes its MFMA operands from there.  With one decoded token per request
+// only the first wave has rows, but all four still fetch, so one workgroup
+// keeps 64 KB of loads in flight.  The next tile's global loads are issued
+// before the current tile is multiplied.  The arithmetic is the same as in
+// the direct variant, instruction for instruction, so both give the same bits.
+//
+// LDS layout: K tile [128 keys][D], V tile [D][128 keys], rows unpadded; the
+// 16-byte pieces of a row are rotated by the row index so that the 16 rows an
+// MFMA operand touches fall into different banks.
+template <typename T, bool PREFETCH>
+__global__ __launch_bounds__(256) void attention_staged_kernel(
+    const T* __restrict__ q, long ldq, const T* __restrict__ k_pages, const T* __restrict__ v_pages, int nkv,
+    int page_size, int page_shift, const int* __restrict__ table, int table_stride,
+    const SeqMeta* __restrict__ seqs, const AttnItem* __restrict__ items, T* __restrict__ out, long ldo,
+    float* __restrict__ part_acc, float* __restrict__ part_ml, int G, float scale, int window) {
+  typedef Atom<T> A;
+  typedef typename A::vec_t vec_t;
+  constexpr int SZ = sizeof(T);
+  constexpr int NC = (D + A::KCHUNK - 1) / A::KCHUNK;
+  constexpr int KROW = D * SZ;              // bytes of one key row
+  constexpr int KPIECES = KROW / 16;        // 16-byte pieces in it
+  constexpr int VROW = kTileKeys * SZ;      // bytes of one column row of the V^T tile
+  constexpr int VPIECES = VROW / 16;
+  constexpr int TOTAL = kTileKeys * KPIECES;  // pieces in the K tile == pieces in the V tile
+  constexpr int PER = (TOTAL + 255) / 256;    // pieces per thread
+  constexpr int TILES_PER_SPLIT = kSplitKeys / kTileKeys;
+  constexpr int LOG_VEC = (A::VEC == 8) ? 3 : 2;
+
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+  unsigned char* k_lds = lds;
+  unsigned char* v_lds = lds + kTileKeys * KROW;
+
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const AttnItem item = items[blockIdx.x];
+  const SeqMeta sm = seqs[item.seq];
+  const int kvh = blockIdx.y;
+  const int rows_total = sm.q_len * G;
+  const int block_r0 = item.row_block * 64;
+  if (block_r0 >= rows_total) return;  // uniform for the workgroup
+  const int block_first_pos = sm.q_start + block_r0 / G;
+  const int block_last_pos = sm.q_start + min(block_r0 + 63, rows_total - 1) / G;
+
+  const int r0 = block_r0 + wave * 16;
+  const bool wave_active = r0 < rows_total;
+  const int row16 = lane & 15;
+  const int g = lane >> 4;
+  const int r = r0 + row16;
+  const bool row_ok = r < rows_total;
+  const int qi = row_ok ? r / G : 0;
+  const int head = kvh * G + (row_ok ? r % G : 0);
+  const int q_pos = sm.q_start + qi;
+  const int wave_first_pos = sm.q_start + min(r0, rows_total - 1) / G;
+  const int wave_last_pos = sm.q_start + min(r0 + 15, rows_total - 1) / G;
+  const int lo_valid = window > 0 ? max(0, sm.q_start - window + 1) : 0;
+  const int* __restrict__ tbl = table + (long)sm.table_row * table_stride;
+  const bool direct = item.part_base < 0;
+  const int vshift = page_shift - LOG_VEC;  // log2 of the pieces of one column inside a page
+
+  vec_t qv[NC];
+#pragma unroll
+  for (int c = 0; c < NC; ++c)
+    qv[c] = load_vec<T>(q + (long)head * D, sm.q_off + qi, c * A::KCHUNK + g * A::VEC, D, ldq, row_ok, true);
+
+  // tiles this workgroup walks: a contiguous range
+  int ti_lo = item.split_begin * TILES_PER_SPLIT;
+  if (window > 0) ti_lo = max(ti_lo, max(0, block_first_pos - window + 1) / kTileKeys);
+  const int ti_hi = min(item.split_end * TILES_PER_SPLIT, block_last_pos / kTileKeys + 1);
+
+  // Without prefetch the pieces go through registers a few at a time.
+  constexpr int GROUP = PREFETCH ? PER : (PER < 4 ? PER : 4);
+  vec_t kreg[GROUP], vreg[GROUP];
+  auto fetch = [&](int ti, int i0) {
+    const int t0 = ti * kTileKeys;
+#pragma unroll
+    for (int j = 0; j < GROUP; ++j) {
+      const int i = i0 + j;
+      if (i >= PER) break;
+      const int p = threadIdx.x + 256 * i;
+      // ---- K piece: key row p / KPIECES, piece p % KPIECES
+      {
+        const int kt = p / KPIECES;
+        const int piece = p % KPIECES;
+        const int key = t0 + kt;
+        bool ok = (TOTAL % 256 == 0 || p < TOTAL) && key < sm.kv_len && key >= lo_valid;
+        int page = tbl[min(key, sm.kv_len - 1) >> page_shift];
+        ok = ok && page >= 0;
+        page = max(page, 0);
+        const int slot = min(key, sm.kv_len - 1) & (page_size - 1);
+        const T* src = k_pages + (((long)page * nkv + kvh) * page_size + slot) * D + piece * A::VEC;
+        vec_t v = *reinterpret_cast<const vec_t*>(src);
+        kreg[j] = ok ? v : A::zero();
+      }
+      // ---- V piece: page pg of the tile, column d, keys kp*VEC.. inside the page
+      {
+        const int q1 = p >> vshift;
+        const int kp = p & ((1 << vshift) - 1);
+        const int pg = q1 / D;
+        const int d = q1 % D;
+        const int key0 = t0 + (pg << page_shift) + (kp << LOG_VEC);
+        bool ok = (TOTAL % 256 == 0 || p < TOTAL) && key0 < sm.kv_len && key0 + A::VEC > lo_valid;
+        int page = tbl[min(key0, sm.kv_len - 1) >> page_shift];
+        ok = ok && page >= 0;
+        page = max(page, 0);
+        const T* src = v_pages + ((((long)page * nkv + kvh) * D + d) << page_shift) + (kp << LOG_VEC);
+        vec_t v = *reinterpret_cast<const vec_t*>(src);
+#pragma unroll
+        for (int e = 0; e < A::VEC; ++e)
+          if (!ok || key0 + e >= sm.kv_len || key0 + e < lo_valid) v[e] = 0;
+        vreg[j] = v;
+      }
+    }
+  };
+  auto stash = [&](int i0) {
+#pragma unroll
+    for (int j = 0; j < GROUP; ++j) {
+      const int i = i0 + j;
+      if (i >= PER) break;
+      const int p = threadIdx.x + 256 * i;
+      if (TOTAL % 256 != 0 && p >= TOTAL) continue;
+      const int kt = p / KPIECES;
+      const int piece = p % KPIECES;
+      *reinterpret_cast<vec_t*>(k_lds + kt * KROW + ((piece + kt) % KPIECES) * 16) = kreg[j];
+      const int q1 = p >> vshift;
+      const int kp = p & ((1 << vshift) - 1);
+      const int pg = q1 / D;
+      const int d = q1 % D;
+      const int vpiece = (pg << vshift) + kp;
+      *reinterpret_cast<vec_t*>(v_lds + d * VROW + ((vpiece + d) % VPIECES) * 16) = vreg[j];
+    }
+  };
+
+  RowState run, cur;
+  run.reset();
+  cur.reset();
+
+  if (PREFETCH && ti_lo < ti_hi) fetch(ti_lo, 0);
+  for (int ti = ti_lo; ti < ti_hi; ++ti) {
+    const int t0 = ti * kTileKeys;
+    __syncthreads();  // the previous tile has been read by every wave
+    if (PREFETCH) {
+      stash(0);
+    } else {
+      for (int i0 = 0; i0 < PER; i0 += GROUP) {
+        fetch(ti, i0);
+        stash(i0);
+      }
+    }
+    __syncthreads();
+    if (PREFETCH && ti + 1 < ti_hi) fetch(ti + 1, 0);
+
+    const bool mine = wave_active && t0 <= wave_last_pos &&
+                      !(window > 0 && t0 + kTileKeys <= wave_first_pos - window + 1);
+    if (mine) {
+      // ---- S^T = K . Q^T ---------------------------------------------------
+      f32x4 s[NB];
+#pragma unroll
+      for (int kb = 0; kb < NB; ++kb) {
+        s[kb] = f32x4{0.f, 0.f, 0.f, 0.f};
+        const int row = kb * 16 + row16;
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+          const int piece = c * 4 + g;
+          vec_t kv = A::zero();
+          if (piece < KPIECES)
+            kv = *reinterpret_cast<const vec_t*>(k_lds + row * KROW + ((piece + row) % KPIECES) * 16);
+          A::mma(s[kb], kv, qv[c]);
+        }
+      }
+      // ---- scale, mask, online softmax --------------------------------------
+      float tile_max = kNegSentinel;
+#pragma unroll
+      for (int kb = 0; kb < NB; ++kb)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int key = t0 + kb * 16 + 4 * g + e;
+          const bool keep = row_ok && key <= q_pos && (window <= 0 || q_pos - key < window);
+          const float v = keep ? s[kb][e] * scale : kNegSentinel;
+          s[kb][e] = v;
+          tile_max = fmaxf(tile_max, v);
+        }
+      tile_max = quad16_max(tile_max);
+      const float m_new = fmaxf(cur.m, tile_max);
+      const float alpha = softmax_exp<T>(cur.m - m_new);
+      float p_sum = 0.f;
+#pragma unroll
+      for (int kb = 0; kb < NB; ++kb)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int key = t0 + kb * 16 + 4 * g + e;
+          const bool keep = row_ok && key <= q_pos && (window <= 0 || q_pos - key < window);
+          const float p = keep ? softmax_exp<T>(s[kb][e] - m_new) : 0.f;
+          s[kb][e] = p;
+          p_sum = p_sum + p;
+        }
+      p_sum = quad16_sum(p_sum);
+      cur.l = cur.l * alpha + p_sum;
+      cur.m = m_new;
+#pragma unroll
+      for (int blk = 0; blk < DB; ++blk)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) cur.acc[blk][e] = cur.acc[blk][e] * alpha;
+      // ---- O^T += V^T . P^T --------------------------------------------------
+      constexpr int KB16 = A::VEC / 4;
+#pragma unroll
+      for (int kb = 0; kb < NB; kb += KB16) {
+        vec_t pv;
+#pragma unroll
+        for (int h = 0; h < KB16; ++h)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) pv[h * 4 + e] = from_f32<T>(s[kb + h][e]);
+#pragma unroll
+        for (int blk = 0; blk < DB; ++blk) {
+          const int d = blk * 16 + row16;
+          vec_t vv;
+#pragma unroll
+          for (int h = 0; h < KB16; ++h) {
+            const int byte = ((kb + h) * 16 + 4 * g) * SZ;  // offset of the lane's four keys in the column row
+            const unsigned char* src = v_lds + d * VROW + (((byte >> 4) + d) % VPIECES) * 16 + (byte & 15);
+            if (SZ == 2) {
+              bf16x4 four = *reinterpret_cast<const bf16x4*>(src);
+#pragma unroll
+              for (int e = 0; e < 4; ++e) vv[h * 4 + e] = four[e];
+            } else {
+              f32x4 four = *reinterpret_cast<const f32x4*>(src);
+#pragma unroll
+              for (int e = 0; e < 4; ++e) vv[h * 4 + e] = four[e];
+            }
+          }
+          A::mma(cur.acc[blk], vv, pv);
+        }
+      }
+    }
+    if (direct && ((ti + 1) % TILES_PER_SPLIT == 0 || ti + 1 == ti_hi)) {
+      fold_split<T>(run, cur.acc, cur.m, cur.l);
+      cur.reset();
+    }
+  }
+
+  if (!row_ok) return;
+  if (direct) {
+    store_output<T>(run, out + (long)(sm.q_off + qi) * ldo + (long)head * D, g);
+  } else {
+    const int split = item.split_begin;
+    const long pr = item.part_base + ((long)kvh * rows_total + r) * item.n_splits + (split - item.split_lo);
+    float* pa = part_acc + pr * D;
+#pragma unroll
+    for (int blk = 0; blk < DB; ++blk) *reinterpret_cast<f32x4*>(pa + blk * 16 + 4 * g) = cur.acc[blk];
+    if (g == 0) {
+      part_ml[pr * 2] = cur.m;
+      part_ml[pr * 2 + 1] = cur.l;
+    }
+  }
+}
+
 struct CombineItem {
   int seq, row_block, part_base, n_splits;
 };
@@ -319,13 +580,35 @@ extern "C" int ls_attn_head_dim() { return D; }
 extern "C" int ls_attn_tile_keys() { return kTileKeys; }
 extern "C" int ls_attn_split_keys() { return kSplitKeys; }
 
+// Whether the staged kernel can have `bytes` of LDS: up to 64 KB always; above
+// that the function attribute is raised once per kernel (the device offers
+// 160 KB per workgroup); if that is refused the direct kernel runs instead.
+static bool staged_fits(int dtype, size_t bytes) {
+  if (bytes <= 64 * 1024) return true;
+  if (bytes > 160 * 1024) return false;
+  static int state[2] = {0, 0};  // 0 unknown, 1 granted, -1 refused
+  int& st = state[dtype == kF32 ? 0 : 1];
+  if (st == 0) {
+    hipError_t e = dtype == kF32
+        ? hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_staged_kernel<float, false>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes)
+        : hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_staged_kernel<bf16_t, true>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+    if (e != hipSuccess) (void)hipGetLastError();
+    st = e == hipSuccess ? 1 : -1;
+  }
+  return st == 1;
+}
+
+// variant: 0 picks the staged kernel where its tiles fit into LDS and the
+// direct one elsewhere, 1 forces the direct kernel, 2 the staged one.
 // q [tokens, ldq]: head h of a token at columns [h*D, (h+1)*D).  out likewise
 // with ldo.  k_pages [pages][nkv][page_size][D], v_pages [pages][nkv][D][page_size].
 // table [rows][table_stride] int32 (page id or -1).  items: n_items AttnItem.
 extern "C" int ls_attention(int dtype, const void* q, long ldq, const void* k_pages, const void* v_pages, int nkv,
                             int page_size, const int* table, int table_stride, const void* seqs, const void* items,
                             int n_items, void* out, long ldo, float* part_acc, float* part_ml, int G, float scale,
-                            int window, void* stream) {
+                            int window, int variant, void* stream) {
   LS_REQUIRE(n_items > 0 && nkv > 0 && G > 0, "attention: bad sizes (items %d, kv heads %d, group %d)", n_items, nkv, G);
   LS_REQUIRE(page_size >= 4 && page_size % 4 == 0 && kTileKeys % page_size == 0,
              "attention: page size %d must be a multiple of 4 that divides the key tile %d", page_size, kTileKeys);
@@ -336,17 +619,39 @@ extern "C" int ls_attention(int dtype, const void* q, long ldq, const void* k_pa
              "attention: operands must be 16-byte aligned");
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   dim3 grid(n_items, nkv);
-  if (dtype == kF32)
-    hipLaunchKernelGGL(attention_kernel<float>, grid, dim3(256), 0, s, (const float*)q, ldq, (const float*)k_pages,
-                       (const float*)v_pages, nkv, page_size, table, table_stride, (const SeqMeta*)seqs,
-                       (const AttnItem*)items, (float*)out, ldo, part_acc, part_ml, G, scale, window);
-  else if (dtype == kBF16)
-    hipLaunchKernelGGL(attention_kernel<bf16_t>, grid, dim3(256), 0, s, (const bf16_t*)q, ldq,
-                       (const bf16_t*)k_pages, (const bf16_t*)v_pages, nkv, page_size, table, table_stride,
-                       (const SeqMeta*)seqs, (const AttnItem*)items, (bf16_t*)out, ldo, part_acc, part_ml, G, scale,
-                       window);
-  else
+  int page_shift = 0;
+  while ((1 << page_shift) < page_size) ++page_shift;
+  LS_REQUIRE((1 << page_shift) == page_size, "attention: page size %d is not a power of two", page_size);
+  const size_t elem = dtype == kF32 ? 4 : 2;
+  const size_t lds_bytes = 2 * (size_t)kTileKeys * D * elem;
+  const bool staged = variant != 1 && staged_fits(dtype, lds_bytes);
+  LS_REQUIRE(variant != 2 || staged, "attention: the staged variant needs %zu bytes of LDS, which is not available",
+             lds_bytes);
+  if (dtype == kF32) {
+    if (staged)
+      hipLaunchKernelGGL((attention_staged_kernel<float, false>), grid, dim3(256), lds_bytes, s, (const float*)q,
+                         ldq, (const float*)k_pages, (const float*)v_pages, nkv, page_size, page_shift, table,
+                         table_stride, (const SeqMeta*)seqs, (const AttnItem*)items, (float*)out, ldo, part_acc,
+                         part_ml, G, scale, window);
+    else
+      hipLaunchKernelGGL(attention_direct_kernel<float>, grid, dim3(256), 0, s, (const float*)q, ldq,
+                         (const float*)k_pages, (const float*)v_pages, nkv, page_size, table, table_stride,
+                         (const SeqMeta*)seqs, (const AttnItem*)items, (float*)out, ldo, part_acc, part_ml, G, scale,
+                         window);
+  } else if (dtype == kBF16) {
+    if (staged)
+      hipLaunchKernelGGL((attention_staged_kernel<bf16_t, true>), grid, dim3(256), lds_bytes, s, (const bf16_t*)q,
+                         ldq, (const bf16_t*)k_pages, (const bf16_t*)v_pages, nkv, page_size, page_shift, table,
+                         table_stride, (const SeqMeta*)seqs, (const AttnItem*)items, (bf16_t*)out, ldo, part_acc,
+                         part_ml, G, scale, window);
+    else
+      hipLaunchKernelGGL(attention_direct_kernel<bf16_t>, grid, dim3(256), 0, s, (const bf16_t*)q, ldq,
+                         (const bf16_t*)k_pages, (const bf16_t*)v_pages, nkv, page_size, table, table_stride,
+                         (const SeqMeta*)seqs, (const AttnItem*)items, (bf16_t*)out, ldo, part_acc, part_ml, G, scale,
+                         window);
+  } else {
     return fail("attention: unknown dtype %d", dtype);
+  }
   return check_launch("attention");
 }
 

@@ -204,8 +204,9 @@ class Kernels:
 
     def attention(self, q: torch.Tensor, nq: int, nkv: int, d: int, k_pages, v_pages, page_size: int, table,
                   seqs, items, n_items: int, out: torch.Tensor, part_acc, part_ml, scale: float,
-                  window: int) -> None:
-        """Launch the attention kernel over ``n_items`` work items (see attention.hip)."""
+                  window: int, variant: int = 0) -> None:
+        """Launch the attention kernel over ``n_items`` work items (see attention.hip).
+        ``variant``: 0 staged through LDS where it fits, 1 direct from global memory, 2 staged or error."""
         lib = self.attention_lib(d)
         _rows_ok(q, "attention q"); _rows_ok(out, "attention out")
         _need(q.dtype in DTYPE_CODE and out.dtype == q.dtype, "attention q/out dtype")
@@ -223,7 +224,7 @@ class Kernels:
             c_int(DTYPE_CODE[q.dtype]), _ptr(q), c_long(q.stride(0)), _ptr(k_pages), _ptr(v_pages), c_int(nkv),
             c_int(page_size), _ptr(table), c_int(table.shape[1]), _ptr(seqs), _ptr(items), c_int(n_items),
             _ptr(out), c_long(out.stride(0)), _ptr(part_acc), _ptr(part_ml), c_int(nq // nkv), c_float(scale),
-            c_int(window), _stream())
+            c_int(window), c_int(variant), _stream())
         self._check(lib, code)
 
     def attention_combine(self, d: int, seqs, items, n_items: int, nq: int, nkv: int, part_acc, part_ml,

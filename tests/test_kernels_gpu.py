@@ -195,7 +195,7 @@ class PagedCase:
         K().qk_rope_kv(qkv, t, self.nq, self.nkv, self.d, q_norm, k_norm, eps, cos, sin, rot, tok_seq, tok_pos,
                        self.seqs(q_start, t), q_start + t - 1, self.table, self.k_pages, self.v_pages, self.ps, True)
 
-    def attend(self, qkv, q_start, scale, window=0, force_split=None):
+    def attend(self, qkv, q_start, scale, window=0, force_split=None, variant=0):
         from lockstep_amd.ops import kernels
 
         t = qkv.shape[0]
@@ -225,7 +225,8 @@ class PagedCase:
         part_acc = torch.full((max(part_rows, 1), self.d), float("nan"), dtype=torch.float32, device="cuda")
         part_ml = torch.full((max(part_rows, 1), 2), float("nan"), dtype=torch.float32, device="cuda")
         K().attention(qkv, self.nq, self.nkv, self.d, self.k_pages, self.v_pages, self.ps, self.table,
-                      self.seqs(q_start, t), items_t, len(items) // 8, out, part_acc, part_ml, scale, window)
+                      self.seqs(q_start, t), items_t, len(items) // 8, out, part_acc, part_ml, scale, window,
+                      variant)
         if combine:
             comb = torch.tensor(combine, dtype=torch.int32).cuda()
             K().attention_combine(self.d, self.seqs(q_start, t), comb, len(combine) // 4, self.nq, self.nkv,
@@ -270,6 +271,8 @@ def test_prefill_attention_matches_naive(dtype, nq, nkv, d, ps, kv_len):
     want = naive_attention(q, k, v, 0, d ** -0.5)
     assert not torch.isnan(out).any()
     assert rel_err(out, want) < ATT_TOL[dtype]
+    # the kernel that loads straight from global memory gives the same bits as the LDS-staged one
+    assert torch.equal(case.attend(dev, 0, d ** -0.5, variant=1), out)
     if kv_len == 1:
         assert torch.equal(out.cpu().float()[0], v.float()[0].repeat_interleave(nq // nkv, dim=0))
 
@@ -290,6 +293,8 @@ def test_attention_row_is_the_same_alone_in_a_portion_and_in_the_whole_prompt(dt
     for p in (0, 1, 15, 16, 17, 127, 128, 255, 256, 257, 511, 512, 699):
         alone = whole.attend(qkv[p:p + 1], p, d ** -0.5)
         assert torch.equal(alone[0], full[p]), f"row {p} alone"
+        alone = whole.attend(qkv[p:p + 1], p, d ** -0.5, variant=1)
+        assert torch.equal(alone[0], full[p]), f"row {p} alone, loaded directly"
         both = whole.attend(qkv[p:p + 1], p, d ** -0.5, force_split=False)
         assert torch.equal(both[0], full[p]), f"row {p} alone, direct"
     for lo, hi in ((250, 262), (0, 3), (500, 700), (255, 257), (690, 700)):
@@ -311,6 +316,7 @@ def test_attention_window(dtype, window):
     q, k, v = split_qkv(qkv.double(), nq, nkv, d)
     want = naive_attention(q, k, v, 0, d ** -0.5, window=window)
     assert rel_err(out, want) < ATT_TOL[dtype]
+    assert torch.equal(case.attend(dev, 0, d ** -0.5, window=window, variant=1), out)
     # pages behind the window may be gone: mark them released and decode the last rows
     for p in (kv_len - 1, 300, 130):
         first_needed = max(0, p - window + 1) // ps
