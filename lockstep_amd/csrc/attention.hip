@@ -13,6 +13,8 @@
 // in ascending order with the online softmax
 //     m' = max(m, rowmax(s)); a = exp(m - m'); p = exp(s - m') (0 if masked);
 //     l = l*a + sum(p); acc = acc*a + round(p) . V
+// (sum(p): a lane adds its four keys of a 16-key block as (p0+p1)+(p2+p3),
+// the eight blocks in ascending order, then the four lanes of the row)
 // and the splits are folded in ascending order with
 //     m' = max(M, m); A = exp(M - m'); B = exp(m - m');
 //     ACC = ACC*A + acc*B; L = L*A + l*B
@@ -43,6 +45,9 @@
 namespace ls {
 
 constexpr int D = LS_HEAD_DIM;
+#ifndef LS_STAGED_MIN_BLOCKS
+#define LS_STAGED_MIN_BLOCKS 1
+#endif
 static_assert(D % 16 == 0 && D >= 16 && D <= 256, "head size must be a multiple of 16 up to 256");
 constexpr int kTileKeys = 128;
 constexpr int kSplitKeys = 256;
@@ -173,7 +178,7 @@ __global__ __launch_bounds__(256) void attention_direct_kernel(
         bool key_ok = key < sm.kv_len && key >= lo_valid && key <= wave_last_pos;
         long page = key_ok ? tbl[key / page_size] : -1;
         key_ok = key_ok && page >= 0;
-        const T* krow = k_pages + ((page * nkv + kvh) * page_size + key % page_size) * D;
+        const T* krow = k_pages + (key_ok ? ((page * nkv + kvh) * page_size + key % page_size) * D : 0);
 #pragma unroll
         for (int c = 0; c < NC; ++c) {
           vec_t kv = load_vec<T>(krow, 0, c * A::KCHUNK + g * A::VEC, D, 0, key_ok, true);
@@ -199,15 +204,15 @@ __global__ __launch_bounds__(256) void attention_direct_kernel(
       const float alpha = softmax_exp<T>(cur.m - m_new);
       float p_sum = 0.f;
 #pragma unroll
-      for (int kb = 0; kb < NB; ++kb)
+      for (int kb = 0; kb < NB; ++kb) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           const int key = t0 + kb * 16 + 4 * g + e;
           const bool keep = row_ok && key <= q_pos && (window <= 0 || q_pos - key < window);
-          const float p = keep ? softmax_exp<T>(s[kb][e] - m_new) : 0.f;
-          s[kb][e] = p;
-          p_sum = p_sum + p;
+          s[kb][e] = keep ? softmax_exp<T>(s[kb][e] - m_new) : 0.f;
         }
+        p_sum = p_sum + ((s[kb][0] + s[kb][1]) + (s[kb][2] + s[kb][3]));
+      }
       p_sum = quad16_sum(p_sum);
       cur.l = cur.l * alpha + p_sum;
       cur.m = m_new;
@@ -290,7 +295,7 @@ __global__ __launch_bounds__(256) void attention_direct_kernel(
 // 16-byte pieces of a row are rotated by the row index so that the 16 rows an
 // MFMA operand touches fall into different banks.
 template <typename T, bool PREFETCH>
-__global__ __launch_bounds__(256) void attention_staged_kernel(
+__global__ __launch_bounds__(256, LS_STAGED_MIN_BLOCKS) void attention_staged_kernel(
     const T* __restrict__ q, long ldq, const T* __restrict__ k_pages, const T* __restrict__ v_pages, int nkv,
     int page_size, int page_shift, const int* __restrict__ table, int table_stride,
     const SeqMeta* __restrict__ seqs, const AttnItem* __restrict__ items, T* __restrict__ out, long ldo,
@@ -351,6 +356,21 @@ __global__ __launch_bounds__(256) void attention_staged_kernel(
 
   // Without prefetch the pieces go through registers a few at a time.
   constexpr int GROUP = PREFETCH ? PER : (PER < 4 ? PER : 4);
+  // Page ids are looked up one tile ahead of the data they address, so the
+  // two dependent loads of a tile do not wait for each other.
+  int kpage[PER], vpage[PER];
+  auto lookup = [&](int ti) {
+    const int t0 = ti * kTileKeys;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const int p = threadIdx.x + 256 * i;
+      const int key = t0 + p / KPIECES;
+      kpage[i] = tbl[min(key, sm.kv_len - 1) >> page_shift];
+      const int q1 = p >> vshift;
+      const int key0 = t0 + ((q1 / D) << page_shift) + ((p & ((1 << vshift) - 1)) << LOG_VEC);
+      vpage[i] = tbl[min(key0, sm.kv_len - 1) >> page_shift];
+    }
+  };
   vec_t kreg[GROUP], vreg[GROUP];
   auto fetch = [&](int ti, int i0) {
     const int t0 = ti * kTileKeys;
@@ -365,7 +385,7 @@ __global__ __launch_bounds__(256) void attention_staged_kernel(
         const int piece = p % KPIECES;
         const int key = t0 + kt;
         bool ok = (TOTAL % 256 == 0 || p < TOTAL) && key < sm.kv_len && key >= lo_valid;
-        int page = tbl[min(key, sm.kv_len - 1) >> page_shift];
+        int page = kpage[i];
         ok = ok && page >= 0;
         page = max(page, 0);
         const int slot = min(key, sm.kv_len - 1) & (page_size - 1);
@@ -381,7 +401,7 @@ __global__ __launch_bounds__(256) void attention_staged_kernel(
         const int d = q1 % D;
         const int key0 = t0 + (pg << page_shift) + (kp << LOG_VEC);
         bool ok = (TOTAL % 256 == 0 || p < TOTAL) && key0 < sm.kv_len && key0 + A::VEC > lo_valid;
-        int page = tbl[min(key0, sm.kv_len - 1) >> page_shift];
+        int page = vpage[i];
         ok = ok && page >= 0;
         page = max(page, 0);
         const T* src = v_pages + ((((long)page * nkv + kvh) * D + d) << page_shift) + (kp << LOG_VEC);
@@ -416,7 +436,11 @@ __global__ __launch_bounds__(256) void attention_staged_kernel(
   run.reset();
   cur.reset();
 
-  if (PREFETCH && ti_lo < ti_hi) fetch(ti_lo, 0);
+  if (ti_lo < ti_hi) lookup(ti_lo);
+  if (PREFETCH && ti_lo < ti_hi) {
+    fetch(ti_lo, 0);
+    if (ti_lo + 1 < ti_hi) lookup(ti_lo + 1);
+  }
   for (int ti = ti_lo; ti < ti_hi; ++ti) {
     const int t0 = ti * kTileKeys;
     __syncthreads();  // the previous tile has been read by every wave
@@ -427,10 +451,17 @@ __global__ __launch_bounds__(256) void attention_staged_kernel(
         fetch(ti, i0);
         stash(i0);
       }
+      if (ti + 1 < ti_hi) lookup(ti + 1);
     }
     __syncthreads();
-    if (PREFETCH && ti + 1 < ti_hi) fetch(ti + 1, 0);
+    if (PREFETCH && ti + 1 < ti_hi) {
+      fetch(ti + 1, 0);
+      if (ti + 2 < ti_hi) lookup(ti + 2);
+    }
 
+#ifdef LS_EXP
+    if (LS_EXP & 1) continue;
+#endif
     const bool mine = wave_active && t0 <= wave_last_pos &&
                       !(window > 0 && t0 + kTileKeys <= wave_first_pos - window + 1);
     if (mine) {
@@ -466,15 +497,15 @@ __global__ __launch_bounds__(256) void attention_staged_kernel(
       const float alpha = softmax_exp<T>(cur.m - m_new);
       float p_sum = 0.f;
 #pragma unroll
-      for (int kb = 0; kb < NB; ++kb)
+      for (int kb = 0; kb < NB; ++kb) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           const int key = t0 + kb * 16 + 4 * g + e;
           const bool keep = row_ok && key <= q_pos && (window <= 0 || q_pos - key < window);
-          const float p = keep ? softmax_exp<T>(s[kb][e] - m_new) : 0.f;
-          s[kb][e] = p;
-          p_sum = p_sum + p;
+          s[kb][e] = keep ? softmax_exp<T>(s[kb][e] - m_new) : 0.f;
         }
+        p_sum = p_sum + ((s[kb][0] + s[kb][1]) + (s[kb][2] + s[kb][3]));
+      }
       p_sum = quad16_sum(p_sum);
       cur.l = cur.l * alpha + p_sum;
       cur.m = m_new;
@@ -535,6 +566,305 @@ __global__ __launch_bounds__(256) void attention_staged_kernel(
   }
 }
 
+
+// Variant 3, "cooperative": for work items with at most 16 rows (one decoded
+// token per request and up to 16 query heads per kv head), where the staged
+// kernel would leave three of its four waves idle.  All four waves hold the
+// same 16 rows.  Wave w computes the score blocks 2w and 2w+1 of a tile and
+// the output columns of the blocks w, w+4, ...; row maxima, per-block sums and
+// probabilities meet in LDS.  Every number is produced by the same
+// instruction sequence as in the other variants, so the bits are the same.
+// STAGE tiles (a whole split when it fits) are fetched at once.
+template <typename T, int STAGE>
+__global__ __launch_bounds__(256) void attention_coop_kernel(
+    const T* __restrict__ q, long ldq, const T* __restrict__ k_pages, const T* __restrict__ v_pages, int nkv,
+    int page_size, int page_shift, const int* __restrict__ table, int table_stride,
+    const SeqMeta* __restrict__ seqs, const AttnItem* __restrict__ items, T* __restrict__ out, long ldo,
+    float* __restrict__ part_acc, float* __restrict__ part_ml, int G, float scale, int window) {
+  typedef Atom<T> A;
+  typedef typename A::vec_t vec_t;
+  constexpr int SZ = sizeof(T);
+  constexpr int NC = (D + A::KCHUNK - 1) / A::KCHUNK;
+  constexpr int KROW = D * SZ;
+  constexpr int KPIECES = KROW / 16;
+  constexpr int VROW = kTileKeys * SZ;
+  constexpr int VPIECES = VROW / 16;
+  constexpr int TOTAL = kTileKeys * KPIECES;
+  constexpr int PER = (TOTAL + 255) / 256;
+  constexpr int TILES_PER_SPLIT = kSplitKeys / kTileKeys;
+  constexpr int LOG_VEC = (A::VEC == 8) ? 3 : 2;
+  constexpr int TILE_BYTES = 2 * kTileKeys * KROW;  // K tile + V tile
+  constexpr int MYDB = (DB + 3) / 4;                 // output blocks of one wave
+
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+  float* wmax = reinterpret_cast<float*>(lds + STAGE * TILE_BYTES);  // [4][16]
+  float* psum = wmax + 64;                                            // [NB][64]
+  f32x4* prob = reinterpret_cast<f32x4*>(psum + NB * 64);             // [NB][64]
+
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const AttnItem item = items[blockIdx.x];
+  const SeqMeta sm = seqs[item.seq];
+  const int kvh = blockIdx.y;
+  const int rows_total = sm.q_len * G;  // <= 16, checked on the host
+  const int row16 = lane & 15;
+  const int g = lane >> 4;
+  const int r = row16;
+  const bool row_ok = r < rows_total;
+  const int qi = row_ok ? r / G : 0;
+  const int head = kvh * G + (row_ok ? r % G : 0);
+  const int q_pos = sm.q_start + qi;
+  const int first_pos = sm.q_start;
+  const int last_pos = sm.q_start + (rows_total - 1) / G;
+  const int lo_valid = window > 0 ? max(0, sm.q_start - window + 1) : 0;
+  const int* __restrict__ tbl = table + (long)sm.table_row * table_stride;
+  const bool direct = item.part_base < 0;
+  const int vshift = page_shift - LOG_VEC;
+
+  vec_t qv[NC];
+#pragma unroll
+  for (int c = 0; c < NC; ++c)
+    qv[c] = load_vec<T>(q + (long)head * D, sm.q_off + qi, c * A::KCHUNK + g * A::VEC, D, ldq, row_ok, true);
+
+  int ti_lo = item.split_begin * TILES_PER_SPLIT;
+  if (window > 0) ti_lo = max(ti_lo, max(0, first_pos - window + 1) / kTileKeys);
+  const int ti_hi = min(item.split_end * TILES_PER_SPLIT, last_pos / kTileKeys + 1);
+
+  // a wave keeps only its own output blocks: block j of the arrays is column block wave + 4j
+  f32x4 cur_acc[MYDB], run_acc[MYDB];
+  float cur_m = kNegSentinel, cur_l = 0.f, run_m = kNegSentinel, run_l = 0.f;
+#pragma unroll
+  for (int j = 0; j < MYDB; ++j) {
+    cur_acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+    run_acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+
+  for (int tb = ti_lo; tb < ti_hi; tb += STAGE) {
+    // ---- fetch STAGE tiles: all page ids, then all data, then LDS ------------
+    int kpage[STAGE][PER], vpage[STAGE][PER];
+#pragma unroll
+    for (int st = 0; st < STAGE; ++st) {
+      const int t0 = (tb + st) * kTileKeys;
+#pragma unroll
+      for (int i = 0; i < PER; ++i) {
+        const int p = threadIdx.x + 256 * i;
+        const int key = t0 + p / KPIECES;
+        kpage[st][i] = tbl[min(key, sm.kv_len - 1) >> page_shift];
+        const int q1 = p >> vshift;
+        const int key0 = t0 + ((q1 / D) << page_shift) + ((p & ((1 << vshift) - 1)) << LOG_VEC);
+        vpage[st][i] = tbl[min(key0, sm.kv_len - 1) >> page_shift];
+      }
+    }
+    vec_t kreg[STAGE][PER], vreg[STAGE][PER];
+#pragma unroll
+    for (int st = 0; st < STAGE; ++st) {
+      const int t0 = (tb + st) * kTileKeys;
+      const bool tile_in = tb + st < ti_hi;
+#pragma unroll
+      for (int i = 0; i < PER; ++i) {
+        const int p = threadIdx.x + 256 * i;
+        {
+          const int kt = p / KPIECES;
+          const int piece = p % KPIECES;
+          const int key = t0 + kt;
+          int page = kpage[st][i];
+          const bool ok = tile_in && key < sm.kv_len && key >= lo_valid && page >= 0;
+          page = max(page, 0);
+          const int slot = min(key, sm.kv_len - 1) & (page_size - 1);
+          const T* src = k_pages + (((long)page * nkv + kvh) * page_size + slot) * D + piece * A::VEC;
+          vec_t v = *reinterpret_cast<const vec_t*>(src);
+          kreg[st][i] = ok ? v : A::zero();
+        }
+        {
+          const int q1 = p >> vshift;
+          const int kp = p & ((1 << vshift) - 1);
+          const int pg = q1 / D;
+          const int d = q1 % D;
+          const int key0 = t0 + (pg << page_shift) + (kp << LOG_VEC);
+          int page = vpage[st][i];
+          const bool ok = tile_in && key0 < sm.kv_len && key0 + A::VEC > lo_valid && page >= 0;
+          page = max(page, 0);
+          const T* src = v_pages + ((((long)page * nkv + kvh) * D + d) << page_shift) + (kp << LOG_VEC);
+          vec_t v = *reinterpret_cast<const vec_t*>(src);
+#pragma unroll
+          for (int e = 0; e < A::VEC; ++e)
+            if (!ok || key0 + e >= sm.kv_len || key0 + e < lo_valid) v[e] = 0;
+          vreg[st][i] = v;
+        }
+      }
+    }
+    __syncthreads();  // the previous stage has been consumed
+#pragma unroll
+    for (int st = 0; st < STAGE; ++st) {
+      unsigned char* k_lds = lds + st * TILE_BYTES;
+      unsigned char* v_lds = k_lds + kTileKeys * KROW;
+#pragma unroll
+      for (int i = 0; i < PER; ++i) {
+        const int p = threadIdx.x + 256 * i;
+        const int kt = p / KPIECES;
+        const int piece = p % KPIECES;
+        *reinterpret_cast<vec_t*>(k_lds + kt * KROW + ((piece + kt) % KPIECES) * 16) = kreg[st][i];
+        const int q1 = p >> vshift;
+        const int kp = p & ((1 << vshift) - 1);
+        const int pg = q1 / D;
+        const int d = q1 % D;
+        const int vpiece = (pg << vshift) + kp;
+        *reinterpret_cast<vec_t*>(v_lds + d * VROW + ((vpiece + d) % VPIECES) * 16) = vreg[st][i];
+      }
+    }
+    __syncthreads();
+
+    // ---- the tiles of this stage ------------------------------------------------
+    for (int st = 0; st < STAGE; ++st) {
+      const int ti = tb + st;
+      if (ti >= ti_hi) break;
+      const int t0 = ti * kTileKeys;
+      const unsigned char* k_lds = lds + st * TILE_BYTES;
+      const unsigned char* v_lds = k_lds + kTileKeys * KROW;
+
+      // score blocks 2w and 2w+1
+      f32x4 s[2];
+      float my_max = kNegSentinel;
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const int kb = 2 * wave + j;
+        s[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+        const int row = kb * 16 + row16;
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+          const int piece = c * 4 + g;
+          vec_t kv = A::zero();
+          if (piece < KPIECES)
+            kv = *reinterpret_cast<const vec_t*>(k_lds + row * KROW + ((piece + row) % KPIECES) * 16);
+          A::mma(s[j], kv, qv[c]);
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int key = t0 + kb * 16 + 4 * g + e;
+          const bool keep = row_ok && key <= q_pos && (window <= 0 || q_pos - key < window);
+          const float v = keep ? s[j][e] * scale : kNegSentinel;
+          s[j][e] = v;
+          my_max = fmaxf(my_max, v);
+        }
+      }
+      my_max = quad16_max(my_max);
+      if (g == 0) wmax[wave * 16 + row16] = my_max;
+      __syncthreads();
+      const float tile_max = fmaxf(fmaxf(wmax[row16], wmax[16 + row16]), fmaxf(wmax[32 + row16], wmax[48 + row16]));
+      const float m_new = fmaxf(cur_m, tile_max);
+      const float alpha = softmax_exp<T>(cur_m - m_new);
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const int kb = 2 * wave + j;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int key = t0 + kb * 16 + 4 * g + e;
+          const bool keep = row_ok && key <= q_pos && (window <= 0 || q_pos - key < window);
+          s[j][e] = keep ? softmax_exp<T>(s[j][e] - m_new) : 0.f;
+        }
+        psum[kb * 64 + lane] = (s[j][0] + s[j][1]) + (s[j][2] + s[j][3]);
+        prob[kb * 64 + lane] = s[j];
+      }
+      __syncthreads();
+      float p_sum = 0.f;
+#pragma unroll
+      for (int kb = 0; kb < NB; ++kb) p_sum = p_sum + psum[kb * 64 + lane];
+      p_sum = quad16_sum(p_sum);
+      cur_l = cur_l * alpha + p_sum;
+      cur_m = m_new;
+#pragma unroll
+      for (int j = 0; j < MYDB; ++j)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) cur_acc[j][e] = cur_acc[j][e] * alpha;
+      constexpr int KB16 = A::VEC / 4;
+#pragma unroll
+      for (int kb = 0; kb < NB; kb += KB16) {
+        vec_t pv;
+#pragma unroll
+        for (int h = 0; h < KB16; ++h) {
+          const f32x4 four = prob[(kb + h) * 64 + lane];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) pv[h * 4 + e] = from_f32<T>(four[e]);
+        }
+#pragma unroll
+        for (int j = 0; j < MYDB; ++j) {
+          const int blk = wave + 4 * j;
+          if (blk >= DB) continue;
+          const int d = blk * 16 + row16;
+          vec_t vv;
+#pragma unroll
+          for (int h = 0; h < KB16; ++h) {
+            const int byte = ((kb + h) * 16 + 4 * g) * SZ;
+            const unsigned char* src = v_lds + d * VROW + (((byte >> 4) + d) % VPIECES) * 16 + (byte & 15);
+            if (SZ == 2) {
+              bf16x4 four = *reinterpret_cast<const bf16x4*>(src);
+#pragma unroll
+              for (int e = 0; e < 4; ++e) vv[h * 4 + e] = four[e];
+            } else {
+              f32x4 four = *reinterpret_cast<const f32x4*>(src);
+#pragma unroll
+              for (int e = 0; e < 4; ++e) vv[h * 4 + e] = four[e];
+            }
+          }
+          A::mma(cur_acc[j], vv, pv);
+        }
+      }
+      if (direct && ((ti + 1) % TILES_PER_SPLIT == 0 || ti + 1 == ti_hi)) {
+        if (cur_l > 0.f) {  // the fold of fold_split, on this wave's blocks
+          const float m_fold = fmaxf(run_m, cur_m);
+          const float fa = softmax_exp<T>(run_m - m_fold);
+          const float fb = softmax_exp<T>(cur_m - m_fold);
+#pragma unroll
+          for (int j = 0; j < MYDB; ++j)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) run_acc[j][e] = run_acc[j][e] * fa + cur_acc[j][e] * fb;
+          run_l = run_l * fa + cur_l * fb;
+          run_m = m_fold;
+        }
+#pragma unroll
+        for (int j = 0; j < MYDB; ++j) cur_acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+        cur_m = kNegSentinel;
+        cur_l = 0.f;
+      }
+    }
+  }
+
+  if (!row_ok) return;
+  if (direct) {
+    T* dst = out + (long)(sm.q_off + qi) * ldo + (long)head * D;
+    const float l = run_l;
+#pragma unroll
+    for (int j = 0; j < MYDB; ++j) {
+      const int blk = wave + 4 * j;
+      if (blk >= DB) continue;
+      float o[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) o[e] = l > 0.f ? run_acc[j][e] / l : 0.f;
+      T* p = dst + blk * 16 + 4 * g;
+      if (SZ == 2) {
+        bf16x4 v;
+        v[0] = (bf16_t)o[0]; v[1] = (bf16_t)o[1]; v[2] = (bf16_t)o[2]; v[3] = (bf16_t)o[3];
+        *reinterpret_cast<bf16x4*>(p) = v;
+      } else {
+        *reinterpret_cast<f32x4*>(p) = f32x4{o[0], o[1], o[2], o[3]};
+      }
+    }
+  } else {
+    const int split = item.split_begin;
+    const long pr = item.part_base + ((long)kvh * rows_total + r) * item.n_splits + (split - item.split_lo);
+    float* pa = part_acc + pr * D;
+#pragma unroll
+    for (int j = 0; j < MYDB; ++j) {
+      const int blk = wave + 4 * j;
+      if (blk < DB) *reinterpret_cast<f32x4*>(pa + blk * 16 + 4 * g) = cur_acc[j];
+    }
+    if (wave == 0 && g == 0) {
+      part_ml[pr * 2] = cur_m;
+      part_ml[pr * 2 + 1] = cur_l;
+    }
+  }
+}
+
 struct CombineItem {
   int seq, row_block, part_base, n_splits;
 };
@@ -579,6 +909,9 @@ using namespace ls;
 extern "C" int ls_attn_head_dim() { return D; }
 extern "C" int ls_attn_tile_keys() { return kTileKeys; }
 extern "C" int ls_attn_split_keys() { return kSplitKeys; }
+static bool coop_supported(int dtype);
+// 1 if the cooperative kernel (work items of at most 16 rows) can run for this dtype.
+extern "C" int ls_attn_coop_supported(int dtype) { return coop_supported(dtype) ? 1 : 0; }
 
 // Whether the staged kernel can have `bytes` of LDS: up to 64 KB always; above
 // that the function attribute is raised once per kernel (the device offers
@@ -600,6 +933,36 @@ static bool staged_fits(int dtype, size_t bytes) {
   return st == 1;
 }
 
+// The cooperative kernel stages two tiles (a whole split) when they fit into
+// 160 KB together with its exchange buffers, else one.
+constexpr size_t kCoopExtra = 64 * 4 + NB * 64 * 4 + NB * 64 * 16;
+constexpr size_t kLdsLimit = 160 * 1024;
+constexpr int coop_stage(size_t elem) { return 2 * (2 * kTileKeys * D * elem) + kCoopExtra <= kLdsLimit ? 2 : 1; }
+constexpr int kCoopStageF32 = coop_stage(4);
+constexpr int kCoopStageBF16 = coop_stage(2);
+static size_t coop_lds_bytes(int dtype) {
+  const size_t elem = dtype == kF32 ? 4 : 2;
+  return (dtype == kF32 ? kCoopStageF32 : kCoopStageBF16) * (2 * (size_t)kTileKeys * D * elem) + kCoopExtra;
+}
+static bool coop_supported(int dtype) {
+  const size_t bytes = coop_lds_bytes(dtype);
+  if (bytes > kLdsLimit) return false;
+  if (bytes <= 64 * 1024) return true;
+  static int state[2] = {0, 0};
+  int& st = state[dtype == kF32 ? 0 : 1];
+  if (st == 0) {
+    hipError_t e = dtype == kF32
+        ? hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_coop_kernel<float, kCoopStageF32>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes)
+        : hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_coop_kernel<bf16_t, kCoopStageBF16>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+    if (e != hipSuccess) (void)hipGetLastError();
+    st = e == hipSuccess ? 1 : -1;
+  }
+  return st == 1;
+}
+
+// variant: 3 runs the cooperative kernel (all items must have at most 16 rows);
 // variant: 0 picks the staged kernel where its tiles fit into LDS and the
 // direct one elsewhere, 1 forces the direct kernel, 2 the staged one.
 // q [tokens, ldq]: head h of a token at columns [h*D, (h+1)*D).  out likewise
@@ -608,7 +971,7 @@ static bool staged_fits(int dtype, size_t bytes) {
 extern "C" int ls_attention(int dtype, const void* q, long ldq, const void* k_pages, const void* v_pages, int nkv,
                             int page_size, const int* table, int table_stride, const void* seqs, const void* items,
                             int n_items, void* out, long ldo, float* part_acc, float* part_ml, int G, float scale,
-                            int window, int variant, void* stream) {
+                            int window, int variant, int max_rows, void* stream) {
   LS_REQUIRE(n_items > 0 && nkv > 0 && G > 0, "attention: bad sizes (items %d, kv heads %d, group %d)", n_items, nkv, G);
   LS_REQUIRE(page_size >= 4 && page_size % 4 == 0 && kTileKeys % page_size == 0,
              "attention: page size %d must be a multiple of 4 that divides the key tile %d", page_size, kTileKeys);
@@ -624,6 +987,25 @@ extern "C" int ls_attention(int dtype, const void* q, long ldq, const void* k_pa
   LS_REQUIRE((1 << page_shift) == page_size, "attention: page size %d is not a power of two", page_size);
   const size_t elem = dtype == kF32 ? 4 : 2;
   const size_t lds_bytes = 2 * (size_t)kTileKeys * D * elem;
+  if (variant == 3) {
+    LS_REQUIRE(max_rows <= 16, "attention: the cooperative variant takes work items of at most 16 rows, got %d",
+               max_rows);
+    LS_REQUIRE(coop_supported(dtype), "attention: the cooperative variant does not fit into LDS for this head size");
+    const size_t bytes = coop_lds_bytes(dtype);
+    if (dtype == kF32)
+      hipLaunchKernelGGL((attention_coop_kernel<float, kCoopStageF32>), grid, dim3(256), bytes, s, (const float*)q,
+                         ldq, (const float*)k_pages, (const float*)v_pages, nkv, page_size, page_shift, table,
+                         table_stride, (const SeqMeta*)seqs, (const AttnItem*)items, (float*)out, ldo, part_acc,
+                         part_ml, G, scale, window);
+    else if (dtype == kBF16)
+      hipLaunchKernelGGL((attention_coop_kernel<bf16_t, kCoopStageBF16>), grid, dim3(256), bytes, s,
+                         (const bf16_t*)q, ldq, (const bf16_t*)k_pages, (const bf16_t*)v_pages, nkv, page_size,
+                         page_shift, table, table_stride, (const SeqMeta*)seqs, (const AttnItem*)items, (bf16_t*)out,
+                         ldo, part_acc, part_ml, G, scale, window);
+    else
+      return fail("attention: unknown dtype %d", dtype);
+    return check_launch("attention (cooperative)");
+  }
   const bool staged = variant != 1 && staged_fits(dtype, lds_bytes);
   LS_REQUIRE(variant != 2 || staged, "attention: the staged variant needs %zu bytes of LDS, which is not available",
              lds_bytes);

@@ -74,18 +74,24 @@ template <> struct Atom<float> {
 
 // Load VEC elements of row `row` at element offset `k` of a row-major matrix
 // with `ld` elements per row, zero where the row is not `ok` or k >= limit.
-// `aligned` (uniform) says every row start and k are 16-byte aligned.
+// `aligned` (uniform) says every row start and k are 16-byte aligned and
+// limit is a multiple of VEC; the load is then unconditional (from a clamped
+// address) and the zero is selected afterwards, so a run of such loads can
+// be in flight together.
 template <typename T>
 __device__ __forceinline__ typename Atom<T>::vec_t load_vec(const T* __restrict__ base, long row, int k,
                                                             int limit, long ld, bool ok, bool aligned) {
   typedef typename Atom<T>::vec_t vec_t;
   constexpr int VEC = Atom<T>::VEC;
+  const bool valid = ok && k < limit;
+  if (aligned) {
+    const T* p = base + (valid ? row * ld + k : 0);
+    vec_t v = *reinterpret_cast<const vec_t*>(p);
+    return valid ? v : Atom<T>::zero();
+  }
   vec_t v = Atom<T>::zero();
-  if (!ok || k >= limit) return v;
-  const T* p = base + row * ld + k;
-  if (aligned && k + VEC <= limit) {
-    v = *reinterpret_cast<const vec_t*>(p);
-  } else {
+  if (valid) {
+    const T* p = base + row * ld + k;
 #pragma unroll
     for (int e = 0; e < VEC; ++e)
       if (k + e < limit) v[e] = p[e];

@@ -93,14 +93,23 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const T* __restric
     for (int j = 0; j < MT; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
     const int k_begin = s * kslice;
     const int k_end = min(K, k_begin + kslice);
-    for (int k0 = k_begin; k0 < k_end; k0 += A::KCHUNK) {
-      const int k = k0 + g * A::VEC;
-      vec_t w = load_vec<T>(W, n, k, K, K, n_ok, aligned);
+    // Four chunks at a time: all their loads are issued before the first
+    // MFMA needs one, so a wave keeps several kilobytes in flight.
+    for (int k0 = k_begin; k0 < k_end; k0 += 4 * A::KCHUNK) {
+      vec_t w[4], x[MT][4];
 #pragma unroll
-      for (int j = 0; j < MT; ++j) {
-        const int m = j * 16 + row16;
-        vec_t x = load_vec<T>(X, m, k, K, ldx, m < M, aligned);
-        A::mma(acc[j], w, x);
+      for (int u = 0; u < 4; ++u) {
+        const int k = k0 + u * A::KCHUNK + g * A::VEC;
+        const bool in = k0 + u * A::KCHUNK < k_end;
+        w[u] = load_vec<T>(W, n, k, K, K, n_ok && in, aligned);
+#pragma unroll
+        for (int j = 0; j < MT; ++j) x[j][u] = load_vec<T>(X, j * 16 + row16, k, K, ldx, j * 16 + row16 < M && in, aligned);
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        if (k0 + u * A::KCHUNK >= k_end) break;  // uniform: a chunk is visited iff it starts inside the slice
+#pragma unroll
+        for (int j = 0; j < MT; ++j) A::mma(acc[j], w[u], x[j][u]);
       }
     }
 #pragma unroll

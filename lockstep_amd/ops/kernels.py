@@ -72,6 +72,10 @@ class Kernels:
             self.attention_paths[head_dim] = str(path)
         return lib
 
+    def coop_supported(self, head_dim: int, dtype: torch.dtype) -> bool:
+        """Whether the cooperative attention kernel can run (its tiles must fit into LDS)."""
+        return bool(self.attention_lib(head_dim).ls_attn_coop_supported(c_int(DTYPE_CODE[dtype])))
+
     def attention_geometry(self, head_dim: int) -> tuple[int, int]:
         """(keys per tile, keys per split) of the attention kernels."""
         lib = self.attention_lib(head_dim)
@@ -204,9 +208,10 @@ class Kernels:
 
     def attention(self, q: torch.Tensor, nq: int, nkv: int, d: int, k_pages, v_pages, page_size: int, table,
                   seqs, items, n_items: int, out: torch.Tensor, part_acc, part_ml, scale: float,
-                  window: int, variant: int = 0) -> None:
+                  window: int, variant: int = 0, max_rows: int = 0) -> None:
         """Launch the attention kernel over ``n_items`` work items (see attention.hip).
-        ``variant``: 0 staged through LDS where it fits, 1 direct from global memory, 2 staged or error."""
+        ``variant``: 0 staged through LDS where it fits, 1 direct from global memory, 2 staged or
+        error, 3 cooperative (every item has at most 16 rows; ``max_rows`` states the largest)."""
         lib = self.attention_lib(d)
         _rows_ok(q, "attention q"); _rows_ok(out, "attention out")
         _need(q.dtype in DTYPE_CODE and out.dtype == q.dtype, "attention q/out dtype")
@@ -224,7 +229,7 @@ class Kernels:
             c_int(DTYPE_CODE[q.dtype]), _ptr(q), c_long(q.stride(0)), _ptr(k_pages), _ptr(v_pages), c_int(nkv),
             c_int(page_size), _ptr(table), c_int(table.shape[1]), _ptr(seqs), _ptr(items), c_int(n_items),
             _ptr(out), c_long(out.stride(0)), _ptr(part_acc), _ptr(part_ml), c_int(nq // nkv), c_float(scale),
-            c_int(window), c_int(variant), _stream())
+            c_int(window), c_int(variant), c_int(max_rows), _stream())
         self._check(lib, code)
 
     def attention_combine(self, d: int, seqs, items, n_items: int, nq: int, nkv: int, part_acc, part_ml,

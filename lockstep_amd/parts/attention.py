@@ -112,8 +112,13 @@ class Attention(Mixer):
         attn = ctx.buf("attention.out", (t, nq * d), rt.dtype)
         window = int(self.window) if self.window is not None else 0
         plan = ctx.attention_plan(nq // nkv, nkv, d, window)
-        k.attention(qkv, nq, nkv, d, key_pages, value_pages, group.page_size, group.table, ctx.seqs,
-                    plan.items, plan.n_items, attn, plan.part_acc, plan.part_ml, self.scale, window)
+        if plan.n_items:
+            k.attention(qkv, nq, nkv, d, key_pages, value_pages, group.page_size, group.table, ctx.seqs,
+                        plan.items, plan.n_items, attn, plan.part_acc, plan.part_ml, self.scale, window)
+        if plan.n_coop:
+            k.attention(qkv, nq, nkv, d, key_pages, value_pages, group.page_size, group.table, ctx.seqs,
+                        plan.coop_items, plan.n_coop, attn, plan.part_acc, plan.part_ml, self.scale, window,
+                        variant=3, max_rows=plan.coop_max_rows)
         if plan.n_combine:
             k.attention_combine(d, ctx.seqs, plan.combine_items, plan.n_combine, nq, nkv, plan.part_acc,
                                 plan.part_ml, attn)

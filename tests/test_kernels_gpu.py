@@ -226,7 +226,7 @@ class PagedCase:
         part_ml = torch.full((max(part_rows, 1), 2), float("nan"), dtype=torch.float32, device="cuda")
         K().attention(qkv, self.nq, self.nkv, self.d, self.k_pages, self.v_pages, self.ps, self.table,
                       self.seqs(q_start, t), items_t, len(items) // 8, out, part_acc, part_ml, scale, window,
-                      variant)
+                      variant, rows)
         if combine:
             comb = torch.tensor(combine, dtype=torch.int32).cuda()
             K().attention_combine(self.d, self.seqs(q_start, t), comb, len(combine) // 4, self.nq, self.nkv,
@@ -295,6 +295,10 @@ def test_attention_row_is_the_same_alone_in_a_portion_and_in_the_whole_prompt(dt
         assert torch.equal(alone[0], full[p]), f"row {p} alone"
         alone = whole.attend(qkv[p:p + 1], p, d ** -0.5, variant=1)
         assert torch.equal(alone[0], full[p]), f"row {p} alone, loaded directly"
+        if K().coop_supported(d, dtype):
+            for split in (True, False):
+                alone = whole.attend(qkv[p:p + 1], p, d ** -0.5, variant=3, force_split=split)
+                assert torch.equal(alone[0], full[p]), f"row {p} alone, cooperative kernel, split={split}"
         both = whole.attend(qkv[p:p + 1], p, d ** -0.5, force_split=False)
         assert torch.equal(both[0], full[p]), f"row {p} alone, direct"
     for lo, hi in ((250, 262), (0, 3), (500, 700), (255, 257), (690, 700)):
@@ -323,8 +327,10 @@ def test_attention_window(dtype, window):
         saved = case.table.clone()
         case.table[1, :first_needed] = -1
         alone = case.attend(dev[p:p + 1], p, d ** -0.5, window=window)
+        coop = case.attend(dev[p:p + 1], p, d ** -0.5, window=window, variant=3)
         case.table.copy_(saved)
         assert torch.equal(alone[0], out[p]), f"row {p}"
+        assert torch.equal(coop[0], out[p]), f"row {p}, cooperative kernel"
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -368,3 +374,30 @@ def test_norm_rotation_and_cache_write(dtype):
     one = qkv[:1].clone().cuda()
     case0.write(one, 0, None, None, eps, cos.cuda(), sin.cuda(), rot)
     assert torch.equal(one.cpu(), qkv[:1])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nq,nkv,d,ps", [(16, 8, 128, 16), (4, 4, 16, 8), (8, 1, 64, 32), (6, 2, 48, 16),
+                                         (32, 2, 80, 64), (2, 2, 256, 128), (3, 3, 32, 8)])
+def test_decode_attention_is_the_same_in_every_kernel(dtype, nq, nkv, d, ps):
+    """The last one or two tokens of a sequence through the staged, the direct
+    and the cooperative kernel, split or not: same bits, and right."""
+    kv_len = 700
+    qkv = rand_qkv(kv_len, nq, nkv, d, dtype, seed=d + nq, sharp=(5,))
+    case = PagedCase(dtype, nq, nkv, d, ps, kv_len, shuffle_seed=7)
+    dev = qkv.cuda()
+    case.write(dev, 0)
+    q, k, v = split_qkv(qkv.double(), nq, nkv, d)
+    want = naive_attention(q, k, v, 0, d ** -0.5)
+    g = nq // nkv
+    for start, n in ((699, 1), (698, 2), (255, 1), (256, 1), (0, 1), (127, 2)):
+        if n * g > 16:
+            n = 1
+        ref = case.attend(dev[start:start + n], start, d ** -0.5, variant=1, force_split=False)
+        assert rel_err(ref, want[start:start + n]) < ATT_TOL[dtype], (start, n)
+        variants = [(0, True), (0, False), (1, True)]
+        if K().coop_supported(d, dtype):
+            variants += [(3, True), (3, False)]
+        for variant, split in variants:
+            got = case.attend(dev[start:start + n], start, d ** -0.5, variant=variant, force_split=split)
+            assert torch.equal(got, ref), f"start={start} n={n} variant={variant} split={split}"
