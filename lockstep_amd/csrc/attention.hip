@@ -71,6 +71,24 @@ template <typename T> __device__ __forceinline__ float softmax_exp(float x);
 template <> __device__ __forceinline__ float softmax_exp<float>(float x) { return expf(x); }
 template <> __device__ __forceinline__ float softmax_exp<bf16_t>(float x) { return __expf(x); }
 
+// Keep elements n_lo <= e < n_hi of a vector of VEC consecutive keys, zero the others.
+__device__ __forceinline__ bf16x8 mask_keys(bf16x8 v, int n_lo, int n_hi) {
+  typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
+  u32x4 w = __builtin_bit_cast(u32x4, v);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const unsigned lo = (2 * i >= n_lo && 2 * i < n_hi) ? 0x0000FFFFu : 0u;
+    const unsigned hi = (2 * i + 1 >= n_lo && 2 * i + 1 < n_hi) ? 0xFFFF0000u : 0u;
+    w[i] = w[i] & (lo | hi);
+  }
+  return __builtin_bit_cast(bf16x8, w);
+}
+__device__ __forceinline__ f32x4 mask_keys(f32x4 v, int n_lo, int n_hi) {
+#pragma unroll
+  for (int e = 0; e < 4; ++e) v[e] = (e >= n_lo && e < n_hi) ? v[e] : 0.f;
+  return v;
+}
+
 struct RowState {
   f32x4 acc[DB];
   float m, l;
@@ -371,64 +389,65 @@ __global__ __launch_bounds__(256, LS_STAGED_MIN_BLOCKS) void attention_staged_ke
       vpage[i] = tbl[min(key0, sm.kv_len - 1) >> page_shift];
     }
   };
+  // fetch() only issues loads (from clamped, always valid addresses), so all
+  // of a tile's loads are in flight together; stash() zeroes what is not a
+  // held key and writes to LDS.
   vec_t kreg[GROUP], vreg[GROUP];
   auto fetch = [&](int ti, int i0) {
+    const int t0 = ti * kTileKeys;
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int j = 0; j < GROUP; ++j) {
+      const int i = i0 + j;
+      if (i >= PER) break;
+      const int p = threadIdx.x + 256 * i;
+      {
+        const int key = min(t0 + p / KPIECES, sm.kv_len - 1);
+        const int page = max(kpage[i], 0);
+        const T* src = k_pages + (((long)page * nkv + kvh) * page_size + (key & (page_size - 1))) * D +
+                       (p % KPIECES) * A::VEC;
+        kreg[j] = *reinterpret_cast<const vec_t*>(src);
+      }
+      {
+        const int q1 = p >> vshift;
+        const int kp = p & ((1 << vshift) - 1);
+        const int page = max(vpage[i], 0);
+        const T* src = v_pages + ((((long)page * nkv + kvh) * D + q1 % D) << page_shift) + (kp << LOG_VEC);
+        vreg[j] = *reinterpret_cast<const vec_t*>(src);
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  // page ids of the tile whose data is in kreg/vreg (fetch() ran with them)
+  int kpage_held[PER], vpage_held[PER];
+  auto hold_pages = [&]() {
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      kpage_held[i] = kpage[i];
+      vpage_held[i] = vpage[i];
+    }
+  };
+  auto stash = [&](int ti, int i0) {
     const int t0 = ti * kTileKeys;
 #pragma unroll
     for (int j = 0; j < GROUP; ++j) {
       const int i = i0 + j;
       if (i >= PER) break;
       const int p = threadIdx.x + 256 * i;
-      // ---- K piece: key row p / KPIECES, piece p % KPIECES
-      {
-        const int kt = p / KPIECES;
-        const int piece = p % KPIECES;
-        const int key = t0 + kt;
-        bool ok = (TOTAL % 256 == 0 || p < TOTAL) && key < sm.kv_len && key >= lo_valid;
-        int page = kpage[i];
-        ok = ok && page >= 0;
-        page = max(page, 0);
-        const int slot = min(key, sm.kv_len - 1) & (page_size - 1);
-        const T* src = k_pages + (((long)page * nkv + kvh) * page_size + slot) * D + piece * A::VEC;
-        vec_t v = *reinterpret_cast<const vec_t*>(src);
-        kreg[j] = ok ? v : A::zero();
-      }
-      // ---- V piece: page pg of the tile, column d, keys kp*VEC.. inside the page
-      {
-        const int q1 = p >> vshift;
-        const int kp = p & ((1 << vshift) - 1);
-        const int pg = q1 / D;
-        const int d = q1 % D;
-        const int key0 = t0 + (pg << page_shift) + (kp << LOG_VEC);
-        bool ok = (TOTAL % 256 == 0 || p < TOTAL) && key0 < sm.kv_len && key0 + A::VEC > lo_valid;
-        int page = vpage[i];
-        ok = ok && page >= 0;
-        page = max(page, 0);
-        const T* src = v_pages + ((((long)page * nkv + kvh) * D + d) << page_shift) + (kp << LOG_VEC);
-        vec_t v = *reinterpret_cast<const vec_t*>(src);
-#pragma unroll
-        for (int e = 0; e < A::VEC; ++e)
-          if (!ok || key0 + e >= sm.kv_len || key0 + e < lo_valid) v[e] = 0;
-        vreg[j] = v;
-      }
-    }
-  };
-  auto stash = [&](int i0) {
-#pragma unroll
-    for (int j = 0; j < GROUP; ++j) {
-      const int i = i0 + j;
-      if (i >= PER) break;
-      const int p = threadIdx.x + 256 * i;
-      if (TOTAL % 256 != 0 && p >= TOTAL) continue;
       const int kt = p / KPIECES;
       const int piece = p % KPIECES;
-      *reinterpret_cast<vec_t*>(k_lds + kt * KROW + ((piece + kt) % KPIECES) * 16) = kreg[j];
+      const int key = t0 + kt;
+      const bool k_ok = key < sm.kv_len && key >= lo_valid && kpage_held[i] >= 0;
+      *reinterpret_cast<vec_t*>(k_lds + kt * KROW + ((piece + kt) % KPIECES) * 16) = k_ok ? kreg[j] : A::zero();
       const int q1 = p >> vshift;
       const int kp = p & ((1 << vshift) - 1);
       const int pg = q1 / D;
       const int d = q1 % D;
+      const int key0 = t0 + (pg << page_shift) + (kp << LOG_VEC);
+      const int n_hi = vpage_held[i] >= 0 ? sm.kv_len - key0 : 0;
       const int vpiece = (pg << vshift) + kp;
-      *reinterpret_cast<vec_t*>(v_lds + d * VROW + ((vpiece + d) % VPIECES) * 16) = vreg[j];
+      *reinterpret_cast<vec_t*>(v_lds + d * VROW + ((vpiece + d) % VPIECES) * 16) =
+          mask_keys(vreg[j], lo_valid - key0, n_hi);
     }
   };
 
@@ -439,29 +458,29 @@ __global__ __launch_bounds__(256, LS_STAGED_MIN_BLOCKS) void attention_staged_ke
   if (ti_lo < ti_hi) lookup(ti_lo);
   if (PREFETCH && ti_lo < ti_hi) {
     fetch(ti_lo, 0);
+    hold_pages();
     if (ti_lo + 1 < ti_hi) lookup(ti_lo + 1);
   }
   for (int ti = ti_lo; ti < ti_hi; ++ti) {
     const int t0 = ti * kTileKeys;
     __syncthreads();  // the previous tile has been read by every wave
     if (PREFETCH) {
-      stash(0);
+      stash(ti, 0);
     } else {
+      hold_pages();
       for (int i0 = 0; i0 < PER; i0 += GROUP) {
         fetch(ti, i0);
-        stash(i0);
+        stash(ti, i0);
       }
       if (ti + 1 < ti_hi) lookup(ti + 1);
     }
     __syncthreads();
     if (PREFETCH && ti + 1 < ti_hi) {
       fetch(ti + 1, 0);
+      hold_pages();
       if (ti + 2 < ti_hi) lookup(ti + 2);
     }
 
-#ifdef LS_EXP
-    if (LS_EXP & 1) continue;
-#endif
     const bool mine = wave_active && t0 <= wave_last_pos &&
                       !(window > 0 && t0 + kTileKeys <= wave_first_pos - window + 1);
     if (mine) {
@@ -655,61 +674,56 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
         vpage[st][i] = tbl[min(key0, sm.kv_len - 1) >> page_shift];
       }
     }
+    __builtin_amdgcn_sched_barrier(0);  // every page id is requested before the first data load is built from one
     vec_t kreg[STAGE][PER], vreg[STAGE][PER];
 #pragma unroll
-    for (int st = 0; st < STAGE; ++st) {
+    for (int st = 0; st < STAGE; ++st) {  // loads only, from clamped addresses
+      const int t0 = (tb + st) * kTileKeys;
+#pragma unroll
+      for (int i = 0; i < PER; ++i) {
+        const int p = threadIdx.x + 256 * i;
+        {
+          const int key = min(t0 + p / KPIECES, sm.kv_len - 1);
+          const int page = max(kpage[st][i], 0);
+          const T* src = k_pages + (((long)page * nkv + kvh) * page_size + (key & (page_size - 1))) * D +
+                         (p % KPIECES) * A::VEC;
+          kreg[st][i] = *reinterpret_cast<const vec_t*>(src);
+        }
+        {
+          const int q1 = p >> vshift;
+          const int kp = p & ((1 << vshift) - 1);
+          const int page = max(vpage[st][i], 0);
+          const T* src = v_pages + ((((long)page * nkv + kvh) * D + q1 % D) << page_shift) + (kp << LOG_VEC);
+          vreg[st][i] = *reinterpret_cast<const vec_t*>(src);
+        }
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);  // ... and every data load is issued before the first one is waited for
+    __syncthreads();  // the previous stage has been consumed
+#pragma unroll
+    for (int st = 0; st < STAGE; ++st) {  // zero what is not a held key, write to LDS
+      unsigned char* k_lds = lds + st * TILE_BYTES;
+      unsigned char* v_lds = k_lds + kTileKeys * KROW;
       const int t0 = (tb + st) * kTileKeys;
       const bool tile_in = tb + st < ti_hi;
 #pragma unroll
       for (int i = 0; i < PER; ++i) {
         const int p = threadIdx.x + 256 * i;
-        {
-          const int kt = p / KPIECES;
-          const int piece = p % KPIECES;
-          const int key = t0 + kt;
-          int page = kpage[st][i];
-          const bool ok = tile_in && key < sm.kv_len && key >= lo_valid && page >= 0;
-          page = max(page, 0);
-          const int slot = min(key, sm.kv_len - 1) & (page_size - 1);
-          const T* src = k_pages + (((long)page * nkv + kvh) * page_size + slot) * D + piece * A::VEC;
-          vec_t v = *reinterpret_cast<const vec_t*>(src);
-          kreg[st][i] = ok ? v : A::zero();
-        }
-        {
-          const int q1 = p >> vshift;
-          const int kp = p & ((1 << vshift) - 1);
-          const int pg = q1 / D;
-          const int d = q1 % D;
-          const int key0 = t0 + (pg << page_shift) + (kp << LOG_VEC);
-          int page = vpage[st][i];
-          const bool ok = tile_in && key0 < sm.kv_len && key0 + A::VEC > lo_valid && page >= 0;
-          page = max(page, 0);
-          const T* src = v_pages + ((((long)page * nkv + kvh) * D + d) << page_shift) + (kp << LOG_VEC);
-          vec_t v = *reinterpret_cast<const vec_t*>(src);
-#pragma unroll
-          for (int e = 0; e < A::VEC; ++e)
-            if (!ok || key0 + e >= sm.kv_len || key0 + e < lo_valid) v[e] = 0;
-          vreg[st][i] = v;
-        }
-      }
-    }
-    __syncthreads();  // the previous stage has been consumed
-#pragma unroll
-    for (int st = 0; st < STAGE; ++st) {
-      unsigned char* k_lds = lds + st * TILE_BYTES;
-      unsigned char* v_lds = k_lds + kTileKeys * KROW;
-#pragma unroll
-      for (int i = 0; i < PER; ++i) {
-        const int p = threadIdx.x + 256 * i;
         const int kt = p / KPIECES;
         const int piece = p % KPIECES;
-        *reinterpret_cast<vec_t*>(k_lds + kt * KROW + ((piece + kt) % KPIECES) * 16) = kreg[st][i];
+        const int key = t0 + kt;
+        const bool k_ok = tile_in && key < sm.kv_len && key >= lo_valid && kpage[st][i] >= 0;
+        *reinterpret_cast<vec_t*>(k_lds + kt * KROW + ((piece + kt) % KPIECES) * 16) =
+            k_ok ? kreg[st][i] : A::zero();
         const int q1 = p >> vshift;
         const int kp = p & ((1 << vshift) - 1);
         const int pg = q1 / D;
         const int d = q1 % D;
+        const int key0 = t0 + (pg << page_shift) + (kp << LOG_VEC);
+        const int n_hi = (tile_in && vpage[st][i] >= 0) ? sm.kv_len - key0 : 0;
         const int vpiece = (pg << vshift) + kp;
-        *reinterpret_cast<vec_t*>(v_lds + d * VROW + ((vpiece + d) % VPIECES) * 16) = vreg[st][i];
+        *reinterpret_cast<vec_t*>(v_lds + d * VROW + ((vpiece + d) % VPIECES) * 16) =
+            mask_keys(vreg[st][i], lo_valid - key0, n_hi);
       }
     }
     __syncthreads();

@@ -23,6 +23,8 @@ enum Epilogue : int {
   kStore = 0,     // C[m][n] = total, in the compute dtype
   kStoreF32 = 1,  // C[m][n] = total, float
   kAddF32 = 2,    // C[m][n] += total, float (residual stream)
+  kSwiGLU = 3,    // W holds gate and up rows interleaved in tiles of 16 (gate rows 16t.., then up rows 16t..);
+                  // C[m][16t + i] = (g * 1/(1 + exp(-g))) * u in float, stored in the compute dtype
 };
 
 __host__ __device__ inline int kslice_for(int K) { return 256 * ((K + 4095) / 4096); }
@@ -65,69 +67,176 @@ __device__ __forceinline__ void epilogue4(void* __restrict__ C, long ldc, int m,
   }
 }
 
+// SwiGLU epilogue on the float totals of a gate tile and the matching up tile.
+template <typename T>
+__device__ __forceinline__ void epilogue_swiglu4(void* __restrict__ C, long ldc, int m, int col, int M, int width,
+                                                 const float gate[4], const float up[4], bool vec_ok) {
+  if (m >= M || col >= width) return;
+  float act[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const float sig = 1.0f / (1.0f + expf(-gate[r]));
+    act[r] = (gate[r] * sig) * up[r];
+  }
+  epilogue4<T, kStore>(C, ldc, m, col, M, width, act, vec_ok);
+}
+
+// RMSNorm of rows of the float residual stream, as a prologue of the skinny
+// kernel (at most 16 rows): the sum of squares of a row is formed exactly as
+// rmsnorm_kernel forms it (thread i of the first 256 adds x[i]^2, x[i+256]^2,
+// ... ascending; butterfly over the wave; the four wave sums in wave order),
+// so the normalised operand has the same bits as the stand-alone kernel's.
+template <int NW>
+__device__ __forceinline__ void row_scales(const float* __restrict__ H, long ldh, int M, int K, float eps,
+                                           float* __restrict__ wave_part /*[16][4]*/, float* __restrict__ scale /*[16]*/) {
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  if (wave < 4) {
+    // all rows together: the loads of one pass over the 16 rows are independent
+    float part[16];
+#pragma unroll
+    for (int m = 0; m < 16; ++m) part[m] = 0.f;
+    for (int e = threadIdx.x; e < K; e += 256) {
+      float v[16];
+#pragma unroll
+      for (int m = 0; m < 16; ++m) v[m] = H[(long)(m < M ? m : 0) * ldh + e];
+#pragma unroll
+      for (int m = 0; m < 16; ++m) part[m] = part[m] + v[m] * v[m];
+    }
+#pragma unroll
+    for (int m = 0; m < 16; ++m) {
+      const float total = wave_sum(part[m]);
+      if (lane == 0) wave_part[m * 4 + wave] = total;
+    }
+  }
+  __syncthreads();
+  if (threadIdx.x < 16) {
+    const float* p = wave_part + threadIdx.x * 4;
+    const float total = ((p[0] + p[1]) + p[2]) + p[3];
+    scale[threadIdx.x] = 1.0f / sqrtf(total / (float)K + eps);
+  }
+  __syncthreads();
+}
+
 // ---------------------------------------------------------------------------
 // Skinny kernel: one workgroup per 16 output columns, NW waves, wave w takes
 // slices w, w + NW, ...; slice sums meet in LDS and are folded in ascending
 // order by the thread that owns the output element.
 // ---------------------------------------------------------------------------
-template <typename T, int MT, int NW, int EPI>
-__global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const T* __restrict__ X, const T* __restrict__ W,
+template <typename T, int MT, int NW, int EPI, bool NORM>
+__global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const void* __restrict__ Xv, const T* __restrict__ W,
                                                                void* __restrict__ C, int M, int N, int K, long ldx,
-                                                               long ldc, int kslice, int aligned, int vec_ok) {
+                                                               long ldc, int kslice, int aligned, int vec_ok,
+                                                               const float* __restrict__ norm_w, float eps,
+                                                               int out_cols) {
   typedef Atom<T> A;
   typedef typename A::vec_t vec_t;
-  extern __shared__ float part[];  // [nslices][MT][256]
+  constexpr int NT = (EPI == kSwiGLU) ? 2 : 1;  // weight tiles per workgroup
+  extern __shared__ float part[];                // [nslices][NT][MT][256] (+ 80 floats with NORM)
 
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
-  const int n0 = blockIdx.x * 16;
+  const int n0 = blockIdx.x * 16 * NT;
   const int row16 = lane & 15;
   const int g = lane >> 4;
   const int nslices = (K + kslice - 1) / kslice;
-  const int n = n0 + row16;
-  const bool n_ok = n < N;
+
+  const T* X = reinterpret_cast<const T*>(Xv);
+  const float* H = reinterpret_cast<const float*>(Xv);
+  float my_scale = 0.f;
+  if (NORM) {
+    float* wave_part = part + nslices * NT * MT * 256;
+    float* scale = wave_part + 64;
+    row_scales<NW>(H, ldx, M, K, eps, wave_part, scale);
+    my_scale = row16 < M ? scale[row16] : 0.f;
+  }
+  const bool norm_vec = NORM && aligned && ldx % 4 == 0 && reinterpret_cast<uintptr_t>(norm_w) % 16 == 0;
 
   for (int s = wave; s < nslices; s += NW) {
-    f32x4 acc[MT];
+    f32x4 acc[NT][MT];
 #pragma unroll
-    for (int j = 0; j < MT; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int j = 0; j < MT; ++j) acc[t][j] = f32x4{0.f, 0.f, 0.f, 0.f};
     const int k_begin = s * kslice;
     const int k_end = min(K, k_begin + kslice);
     // Four chunks at a time: all their loads are issued before the first
     // MFMA needs one, so a wave keeps several kilobytes in flight.
     for (int k0 = k_begin; k0 < k_end; k0 += 4 * A::KCHUNK) {
-      vec_t w[4], x[MT][4];
+      vec_t w[NT][4], x[MT][4];
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
         const int k = k0 + u * A::KCHUNK + g * A::VEC;
         const bool in = k0 + u * A::KCHUNK < k_end;
-        w[u] = load_vec<T>(W, n, k, K, K, n_ok && in, aligned);
 #pragma unroll
-        for (int j = 0; j < MT; ++j) x[j][u] = load_vec<T>(X, j * 16 + row16, k, K, ldx, j * 16 + row16 < M && in, aligned);
+        for (int t = 0; t < NT; ++t) {
+          const int n = n0 + t * 16 + row16;
+          w[t][u] = load_vec<T>(W, n, k, K, K, n < N && in, aligned);
+        }
+        if (NORM) {
+          // normalise on the fly: (x * scale) * weight, rounded to the compute dtype
+          vec_t v = A::zero();
+          const bool valid = row16 < M && in && k < K;
+          if (norm_vec) {  // uniform: rows and k are 16-byte aligned and K is a multiple of VEC
+            const float* src = H + (valid ? (long)row16 * ldx + k : 0);
+            const float* wsrc = norm_w + (valid ? k : 0);
+#pragma unroll
+            for (int q4 = 0; q4 < A::VEC / 4; ++q4) {
+              const f32x4 xs = *reinterpret_cast<const f32x4*>(src + 4 * q4);
+              const f32x4 ws = *reinterpret_cast<const f32x4*>(wsrc + 4 * q4);
+#pragma unroll
+              for (int e = 0; e < 4; ++e) v[4 * q4 + e] = from_f32<T>((xs[e] * my_scale) * ws[e]);
+            }
+            if (!valid) v = A::zero();
+          } else if (valid) {
+            const float* src = H + (long)row16 * ldx + k;
+#pragma unroll
+            for (int e = 0; e < A::VEC; ++e)
+              if (k + e < K) v[e] = from_f32<T>((src[e] * my_scale) * norm_w[k + e]);
+          }
+          x[0][u] = v;
+        } else {
+#pragma unroll
+          for (int j = 0; j < MT; ++j)
+            x[j][u] = load_vec<T>(X, j * 16 + row16, k, K, ldx, j * 16 + row16 < M && in, aligned);
+        }
       }
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
         if (k0 + u * A::KCHUNK >= k_end) break;  // uniform: a chunk is visited iff it starts inside the slice
 #pragma unroll
-        for (int j = 0; j < MT; ++j) A::mma(acc[j], w[u], x[j][u]);
+        for (int t = 0; t < NT; ++t)
+#pragma unroll
+          for (int j = 0; j < MT; ++j) A::mma(acc[t][j], w[t][u], x[j][u]);
       }
     }
 #pragma unroll
-    for (int j = 0; j < MT; ++j)
-      *reinterpret_cast<f32x4*>(&part[((s * MT + j) * 64 + lane) * 4]) = acc[j];
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int j = 0; j < MT; ++j)
+        *reinterpret_cast<f32x4*>(&part[(((s * NT + t) * MT + j) * 64 + lane) * 4]) = acc[t][j];
   }
   __syncthreads();
 
   for (int idx = threadIdx.x; idx < MT * 64; idx += NW * 64) {
     const int j = idx >> 6;
     const int l = idx & 63;
-    float total[4] = {0.f, 0.f, 0.f, 0.f};
-    for (int s = 0; s < nslices; ++s) {
-      f32x4 p = *reinterpret_cast<const f32x4*>(&part[((s * MT + j) * 64 + l) * 4]);
+    float total[NT][4];
 #pragma unroll
-      for (int r = 0; r < 4; ++r) total[r] = total[r] + p[r];
+    for (int t = 0; t < NT; ++t) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) total[t][r] = 0.f;
+      for (int s = 0; s < nslices; ++s) {
+        f32x4 p = *reinterpret_cast<const f32x4*>(&part[(((s * NT + t) * MT + j) * 64 + l) * 4]);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) total[t][r] = total[t][r] + p[r];
+      }
     }
-    epilogue4<T, EPI>(C, ldc, j * 16 + (l & 15), n0 + (l >> 4) * 4, M, N, total, vec_ok);
+    const int m = j * 16 + (l & 15);
+    if (EPI == kSwiGLU)
+      epilogue_swiglu4<T>(C, ldc, m, blockIdx.x * 16 + (l >> 4) * 4, M, out_cols, total[0], total[NT - 1], vec_ok);
+    else
+      epilogue4<T, EPI>(C, ldc, m, n0 + (l >> 4) * 4, M, N, total[0], vec_ok);
   }
 }
 
@@ -142,7 +251,7 @@ template <typename T, int EPI>
 __global__ __launch_bounds__(256) void gemm_tiled_kernel(const T* __restrict__ X, const T* __restrict__ W,
                                                          void* __restrict__ C, int M, int N, int K, long ldx,
                                                          long ldc, int kslice, int aligned, int vec_ok,
-                                                         int tiles_m) {
+                                                         int tiles_m, int out_cols) {
   typedef Atom<T> A;
   typedef typename A::vec_t vec_t;
   constexpr int BK = kRowBytes / sizeof(T);  // elements of K per stage
@@ -236,6 +345,19 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const T* __restrict__ X
 #pragma unroll
       for (int r = 0; r < 4; ++r) total[i][j][r] = total[i][j][r] + acc[i][j][r];
 
+  if (EPI == kSwiGLU) {
+    // the wave's four weight tiles are (gate t, up t, gate t+1, up t+1)
+#pragma unroll
+    for (int i = 0; i < 4; i += 2)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        float gate[4] = {total[i][j][0], total[i][j][1], total[i][j][2], total[i][j][3]};
+        float up[4] = {total[i + 1][j][0], total[i + 1][j][1], total[i + 1][j][2], total[i + 1][j][3]};
+        epilogue_swiglu4<T>(C, ldc, m_base + wm + j * 16 + row16, (n_base + wn + i * 16) / 2 + g * 4, M, out_cols, gate,
+                            up, vec_ok);
+      }
+    return;
+  }
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
@@ -246,35 +368,41 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const T* __restrict__ X
 }
 
 template <typename T, int EPI>
-int launch_gemm(const void* X, const void* W, void* C, int M, int N, int K, long ldx, long ldc, hipStream_t stream) {
+int launch_gemm(const void* X, const void* W, void* C, int M, int N, int K, long ldx, long ldc, const float* norm_w,
+                float eps, int out_cols, hipStream_t stream) {
   const int kslice = kslice_for(K);
   const int nslices = (K + kslice - 1) / kslice;
   constexpr int VEC = Atom<T>::VEC;
-  const int aligned = (K % VEC == 0) && (ldx % VEC == 0) && (reinterpret_cast<uintptr_t>(X) % 16 == 0) &&
+  constexpr int NT = (EPI == kSwiGLU) ? 2 : 1;
+  const int aligned = (K % VEC == 0) && (norm_w || ldx % VEC == 0) && (reinterpret_cast<uintptr_t>(X) % 16 == 0) &&
                       (reinterpret_cast<uintptr_t>(W) % 16 == 0);
-  const size_t out_size = (EPI == kStore) ? sizeof(T) : sizeof(float);
+  const size_t out_size = (EPI == kStore || EPI == kSwiGLU) ? sizeof(T) : sizeof(float);
   const int vec_ok = (ldc % 4 == 0) && (reinterpret_cast<uintptr_t>(C) % (4 * out_size) == 0);
-  const T* x = reinterpret_cast<const T*>(X);
   const T* w = reinterpret_cast<const T*>(W);
+  if (norm_w && M > 16) return fail("gemm: the fused norm prologue takes at most 16 rows, got %d", M);
   if (M <= 64) {
     const int mt = (M + 15) / 16;
     const int nw = nslices >= 8 ? 8 : 4;
-    dim3 grid((N + 15) / 16);
-    const size_t lds = (size_t)nslices * mt * 256 * sizeof(float);
-#define LS_SKINNY(MT_, NW_)                                                                            \
-  hipLaunchKernelGGL((gemm_skinny_kernel<T, MT_, NW_, EPI>), grid, dim3(NW_ * 64), lds, stream, x, w, C, M, N, K, \
-                     ldx, ldc, kslice, aligned, vec_ok)
-    if (nw == 8) {
-      if (mt == 1) LS_SKINNY(1, 8); else if (mt == 2) LS_SKINNY(2, 8); else if (mt == 3) LS_SKINNY(3, 8); else LS_SKINNY(4, 8);
+    dim3 grid((N + 16 * NT - 1) / (16 * NT));
+    const size_t lds = ((size_t)nslices * NT * mt * 256 + (norm_w ? 80 : 0)) * sizeof(float);
+#define LS_SKINNY(MT_, NW_, NORM_)                                                                              \
+  hipLaunchKernelGGL((gemm_skinny_kernel<T, MT_, NW_, EPI, NORM_>), grid, dim3(NW_ * 64), lds, stream, X, w, C, M, N, \
+                     K, ldx, ldc, kslice, aligned, vec_ok, norm_w, eps, out_cols)
+    if (norm_w) {
+      if (nw == 8) LS_SKINNY(1, 8, true); else LS_SKINNY(1, 4, true);
+    } else if (nw == 8) {
+      if (mt == 1) LS_SKINNY(1, 8, false); else if (mt == 2) LS_SKINNY(2, 8, false);
+      else if (mt == 3) LS_SKINNY(3, 8, false); else LS_SKINNY(4, 8, false);
     } else {
-      if (mt == 1) LS_SKINNY(1, 4); else if (mt == 2) LS_SKINNY(2, 4); else if (mt == 3) LS_SKINNY(3, 4); else LS_SKINNY(4, 4);
+      if (mt == 1) LS_SKINNY(1, 4, false); else if (mt == 2) LS_SKINNY(2, 4, false);
+      else if (mt == 3) LS_SKINNY(3, 4, false); else LS_SKINNY(4, 4, false);
     }
 #undef LS_SKINNY
   } else {
     const int tiles_m = (M + kTile - 1) / kTile;
     const int tiles_n = (N + kTile - 1) / kTile;
-    hipLaunchKernelGGL((gemm_tiled_kernel<T, EPI>), dim3(tiles_m * tiles_n), dim3(256), 0, stream, x, w, C, M, N, K,
-                       ldx, ldc, kslice, aligned, vec_ok, tiles_m);
+    hipLaunchKernelGGL((gemm_tiled_kernel<T, EPI>), dim3(tiles_m * tiles_n), dim3(256), 0, stream,
+                       reinterpret_cast<const T*>(X), w, C, M, N, K, ldx, ldc, kslice, aligned, vec_ok, tiles_m, out_cols);
   }
   return check_launch("gemm");
 }
@@ -282,21 +410,29 @@ int launch_gemm(const void* X, const void* W, void* C, int M, int N, int K, long
 }  // namespace ls
 
 // dtype: 0 float32, 1 bfloat16.  epilogue: 0 store in dtype, 1 store float,
-// 2 add to float.  X [M,K] with ldx elements per row, W [N,K] contiguous,
-// C [M,N] with ldc elements per row.
+// 2 add to float, 3 SwiGLU of interleaved gate/up tiles (N = rows of W, the
+// output has out_cols <= N/2 columns; rows of W beyond them are padding).  X [M,K] with ldx elements per row, W [N,K]
+// contiguous, C with ldc elements per row.  With norm_w (float [K]) X is the
+// float residual stream and is RMS-normalised on the fly (M <= 16).
 extern "C" int ls_gemm(int dtype, int epilogue, const void* X, const void* W, void* C, int M, int N, int K, long ldx,
-                       long ldc, void* stream) {
+                       long ldc, const float* norm_w, float eps, int out_cols, void* stream) {
   using namespace ls;
   LS_REQUIRE(M > 0 && N > 0 && K > 0, "gemm: sizes must be positive, got M=%d N=%d K=%d", M, N, K);
-  LS_REQUIRE(ldx >= K && ldc >= N, "gemm: row strides ldx=%ld ldc=%ld are shorter than K=%d / N=%d", ldx, ldc, K, N);
+  if (epilogue != kSwiGLU) out_cols = N;
+  LS_REQUIRE(out_cols > 0 && (epilogue != kSwiGLU || (out_cols <= N / 2 && out_cols > N / 2 - 16)),
+             "gemm: %d output columns do not fit %d interleaved weight rows", out_cols, N);
+  LS_REQUIRE(ldx >= K && ldc >= out_cols, "gemm: row strides ldx=%ld ldc=%ld are shorter than K=%d / %d columns", ldx,
+             ldc, K, out_cols);
+  LS_REQUIRE(epilogue != kSwiGLU || N % 32 == 0, "gemm: the SwiGLU epilogue needs interleaved tiles, N=%d", N);
   LS_REQUIRE(X && W && C, "gemm: null operand");
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-#define LS_GEMM_CASE(T_)                                                             \
-  switch (epilogue) {                                                                \
-    case kStore: return launch_gemm<T_, kStore>(X, W, C, M, N, K, ldx, ldc, s);      \
-    case kStoreF32: return launch_gemm<T_, kStoreF32>(X, W, C, M, N, K, ldx, ldc, s); \
-    case kAddF32: return launch_gemm<T_, kAddF32>(X, W, C, M, N, K, ldx, ldc, s);    \
-    default: return fail("gemm: unknown epilogue %d", epilogue);                     \
+#define LS_GEMM_CASE(T_)                                                                              \
+  switch (epilogue) {                                                                                 \
+    case kStore: return launch_gemm<T_, kStore>(X, W, C, M, N, K, ldx, ldc, norm_w, eps, out_cols, s);          \
+    case kStoreF32: return launch_gemm<T_, kStoreF32>(X, W, C, M, N, K, ldx, ldc, norm_w, eps, out_cols, s);    \
+    case kAddF32: return launch_gemm<T_, kAddF32>(X, W, C, M, N, K, ldx, ldc, norm_w, eps, out_cols, s);        \
+    case kSwiGLU: return launch_gemm<T_, kSwiGLU>(X, W, C, M, N, K, ldx, ldc, norm_w, eps, out_cols, s);        \
+    default: return fail("gemm: unknown epilogue %d", epilogue);                                      \
   }
   if (dtype == kF32) { LS_GEMM_CASE(float) }
   if (dtype == kBF16) { LS_GEMM_CASE(bf16_t) }

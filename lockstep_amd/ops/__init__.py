@@ -1,5 +1,6 @@
 """Hand-written gfx950 kernels and the code that builds and loads them."""
 
-from .kernels import ADD_F32, STORE, STORE_F32, KernelError, Kernels, kernels
+from .kernels import (ADD_F32, STORE, STORE_F32, SWIGLU, KernelError, Kernels, interleave_gate_up,
+                      kernels)
 
-__all__ = ["ADD_F32", "STORE", "STORE_F32", "KernelError", "Kernels", "kernels"]
+__all__ = ["ADD_F32", "STORE", "STORE_F32", "SWIGLU", "KernelError", "Kernels", "interleave_gate_up", "kernels"]

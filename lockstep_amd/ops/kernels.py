@@ -18,7 +18,22 @@ import torch
 from . import build as _build
 
 DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1}
-STORE, STORE_F32, ADD_F32 = 0, 1, 2
+STORE, STORE_F32, ADD_F32, SWIGLU = 0, 1, 2, 3
+
+
+def interleave_gate_up(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
+    """Rows of ``gate`` and ``up`` (``[I, K]`` each) interleaved in tiles of 16 rows:
+    gate rows 0..15, up rows 0..15, gate rows 16..31, ...; the last tile of each is
+    padded with zero rows.  This is the weight layout of the SwiGLU epilogue."""
+    inter, k = gate.shape
+    tiles = -(-inter // 16)
+    out = torch.zeros((tiles, 2, 16, k), dtype=gate.dtype)
+    pad = tiles * 16 - inter
+    g = torch.cat([gate, gate.new_zeros((pad, k))]) if pad else gate
+    u = torch.cat([up, up.new_zeros((pad, k))]) if pad else up
+    out[:, 0] = g.view(tiles, 16, k)
+    out[:, 1] = u.view(tiles, 16, k)
+    return out.view(tiles * 32, k)
 MAX_HEAD_DIM = 256
 
 
@@ -82,21 +97,39 @@ class Kernels:
         return lib.ls_attn_tile_keys(), lib.ls_attn_split_keys()
 
     # -- matrix product -------------------------------------------------------
-    def gemm(self, x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, epilogue: int = STORE) -> None:
-        """``out (+)= x @ w.T``; ``x [M,K]``, ``w [N,K]`` contiguous, ``out [M,N]``."""
+    def gemm(self, x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, epilogue: int = STORE,
+             norm_weight: torch.Tensor | None = None, eps: float = 0.0) -> None:
+        """``out (+)= x @ w.T``; ``x [M,K]``, ``w [N,K]`` contiguous, ``out [M,N]``.
+
+        ``epilogue=SWIGLU``: ``w`` holds gate and up rows interleaved in tiles of
+        16 (see ``interleave_gate_up``) and ``out [M, I]`` gets ``silu(gate) * up``.
+        ``norm_weight`` (float32 ``[K]``): ``x`` is the float32 residual stream and is
+        RMS-normalised on the fly with this weight and ``eps`` (at most 16 rows)."""
         _rows_ok(x, "gemm x"); _rows_ok(w, "gemm w"); _rows_ok(out, "gemm out")
-        _need(x.dtype in DTYPE_CODE and w.dtype == x.dtype, f"gemm operands must share float32 or bfloat16, got "
-              f"{x.dtype} and {w.dtype}")
+        _need(w.dtype in DTYPE_CODE, f"gemm weights must be float32 or bfloat16, got {w.dtype}")
+        if norm_weight is None:
+            _need(x.dtype == w.dtype, f"gemm operands must share a dtype, got {x.dtype} and {w.dtype}")
+        else:
+            _need(x.dtype == torch.float32 and x.shape[0] <= 16, "the fused norm reads at most 16 float32 rows")
+            _need(norm_weight.is_cuda and norm_weight.dtype == torch.float32 and norm_weight.is_contiguous()
+                  and norm_weight.shape == (x.shape[1],), f"norm weight must be float32 [{x.shape[1]}]")
         m, k = x.shape
         n = w.shape[0]
         _need(w.shape[1] == k and w.is_contiguous(), f"gemm w must be contiguous [N,{k}], got {tuple(w.shape)}")
-        _need(tuple(out.shape) == (m, n), f"gemm out must be [{m},{n}], got {tuple(out.shape)}")
-        want = x.dtype if epilogue == STORE else torch.float32
+        if epilogue == SWIGLU:
+            cols = out.shape[1]
+            _need(n % 32 == 0 and n // 2 - 16 < cols <= n // 2 and out.shape[0] == m,
+                  f"SwiGLU output [{m},{cols}] does not fit {n} interleaved weight rows")
+        else:
+            cols = n
+            _need(tuple(out.shape) == (m, n), f"gemm out must be [{m},{n}], got {tuple(out.shape)}")
+        want = w.dtype if epilogue in (STORE, SWIGLU) else torch.float32
         _need(out.dtype == want, f"gemm out dtype {out.dtype} does not fit epilogue {epilogue}")
         if m == 0:
             return
-        code = self.core.ls_gemm(c_int(DTYPE_CODE[x.dtype]), c_int(epilogue), _ptr(x), _ptr(w), _ptr(out),
-                                 c_int(m), c_int(n), c_int(k), c_long(x.stride(0)), c_long(out.stride(0)), _stream())
+        code = self.core.ls_gemm(c_int(DTYPE_CODE[w.dtype]), c_int(epilogue), _ptr(x), _ptr(w), _ptr(out),
+                                 c_int(m), c_int(n), c_int(k), c_long(x.stride(0)), c_long(out.stride(0)),
+                                 _ptr(norm_weight), c_float(eps), c_int(cols), _stream())
         self._check(self.core, code)
 
     # -- rows -------------------------------------------------------------------

@@ -94,7 +94,9 @@ class Attention(Mixer):
         self.position.ensure(ctx.max_position + 1, ctx.rt)
         ctx.plan_attention(self.nq // self.nkv, self.nkv, self.d, int(self.window) if self.window is not None else 0)
 
-    def forward(self, ctx, run, x, out, accumulate: bool) -> None:
+    def forward(self, ctx, run, x, out, accumulate: bool, norm=None) -> None:
+        """``norm``: when given, ``x`` is the float32 residual stream and ``norm``
+        (an RMSNorm part) is applied inside the projection."""
         rt = ctx.rt
         k = rt.kernels
         t = ctx.n_tokens
@@ -102,10 +104,11 @@ class Attention(Mixer):
         group, key_pages, value_pages = ctx.cache.unit_pages(run.cache)
         width = (nq + 2 * nkv) * d
         qkv = ctx.buf("attention.qkv", (t, width), rt.dtype)
+        fused = {} if norm is None else {"norm_weight": norm.weight, "eps": norm.eps}
         if run.writes_cache:
-            k.gemm(x, self.w_qkv, qkv)
+            k.gemm(x, self.w_qkv, qkv, **fused)
         else:
-            k.gemm(x, self.w_q, qkv[:, : nq * d])
+            k.gemm(x, self.w_q, qkv[:, : nq * d], **fused)
         k.qk_rope_kv(qkv, t, nq, nkv, d, self.q_norm, self.k_norm, self.norm_eps, self.position.cos,
                      self.position.sin, self.position.rotary_dim, ctx.tok_seq, ctx.tok_pos, ctx.seqs,
                      ctx.max_position, group.table, key_pages, value_pages, group.page_size, run.writes_cache)

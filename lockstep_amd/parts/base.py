@@ -20,6 +20,11 @@ Kinds of part and what each must provide:
                     cache, writes this step's part of it, and writes (or adds)
                     ``[T, H]`` into the 32-bit ``out``.
 ``FeedForward``     ``forward(ctx, x, out, accumulate)``: token-wise.
+                    A mixer or feed-forward whose ``forward`` also takes
+                    ``norm=None`` may be handed the residual stream itself and
+                    the norm part to apply inside its first kernel (the
+                    arrangement does so for small steps); it must give the
+                    bits it would give on the separately normalised input.
 ``Arrangement``     owns one layer's parts and the order they run in.
 
 Rule for every ``forward``: a row's result depends on rows of the same

@@ -24,6 +24,8 @@ class PreNormResidual(Arrangement):
         self.feed_forward_norm = build_part(layer_spec.feed_forward_norm,
                                             self.join(base, p["feed_forward_norm_name"]))
         self.feed_forward = build_part(layer_spec.feed_forward, self.join(base, p["feed_forward_prefix"]))
+        self._fuse_mixer = self._fuses(self._mixer, self.mixer_norm)
+        self._fuse_ff = self._fuses(self.feed_forward, self.feed_forward_norm)
 
     @classmethod
     def weight_specs(cls, layer_spec, prefix: str = ""):
@@ -50,10 +52,31 @@ class PreNormResidual(Arrangement):
         for part in self.parts():
             part.load(weights, rt)
 
+    #: a step of at most this many tokens lets the consumer's first matrix
+    #: product normalise its input itself (one launch less per norm).  Off by
+    #: default: on MI355X the longer dependent chain inside the product costs
+    #: more than the launch it saves (Qwen3-0.6B sizes, batch 1 and 8: 7 % slower).
+    FUSE_NORM_ROWS = int(__import__("os").environ.get("LOCKSTEP_FUSE_NORM_ROWS", "0"))
+
+    @staticmethod
+    def _fuses(part, norm) -> bool:
+        import inspect
+
+        return (getattr(norm, "kind", "") == "rmsnorm"
+                and "norm" in inspect.signature(part.forward).parameters)
+
     def forward(self, ctx, run, h) -> None:
         rt = ctx.rt
-        x = ctx.buf("block.normed", (ctx.n_tokens, h.shape[1]), rt.dtype)
-        self.mixer_norm.forward(ctx, h, x)
-        self._mixer.forward(ctx, run, x, h, accumulate=True)
-        self.feed_forward_norm.forward(ctx, h, x)
-        self.feed_forward.forward(ctx, x, h, accumulate=True)
+        small = ctx.n_tokens <= self.FUSE_NORM_ROWS
+        if small and self._fuse_mixer:
+            self._mixer.forward(ctx, run, h, h, accumulate=True, norm=self.mixer_norm)
+        else:
+            x = ctx.buf("block.normed", (ctx.n_tokens, h.shape[1]), rt.dtype)
+            self.mixer_norm.forward(ctx, h, x)
+            self._mixer.forward(ctx, run, x, h, accumulate=True)
+        if small and self._fuse_ff:
+            self.feed_forward.forward(ctx, h, h, accumulate=True, norm=self.feed_forward_norm)
+        else:
+            x = ctx.buf("block.normed", (ctx.n_tokens, h.shape[1]), rt.dtype)
+            self.feed_forward_norm.forward(ctx, h, x)
+            self.feed_forward.forward(ctx, x, h, accumulate=True)

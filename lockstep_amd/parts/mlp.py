@@ -1,14 +1,16 @@
 """Gated feed-forward: ``down(act(gate(x)) * up(x))`` without biases; with the
 SiLU activation this is the reference's SwiGLU MLP
 (engine/model/qwen3.py:368-370, engine/kernels/swiglu.py:25-29).  Gate and up
-are one matrix product over ``[Wg; Wu]``."""
+are one matrix product over their rows interleaved in tiles of 16, whose
+epilogue applies the activation, so the two projections never leave the
+kernel."""
 
 from __future__ import annotations
 
 import torch
 
 from ..config.base import PartSpec
-from ..ops import ADD_F32, STORE_F32
+from ..ops import ADD_F32, STORE_F32, SWIGLU, interleave_gate_up
 from .base import FeedForward, WeightSpec, register_part
 
 
@@ -36,14 +38,16 @@ class GatedMLP(FeedForward):
         up = weights.get(f"{self.prefix}.up_proj.weight")
         if gate.dtype != up.dtype:
             gate, up = gate.to(torch.float32), up.to(torch.float32)
-        self.w_gate_up = rt.matrix(torch.cat([gate, up], dim=0))
+        self.w_gate_up = rt.matrix(interleave_gate_up(gate, up))
         self.w_down = rt.matrix(weights.get(f"{self.prefix}.down_proj.weight"))
 
-    def forward(self, ctx, x, out, accumulate: bool) -> None:
+    def forward(self, ctx, x, out, accumulate: bool, norm=None) -> None:
+        """``norm``: when given, ``x`` is the float32 residual stream and ``norm``
+        (an RMSNorm part) is applied inside the first matrix product."""
         rt = ctx.rt
-        t = ctx.n_tokens
-        gate_up = ctx.buf("mlp.gate_up", (t, 2 * self.inter), rt.dtype)
-        rt.kernels.gemm(x, self.w_gate_up, gate_up)
-        act = ctx.buf("mlp.act", (t, self.inter), rt.dtype)
-        rt.kernels.swiglu(gate_up, act)
+        act = ctx.buf("mlp.act", (ctx.n_tokens, self.inter), rt.dtype)
+        if norm is None:
+            rt.kernels.gemm(x, self.w_gate_up, act, SWIGLU)
+        else:
+            rt.kernels.gemm(x, self.w_gate_up, act, SWIGLU, norm_weight=norm.weight, eps=norm.eps)
         rt.kernels.gemm(act, self.w_down, out, ADD_F32 if accumulate else STORE_F32)

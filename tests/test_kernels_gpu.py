@@ -401,3 +401,59 @@ def test_decode_attention_is_the_same_in_every_kernel(dtype, nq, nkv, d, ps):
         for variant, split in variants:
             got = case.attend(dev[start:start + n], start, d ** -0.5, variant=variant, force_split=split)
             assert torch.equal(got, ref), f"start={start} n={n} variant={variant} split={split}"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("m", [1, 9, 16, 40, 200])
+@pytest.mark.parametrize("inter,k", [(136, 96), (3072, 1024), (48, 260)])
+def test_gemm_with_swiglu_epilogue(dtype, m, inter, k):
+    """Gate and up interleaved in tiles of 16 rows, activation in the epilogue:
+    equals silu(x Wg^T) * (x Wu^T); a row has the same bits at any batch size."""
+    from lockstep_amd.ops import SWIGLU, interleave_gate_up
+
+    g = torch.Generator().manual_seed(inter + k)
+    x = torch.randn(m, k, generator=g).to(dtype)
+    gate = (torch.randn(inter, k, generator=g) * 0.2).to(dtype)
+    up = (torch.randn(inter, k, generator=g) * 0.2).to(dtype)
+    w = interleave_gate_up(gate, up).cuda()
+    assert w.shape[0] % 32 == 0 and torch.equal(w[16:32, :].cpu(), up[:16])
+    out = torch.empty(m, inter, dtype=dtype, device="cuda")
+    K().gemm(x.cuda(), w, out, SWIGLU)
+    want = torch.nn.functional.silu(x.double() @ gate.double().T) * (x.double() @ up.double().T)
+    assert rel_err(out, want) < TOL[dtype]
+    one = torch.empty(1, inter, dtype=dtype, device="cuda")
+    K().gemm(x[m - 1:].cuda(), w, one, SWIGLU)
+    assert torch.equal(one[0], out[m - 1])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("m,n,k", [(1, 64, 1024), (8, 272, 96), (16, 100, 3072), (5, 48, 200)])
+def test_gemm_with_fused_norm_equals_norm_then_gemm(dtype, m, n, k):
+    """The RMSNorm prologue of the skinny kernel gives the bits of the
+    stand-alone norm kernel followed by the plain product, also with the
+    SwiGLU epilogue."""
+    from lockstep_amd.ops import STORE, SWIGLU, interleave_gate_up
+
+    g = torch.Generator().manual_seed(m + n + k)
+    h = (torch.randn(m, k, generator=g) * 3).cuda()
+    nw = (1 + 0.2 * torch.randn(k, generator=g)).cuda()
+    w = (torch.randn(n, k, generator=g) * 0.1).to(dtype).cuda()
+    eps = 1e-5
+    normed = torch.empty(m, k, dtype=dtype, device="cuda")
+    K().rmsnorm(h, nw, normed, eps)
+    want = torch.empty(m, n, dtype=dtype, device="cuda")
+    K().gemm(normed, w, want, STORE)
+    got = torch.empty(m, n, dtype=dtype, device="cuda")
+    K().gemm(h, w, got, STORE, norm_weight=nw, eps=eps)
+    assert torch.equal(got, want)
+    inter = n // 2
+    wi = interleave_gate_up(w[:inter].cpu(), w[inter:2 * inter].cpu()).cuda()
+    want2 = torch.empty(m, inter, dtype=dtype, device="cuda")
+    K().gemm(normed, wi, want2, SWIGLU)
+    got2 = torch.empty(m, inter, dtype=dtype, device="cuda")
+    K().gemm(h, wi, got2, SWIGLU, norm_weight=nw, eps=eps)
+    assert torch.equal(got2, want2)
+    from lockstep_amd.ops import KernelError
+    with pytest.raises(KernelError):
+        K().gemm(torch.zeros(17, k, device="cuda"), w, torch.empty(17, n, dtype=dtype, device="cuda"), STORE,
+                 norm_weight=nw, eps=eps)
