@@ -160,12 +160,13 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const void* __rest
       for (int j = 0; j < MT; ++j) acc[t][j] = f32x4{0.f, 0.f, 0.f, 0.f};
     const int k_begin = s * kslice;
     const int k_end = min(K, k_begin + kslice);
-    // Four chunks at a time: all their loads are issued before the first
-    // MFMA needs one, so a wave keeps several kilobytes in flight.
-    for (int k0 = k_begin; k0 < k_end; k0 += 4 * A::KCHUNK) {
-      vec_t w[NT][4], x[MT][4];
+    // UNR chunks at a time: all their loads are issued before the first MFMA
+    // needs one, so a wave keeps several kilobytes in flight.
+    constexpr int UNR = (NT * MT == 1 && !NORM) ? 8 : 4;
+    for (int k0 = k_begin; k0 < k_end; k0 += UNR * A::KCHUNK) {
+      vec_t w[NT][UNR], x[MT][UNR];
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
+      for (int u = 0; u < UNR; ++u) {
         const int k = k0 + u * A::KCHUNK + g * A::VEC;
         const bool in = k0 + u * A::KCHUNK < k_end;
 #pragma unroll
@@ -202,7 +203,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const void* __rest
         }
       }
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
+      for (int u = 0; u < UNR; ++u) {
         if (k0 + u * A::KCHUNK >= k_end) break;  // uniform: a chunk is visited iff it starts inside the slice
 #pragma unroll
         for (int t = 0; t < NT; ++t)
@@ -382,14 +383,17 @@ int launch_gemm(const void* X, const void* W, void* C, int M, int N, int K, long
   if (norm_w && M > 16) return fail("gemm: the fused norm prologue takes at most 16 rows, got %d", M);
   if (M <= 64) {
     const int mt = (M + 15) / 16;
-    const int nw = nslices >= 8 ? 8 : 4;
+    // 16 waves leave 128 registers a lane: only for one or two row tiles
+    const int nw = (nslices > 8 && mt * NT <= 2) ? 16 : (nslices > 4 ? 8 : 4);
     dim3 grid((N + 16 * NT - 1) / (16 * NT));
     const size_t lds = ((size_t)nslices * NT * mt * 256 + (norm_w ? 80 : 0)) * sizeof(float);
 #define LS_SKINNY(MT_, NW_, NORM_)                                                                              \
   hipLaunchKernelGGL((gemm_skinny_kernel<T, MT_, NW_, EPI, NORM_>), grid, dim3(NW_ * 64), lds, stream, X, w, C, M, N, \
                      K, ldx, ldc, kslice, aligned, vec_ok, norm_w, eps, out_cols)
     if (norm_w) {
-      if (nw == 8) LS_SKINNY(1, 8, true); else LS_SKINNY(1, 4, true);
+      if (nw >= 8) LS_SKINNY(1, 8, true); else LS_SKINNY(1, 4, true);
+    } else if (nw == 16) {
+      if (mt == 1) LS_SKINNY(1, 16, false); else LS_SKINNY(2, 16, false);
     } else if (nw == 8) {
       if (mt == 1) LS_SKINNY(1, 8, false); else if (mt == 2) LS_SKINNY(2, 8, false);
       else if (mt == 3) LS_SKINNY(3, 8, false); else LS_SKINNY(4, 8, false);
