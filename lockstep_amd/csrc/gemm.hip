@@ -19,6 +19,16 @@
 
 namespace ls {
 
+#ifndef LS_GEMM_BIG
+#define LS_GEMM_BIG 512       // from this many 128 x 128 tiles on, use them
+#endif
+#ifndef LS_GEMM_PD_BIG
+#define LS_GEMM_PD_BIG 1      // register prefetch depth (stages) of the 128 x 128 kernel
+#endif
+#ifndef LS_GEMM_PD_SMALL
+#define LS_GEMM_PD_SMALL 2    // ... and of the 64 x 64 kernel
+#endif
+
 enum Epilogue : int {
   kStore = 0,     // C[m][n] = total, in the compute dtype
   kStoreF32 = 1,  // C[m][n] = total, float
@@ -242,116 +252,147 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const void* __rest
 }
 
 // ---------------------------------------------------------------------------
-// Tiled kernel: 128 x 128 outputs per workgroup, four waves of 64 x 64.
+// Tiled kernel: BM x BN outputs per workgroup, four waves in a 2 x 2 grid,
+// each (BM/2) x (BN/2).  Both operands go through LDS in stages of 128 bytes
+// of K per row, double buffered: while stage i is multiplied, stage i+1 is
+// written to the other buffer and the global loads of stage i+2 are in
+// flight.  Accumulators are small enough for two or three workgroups a CU,
+// which is what hides the LDS and barrier latency.  Workgroups are numbered
+// so that those that share a weight tile run on the same XCD (each XCD has
+// its own L2).
 // ---------------------------------------------------------------------------
-constexpr int kTile = 128;
-constexpr int kRowBytes = 128;            // bytes of K per row per stage (two chunks)
-constexpr int kRowStride = kRowBytes + 16;  // padded LDS row
+constexpr int kRowBytes = 128;               // bytes of K per row per stage (two chunks)
+constexpr int kRowStride = kRowBytes + 16;   // padded LDS row
 
-template <typename T, int EPI>
+template <typename T, int EPI, int BM, int BN, int PD>
 __global__ __launch_bounds__(256) void gemm_tiled_kernel(const T* __restrict__ X, const T* __restrict__ W,
                                                          void* __restrict__ C, int M, int N, int K, long ldx,
                                                          long ldc, int kslice, int aligned, int vec_ok,
-                                                         int tiles_m, int out_cols) {
+                                                         int tiles_m, int tiles_n, int out_cols) {
   typedef Atom<T> A;
   typedef typename A::vec_t vec_t;
   constexpr int BK = kRowBytes / sizeof(T);  // elements of K per stage
-  __shared__ __attribute__((aligned(16))) unsigned char w_lds[kTile * kRowStride];
-  __shared__ __attribute__((aligned(16))) unsigned char x_lds[kTile * kRowStride];
+  constexpr int TI = BN / 32;                // weight tiles (16 columns) per wave
+  constexpr int TJ = BM / 32;                // row tiles per wave
+  constexpr int WP = BN / 32;                // staging passes over the weight tile (32 rows each)
+  constexpr int XP = BM / 32;
+  constexpr int STAGE_BYTES = (BM + BN) * kRowStride;
+  __shared__ __attribute__((aligned(16))) unsigned char lds[2 * STAGE_BYTES];
 
-  const int tile_m = blockIdx.x % tiles_m;
-  const int tile_n = blockIdx.x / tiles_m;
-  const int m_base = tile_m * kTile;
-  const int n_base = tile_n * kTile;
+  // XCD-aware numbering: consecutive ids on one XCD walk the row tiles of one weight tile
+  int id = blockIdx.x;
+  const int total_tiles = tiles_m * tiles_n;
+  if (total_tiles % 8 == 0) id = (id % 8) * (total_tiles / 8) + id / 8;
+  const int tile_m = id % tiles_m;
+  const int tile_n = id / tiles_m;
+  const int m_base = tile_m * BM;
+  const int n_base = tile_n * BN;
 
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
-  const int wn = (wave & 1) * 64;
-  const int wm = (wave >> 1) * 64;
+  const int wn = (wave & 1) * (BN / 2);
+  const int wm = (wave >> 1) * (BM / 2);
   const int row16 = lane & 15;
   const int g = lane >> 4;
-
-  // staging assignment: 8 threads per row (16 bytes each), 32 rows per pass
-  const int st_row = threadIdx.x >> 3;
+  const int st_row = threadIdx.x >> 3;             // staging: 8 threads per row, 32 rows per pass
   const int st_col = (threadIdx.x & 7) * A::VEC;
 
-  f32x4 total[4][4];
-  f32x4 acc[4][4];
+  f32x4 total[TI][TJ];
+  f32x4 acc[TI][TJ];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < TI; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < TJ; ++j) {
       total[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
       acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
 
-  // Stages of BK elements; kslice is a multiple of BK, so a stage never
-  // straddles a slice.  The next stage's global loads are in flight while the
-  // current one is multiplied out of LDS.
-  vec_t wv[4], xv[4];
+  // PD stages of global loads are in flight in registers (slot = stage % PD)
+  vec_t wv[PD][WP], xv[PD][XP];
+  auto fetch = [&](int slot, int k0) {
 #pragma unroll
-  for (int p = 0; p < 4; ++p) {
-    const int r = st_row + 32 * p;
-    wv[p] = load_vec<T>(W, n_base + r, st_col, K, K, n_base + r < N, aligned);
-    xv[p] = load_vec<T>(X, m_base + r, st_col, K, ldx, m_base + r < M, aligned);
-  }
-  for (int k0 = 0; k0 < K; k0 += BK) {
-    if (k0 > 0 && k0 % kslice == 0) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-#pragma unroll
-          for (int r = 0; r < 4; ++r) total[i][j][r] = total[i][j][r] + acc[i][j][r];
-          acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
-        }
-    }
-    __syncthreads();  // previous stage fully consumed
-#pragma unroll
-    for (int p = 0; p < 4; ++p) {
+    for (int p = 0; p < WP; ++p) {
       const int r = st_row + 32 * p;
-      *reinterpret_cast<vec_t*>(&w_lds[r * kRowStride + st_col * sizeof(T)]) = wv[p];
-      *reinterpret_cast<vec_t*>(&x_lds[r * kRowStride + st_col * sizeof(T)]) = xv[p];
+      wv[slot][p] = load_vec<T>(W, n_base + r, k0 + st_col, K, K, n_base + r < N, aligned);
     }
-    __syncthreads();
-    if (k0 + BK < K) {
 #pragma unroll
-      for (int p = 0; p < 4; ++p) {
-        const int r = st_row + 32 * p;
-        wv[p] = load_vec<T>(W, n_base + r, k0 + BK + st_col, K, K, n_base + r < N, aligned);
-        xv[p] = load_vec<T>(X, m_base + r, k0 + BK + st_col, K, ldx, m_base + r < M, aligned);
+    for (int p = 0; p < XP; ++p) {
+      const int r = st_row + 32 * p;
+      xv[slot][p] = load_vec<T>(X, m_base + r, k0 + st_col, K, ldx, m_base + r < M, aligned);
+    }
+  };
+  auto stash = [&](int slot, int buf) {
+    unsigned char* w_lds = lds + buf * STAGE_BYTES;
+    unsigned char* x_lds = w_lds + BN * kRowStride;
+#pragma unroll
+    for (int p = 0; p < WP; ++p)
+      *reinterpret_cast<vec_t*>(&w_lds[(st_row + 32 * p) * kRowStride + st_col * sizeof(T)]) = wv[slot][p];
+#pragma unroll
+    for (int p = 0; p < XP; ++p)
+      *reinterpret_cast<vec_t*>(&x_lds[(st_row + 32 * p) * kRowStride + st_col * sizeof(T)]) = xv[slot][p];
+  };
+
+  const int stages = (K + BK - 1) / BK;
+  // stage s lives in register slot s % PD until it is written to LDS buffer s % 2
+  fetch(0, 0);
+  stash(0, 0);
+#pragma unroll
+  for (int u = 1; u <= PD; ++u)
+    if (u < stages) fetch(u % PD, u * BK);
+  for (int base = 0; base < stages; base += PD) {
+#pragma unroll
+    for (int u = 0; u < PD; ++u) {  // unrolled so that the register slots are static
+      const int st = base + u;
+      if (st >= stages) break;
+      const int k0 = st * BK;
+      if (k0 > 0 && k0 % kslice == 0) {  // a stage never straddles a slice: kslice is a multiple of BK
+#pragma unroll
+        for (int i = 0; i < TI; ++i)
+#pragma unroll
+          for (int j = 0; j < TJ; ++j) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) total[i][j][r] = total[i][j][r] + acc[i][j][r];
+            acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+          }
+      }
+      __syncthreads();  // stage st is in its buffer; the other buffer has been read by every wave
+      if (st + 1 < stages) {
+        stash((u + 1) % PD, (st + 1) & 1);
+        if (st + 1 + PD < stages) fetch((u + 1) % PD, (st + 1 + PD) * BK);
+      }
+      const unsigned char* w_lds = lds + (st & 1) * STAGE_BYTES;
+      const unsigned char* x_lds = w_lds + BN * kRowStride;
+#pragma unroll
+      for (int c = 0; c < 2; ++c) {
+        // The skinny kernel visits a chunk iff it starts below K; do the same.
+        if (k0 + c * A::KCHUNK >= K) break;
+        vec_t a[TI], b[TJ];
+#pragma unroll
+        for (int i = 0; i < TI; ++i)
+          a[i] = *reinterpret_cast<const vec_t*>(&w_lds[(wn + i * 16 + row16) * kRowStride + c * 64 + g * 16]);
+#pragma unroll
+        for (int j = 0; j < TJ; ++j)
+          b[j] = *reinterpret_cast<const vec_t*>(&x_lds[(wm + j * 16 + row16) * kRowStride + c * 64 + g * 16]);
+#pragma unroll
+        for (int i = 0; i < TI; ++i)
+#pragma unroll
+          for (int j = 0; j < TJ; ++j) A::mma(acc[i][j], a[i], b[j]);
       }
     }
-#pragma unroll
-    for (int c = 0; c < 2; ++c) {
-      // The skinny kernel visits a chunk iff it starts below K; do the same.
-      if (k0 + c * A::KCHUNK >= K) break;
-      vec_t a[4], b[4];
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-        a[i] = *reinterpret_cast<const vec_t*>(&w_lds[(wn + i * 16 + row16) * kRowStride + c * 64 + g * 16]);
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-        b[j] = *reinterpret_cast<const vec_t*>(&x_lds[(wm + j * 16 + row16) * kRowStride + c * 64 + g * 16]);
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) A::mma(acc[i][j], a[i], b[j]);
-    }
   }
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < TI; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < TJ; ++j)
 #pragma unroll
       for (int r = 0; r < 4; ++r) total[i][j][r] = total[i][j][r] + acc[i][j][r];
 
   if (EPI == kSwiGLU) {
-    // the wave's four weight tiles are (gate t, up t, gate t+1, up t+1)
+    // the wave's weight tiles come in pairs (gate t, up t)
 #pragma unroll
-    for (int i = 0; i < 4; i += 2)
+    for (int i = 0; i < TI; i += 2)
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
+      for (int j = 0; j < TJ; ++j) {
         float gate[4] = {total[i][j][0], total[i][j][1], total[i][j][2], total[i][j][3]};
         float up[4] = {total[i + 1][j][0], total[i + 1][j][1], total[i + 1][j][2], total[i + 1][j][3]};
         epilogue_swiglu4<T>(C, ldc, m_base + wm + j * 16 + row16, (n_base + wn + i * 16) / 2 + g * 4, M, out_cols, gate,
@@ -360,9 +401,9 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const T* __restrict__ X
     return;
   }
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < TI; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < TJ; ++j) {
       float t[4] = {total[i][j][0], total[i][j][1], total[i][j][2], total[i][j][3]};
       epilogue4<T, EPI>(C, ldc, m_base + wm + j * 16 + row16, n_base + wn + i * 16 + g * 4, M, N, t, vec_ok);
     }
@@ -403,10 +444,18 @@ int launch_gemm(const void* X, const void* W, void* C, int M, int N, int K, long
     }
 #undef LS_SKINNY
   } else {
-    const int tiles_m = (M + kTile - 1) / kTile;
-    const int tiles_n = (N + kTile - 1) / kTile;
-    hipLaunchKernelGGL((gemm_tiled_kernel<T, EPI>), dim3(tiles_m * tiles_n), dim3(256), 0, stream,
-                       reinterpret_cast<const T*>(X), w, C, M, N, K, ldx, ldc, kslice, aligned, vec_ok, tiles_m, out_cols);
+    // Large products take 128 x 128 tiles (least LDS traffic per MFMA); smaller ones take
+    // 64 x 64 tiles so that every CU has several workgroups, with a deeper register prefetch.
+    const long big_tiles = (long)((M + 127) / 128) * ((N + 127) / 128);
+#define LS_TILED(BM_, BN_, PD_)                                                                                 \
+  {                                                                                                             \
+    const int tiles_m = (M + BM_ - 1) / BM_, tiles_n = (N + BN_ - 1) / BN_;                                       \
+    hipLaunchKernelGGL((gemm_tiled_kernel<T, EPI, BM_, BN_, PD_>), dim3(tiles_m * tiles_n), dim3(256), 0, stream, \
+                       reinterpret_cast<const T*>(X), w, C, M, N, K, ldx, ldc, kslice, aligned, vec_ok, tiles_m,  \
+                       tiles_n, out_cols);                                                                      \
+  }
+    if (big_tiles >= LS_GEMM_BIG) LS_TILED(128, 128, LS_GEMM_PD_BIG) else LS_TILED(64, 64, LS_GEMM_PD_SMALL)
+#undef LS_TILED
   }
   return check_launch("gemm");
 }
