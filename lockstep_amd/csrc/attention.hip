@@ -11,7 +11,7 @@
 // kTileKeys, and in splits of kSplitKeys anchored at multiples of kSplitKeys,
 // whatever the step's first position is.  Inside a split the tiles are walked
 // in ascending order with the online softmax
-//     m' = max(m, rowmax(s)); a = exp(m - m'); p = exp(s - m') (0 if masked);
+//     m' = max(m, rowmax(s)); a = exp(m - m'); p = exp(s - m') (s = -inf if masked, so p = 0);
 //     l = l*a + sum(p); acc = acc*a + round(p) . V
 // (sum(p): a lane adds its four keys of a 16-key block as (p0+p1)+(p2+p3),
 // the eight blocks in ascending order, then the four lanes of the row)
@@ -66,6 +66,11 @@ struct AttnItem {  // one workgroup column of the attention launch
   int split_lo;    // first of them (splits below lie behind the window)
   int reserved;
 };
+
+// A masked score is minus infinity, so its probability exp(-inf - m) is an
+// exact zero without a select; running maxima start at the finite -1e30, so
+// "m" never becomes infinite and no difference of infinities can arise.
+constexpr float kMasked = -__builtin_huge_valf();
 
 template <typename T> __device__ __forceinline__ float softmax_exp(float x);
 template <> __device__ __forceinline__ float softmax_exp<float>(float x) { return expf(x); }
@@ -164,6 +169,9 @@ __global__ __launch_bounds__(256) void attention_direct_kernel(
   const int qi = row_ok ? r / G : 0;
   const int head = kvh * G + (row_ok ? r % G : 0);
   const int q_pos = sm.q_start + qi;
+  // this row sees the keys key_lo <= key <= key_hi (none if the row does not exist)
+  const int key_hi = row_ok ? q_pos : -1;
+  const int key_lo = window > 0 ? q_pos - window + 1 : 0;
   const int wave_first_pos = sm.q_start + r0 / G;
   const int wave_last_pos = sm.q_start + min(r0 + 15, rows_total - 1) / G;
   const int lo_valid = window > 0 ? max(0, sm.q_start - window + 1) : 0;
@@ -206,17 +214,29 @@ __global__ __launch_bounds__(256) void attention_direct_kernel(
 
       // ---- scale, mask, online softmax --------------------------------------
       // lane holds keys t0 + kb*16 + 4g + e of its row
+      // uniform: every key of the tile is visible to every row of the wave (no mask needed)
+      const bool all_visible = t0 + kTileKeys - 1 <= wave_first_pos && r0 + 15 < rows_total &&
+                               (window <= 0 || wave_last_pos - t0 < window);
       float tile_max = kNegSentinel;
+      if (all_visible) {
 #pragma unroll
-      for (int kb = 0; kb < NB; ++kb)
+        for (int kb = 0; kb < NB; ++kb)
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int key = t0 + kb * 16 + 4 * g + e;
-          const bool keep = row_ok && key <= q_pos && (window <= 0 || q_pos - key < window);
-          const float v = keep ? s[kb][e] * scale : kNegSentinel;
-          s[kb][e] = v;
-          tile_max = fmaxf(tile_max, v);
-        }
+          for (int e = 0; e < 4; ++e) {
+            s[kb][e] = s[kb][e] * scale;
+            tile_max = fmaxf(tile_max, s[kb][e]);
+          }
+      } else {
+#pragma unroll
+        for (int kb = 0; kb < NB; ++kb)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const int key = t0 + kb * 16 + 4 * g + e;
+            const float v = ((key <= key_hi) & (key >= key_lo)) ? s[kb][e] * scale : kMasked;
+            s[kb][e] = v;
+            tile_max = fmaxf(tile_max, v);
+          }
+      }
       tile_max = quad16_max(tile_max);
       const float m_new = fmaxf(cur.m, tile_max);
       const float alpha = softmax_exp<T>(cur.m - m_new);
@@ -224,11 +244,7 @@ __global__ __launch_bounds__(256) void attention_direct_kernel(
 #pragma unroll
       for (int kb = 0; kb < NB; ++kb) {
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int key = t0 + kb * 16 + 4 * g + e;
-          const bool keep = row_ok && key <= q_pos && (window <= 0 || q_pos - key < window);
-          s[kb][e] = keep ? softmax_exp<T>(s[kb][e] - m_new) : 0.f;
-        }
+        for (int e = 0; e < 4; ++e) s[kb][e] = softmax_exp<T>(s[kb][e] - m_new);  // masked: exp(-inf) = 0
         p_sum = p_sum + ((s[kb][0] + s[kb][1]) + (s[kb][2] + s[kb][3]));
       }
       p_sum = quad16_sum(p_sum);
@@ -355,6 +371,9 @@ __global__ __launch_bounds__(256, LS_STAGED_MIN_BLOCKS) void attention_staged_ke
   const int qi = row_ok ? r / G : 0;
   const int head = kvh * G + (row_ok ? r % G : 0);
   const int q_pos = sm.q_start + qi;
+  // this row sees the keys key_lo <= key <= key_hi (none if the row does not exist)
+  const int key_hi = row_ok ? q_pos : -1;
+  const int key_lo = window > 0 ? q_pos - window + 1 : 0;
   const int wave_first_pos = sm.q_start + min(r0, rows_total - 1) / G;
   const int wave_last_pos = sm.q_start + min(r0 + 15, rows_total - 1) / G;
   const int lo_valid = window > 0 ? max(0, sm.q_start - window + 1) : 0;
@@ -500,17 +519,29 @@ __global__ __launch_bounds__(256, LS_STAGED_MIN_BLOCKS) void attention_staged_ke
         }
       }
       // ---- scale, mask, online softmax --------------------------------------
+      // uniform: every key of the tile is visible to every row of the wave (no mask needed)
+      const bool all_visible = t0 + kTileKeys - 1 <= wave_first_pos && r0 + 15 < rows_total &&
+                               (window <= 0 || wave_last_pos - t0 < window);
       float tile_max = kNegSentinel;
+      if (all_visible) {
 #pragma unroll
-      for (int kb = 0; kb < NB; ++kb)
+        for (int kb = 0; kb < NB; ++kb)
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int key = t0 + kb * 16 + 4 * g + e;
-          const bool keep = row_ok && key <= q_pos && (window <= 0 || q_pos - key < window);
-          const float v = keep ? s[kb][e] * scale : kNegSentinel;
-          s[kb][e] = v;
-          tile_max = fmaxf(tile_max, v);
-        }
+          for (int e = 0; e < 4; ++e) {
+            s[kb][e] = s[kb][e] * scale;
+            tile_max = fmaxf(tile_max, s[kb][e]);
+          }
+      } else {
+#pragma unroll
+        for (int kb = 0; kb < NB; ++kb)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const int key = t0 + kb * 16 + 4 * g + e;
+            const float v = ((key <= key_hi) & (key >= key_lo)) ? s[kb][e] * scale : kMasked;
+            s[kb][e] = v;
+            tile_max = fmaxf(tile_max, v);
+          }
+      }
       tile_max = quad16_max(tile_max);
       const float m_new = fmaxf(cur.m, tile_max);
       const float alpha = softmax_exp<T>(cur.m - m_new);
@@ -518,11 +549,7 @@ __global__ __launch_bounds__(256, LS_STAGED_MIN_BLOCKS) void attention_staged_ke
 #pragma unroll
       for (int kb = 0; kb < NB; ++kb) {
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int key = t0 + kb * 16 + 4 * g + e;
-          const bool keep = row_ok && key <= q_pos && (window <= 0 || q_pos - key < window);
-          s[kb][e] = keep ? softmax_exp<T>(s[kb][e] - m_new) : 0.f;
-        }
+        for (int e = 0; e < 4; ++e) s[kb][e] = softmax_exp<T>(s[kb][e] - m_new);  // masked: exp(-inf) = 0
         p_sum = p_sum + ((s[kb][0] + s[kb][1]) + (s[kb][2] + s[kb][3]));
       }
       p_sum = quad16_sum(p_sum);
@@ -633,6 +660,9 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
   const int qi = row_ok ? r / G : 0;
   const int head = kvh * G + (row_ok ? r % G : 0);
   const int q_pos = sm.q_start + qi;
+  // this row sees the keys key_lo <= key <= key_hi (none if the row does not exist)
+  const int key_hi = row_ok ? q_pos : -1;
+  const int key_lo = window > 0 ? q_pos - window + 1 : 0;
   const int first_pos = sm.q_start;
   const int last_pos = sm.q_start + (rows_total - 1) / G;
   const int lo_valid = window > 0 ? max(0, sm.q_start - window + 1) : 0;
@@ -755,8 +785,7 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           const int key = t0 + kb * 16 + 4 * g + e;
-          const bool keep = row_ok && key <= q_pos && (window <= 0 || q_pos - key < window);
-          const float v = keep ? s[j][e] * scale : kNegSentinel;
+          const float v = ((key <= key_hi) & (key >= key_lo)) ? s[j][e] * scale : kMasked;
           s[j][e] = v;
           my_max = fmaxf(my_max, v);
         }
@@ -771,11 +800,7 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
       for (int j = 0; j < 2; ++j) {
         const int kb = 2 * wave + j;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int key = t0 + kb * 16 + 4 * g + e;
-          const bool keep = row_ok && key <= q_pos && (window <= 0 || q_pos - key < window);
-          s[j][e] = keep ? softmax_exp<T>(s[j][e] - m_new) : 0.f;
-        }
+        for (int e = 0; e < 4; ++e) s[j][e] = softmax_exp<T>(s[j][e] - m_new);  // masked: exp(-inf) = 0
         psum[kb * 64 + lane] = (s[j][0] + s[j][1]) + (s[j][2] + s[j][3]);
         prob[kb * 64 + lane] = s[j];
       }
