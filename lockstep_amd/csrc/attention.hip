@@ -51,6 +51,10 @@ constexpr int D = LS_HEAD_DIM;
 static_assert(D % 16 == 0 && D >= 16 && D <= 256, "head size must be a multiple of 16 up to 256");
 constexpr int kTileKeys = 128;
 constexpr int kSplitKeys = 256;
+#ifndef LS_ATTN_RING
+#define LS_ATTN_RING 8
+#endif
+constexpr int kRing = LS_ATTN_RING;  // LDS operand reads kept in flight ahead of the MFMAs
 constexpr int NB = kTileKeys / 16;  // 16-key blocks per tile
 constexpr int DB = D / 16;          // 16-column blocks of the head
 
@@ -504,18 +508,29 @@ __global__ __launch_bounds__(256, LS_STAGED_MIN_BLOCKS) void attention_staged_ke
                       !(window > 0 && t0 + kTileKeys <= wave_first_pos - window + 1);
     if (mine) {
       // ---- S^T = K . Q^T ---------------------------------------------------
+      // Operands come from LDS through a ring of registers, read RING products
+      // ahead of the MFMA that uses them, so the reads' latency overlaps the
+      // matrix work.  The order of the products of one accumulator is unchanged.
       f32x4 s[NB];
+      {
+        constexpr int NS = NB * NC;
+        constexpr int RING = NS < kRing ? NS : kRing;
+        auto k_read = [&](int idx) -> vec_t {
+          const int row = (idx / NC) * 16 + row16;
+          const int piece = (idx % NC) * 4 + g;
+          const int pc = (4 * NC == KPIECES) ? piece : min(piece, KPIECES - 1);
+          vec_t kv = *reinterpret_cast<const vec_t*>(k_lds + row * KROW + ((pc + row) % KPIECES) * 16);
+          if (4 * NC != KPIECES) kv = piece < KPIECES ? kv : A::zero();
+          return kv;
+        };
+        vec_t ring[RING];
 #pragma unroll
-      for (int kb = 0; kb < NB; ++kb) {
-        s[kb] = f32x4{0.f, 0.f, 0.f, 0.f};
-        const int row = kb * 16 + row16;
+        for (int i = 0; i < RING; ++i) ring[i] = k_read(i);
 #pragma unroll
-        for (int c = 0; c < NC; ++c) {
-          const int piece = c * 4 + g;
-          vec_t kv = A::zero();
-          if (piece < KPIECES)
-            kv = *reinterpret_cast<const vec_t*>(k_lds + row * KROW + ((piece + row) % KPIECES) * 16);
-          A::mma(s[kb], kv, qv[c]);
+        for (int idx = 0; idx < NS; ++idx) {
+          if (idx % NC == 0) s[idx / NC] = f32x4{0.f, 0.f, 0.f, 0.f};
+          A::mma(s[idx / NC], ring[idx % RING], qv[idx % NC]);
+          if (idx + RING < NS) ring[idx % RING] = k_read(idx + RING);
         }
       }
       // ---- scale, mask, online softmax --------------------------------------
@@ -561,16 +576,12 @@ __global__ __launch_bounds__(256, LS_STAGED_MIN_BLOCKS) void attention_staged_ke
         for (int e = 0; e < 4; ++e) cur.acc[blk][e] = cur.acc[blk][e] * alpha;
       // ---- O^T += V^T . P^T --------------------------------------------------
       constexpr int KB16 = A::VEC / 4;
-#pragma unroll
-      for (int kb = 0; kb < NB; kb += KB16) {
-        vec_t pv;
-#pragma unroll
-        for (int h = 0; h < KB16; ++h)
-#pragma unroll
-          for (int e = 0; e < 4; ++e) pv[h * 4 + e] = from_f32<T>(s[kb + h][e]);
-#pragma unroll
-        for (int blk = 0; blk < DB; ++blk) {
-          const int d = blk * 16 + row16;
+      {
+        constexpr int NP = (NB / KB16) * DB;
+        constexpr int RING = NP < kRing ? NP : kRing;
+        auto v_read = [&](int idx) -> vec_t {
+          const int kb = (idx / DB) * KB16;
+          const int d = (idx % DB) * 16 + row16;
           vec_t vv;
 #pragma unroll
           for (int h = 0; h < KB16; ++h) {
@@ -586,7 +597,23 @@ __global__ __launch_bounds__(256, LS_STAGED_MIN_BLOCKS) void attention_staged_ke
               for (int e = 0; e < 4; ++e) vv[h * 4 + e] = four[e];
             }
           }
-          A::mma(cur.acc[blk], vv, pv);
+          return vv;
+        };
+        vec_t ring[RING];
+#pragma unroll
+        for (int i = 0; i < RING; ++i) ring[i] = v_read(i);
+        vec_t pv;
+#pragma unroll
+        for (int idx = 0; idx < NP; ++idx) {
+          if (idx % DB == 0) {
+            const int kb = (idx / DB) * KB16;
+#pragma unroll
+            for (int h = 0; h < KB16; ++h)
+#pragma unroll
+              for (int e = 0; e < 4; ++e) pv[h * 4 + e] = from_f32<T>(s[kb + h][e]);
+          }
+          A::mma(cur.acc[idx % DB], ring[idx % RING], pv);
+          if (idx + RING < NP) ring[idx % RING] = v_read(idx + RING);
         }
       }
     }
