@@ -162,6 +162,8 @@ def main(argv=None) -> int:
     p.add_argument("--page-size", type=int, default=16)
     p.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     p.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points and the prefill")
+    p.add_argument("--only-prefill", action="store_true",
+                   help="run the prefill measurement alone and print its record (for profiling)")
     args = p.parse_args(argv)
 
     if args.gpus != 1:
@@ -172,6 +174,12 @@ def main(argv=None) -> int:
 
     model, cfg, full_layers = build_model(args)
     element = 2 if args.dtype == "bf16" else 4
+
+    if args.only_prefill:
+        seconds = measure_prefill(model, cfg, args.prefill_len, args.page_size)
+        print(json.dumps({"prefill": {"value": round(args.prefill_len / seconds, 1), "tokens": args.prefill_len,
+                                      "ms": round(1e3 * seconds, 3)}}))
+        return 0
 
     elapsed, context = measure_decode(model, cfg, args.batch, args.prompt_len, args.steps, args.warmup,
                                       args.page_size)

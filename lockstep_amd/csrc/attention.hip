@@ -55,6 +55,11 @@ constexpr int kSplitKeys = 256;
 #define LS_ATTN_RING 8
 #endif
 constexpr int kRing = LS_ATTN_RING;  // LDS operand reads kept in flight ahead of the MFMAs
+#ifdef LS_ATTN_PROBE
+#define PROBE(i) { long long now_ = clock64(); pr_t[i] += now_ - pr_last; pr_last = now_; }
+#else
+#define PROBE(i)
+#endif
 constexpr int NB = kTileKeys / 16;  // 16-key blocks per tile
 constexpr int DB = D / 16;          // 16-column blocks of the head
 
@@ -484,9 +489,15 @@ __global__ __launch_bounds__(256, LS_STAGED_MIN_BLOCKS) void attention_staged_ke
     hold_pages();
     if (ti_lo + 1 < ti_hi) lookup(ti_lo + 1);
   }
+#ifdef LS_ATTN_PROBE
+  long long pr_t[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  long long pr_last = clock64();
+  const long long pr_begin = pr_last;
+#endif
   for (int ti = ti_lo; ti < ti_hi; ++ti) {
     const int t0 = ti * kTileKeys;
     __syncthreads();  // the previous tile has been read by every wave
+    PROBE(0)
     if (PREFETCH) {
       stash(ti, 0);
     } else {
@@ -497,12 +508,15 @@ __global__ __launch_bounds__(256, LS_STAGED_MIN_BLOCKS) void attention_staged_ke
       }
       if (ti + 1 < ti_hi) lookup(ti + 1);
     }
+    PROBE(1)
     __syncthreads();
+    PROBE(2)
     if (PREFETCH && ti + 1 < ti_hi) {
       fetch(ti + 1, 0);
       hold_pages();
       if (ti + 2 < ti_hi) lookup(ti + 2);
     }
+    PROBE(3)
 
     const bool mine = wave_active && t0 <= wave_last_pos &&
                       !(window > 0 && t0 + kTileKeys <= wave_first_pos - window + 1);
@@ -533,6 +547,7 @@ __global__ __launch_bounds__(256, LS_STAGED_MIN_BLOCKS) void attention_staged_ke
           if (idx + RING < NS) ring[idx % RING] = k_read(idx + RING);
         }
       }
+      PROBE(4)
       // ---- scale, mask, online softmax --------------------------------------
       // uniform: every key of the tile is visible to every row of the wave (no mask needed)
       const bool all_visible = t0 + kTileKeys - 1 <= wave_first_pos && r0 + 15 < rows_total &&
@@ -574,6 +589,7 @@ __global__ __launch_bounds__(256, LS_STAGED_MIN_BLOCKS) void attention_staged_ke
       for (int blk = 0; blk < DB; ++blk)
 #pragma unroll
         for (int e = 0; e < 4; ++e) cur.acc[blk][e] = cur.acc[blk][e] * alpha;
+      PROBE(5)
       // ---- O^T += V^T . P^T --------------------------------------------------
       constexpr int KB16 = A::VEC / 4;
       {
@@ -617,12 +633,317 @@ __global__ __launch_bounds__(256, LS_STAGED_MIN_BLOCKS) void attention_staged_ke
         }
       }
     }
+    PROBE(6)
     if (direct && ((ti + 1) % TILES_PER_SPLIT == 0 || ti + 1 == ti_hi)) {
       fold_split<T>(run, cur.acc, cur.m, cur.l);
       cur.reset();
     }
   }
 
+#ifdef LS_ATTN_PROBE
+  if (threadIdx.x == 0 && kvh == 0 && part_ml != nullptr) {
+    long long* dst = reinterpret_cast<long long*>(part_ml + (1 << 20)) + blockIdx.x * 10;
+    for (int i = 0; i < 8; ++i) dst[i] = pr_t[i];
+    dst[8] = clock64() - pr_begin;
+    dst[9] = ti_hi - ti_lo;
+  }
+#endif
+  if (!row_ok) return;
+  if (direct) {
+    store_output<T>(run, out + (long)(sm.q_off + qi) * ldo + (long)head * D, g);
+  } else {
+    const int split = item.split_begin;
+    const long pr = item.part_base + ((long)kvh * rows_total + r) * item.n_splits + (split - item.split_lo);
+    float* pa = part_acc + pr * D;
+#pragma unroll
+    for (int blk = 0; blk < DB; ++blk) *reinterpret_cast<f32x4*>(pa + blk * 16 + 4 * g) = cur.acc[blk];
+    if (g == 0) {
+      part_ml[pr * 2] = cur.m;
+      part_ml[pr * 2 + 1] = cur.l;
+    }
+  }
+}
+
+
+// Variant 4, "wide": prompt portions.  A workgroup of NW waves owns 16*NW rows
+// and walks the key tiles with two LDS buffers.  The tiles go from global
+// memory straight into LDS (no registers in between): a load instruction of a
+// wave fills 64 consecutive 16-byte pieces of LDS, and each lane chooses the
+// source of its piece, so the K tile arrives in the rotated layout of the
+// staged kernel and the V tile as [8 or 4 keys][column][16 bytes].  While a
+// tile is multiplied the next one is in flight.  Keys outside the held range
+// need no zeroing in K (their scores are replaced by -inf), and the V tile of
+// a boundary tile is cleaned in LDS before use.  The arithmetic of a row is
+// the instruction sequence of the other variants, so the bits are the same.
+template <typename T, int NW>
+__global__ __launch_bounds__(64 * NW) void attention_wide_kernel(
+    const T* __restrict__ q, long ldq, const T* __restrict__ k_pages, const T* __restrict__ v_pages, int nkv,
+    int page_size, int page_shift, const int* __restrict__ table, int table_stride,
+    const SeqMeta* __restrict__ seqs, const AttnItem* __restrict__ items, T* __restrict__ out, long ldo,
+    float* __restrict__ part_acc, float* __restrict__ part_ml, int G, float scale, int window) {
+  typedef Atom<T> A;
+  typedef typename A::vec_t vec_t;
+  constexpr int SZ = sizeof(T);
+  constexpr int NT = 64 * NW;
+  constexpr int ROWS = 16 * NW;
+  constexpr int VEC = A::VEC;
+  constexpr int NC = (D + A::KCHUNK - 1) / A::KCHUNK;
+  constexpr int KROW = D * SZ;
+  constexpr int KPIECES = KROW / 16;
+  constexpr int TOTAL = kTileKeys * KPIECES;  // pieces of the K tile == pieces of the V tile
+  constexpr int PER = (TOTAL + NT - 1) / NT;
+  constexpr int TILE_BYTES = TOTAL * 16;
+  constexpr int BUF_BYTES = 2 * TILE_BYTES;
+  constexpr int TILES_PER_SPLIT = kSplitKeys / kTileKeys;
+  typedef const __attribute__((address_space(1))) void* gptr_t;
+  typedef __attribute__((address_space(3))) void* lptr_t;
+
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+  int* tile_pages = reinterpret_cast<int*>(lds + 2 * BUF_BYTES);  // [2][16]
+
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const AttnItem item = items[blockIdx.x];
+  const SeqMeta sm = seqs[item.seq];
+  const int kvh = blockIdx.y;
+  const int rows_total = sm.q_len * G;
+  const int block_r0 = item.row_block * ROWS;
+  if (block_r0 >= rows_total) return;  // uniform for the workgroup
+  const int block_first_pos = sm.q_start + block_r0 / G;
+  const int block_last_pos = sm.q_start + min(block_r0 + ROWS - 1, rows_total - 1) / G;
+
+  const int r0 = block_r0 + wave * 16;
+  const bool wave_active = r0 < rows_total;
+  const int row16 = lane & 15;
+  const int g = lane >> 4;
+  const int r = r0 + row16;
+  const bool row_ok = r < rows_total;
+  const int qi = row_ok ? r / G : 0;
+  const int head = kvh * G + (row_ok ? r % G : 0);
+  const int q_pos = sm.q_start + qi;
+  const int key_hi = row_ok ? q_pos : -1;
+  const int key_lo = window > 0 ? q_pos - window + 1 : 0;
+  const int wave_first_pos = sm.q_start + min(r0, rows_total - 1) / G;
+  const int wave_last_pos = sm.q_start + min(r0 + 15, rows_total - 1) / G;
+  const int lo_valid = window > 0 ? max(0, sm.q_start - window + 1) : 0;
+  const int* __restrict__ tbl = table + (long)sm.table_row * table_stride;
+  const bool direct = item.part_base < 0;
+  const int pages_per_tile = kTileKeys >> page_shift;
+
+  vec_t qv[NC];
+#pragma unroll
+  for (int c = 0; c < NC; ++c)
+    qv[c] = load_vec<T>(q + (long)head * D, sm.q_off + qi, c * A::KCHUNK + g * VEC, D, ldq, row_ok, true);
+
+  int ti_lo = item.split_begin * TILES_PER_SPLIT;
+  if (window > 0) ti_lo = max(ti_lo, max(0, block_first_pos - window + 1) / kTileKeys);
+  const int ti_hi = min(item.split_end * TILES_PER_SPLIT, block_last_pos / kTileKeys + 1);
+
+  // page id of page `threadIdx.x` of a tile (for the first pages_per_tile threads)
+  auto table_entry = [&](int ti) -> int {
+    const int key = min(ti * kTileKeys + ((int)threadIdx.x << page_shift), sm.kv_len - 1);
+    return tbl[key >> page_shift];
+  };
+  // Start the loads of a tile into its buffer.  Every address is clamped to a
+  // held key of a held page, so nothing outside the cache is touched.
+  auto issue = [&](int ti) {
+    const int t0 = ti * kTileKeys;
+    const int* pages = tile_pages + (ti & 1) * 16;
+    unsigned char* k_buf = lds + (ti & 1) * BUF_BYTES;
+    unsigned char* v_buf = k_buf + TILE_BYTES;
+    const int last_key = sm.kv_len - 1;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const int p = i * NT + (int)threadIdx.x;
+      if (PER * NT != TOTAL && i * NT + wave * 64 >= TOTAL) break;  // uniform for the wave
+      {
+        const int row = p / KPIECES;
+        const int slot = p % KPIECES;
+        const int piece = (slot - row % KPIECES + KPIECES) % KPIECES;
+        const int key = min(t0 + row, last_key);
+        const int page = max(pages[(key - t0) >> page_shift], 0);
+        const T* src = k_pages + (((long)page * nkv + kvh) * page_size + (key & (page_size - 1))) * D + piece * VEC;
+        __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(k_buf + (i * NT + wave * 64) * 16), 16, 0, 0);
+      }
+      {
+        const int c = p / D;
+        const int d = p % D;
+        const int key = min(t0 + c * VEC, last_key & ~(VEC - 1));
+        const int page = max(pages[(key - t0) >> page_shift], 0);
+        const T* src = v_pages + ((((long)page * nkv + kvh) * D + d) << page_shift) + (key & (page_size - 1));
+        __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(v_buf + (i * NT + wave * 64) * 16), 16, 0, 0);
+      }
+    }
+  };
+
+  RowState run, cur;
+  run.reset();
+  cur.reset();
+
+  int held = 0;
+  if (ti_lo < ti_hi) {
+    if ((int)threadIdx.x < pages_per_tile) tile_pages[(ti_lo & 1) * 16 + threadIdx.x] = table_entry(ti_lo);
+    __syncthreads();
+    issue(ti_lo);
+    if (ti_lo + 1 < ti_hi && (int)threadIdx.x < pages_per_tile) held = table_entry(ti_lo + 1);
+  }
+#ifdef LS_ATTN_PROBE
+  long long pr_t[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  long long pr_last = clock64();
+  const long long pr_begin = pr_last;
+#endif
+  for (int ti = ti_lo; ti < ti_hi; ++ti) {
+    const int t0 = ti * kTileKeys;
+    const unsigned char* k_lds = lds + (ti & 1) * BUF_BYTES;
+    unsigned char* v_lds = lds + (ti & 1) * BUF_BYTES + TILE_BYTES;
+    __asm__ volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this thread's pieces of the tile have landed
+    if (ti + 1 < ti_hi && (int)threadIdx.x < pages_per_tile) tile_pages[((ti + 1) & 1) * 16 + threadIdx.x] = held;
+    PROBE(0)
+    __syncthreads();  // the tile is complete, and the other buffer has been read by every wave
+    PROBE(1)
+    if (t0 + kTileKeys > sm.kv_len || t0 < lo_valid) {  // uniform: clean the values of keys that are not held
+#pragma unroll
+      for (int i = 0; i < PER; ++i) {
+        const int p = i * NT + (int)threadIdx.x;
+        if (PER * NT != TOTAL && p >= TOTAL) break;
+        const int key0 = t0 + (p / D) * VEC;
+        vec_t* at = reinterpret_cast<vec_t*>(v_lds + p * 16);
+        *at = mask_keys(*at, lo_valid - key0, sm.kv_len - key0);
+      }
+      __syncthreads();
+    }
+    if (ti + 1 < ti_hi) {
+      issue(ti + 1);
+      if (ti + 2 < ti_hi && (int)threadIdx.x < pages_per_tile) held = table_entry(ti + 2);
+    }
+
+    PROBE(2)
+    const bool mine = wave_active && t0 <= wave_last_pos &&
+                      !(window > 0 && t0 + kTileKeys <= wave_first_pos - window + 1);
+    if (mine) {
+      // ---- S^T = K . Q^T ---------------------------------------------------
+      f32x4 s[NB];
+      {
+        constexpr int NS = NB * NC;
+        constexpr int RING = NS < kRing ? NS : kRing;
+        auto k_read = [&](int idx) -> vec_t {
+          const int row = (idx / NC) * 16 + row16;
+          const int piece = (idx % NC) * 4 + g;
+          const int pc = (4 * NC == KPIECES) ? piece : min(piece, KPIECES - 1);
+          vec_t kv = *reinterpret_cast<const vec_t*>(k_lds + row * KROW + ((pc + row) % KPIECES) * 16);
+          if (4 * NC != KPIECES) kv = piece < KPIECES ? kv : A::zero();
+          return kv;
+        };
+        vec_t ring[RING];
+#pragma unroll
+        for (int i = 0; i < RING; ++i) ring[i] = k_read(i);
+#pragma unroll
+        for (int idx = 0; idx < NS; ++idx) {
+          if (idx % NC == 0) s[idx / NC] = f32x4{0.f, 0.f, 0.f, 0.f};
+          A::mma(s[idx / NC], ring[idx % RING], qv[idx % NC]);
+          if (idx + RING < NS) ring[idx % RING] = k_read(idx + RING);
+        }
+      }
+      PROBE(3)
+      // ---- scale, mask, online softmax --------------------------------------
+      const bool all_visible = t0 + kTileKeys - 1 <= wave_first_pos && r0 + 15 < rows_total &&
+                               (window <= 0 || wave_last_pos - t0 < window);
+      float tile_max = kNegSentinel;
+      if (all_visible) {
+#pragma unroll
+        for (int kb = 0; kb < NB; ++kb)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            s[kb][e] = s[kb][e] * scale;
+            tile_max = fmaxf(tile_max, s[kb][e]);
+          }
+      } else {
+#pragma unroll
+        for (int kb = 0; kb < NB; ++kb)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const int key = t0 + kb * 16 + 4 * g + e;
+            const float v = ((key <= key_hi) & (key >= key_lo)) ? s[kb][e] * scale : kMasked;
+            s[kb][e] = v;
+            tile_max = fmaxf(tile_max, v);
+          }
+      }
+      tile_max = quad16_max(tile_max);
+      const float m_new = fmaxf(cur.m, tile_max);
+      const float alpha = softmax_exp<T>(cur.m - m_new);
+      float p_sum = 0.f;
+#pragma unroll
+      for (int kb = 0; kb < NB; ++kb) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) s[kb][e] = softmax_exp<T>(s[kb][e] - m_new);  // masked: exp(-inf) = 0
+        p_sum = p_sum + ((s[kb][0] + s[kb][1]) + (s[kb][2] + s[kb][3]));
+      }
+      p_sum = quad16_sum(p_sum);
+      cur.l = cur.l * alpha + p_sum;
+      cur.m = m_new;
+#pragma unroll
+      for (int blk = 0; blk < DB; ++blk)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) cur.acc[blk][e] = cur.acc[blk][e] * alpha;
+      PROBE(4)
+      // ---- O^T += V^T . P^T --------------------------------------------------
+      constexpr int KB16 = VEC / 4;
+      {
+        constexpr int NP = (NB / KB16) * DB;
+        constexpr int RING = NP < kRing ? NP : kRing;
+        auto v_read = [&](int idx) -> vec_t {
+          const int kb = (idx / DB) * KB16;
+          const int d = (idx % DB) * 16 + row16;
+          vec_t vv;
+#pragma unroll
+          for (int h = 0; h < KB16; ++h) {
+            const int key = (kb + h) * 16 + 4 * g;  // the lane's four keys inside the tile
+            const unsigned char* src = v_lds + ((key / VEC) * D + d) * 16 + (key % VEC) * SZ;
+            if (SZ == 2) {
+              bf16x4 four = *reinterpret_cast<const bf16x4*>(src);
+#pragma unroll
+              for (int e = 0; e < 4; ++e) vv[h * 4 + e] = four[e];
+            } else {
+              f32x4 four = *reinterpret_cast<const f32x4*>(src);
+#pragma unroll
+              for (int e = 0; e < 4; ++e) vv[h * 4 + e] = four[e];
+            }
+          }
+          return vv;
+        };
+        vec_t ring[RING];
+#pragma unroll
+        for (int i = 0; i < RING; ++i) ring[i] = v_read(i);
+        vec_t pv;
+#pragma unroll
+        for (int idx = 0; idx < NP; ++idx) {
+          if (idx % DB == 0) {
+            const int kb = (idx / DB) * KB16;
+#pragma unroll
+            for (int h = 0; h < KB16; ++h)
+#pragma unroll
+              for (int e = 0; e < 4; ++e) pv[h * 4 + e] = from_f32<T>(s[kb + h][e]);
+          }
+          A::mma(cur.acc[idx % DB], ring[idx % RING], pv);
+          if (idx + RING < NP) ring[idx % RING] = v_read(idx + RING);
+        }
+      }
+    }
+    PROBE(5)
+    if (direct && ((ti + 1) % TILES_PER_SPLIT == 0 || ti + 1 == ti_hi)) {
+      fold_split<T>(run, cur.acc, cur.m, cur.l);
+      cur.reset();
+    }
+  }
+
+#ifdef LS_ATTN_PROBE
+  if ((threadIdx.x == 0 || threadIdx.x == 64 * (NW - 1)) && kvh == 0 && part_ml != nullptr) {
+    long long* dst = reinterpret_cast<long long*>(part_ml + (1 << 20)) + (blockIdx.x * 2 + (threadIdx.x ? 1 : 0)) * 10;
+    for (int i = 0; i < 8; ++i) dst[i] = pr_t[i];
+    dst[8] = clock64() - pr_begin;
+    dst[9] = ti_hi - ti_lo;
+  }
+#endif
   if (!row_ok) return;
   if (direct) {
     store_output<T>(run, out + (long)(sm.q_off + qi) * ldo + (long)head * D, g);
@@ -1028,6 +1349,32 @@ static bool coop_supported(int dtype) {
   return st == 1;
 }
 
+// The wide kernel: two buffers of a K and a V tile, and two rows of page ids.
+constexpr int kWideWaves = 8;
+static size_t wide_lds_bytes(int dtype) { return 4 * (size_t)kTileKeys * D * (dtype == kF32 ? 4 : 2) + 2 * 16 * sizeof(int); }
+static bool wide_supported(int dtype) {
+  const size_t bytes = wide_lds_bytes(dtype);
+  if (bytes > kLdsLimit) return false;
+  if (bytes <= 64 * 1024) return true;
+  static int state[2] = {0, 0};
+  int& st = state[dtype == kF32 ? 0 : 1];
+  if (st == 0) {
+    hipError_t e = dtype == kF32
+        ? hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_wide_kernel<float, kWideWaves>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes)
+        : hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_wide_kernel<bf16_t, kWideWaves>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+    if (e != hipSuccess) (void)hipGetLastError();
+    st = e == hipSuccess ? 1 : -1;
+  }
+  return st == 1;
+}
+// 1 if the wide kernel (variant 4) can run for this dtype.
+extern "C" int ls_attn_wide_supported(int dtype) { return wide_supported(dtype) ? 1 : 0; }
+// Rows of one work item's row block: AttnItem.row_block counts blocks of this many rows.
+extern "C" int ls_attn_block_rows(int variant) { return variant == 4 ? 16 * kWideWaves : 64; }
+
+// variant: 4 runs the wide kernel (row blocks of ls_attn_block_rows(4) rows);
 // variant: 3 runs the cooperative kernel (all items must have at most 16 rows);
 // variant: 0 picks the staged kernel where its tiles fit into LDS and the
 // direct one elsewhere, 1 forces the direct kernel, 2 the staged one.
@@ -1071,6 +1418,24 @@ extern "C" int ls_attention(int dtype, const void* q, long ldq, const void* k_pa
     else
       return fail("attention: unknown dtype %d", dtype);
     return check_launch("attention (cooperative)");
+  }
+  if (variant == 4) {
+    LS_REQUIRE(wide_supported(dtype), "attention: the wide variant does not fit into LDS for this head size");
+    LS_REQUIRE(page_size >= 8, "attention: the wide variant needs pages of at least 8 keys, got %d", page_size);
+    const size_t bytes = wide_lds_bytes(dtype);
+    if (dtype == kF32)
+      hipLaunchKernelGGL((attention_wide_kernel<float, kWideWaves>), grid, dim3(64 * kWideWaves), bytes, s,
+                         (const float*)q, ldq, (const float*)k_pages, (const float*)v_pages, nkv, page_size,
+                         page_shift, table, table_stride, (const SeqMeta*)seqs, (const AttnItem*)items, (float*)out,
+                         ldo, part_acc, part_ml, G, scale, window);
+    else if (dtype == kBF16)
+      hipLaunchKernelGGL((attention_wide_kernel<bf16_t, kWideWaves>), grid, dim3(64 * kWideWaves), bytes, s,
+                         (const bf16_t*)q, ldq, (const bf16_t*)k_pages, (const bf16_t*)v_pages, nkv, page_size,
+                         page_shift, table, table_stride, (const SeqMeta*)seqs, (const AttnItem*)items, (bf16_t*)out,
+                         ldo, part_acc, part_ml, G, scale, window);
+    else
+      return fail("attention: unknown dtype %d", dtype);
+    return check_launch("attention (wide)");
   }
   const bool staged = variant != 1 && staged_fits(dtype, lds_bytes);
   LS_REQUIRE(variant != 2 || staged, "attention: the staged variant needs %zu bytes of LDS, which is not available",

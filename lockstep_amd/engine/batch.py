@@ -38,6 +38,8 @@ class AttentionPlan:
     coop_items: torch.Tensor | None
     n_coop: int
     coop_max_rows: int
+    wide_items: torch.Tensor | None
+    n_wide: int
     combine_items: torch.Tensor | None
     n_combine: int
     part_acc: torch.Tensor | None
@@ -117,7 +119,9 @@ class StepContext:
             return
         tile, split = self.rt.kernels.attention_geometry(head_dim)
         coop_ok = self.rt.kernels.coop_supported(head_dim, self.rt.dtype)
-        items, coop, combine = [], [], []
+        wide_ok = self.rt.kernels.wide_supported(head_dim, self.rt.dtype, self.cache.page_size)
+        wide_rows = self.rt.kernels.attention_block_rows(head_dim, 4)
+        items, coop, wide, combine = [], [], [], []
         coop_max_rows = 0
         part_rows = 0
         bucket = 0
@@ -145,22 +149,30 @@ class StepContext:
                     target.append((i, 0, s, s + 1, base, n_splits, split_lo, 0))
                 combine.append((i, 0, base, n_splits))
             else:
-                for block in range(-(-rows // 64)):
-                    first_pos = q_start + (block * 64) // group_size
-                    last_pos = q_start + min(block * 64 + 63, rows - 1) // group_size
+                # long portions go to the wide kernel, in larger row blocks
+                if wide_ok and rows > 64:
+                    target, block_rows = wide, wide_rows
+                else:
+                    block_rows = 64
+                for block in range(-(-rows // block_rows)):
+                    first_pos = q_start + (block * block_rows) // group_size
+                    last_pos = q_start + min((block + 1) * block_rows - 1, rows - 1) // group_size
                     begin = (max(0, first_pos - window + 1) // split) if window > 0 else 0
                     target.append((i, block, begin, last_pos // split + 1, -1, 0, 0, 0))
+        # the longest row blocks first: they decide when the launch ends
+        wide.sort(key=lambda it: it[2] - it[3])
         self._plans[key] = (np.asarray(items, dtype=np.int64).reshape(-1),
                             np.asarray(combine, dtype=np.int64).reshape(-1), len(items), len(combine), part_rows,
-                            np.asarray(coop, dtype=np.int64).reshape(-1), len(coop), coop_max_rows)
+                            np.asarray(coop, dtype=np.int64).reshape(-1), len(coop), coop_max_rows,
+                            np.asarray(wide, dtype=np.int64).reshape(-1), len(wide))
         self._plan_specs.append(key)
 
     def upload(self) -> None:
         """Copy all metadata to the device in one transfer."""
         parts = list(self._host_parts)
         for key in self._plan_specs:
-            items, combine, _, _, _, coop, _, _ = self._plans[key]
-            parts += [items, combine, coop]
+            items, combine, _, _, _, coop, _, _, wide, _ = self._plans[key]
+            parts += [items, combine, coop, wide]
         flat = np.concatenate(parts).astype(np.int32)
         host = torch.from_numpy(flat)
         dev = self.workspace.get("step.meta", (flat.shape[0],), torch.int32)
@@ -179,21 +191,24 @@ class StepContext:
         self.want_rows = take(self.n_want)
         self._device_plans: dict[tuple, AttentionPlan] = {}
         for key in self._plan_specs:
-            items, combine, n_items, n_combine, part_rows, coop, n_coop, coop_max_rows = self._plans[key]
+            items, combine, n_items, n_combine, part_rows, coop, n_coop, coop_max_rows, wide, n_wide = self._plans[key]
             head_dim = key[2]
             d_items, d_combine, d_coop = take(items.shape[0]), take(combine.shape[0]), take(coop.shape[0])
+            d_wide = take(wide.shape[0])
             part_acc = part_ml = None
             if part_rows:
                 part_acc = self.workspace.get(f"attention.part_acc.{head_dim}", (part_rows, head_dim), torch.float32)
                 part_ml = self.workspace.get("attention.part_ml", (part_rows, 2), torch.float32)
             self._device_plans[key] = AttentionPlan(d_items, n_items, d_coop if n_coop else None, n_coop,
-                                                    coop_max_rows, d_combine if n_combine else None,
+                                                    coop_max_rows, d_wide if n_wide else None, n_wide,
+                                                    d_combine if n_combine else None,
                                                     n_combine, part_acc, part_ml)
         self._uploaded = True
 
     def plan_signature(self) -> tuple:
         """Sizes of the work lists: equal signatures mean an equal device layout."""
-        return tuple((key, self._plans[key][2], self._plans[key][3], self._plans[key][4], self._plans[key][6])
+        return tuple((key, self._plans[key][2], self._plans[key][3], self._plans[key][4], self._plans[key][6],
+                      self._plans[key][9])
                      for key in self._plan_specs) + (self.n_tokens, self.n_want)
 
     def attention_plan(self, group_size: int, nkv: int, head_dim: int, window: int) -> AttentionPlan:

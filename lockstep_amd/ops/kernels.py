@@ -91,6 +91,14 @@ class Kernels:
         """Whether the cooperative attention kernel can run (its tiles must fit into LDS)."""
         return bool(self.attention_lib(head_dim).ls_attn_coop_supported(c_int(DTYPE_CODE[dtype])))
 
+    def wide_supported(self, head_dim: int, dtype: torch.dtype, page_size: int) -> bool:
+        """Whether the wide attention kernel (variant 4, for prompt portions) can run."""
+        return page_size >= 8 and bool(self.attention_lib(head_dim).ls_attn_wide_supported(c_int(DTYPE_CODE[dtype])))
+
+    def attention_block_rows(self, head_dim: int, variant: int) -> int:
+        """Rows of the row blocks that work items of this variant count in."""
+        return int(self.attention_lib(head_dim).ls_attn_block_rows(c_int(variant)))
+
     def attention_geometry(self, head_dim: int) -> tuple[int, int]:
         """(keys per tile, keys per split) of the attention kernels."""
         lib = self.attention_lib(head_dim)
@@ -244,7 +252,8 @@ class Kernels:
                   window: int, variant: int = 0, max_rows: int = 0) -> None:
         """Launch the attention kernel over ``n_items`` work items (see attention.hip).
         ``variant``: 0 staged through LDS where it fits, 1 direct from global memory, 2 staged or
-        error, 3 cooperative (every item has at most 16 rows; ``max_rows`` states the largest)."""
+        error, 3 cooperative (every item has at most 16 rows; ``max_rows`` states the largest),
+        4 wide (tiles loaded straight into LDS; items count row blocks of ``attention_block_rows``)."""
         lib = self.attention_lib(d)
         _rows_ok(q, "attention q"); _rows_ok(out, "attention out")
         _need(q.dtype in DTYPE_CODE and out.dtype == q.dtype, "attention q/out dtype")

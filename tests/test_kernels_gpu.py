@@ -208,16 +208,18 @@ class PagedCase:
         n_splits = (kv_len - 1) // split + 1 - split_lo
         use_split = (rows <= 64 and n_splits > 1) if force_split is None else force_split
         items, combine, part_rows = [], [], 0
+        br = kernels().attention_block_rows(self.d, variant)       # rows of a work item's row block
         if use_split:
             part_rows = self.nkv * rows * n_splits
-            for b in range(-(-rows // 64)):
+            for b in range(-(-rows // br)):
                 for s in range(split_lo, split_lo + n_splits):
                     items += [0, b, s, s + 1, 0, n_splits, split_lo, 0]
+            for b in range(-(-rows // 64)):
                 combine += [0, b, 0, n_splits]
         else:
-            for b in range(-(-rows // 64)):
-                first = q_start + (b * 64) // g
-                last = q_start + min(b * 64 + 63, rows - 1) // g
+            for b in range(-(-rows // br)):
+                first = q_start + (b * br) // g
+                last = q_start + min(b * br + br - 1, rows - 1) // g
                 begin = (max(0, first - window + 1) // split) if window else 0
                 items += [0, b, begin, last // split + 1, -1, 0, 0, 0]
         items_t = torch.tensor(items, dtype=torch.int32).cuda()
@@ -273,6 +275,8 @@ def test_prefill_attention_matches_naive(dtype, nq, nkv, d, ps, kv_len):
     assert rel_err(out, want) < ATT_TOL[dtype]
     # the kernel that loads straight from global memory gives the same bits as the LDS-staged one
     assert torch.equal(case.attend(dev, 0, d ** -0.5, variant=1), out)
+    if K().wide_supported(d, dtype, ps):
+        assert torch.equal(case.attend(dev, 0, d ** -0.5, variant=4), out), "wide kernel"
     if kv_len == 1:
         assert torch.equal(out.cpu().float()[0], v.float()[0].repeat_interleave(nq // nkv, dim=0))
 
@@ -306,6 +310,10 @@ def test_attention_row_is_the_same_alone_in_a_portion_and_in_the_whole_prompt(dt
         assert torch.equal(part, full[lo:hi]), f"portion {lo}:{hi}"
         part = whole.attend(qkv[lo:hi], lo, d ** -0.5, force_split=True)
         assert torch.equal(part, full[lo:hi]), f"portion {lo}:{hi} split"
+        if K().wide_supported(d, dtype, ps):
+            for split in (False, True):
+                part = whole.attend(qkv[lo:hi], lo, d ** -0.5, variant=4, force_split=split)
+                assert torch.equal(part, full[lo:hi]), f"portion {lo}:{hi}, wide kernel, split={split}"
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -321,6 +329,7 @@ def test_attention_window(dtype, window):
     want = naive_attention(q, k, v, 0, d ** -0.5, window=window)
     assert rel_err(out, want) < ATT_TOL[dtype]
     assert torch.equal(case.attend(dev, 0, d ** -0.5, window=window, variant=1), out)
+    assert torch.equal(case.attend(dev, 0, d ** -0.5, window=window, variant=4), out)
     # pages behind the window may be gone: mark them released and decode the last rows
     for p in (kv_len - 1, 300, 130):
         first_needed = max(0, p - window + 1) // ps
@@ -329,8 +338,13 @@ def test_attention_window(dtype, window):
         alone = case.attend(dev[p:p + 1], p, d ** -0.5, window=window)
         coop = case.attend(dev[p:p + 1], p, d ** -0.5, window=window, variant=3)
         case.table.copy_(saved)
+        lo = max(0, p - 70)                     # a portion: what its first row needs must be held
+        case.table[1, :max(0, lo - window + 1) // ps] = -1
+        wide = case.attend(dev[lo:p + 1], lo, d ** -0.5, window=window, variant=4)
+        case.table.copy_(saved)
         assert torch.equal(alone[0], out[p]), f"row {p}"
         assert torch.equal(coop[0], out[p]), f"row {p}, cooperative kernel"
+        assert torch.equal(wide, out[lo:p + 1]), f"rows {lo}..{p}, wide kernel"
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -398,6 +412,8 @@ def test_decode_attention_is_the_same_in_every_kernel(dtype, nq, nkv, d, ps):
         variants = [(0, True), (0, False), (1, True)]
         if K().coop_supported(d, dtype):
             variants += [(3, True), (3, False)]
+        if K().wide_supported(d, dtype, ps):
+            variants += [(4, True), (4, False)]
         for variant, split in variants:
             got = case.attend(dev[start:start + n], start, d ** -0.5, variant=variant, force_split=split)
             assert torch.equal(got, ref), f"start={start} n={n} variant={variant} split={split}"
