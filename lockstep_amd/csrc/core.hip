@@ -166,34 +166,84 @@ __global__ __launch_bounds__(256) void swiglu_kernel(const T* __restrict__ gu, T
 }
 
 // ---------------------------------------------------------------------------
-// Arg-max of float rows with the lowest index among equal maxima.
+// Arg-max of float rows with the lowest index among equal maxima (NaN never
+// wins; a row without a winner gives 0).  A row is cut into chunks of
+// kArgmaxChunk elements, one workgroup each, whose winners a second small
+// launch reduces; a row of one chunk is finished by the first launch.
 // ---------------------------------------------------------------------------
-__global__ __launch_bounds__(1024) void argmax_kernel(const float* __restrict__ x, int* __restrict__ out, int width,
-                                                      long ld) {
-  __shared__ float best_v[1024];
-  __shared__ int best_i[1024];
-  const float* row = x + (long)blockIdx.x * ld;
+constexpr int kArgmaxChunk = 4096;
+
+__device__ __forceinline__ void argmax_take(float& bv, int& bi, float v, int i) {
+  if (v > bv || (v == bv && i < bi)) { bv = v; bi = i; }
+}
+
+// Reduce (bv, bi) over the 256 threads of the workgroup; valid in thread 0.
+__device__ __forceinline__ void argmax_reduce(float& bv, int& bi) {
+  __shared__ float wave_v[4];
+  __shared__ int wave_i[4];
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    const float ov = __shfl_xor(bv, off, 64);
+    const int oi = __shfl_xor(bi, off, 64);
+    argmax_take(bv, bi, ov, oi);
+  }
+  if ((threadIdx.x & 63) == 0) {
+    wave_v[threadIdx.x >> 6] = bv;
+    wave_i[threadIdx.x >> 6] = bi;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0)
+    for (int w = 1; w < 4; ++w) argmax_take(bv, bi, wave_v[w], wave_i[w]);
+}
+
+__global__ __launch_bounds__(256) void argmax_chunk_kernel(const float* __restrict__ x, int* __restrict__ out,
+                                                           float* __restrict__ part_v, int* __restrict__ part_i,
+                                                           int width, long ld, int chunks) {
+  const float* row = x + (long)blockIdx.y * ld;
+  const int lo = blockIdx.x * kArgmaxChunk;
+  const int hi = min(width, lo + kArgmaxChunk);
   float bv = -INFINITY;
   int bi = 0x7fffffff;
-  for (int e = threadIdx.x; e < width; e += 1024) {
-    const float v = row[e];
-    if (v > bv || (v == bv && e < bi)) { bv = v; bi = e; }
-  }
-  best_v[threadIdx.x] = bv;
-  best_i[threadIdx.x] = bi;
-  __syncthreads();
-  for (int stride = 512; stride > 0; stride >>= 1) {
-    if (threadIdx.x < stride) {
-      const float ov = best_v[threadIdx.x + stride];
-      const int oi = best_i[threadIdx.x + stride];
-      if (ov > best_v[threadIdx.x] || (ov == best_v[threadIdx.x] && oi < best_i[threadIdx.x])) {
-        best_v[threadIdx.x] = ov;
-        best_i[threadIdx.x] = oi;
-      }
+  if ((ld & 3) == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0) {
+    // four loads in flight per thread
+    constexpr int PER = kArgmaxChunk / (256 * 4);
+    f32x4 v[PER];
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      const int e = lo + (j * 256 + threadIdx.x) * 4;
+      v[j] = e + 3 < hi ? *reinterpret_cast<const f32x4*>(row + e) : f32x4{-INFINITY, -INFINITY, -INFINITY, -INFINITY};
+      if (e + 3 >= hi)
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+          if (e + k < hi) v[j][k] = row[e + k];
     }
-    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < PER; ++j)
+#pragma unroll
+      for (int k = 0; k < 4; ++k) argmax_take(bv, bi, v[j][k], lo + (j * 256 + threadIdx.x) * 4 + k);
+  } else {
+    for (int e = lo + threadIdx.x; e < hi; e += 256) argmax_take(bv, bi, row[e], e);
   }
-  if (threadIdx.x == 0) out[blockIdx.x] = best_i[0] == 0x7fffffff ? 0 : best_i[0];
+  argmax_reduce(bv, bi);
+  if (threadIdx.x == 0) {
+    if (chunks == 1) {
+      out[blockIdx.y] = bi == 0x7fffffff ? 0 : bi;
+    } else {
+      part_v[(long)blockIdx.y * chunks + blockIdx.x] = bv;
+      part_i[(long)blockIdx.y * chunks + blockIdx.x] = bi;
+    }
+  }
+}
+
+__global__ __launch_bounds__(256) void argmax_final_kernel(const float* __restrict__ part_v,
+                                                           const int* __restrict__ part_i, int* __restrict__ out,
+                                                           int chunks) {
+  float bv = -INFINITY;
+  int bi = 0x7fffffff;
+  for (int c = threadIdx.x; c < chunks; c += 256)
+    argmax_take(bv, bi, part_v[(long)blockIdx.x * chunks + c], part_i[(long)blockIdx.x * chunks + c]);
+  argmax_reduce(bv, bi);
+  if (threadIdx.x == 0) out[blockIdx.x] = bi == 0x7fffffff ? 0 : bi;
 }
 
 }  // namespace ls
@@ -277,9 +327,20 @@ extern "C" int ls_swiglu(int dtype, const void* gu, void* out, int rows, int int
   return check_launch("swiglu");
 }
 
-extern "C" int ls_argmax(const float* x, int* out, int rows, int width, long ld, void* stream) {
+// Chunks a row of this width is cut into; scratch must hold 2 * rows * chunks 4-byte words when chunks > 1.
+extern "C" int ls_argmax_chunks(int width) { return (width + kArgmaxChunk - 1) / kArgmaxChunk; }
+
+extern "C" int ls_argmax(const float* x, int* out, int rows, int width, long ld, void* scratch, long scratch_words,
+                         void* stream) {
   LS_REQUIRE(rows > 0 && width > 0 && ld >= width, "argmax: bad sizes");
-  hipLaunchKernelGGL(argmax_kernel, dim3(rows), dim3(1024), 0, reinterpret_cast<hipStream_t>(stream), x, out, width,
-                     ld);
+  const int chunks = ls_argmax_chunks(width);
+  LS_REQUIRE(chunks == 1 || (scratch != nullptr && scratch_words >= 2L * rows * chunks),
+             "argmax: scratch of %ld words is too small for %d rows of %d chunks", scratch_words, rows, chunks);
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  float* part_v = reinterpret_cast<float*>(scratch);
+  int* part_i = reinterpret_cast<int*>(scratch) + (long)rows * chunks;
+  hipLaunchKernelGGL(argmax_chunk_kernel, dim3(chunks, rows), dim3(256), 0, s, x, out, part_v, part_i, width, ld,
+                     chunks);
+  if (chunks > 1) hipLaunchKernelGGL(argmax_final_kernel, dim3(rows), dim3(256), 0, s, part_v, part_i, out, chunks);
   return check_launch("argmax");
 }

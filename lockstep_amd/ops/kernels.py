@@ -69,6 +69,7 @@ class Kernels:
         self.core.ls_last_error.restype = ctypes.c_char_p
         self._attention: dict[int, ctypes.CDLL] = {}
         self.attention_paths: dict[int, str] = {}
+        self._argmax_scratch: dict = {}
 
     # -- helpers ------------------------------------------------------------
     @staticmethod
@@ -194,8 +195,13 @@ class Kernels:
               f"argmax out must be int32 [{logits.shape[0]}]")
         if logits.shape[0] == 0:
             return
+        words = 2 * logits.shape[0] * self.core.ls_argmax_chunks(c_int(logits.shape[1]))
+        scratch = self._argmax_scratch.get(logits.device)
+        if scratch is None or scratch.numel() < words:
+            scratch = torch.empty(max(words, 4096), dtype=torch.int32, device=logits.device)
+            self._argmax_scratch[logits.device] = scratch
         code = self.core.ls_argmax(_ptr(logits), _ptr(out), c_int(logits.shape[0]), c_int(logits.shape[1]),
-                                   c_long(logits.stride(0)), _stream())
+                                   c_long(logits.stride(0)), _ptr(scratch), c_long(scratch.numel()), _stream())
         self._check(self.core, code)
 
     # -- attention ----------------------------------------------------------------

@@ -145,6 +145,23 @@ def test_argmax_takes_the_lowest_index_among_maxima():
     one = torch.empty(1, dtype=torch.int32, device="cuda")
     K().argmax(small, one)
     assert one.item() == 1
+    # widths and row strides that are no multiple of four, maxima at the edges of a chunk, NaN, a view
+    g = torch.Generator().manual_seed(3)
+    for width in (4095, 4096, 4097, 8191, 12289, 50001):
+        y = torch.randn(5, width + 3, generator=g)
+        y[0, min(4095, width - 1)] = 9.0
+        y[1, min(4096, width - 1)] = 9.0
+        y[2, width - 1] = 9.0
+        y[3, 0] = float("nan")
+        y[4, :] = float("nan")
+        view = y.cuda()[:, :width]
+        got = torch.empty(5, dtype=torch.int32, device="cuda")
+        K().argmax(view, got)
+        ref = y[:, :width].clone()
+        ref[ref != ref] = float("-inf")
+        want = [int(torch.nonzero(r == r.max())[0]) for r in ref]
+        want[4] = 0
+        assert got.cpu().tolist() == want, width
 
 
 # -- norm + rotation + cache write, attention ---------------------------------------------
