@@ -119,6 +119,29 @@ __device__ __forceinline__ float wave_sum(float v) {
   return v;
 }
 
+// Sum of squares of a float row as every kernel that normalises computes it:
+// thread t of 256 adds the squares of the elements 1024*c + 4*t + {0,1,2,3},
+// c = 0, 1, ... in ascending order; then a butterfly over the wave (wave_sum)
+// and the four wave sums in wave order.  This returns the thread's part.
+__device__ __forceinline__ float row_sumsq_part(const float* __restrict__ src, int width, int t, bool vec_ok) {
+  float part = 0.f;
+  for (int base = 4 * t; base < width; base += 1024) {
+    if (vec_ok && base + 3 < width) {
+      const f32x4 v = *reinterpret_cast<const f32x4*>(src + base);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) part = part + v[e] * v[e];
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (base + e < width) {
+          const float v = src[base + e];
+          part = part + v * v;
+        }
+    }
+  }
+  return part;
+}
+
 }  // namespace ls
 
 // Error reporting across the C interface: every entry point returns 0 or a

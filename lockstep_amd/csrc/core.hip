@@ -40,12 +40,8 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ 
   const int r_out = blockIdx.x;
   const long r_in = rows ? rows[r_out] : r_out;
   const float* src = x + r_in * ldx;
-  float part = 0.f;
-  for (int e = threadIdx.x; e < width; e += 256) {
-    const float v = src[e];
-    part = part + v * v;
-  }
-  part = wave_sum(part);
+  const bool vec_ok = (ldx & 3) == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0;
+  float part = wave_sum(row_sumsq_part(src, width, threadIdx.x, vec_ok));
   if ((threadIdx.x & 63) == 0) wave_part[threadIdx.x >> 6] = part;
   __syncthreads();
   const float total = ((wave_part[0] + wave_part[1]) + wave_part[2]) + wave_part[3];
@@ -220,7 +216,10 @@ __global__ __launch_bounds__(256) void argmax_chunk_kernel(const float* __restri
 #pragma unroll
     for (int j = 0; j < PER; ++j)
 #pragma unroll
-      for (int k = 0; k < 4; ++k) argmax_take(bv, bi, v[j][k], lo + (j * 256 + threadIdx.x) * 4 + k);
+      for (int k = 0; k < 4; ++k) {
+        const int e = lo + (j * 256 + threadIdx.x) * 4 + k;
+        argmax_take(bv, bi, v[j][k], e < hi ? e : 0x7fffffff);  // padding never wins
+      }
   } else {
     for (int e = lo + threadIdx.x; e < hi; e += 256) argmax_take(bv, bi, row[e], e);
   }

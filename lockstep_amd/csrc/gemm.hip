@@ -93,30 +93,27 @@ __device__ __forceinline__ void epilogue_swiglu4(void* __restrict__ C, long ldc,
 
 // RMSNorm of rows of the float residual stream, as a prologue of the skinny
 // kernel (at most 16 rows): the sum of squares of a row is formed exactly as
-// rmsnorm_kernel forms it (thread i of the first 256 adds x[i]^2, x[i+256]^2,
-// ... ascending; butterfly over the wave; the four wave sums in wave order),
-// so the normalised operand has the same bits as the stand-alone kernel's.
+// rmsnorm_kernel forms it (row_sumsq_part over the first 256 threads, a
+// butterfly over the wave, the four wave sums in wave order), so the
+// normalised operand has the same bits as the stand-alone kernel's.
 template <int NW>
 __device__ __forceinline__ void row_scales(const float* __restrict__ H, long ldh, int M, int K, float eps,
                                            float* __restrict__ wave_part /*[16][4]*/, float* __restrict__ scale /*[16]*/) {
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   if (wave < 4) {
-    // all rows together: the loads of one pass over the 16 rows are independent
-    float part[16];
+    const bool vec_ok = (ldh & 3) == 0 && (reinterpret_cast<uintptr_t>(H) & 15) == 0;
+    // four rows at a time, so that their loads are in flight together
+    for (int m0 = 0; m0 < M; m0 += 4) {
+      float part[4];
 #pragma unroll
-    for (int m = 0; m < 16; ++m) part[m] = 0.f;
-    for (int e = threadIdx.x; e < K; e += 256) {
-      float v[16];
+      for (int j = 0; j < 4; ++j)
+        part[j] = row_sumsq_part(H + (long)min(m0 + j, M - 1) * ldh, K, threadIdx.x, vec_ok);
 #pragma unroll
-      for (int m = 0; m < 16; ++m) v[m] = H[(long)(m < M ? m : 0) * ldh + e];
-#pragma unroll
-      for (int m = 0; m < 16; ++m) part[m] = part[m] + v[m] * v[m];
-    }
-#pragma unroll
-    for (int m = 0; m < 16; ++m) {
-      const float total = wave_sum(part[m]);
-      if (lane == 0) wave_part[m * 4 + wave] = total;
+      for (int j = 0; j < 4; ++j) {
+        const float total = wave_sum(part[j]);
+        if (lane == 0 && m0 + j < M) wave_part[(m0 + j) * 4 + wave] = total;
+      }
     }
   }
   __syncthreads();
@@ -153,8 +150,25 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const void* __rest
 
   const T* X = reinterpret_cast<const T*>(Xv);
   const float* H = reinterpret_cast<const float*>(Xv);
+  // UNR chunks at a time: all their loads are issued before the first MFMA
+  // needs one, so a wave keeps several kilobytes in flight.
+  constexpr int UNR = (NT * MT == 1 && !NORM) ? 8 : 4;
+  auto load_w = [&](int k0, int k_end, vec_t (&w)[NT][UNR]) {
+#pragma unroll
+    for (int u = 0; u < UNR; ++u) {
+      const int k = k0 + u * A::KCHUNK + g * A::VEC;
+      const bool in = k0 + u * A::KCHUNK < k_end;
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        const int n = n0 + t * 16 + row16;
+        w[t][u] = load_vec<T>(W, n, k, K, K, n < N && in, aligned);
+      }
+    }
+  };
   float my_scale = 0.f;
+  vec_t w_first[NT][UNR];  // with NORM: the wave's first weights are in flight while the rows are reduced
   if (NORM) {
+    if (wave < nslices) load_w(wave * kslice, min(K, (wave + 1) * kslice), w_first);
     float* wave_part = part + nslices * NT * MT * 256;
     float* scale = wave_part + 64;
     row_scales<NW>(H, ldx, M, K, eps, wave_part, scale);
@@ -170,20 +184,20 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const void* __rest
       for (int j = 0; j < MT; ++j) acc[t][j] = f32x4{0.f, 0.f, 0.f, 0.f};
     const int k_begin = s * kslice;
     const int k_end = min(K, k_begin + kslice);
-    // UNR chunks at a time: all their loads are issued before the first MFMA
-    // needs one, so a wave keeps several kilobytes in flight.
-    constexpr int UNR = (NT * MT == 1 && !NORM) ? 8 : 4;
     for (int k0 = k_begin; k0 < k_end; k0 += UNR * A::KCHUNK) {
       vec_t w[NT][UNR], x[MT][UNR];
+      if (NORM && s == wave && k0 == k_begin) {
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+#pragma unroll
+          for (int u = 0; u < UNR; ++u) w[t][u] = w_first[t][u];
+      } else {
+        load_w(k0, k_end, w);
+      }
 #pragma unroll
       for (int u = 0; u < UNR; ++u) {
         const int k = k0 + u * A::KCHUNK + g * A::VEC;
         const bool in = k0 + u * A::KCHUNK < k_end;
-#pragma unroll
-        for (int t = 0; t < NT; ++t) {
-          const int n = n0 + t * 16 + row16;
-          w[t][u] = load_vec<T>(W, n, k, K, K, n < N && in, aligned);
-        }
         if (NORM) {
           // normalise on the fly: (x * scale) * weight, rounded to the compute dtype
           vec_t v = A::zero();
