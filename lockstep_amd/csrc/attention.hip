@@ -1252,6 +1252,303 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
   }
 }
 
+// Variant 5, "cooperative, streamed": the cooperative kernel's arithmetic with
+// the wide kernel's data path.  The K and V tiles go from global memory
+// straight into LDS; with NBUF == 2 the next tile is in flight while the four
+// waves work on the current one, with NBUF == 1 (large heads) a tile is loaded
+// after the previous one has been consumed.
+template <typename T, int NBUF>
+__global__ __launch_bounds__(256) void attention_coop_dma_kernel(
+    const T* __restrict__ q, long ldq, const T* __restrict__ k_pages, const T* __restrict__ v_pages, int nkv,
+    int page_size, int page_shift, const int* __restrict__ table, int table_stride,
+    const SeqMeta* __restrict__ seqs, const AttnItem* __restrict__ items, T* __restrict__ out, long ldo,
+    float* __restrict__ part_acc, float* __restrict__ part_ml, int G, float scale, int window) {
+  typedef Atom<T> A;
+  typedef typename A::vec_t vec_t;
+  constexpr int SZ = sizeof(T);
+  constexpr int NT = 256;
+  constexpr int VEC = A::VEC;
+  constexpr int NC = (D + A::KCHUNK - 1) / A::KCHUNK;
+  constexpr int KROW = D * SZ;
+  constexpr int KPIECES = KROW / 16;
+  constexpr int TOTAL = kTileKeys * KPIECES;
+  constexpr int PER = (TOTAL + NT - 1) / NT;
+  constexpr int TILE_BYTES = TOTAL * 16;
+  constexpr int BUF_BYTES = 2 * TILE_BYTES;
+  constexpr int TILES_PER_SPLIT = kSplitKeys / kTileKeys;
+  constexpr int MYDB = (DB + 3) / 4;  // output blocks of one wave
+  typedef const __attribute__((address_space(1))) void* gptr_t;
+  typedef __attribute__((address_space(3))) void* lptr_t;
+
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+  int* tile_pages = reinterpret_cast<int*>(lds + NBUF * BUF_BYTES);      // [2][16]
+  float* wmax = reinterpret_cast<float*>(tile_pages + 32);               // [4][16]
+  float* psum = wmax + 64;                                               // [NB][64]
+  f32x4* prob = reinterpret_cast<f32x4*>(psum + NB * 64);                // [NB][64]
+
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const AttnItem item = items[blockIdx.x];
+  const SeqMeta sm = seqs[item.seq];
+  const int kvh = blockIdx.y;
+  const int rows_total = sm.q_len * G;  // <= 16, checked on the host
+  const int row16 = lane & 15;
+  const int g = lane >> 4;
+  const int r = row16;
+  const bool row_ok = r < rows_total;
+  const int qi = row_ok ? r / G : 0;
+  const int head = kvh * G + (row_ok ? r % G : 0);
+  const int q_pos = sm.q_start + qi;
+  const int key_hi = row_ok ? q_pos : -1;
+  const int key_lo = window > 0 ? q_pos - window + 1 : 0;
+  const int first_pos = sm.q_start;
+  const int last_pos = sm.q_start + (rows_total - 1) / G;
+  const int lo_valid = window > 0 ? max(0, sm.q_start - window + 1) : 0;
+  const int* __restrict__ tbl = table + (long)sm.table_row * table_stride;
+  const bool direct = item.part_base < 0;
+  const int pages_per_tile = kTileKeys >> page_shift;
+
+  vec_t qv[NC];
+#pragma unroll
+  for (int c = 0; c < NC; ++c)
+    qv[c] = load_vec<T>(q + (long)head * D, sm.q_off + qi, c * A::KCHUNK + g * VEC, D, ldq, row_ok, true);
+
+  int ti_lo = item.split_begin * TILES_PER_SPLIT;
+  if (window > 0) ti_lo = max(ti_lo, max(0, first_pos - window + 1) / kTileKeys);
+  const int ti_hi = min(item.split_end * TILES_PER_SPLIT, last_pos / kTileKeys + 1);
+
+  auto table_entry = [&](int ti) -> int {
+    const int key = min(ti * kTileKeys + ((int)threadIdx.x << page_shift), sm.kv_len - 1);
+    return tbl[key >> page_shift];
+  };
+  auto issue = [&](int ti) {
+    const int t0 = ti * kTileKeys;
+    const int* pages = tile_pages + (ti & 1) * 16;
+    unsigned char* k_buf = lds + (NBUF == 2 ? (ti & 1) : 0) * BUF_BYTES;
+    unsigned char* v_buf = k_buf + TILE_BYTES;
+    const int last_key = sm.kv_len - 1;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const int p = i * NT + (int)threadIdx.x;
+      if (PER * NT != TOTAL && i * NT + wave * 64 >= TOTAL) break;  // uniform for the wave
+      {
+        const int row = p / KPIECES;
+        const int slot = p % KPIECES;
+        const int piece = (slot - row % KPIECES + KPIECES) % KPIECES;
+        const int key = min(t0 + row, last_key);
+        const int page = max(pages[(key - t0) >> page_shift], 0);
+        const T* src = k_pages + (((long)page * nkv + kvh) * page_size + (key & (page_size - 1))) * D + piece * VEC;
+        __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(k_buf + (i * NT + wave * 64) * 16), 16, 0, 0);
+      }
+      {
+        const int c = p / D;
+        const int d = p % D;
+        const int key = min(t0 + c * VEC, last_key & ~(VEC - 1));
+        const int page = max(pages[(key - t0) >> page_shift], 0);
+        const T* src = v_pages + ((((long)page * nkv + kvh) * D + d) << page_shift) + (key & (page_size - 1));
+        __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(v_buf + (i * NT + wave * 64) * 16), 16, 0, 0);
+      }
+    }
+  };
+
+  // a wave keeps only its own output blocks: block j of the arrays is column block wave + 4j
+  f32x4 cur_acc[MYDB], run_acc[MYDB];
+  float cur_m = kNegSentinel, cur_l = 0.f, run_m = kNegSentinel, run_l = 0.f;
+#pragma unroll
+  for (int j = 0; j < MYDB; ++j) {
+    cur_acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+    run_acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+
+  int held = 0;
+  if (ti_lo < ti_hi) {
+    if ((int)threadIdx.x < pages_per_tile) tile_pages[(ti_lo & 1) * 16 + threadIdx.x] = table_entry(ti_lo);
+    __syncthreads();
+    issue(ti_lo);
+    if (ti_lo + 1 < ti_hi && (int)threadIdx.x < pages_per_tile) held = table_entry(ti_lo + 1);
+  }
+  for (int ti = ti_lo; ti < ti_hi; ++ti) {
+    const int t0 = ti * kTileKeys;
+    const unsigned char* k_lds = lds + (NBUF == 2 ? (ti & 1) : 0) * BUF_BYTES;
+    unsigned char* v_lds = lds + (NBUF == 2 ? (ti & 1) : 0) * BUF_BYTES + TILE_BYTES;
+    __asm__ volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this thread's pieces of the tile have landed
+    if (ti + 1 < ti_hi && (int)threadIdx.x < pages_per_tile) tile_pages[((ti + 1) & 1) * 16 + threadIdx.x] = held;
+    __syncthreads();  // the tile is complete (and the other buffer has been read by every wave)
+    if (t0 + kTileKeys > sm.kv_len || t0 < lo_valid) {  // uniform: clean the values of keys that are not held
+#pragma unroll
+      for (int i = 0; i < PER; ++i) {
+        const int p = i * NT + (int)threadIdx.x;
+        if (PER * NT != TOTAL && p >= TOTAL) break;
+        const int key0 = t0 + (p / D) * VEC;
+        vec_t* at = reinterpret_cast<vec_t*>(v_lds + p * 16);
+        *at = mask_keys(*at, lo_valid - key0, sm.kv_len - key0);
+      }
+      __syncthreads();
+    }
+    if (NBUF == 2 && ti + 1 < ti_hi) {
+      issue(ti + 1);
+      if (ti + 2 < ti_hi && (int)threadIdx.x < pages_per_tile) held = table_entry(ti + 2);
+    }
+
+    // score blocks 2w and 2w+1
+    f32x4 s[2];
+    float my_max = kNegSentinel;
+    {
+      vec_t kop[2][NC];
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const int row = (2 * wave + j) * 16 + row16;
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+          const int piece = c * 4 + g;
+          const int pc = (4 * NC == KPIECES) ? piece : min(piece, KPIECES - 1);
+          vec_t kv = *reinterpret_cast<const vec_t*>(k_lds + row * KROW + ((pc + row) % KPIECES) * 16);
+          if (4 * NC != KPIECES) kv = piece < KPIECES ? kv : A::zero();
+          kop[j][c] = kv;
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const int kb = 2 * wave + j;
+        s[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int c = 0; c < NC; ++c) A::mma(s[j], kop[j][c], qv[c]);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int key = t0 + kb * 16 + 4 * g + e;
+          const float v = ((key <= key_hi) & (key >= key_lo)) ? s[j][e] * scale : kMasked;
+          s[j][e] = v;
+          my_max = fmaxf(my_max, v);
+        }
+      }
+    }
+    my_max = quad16_max(my_max);
+    if (g == 0) wmax[wave * 16 + row16] = my_max;
+    __syncthreads();
+    const float tile_max = fmaxf(fmaxf(wmax[row16], wmax[16 + row16]), fmaxf(wmax[32 + row16], wmax[48 + row16]));
+    const float m_new = fmaxf(cur_m, tile_max);
+    const float alpha = softmax_exp<T>(cur_m - m_new);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int kb = 2 * wave + j;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) s[j][e] = softmax_exp<T>(s[j][e] - m_new);  // masked: exp(-inf) = 0
+      psum[kb * 64 + lane] = (s[j][0] + s[j][1]) + (s[j][2] + s[j][3]);
+      prob[kb * 64 + lane] = s[j];
+    }
+    // this wave's value operands do not depend on the probabilities: read them before the barrier
+    constexpr int KB16 = VEC / 4;
+    constexpr int NPAIR = NB / KB16;
+    vec_t vop[NPAIR][MYDB];
+#pragma unroll
+    for (int kp = 0; kp < NPAIR; ++kp)
+#pragma unroll
+      for (int j = 0; j < MYDB; ++j) {
+        const int blk = wave + 4 * j;
+        const int d = (blk < DB ? blk : 0) * 16 + row16;
+        vec_t vv;
+#pragma unroll
+        for (int h = 0; h < KB16; ++h) {
+          const int key = (kp * KB16 + h) * 16 + 4 * g;
+          const unsigned char* src = v_lds + ((key / VEC) * D + d) * 16 + (key % VEC) * SZ;
+          if (SZ == 2) {
+            bf16x4 four = *reinterpret_cast<const bf16x4*>(src);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) vv[h * 4 + e] = four[e];
+          } else {
+            f32x4 four = *reinterpret_cast<const f32x4*>(src);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) vv[h * 4 + e] = four[e];
+          }
+        }
+        vop[kp][j] = vv;
+      }
+    __syncthreads();
+    float p_sum = 0.f;
+#pragma unroll
+    for (int kb = 0; kb < NB; ++kb) p_sum = p_sum + psum[kb * 64 + lane];
+    p_sum = quad16_sum(p_sum);
+    cur_l = cur_l * alpha + p_sum;
+    cur_m = m_new;
+#pragma unroll
+    for (int j = 0; j < MYDB; ++j)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) cur_acc[j][e] = cur_acc[j][e] * alpha;
+#pragma unroll
+    for (int kp = 0; kp < NPAIR; ++kp) {
+      vec_t pv;
+#pragma unroll
+      for (int h = 0; h < KB16; ++h) {
+        const f32x4 four = prob[(kp * KB16 + h) * 64 + lane];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) pv[h * 4 + e] = from_f32<T>(four[e]);
+      }
+#pragma unroll
+      for (int j = 0; j < MYDB; ++j) {
+        if (wave + 4 * j >= DB) continue;
+        A::mma(cur_acc[j], vop[kp][j], pv);
+      }
+    }
+    if (direct && ((ti + 1) % TILES_PER_SPLIT == 0 || ti + 1 == ti_hi)) {
+      if (cur_l > 0.f) {  // the fold of fold_split, on this wave's blocks
+        const float m_fold = fmaxf(run_m, cur_m);
+        const float fa = softmax_exp<T>(run_m - m_fold);
+        const float fb = softmax_exp<T>(cur_m - m_fold);
+#pragma unroll
+        for (int j = 0; j < MYDB; ++j)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) run_acc[j][e] = run_acc[j][e] * fa + cur_acc[j][e] * fb;
+        run_l = run_l * fa + cur_l * fb;
+        run_m = m_fold;
+      }
+#pragma unroll
+      for (int j = 0; j < MYDB; ++j) cur_acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+      cur_m = kNegSentinel;
+      cur_l = 0.f;
+    }
+    if (NBUF == 1 && ti + 1 < ti_hi) {
+      __syncthreads();  // every wave is done with the buffer
+      issue(ti + 1);
+      if (ti + 2 < ti_hi && (int)threadIdx.x < pages_per_tile) held = table_entry(ti + 2);
+    }
+  }
+
+  if (!row_ok) return;
+  if (direct) {
+    T* dst = out + (long)(sm.q_off + qi) * ldo + (long)head * D;
+    const float l = run_l;
+#pragma unroll
+    for (int j = 0; j < MYDB; ++j) {
+      const int blk = wave + 4 * j;
+      if (blk >= DB) continue;
+      float o[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) o[e] = l > 0.f ? run_acc[j][e] / l : 0.f;
+      T* p = dst + blk * 16 + 4 * g;
+      if (SZ == 2) {
+        bf16x4 v;
+        v[0] = (bf16_t)o[0]; v[1] = (bf16_t)o[1]; v[2] = (bf16_t)o[2]; v[3] = (bf16_t)o[3];
+        *reinterpret_cast<bf16x4*>(p) = v;
+      } else {
+        *reinterpret_cast<f32x4*>(p) = f32x4{o[0], o[1], o[2], o[3]};
+      }
+    }
+  } else {
+    const int split = item.split_begin;
+    const long pr = item.part_base + ((long)kvh * rows_total + r) * item.n_splits + (split - item.split_lo);
+    float* pa = part_acc + pr * D;
+#pragma unroll
+    for (int j = 0; j < MYDB; ++j) {
+      const int blk = wave + 4 * j;
+      if (blk < DB) *reinterpret_cast<f32x4*>(pa + blk * 16 + 4 * g) = cur_acc[j];
+    }
+    if (wave == 0 && g == 0) {
+      part_ml[pr * 2] = cur_m;
+      part_ml[pr * 2 + 1] = cur_l;
+    }
+  }
+}
+
 struct CombineItem {
   int seq, row_block, part_base, n_splits;
 };
@@ -1349,6 +1646,38 @@ static bool coop_supported(int dtype) {
   return st == 1;
 }
 
+// The streamed cooperative kernel: one or two buffers of a K and a V tile,
+// two rows of page ids and the exchange buffers of the cooperative kernel.
+constexpr size_t kDmaExtra = 2 * 16 * sizeof(int) + kCoopExtra;
+constexpr int coop_dma_bufs(size_t elem) {
+  return 2 * (2 * kTileKeys * D * elem) + kDmaExtra <= kLdsLimit ? 2 : 1;
+}
+constexpr int kDmaBufsF32 = coop_dma_bufs(4);
+constexpr int kDmaBufsBF16 = coop_dma_bufs(2);
+static size_t coop_dma_lds_bytes(int dtype) {
+  const size_t elem = dtype == kF32 ? 4 : 2;
+  return (dtype == kF32 ? kDmaBufsF32 : kDmaBufsBF16) * (2 * (size_t)kTileKeys * D * elem) + kDmaExtra;
+}
+static bool coop_dma_supported(int dtype) {
+  const size_t bytes = coop_dma_lds_bytes(dtype);
+  if (bytes > kLdsLimit) return false;
+  if (bytes <= 64 * 1024) return true;
+  static int state[2] = {0, 0};
+  int& st = state[dtype == kF32 ? 0 : 1];
+  if (st == 0) {
+    hipError_t e = dtype == kF32
+        ? hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_coop_dma_kernel<float, kDmaBufsF32>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes)
+        : hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_coop_dma_kernel<bf16_t, kDmaBufsBF16>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+    if (e != hipSuccess) (void)hipGetLastError();
+    st = e == hipSuccess ? 1 : -1;
+  }
+  return st == 1;
+}
+// 1 if the streamed cooperative kernel (variant 5) can run for this dtype.
+extern "C" int ls_attn_coop_dma_supported(int dtype) { return coop_dma_supported(dtype) ? 1 : 0; }
+
 // The wide kernel: two buffers of a K and a V tile, and two rows of page ids.
 constexpr int kWideWaves = 8;
 static size_t wide_lds_bytes(int dtype) { return 4 * (size_t)kTileKeys * D * (dtype == kF32 ? 4 : 2) + 2 * 16 * sizeof(int); }
@@ -1418,6 +1747,26 @@ extern "C" int ls_attention(int dtype, const void* q, long ldq, const void* k_pa
     else
       return fail("attention: unknown dtype %d", dtype);
     return check_launch("attention (cooperative)");
+  }
+  if (variant == 5) {
+    LS_REQUIRE(max_rows <= 16, "attention: the cooperative variants take work items of at most 16 rows, got %d",
+               max_rows);
+    LS_REQUIRE(coop_dma_supported(dtype), "attention: the streamed cooperative variant does not fit into LDS");
+    LS_REQUIRE(page_size >= 8, "attention: the streamed variants need pages of at least 8 keys, got %d", page_size);
+    const size_t bytes = coop_dma_lds_bytes(dtype);
+    if (dtype == kF32)
+      hipLaunchKernelGGL((attention_coop_dma_kernel<float, kDmaBufsF32>), grid, dim3(256), bytes, s, (const float*)q,
+                         ldq, (const float*)k_pages, (const float*)v_pages, nkv, page_size, page_shift, table,
+                         table_stride, (const SeqMeta*)seqs, (const AttnItem*)items, (float*)out, ldo, part_acc,
+                         part_ml, G, scale, window);
+    else if (dtype == kBF16)
+      hipLaunchKernelGGL((attention_coop_dma_kernel<bf16_t, kDmaBufsBF16>), grid, dim3(256), bytes, s,
+                         (const bf16_t*)q, ldq, (const bf16_t*)k_pages, (const bf16_t*)v_pages, nkv, page_size,
+                         page_shift, table, table_stride, (const SeqMeta*)seqs, (const AttnItem*)items, (bf16_t*)out,
+                         ldo, part_acc, part_ml, G, scale, window);
+    else
+      return fail("attention: unknown dtype %d", dtype);
+    return check_launch("attention (cooperative, streamed)");
   }
   if (variant == 4) {
     LS_REQUIRE(wide_supported(dtype), "attention: the wide variant does not fit into LDS for this head size");

@@ -38,6 +38,7 @@ class AttentionPlan:
     coop_items: torch.Tensor | None
     n_coop: int
     coop_max_rows: int
+    coop_variant: int
     wide_items: torch.Tensor | None
     n_wide: int
     combine_items: torch.Tensor | None
@@ -118,7 +119,14 @@ class StepContext:
         if key in self._plans:
             return
         tile, split = self.rt.kernels.attention_geometry(head_dim)
-        coop_ok = self.rt.kernels.coop_supported(head_dim, self.rt.dtype)
+        kernels = self.rt.kernels
+        # rows of decoded tokens: the streamed cooperative kernel, else the cooperative one
+        if kernels.coop_dma_supported(head_dim, self.rt.dtype, self.cache.page_size):
+            coop_ok, coop_variant = True, 5
+        else:
+            coop_ok, coop_variant = kernels.coop_supported(head_dim, self.rt.dtype), 3
+        # with a workgroup per CU anyway, one workgroup walks all splits of a request itself
+        whole_requests = self.n_seqs * nkv >= 256
         wide_ok = self.rt.kernels.wide_supported(head_dim, self.rt.dtype, self.cache.page_size)
         wide_rows = self.rt.kernels.attention_block_rows(head_dim, 4)
         items, coop, wide, combine = [], [], [], []
@@ -142,7 +150,7 @@ class StepContext:
             target = coop if (coop_ok and rows <= 16) else items
             if target is coop:
                 coop_max_rows = max(coop_max_rows, rows)
-            if rows <= 64 and (n_splits > 1 or self.fixed_shape):
+            if rows <= 64 and (n_splits > 1 or self.fixed_shape) and not (target is coop and whole_requests):
                 base = part_rows
                 part_rows += nkv * rows * n_splits
                 for s in range(split_lo, split_lo + n_splits):
@@ -164,14 +172,14 @@ class StepContext:
         self._plans[key] = (np.asarray(items, dtype=np.int64).reshape(-1),
                             np.asarray(combine, dtype=np.int64).reshape(-1), len(items), len(combine), part_rows,
                             np.asarray(coop, dtype=np.int64).reshape(-1), len(coop), coop_max_rows,
-                            np.asarray(wide, dtype=np.int64).reshape(-1), len(wide))
+                            np.asarray(wide, dtype=np.int64).reshape(-1), len(wide), coop_variant)
         self._plan_specs.append(key)
 
     def upload(self) -> None:
         """Copy all metadata to the device in one transfer."""
         parts = list(self._host_parts)
         for key in self._plan_specs:
-            items, combine, _, _, _, coop, _, _, wide, _ = self._plans[key]
+            items, combine, _, _, _, coop, _, _, wide, _, _ = self._plans[key]
             parts += [items, combine, coop, wide]
         flat = np.concatenate(parts).astype(np.int32)
         host = torch.from_numpy(flat)
@@ -191,7 +199,8 @@ class StepContext:
         self.want_rows = take(self.n_want)
         self._device_plans: dict[tuple, AttentionPlan] = {}
         for key in self._plan_specs:
-            items, combine, n_items, n_combine, part_rows, coop, n_coop, coop_max_rows, wide, n_wide = self._plans[key]
+            (items, combine, n_items, n_combine, part_rows, coop, n_coop, coop_max_rows, wide, n_wide,
+             coop_variant) = self._plans[key]
             head_dim = key[2]
             d_items, d_combine, d_coop = take(items.shape[0]), take(combine.shape[0]), take(coop.shape[0])
             d_wide = take(wide.shape[0])
@@ -200,7 +209,7 @@ class StepContext:
                 part_acc = self.workspace.get(f"attention.part_acc.{head_dim}", (part_rows, head_dim), torch.float32)
                 part_ml = self.workspace.get("attention.part_ml", (part_rows, 2), torch.float32)
             self._device_plans[key] = AttentionPlan(d_items, n_items, d_coop if n_coop else None, n_coop,
-                                                    coop_max_rows, d_wide if n_wide else None, n_wide,
+                                                    coop_max_rows, coop_variant, d_wide if n_wide else None, n_wide,
                                                     d_combine if n_combine else None,
                                                     n_combine, part_acc, part_ml)
         self._uploaded = True

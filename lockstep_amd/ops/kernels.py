@@ -92,6 +92,11 @@ class Kernels:
         """Whether the cooperative attention kernel can run (its tiles must fit into LDS)."""
         return bool(self.attention_lib(head_dim).ls_attn_coop_supported(c_int(DTYPE_CODE[dtype])))
 
+    def coop_dma_supported(self, head_dim: int, dtype: torch.dtype, page_size: int) -> bool:
+        """Whether the streamed cooperative attention kernel (variant 5) can run."""
+        lib = self.attention_lib(head_dim)
+        return page_size >= 8 and bool(lib.ls_attn_coop_dma_supported(c_int(DTYPE_CODE[dtype])))
+
     def wide_supported(self, head_dim: int, dtype: torch.dtype, page_size: int) -> bool:
         """Whether the wide attention kernel (variant 4, for prompt portions) can run."""
         return page_size >= 8 and bool(self.attention_lib(head_dim).ls_attn_wide_supported(c_int(DTYPE_CODE[dtype])))
@@ -259,7 +264,8 @@ class Kernels:
         """Launch the attention kernel over ``n_items`` work items (see attention.hip).
         ``variant``: 0 staged through LDS where it fits, 1 direct from global memory, 2 staged or
         error, 3 cooperative (every item has at most 16 rows; ``max_rows`` states the largest),
-        4 wide (tiles loaded straight into LDS; items count row blocks of ``attention_block_rows``)."""
+        4 wide (tiles loaded straight into LDS; items count row blocks of ``attention_block_rows``),
+        5 cooperative with tiles loaded straight into LDS (same items as 3)."""
         lib = self.attention_lib(d)
         _rows_ok(q, "attention q"); _rows_ok(out, "attention out")
         _need(q.dtype in DTYPE_CODE and out.dtype == q.dtype, "attention q/out dtype")

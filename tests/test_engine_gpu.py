@@ -233,3 +233,34 @@ def test_decode_steps_from_a_captured_graph_equal_eager_steps(plain_logits, dtyp
     assert model.graph_replays > 100
     assert torch.equal(torch.cat(got_a), want_a)
     assert torch.equal(torch.cat(got_b), want_b)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_a_large_decode_batch_gives_each_request_the_bits_it_gets_alone(plain_logits, dtype):
+    """With many requests in a decode step the attention plan gives each
+    (request, kv head) to one workgroup that walks all splits itself; a request
+    alone is cut into splits and combined.  Same bits, also from the graph."""
+    from lockstep_amd.engine.batch import StepEntry
+
+    folder, _ = plain_logits["B"]
+    model = load(folder, dtype)
+    n_req, n_decode = 90, 5
+    lengths = [3 + (37 * i) % 290 for i in range(n_req)]          # contexts on both sides of a split's edge
+    prompts = [random_tokens(n + n_decode, 1000, seed=500 + i) for i, n in enumerate(lengths)]
+    cache = model.make_cache(num_pages=sum(-(-(n + n_decode) // 8) for n in lengths) + 4, page_size=8,
+                             max_requests=n_req + 1)
+    for lo in range(0, n_req, 4):                                  # prompts, four requests a step
+        group = range(lo, min(lo + 4, n_req))
+        for i in group:
+            cache.open(f"r{i}")
+        model.step(cache, [StepEntry(f"r{i}", prompts[i][:lengths[i]], []) for i in group])
+    together = []
+    for k in range(n_decode):
+        logits = model.step(cache, [StepEntry(f"r{i}", [prompts[i][lengths[i] + k]], [0]) for i in range(n_req)])
+        together.append(logits.cpu())
+    assert model.graph_replays >= n_decode - 2
+    for i in (0, 7, 8, 33, 60, 89):
+        alone = model.make_cache(num_pages=64, page_size=8)
+        want = feed(model, alone, "x", prompts[i], [lengths[i]] + [1] * n_decode)[lengths[i]:]
+        got = torch.stack([t[i] for t in together])
+        assert torch.equal(got, want), f"request {i} (context {lengths[i]})"
