@@ -1257,12 +1257,34 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
 // straight into LDS; with NBUF == 2 the next tile is in flight while the four
 // waves work on the current one, with NBUF == 1 (large heads) a tile is loaded
 // after the previous one has been consumed.
-template <typename T, int NBUF>
+//
+// With FUSE the kernel also does what qk_rope_kv_kernel does for a step of
+// single decoded tokens: `q` is then the raw fused projection (query heads,
+// key heads, value heads in a row); the workgroup normalises and rotates its
+// query heads into LDS, and the workgroup whose tiles hold the new position
+// does the same for the new key, writes key and value to the cache pages and
+// patches them into its LDS tile.  Each head goes through head_norm_rope, as
+// in the stand-alone kernel, so the bits are the same.
+template <typename T>
+struct DecodeFuse {
+  const float* q_weight;   // per-head norm weights or nullptr
+  const float* k_weight;
+  float eps;
+  const float* cos_table;  // [positions][rot / 2] or nullptr
+  const float* sin_table;
+  int rot;
+  int nq;                  // query heads in a row of the projection
+  int write_kv;            // 0: the cache already holds this step's keys and values
+  T* k_out;                // the cache pages, writable
+  T* v_out;
+};
+
+template <typename T, int NBUF, bool FUSE>
 __global__ __launch_bounds__(256) void attention_coop_dma_kernel(
     const T* __restrict__ q, long ldq, const T* __restrict__ k_pages, const T* __restrict__ v_pages, int nkv,
     int page_size, int page_shift, const int* __restrict__ table, int table_stride,
     const SeqMeta* __restrict__ seqs, const AttnItem* __restrict__ items, T* __restrict__ out, long ldo,
-    float* __restrict__ part_acc, float* __restrict__ part_ml, int G, float scale, int window) {
+    float* __restrict__ part_acc, float* __restrict__ part_ml, int G, float scale, int window, DecodeFuse<T> fz) {
   typedef Atom<T> A;
   typedef typename A::vec_t vec_t;
   constexpr int SZ = sizeof(T);
@@ -1285,6 +1307,8 @@ __global__ __launch_bounds__(256) void attention_coop_dma_kernel(
   float* wmax = reinterpret_cast<float*>(tile_pages + 32);               // [4][16]
   float* psum = wmax + 64;                                               // [NB][64]
   f32x4* prob = reinterpret_cast<f32x4*>(psum + NB * 64);                // [NB][64]
+  T* knew = reinterpret_cast<T*>(prob + NB * 64);                        // FUSE: [D] new key, [D] new value
+  T* vnew = knew + D;
 
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -1309,9 +1333,11 @@ __global__ __launch_bounds__(256) void attention_coop_dma_kernel(
   const int pages_per_tile = kTileKeys >> page_shift;
 
   vec_t qv[NC];
+  if (!FUSE) {
 #pragma unroll
-  for (int c = 0; c < NC; ++c)
-    qv[c] = load_vec<T>(q + (long)head * D, sm.q_off + qi, c * A::KCHUNK + g * VEC, D, ldq, row_ok, true);
+    for (int c = 0; c < NC; ++c)
+      qv[c] = load_vec<T>(q + (long)head * D, sm.q_off + qi, c * A::KCHUNK + g * VEC, D, ldq, row_ok, true);
+  }
 
   int ti_lo = item.split_begin * TILES_PER_SPLIT;
   if (window > 0) ti_lo = max(ti_lo, max(0, first_pos - window + 1) / kTileKeys);
@@ -1361,11 +1387,69 @@ __global__ __launch_bounds__(256) void attention_coop_dma_kernel(
   }
 
   int held = 0;
+  int first_page = 0;
+  if (ti_lo < ti_hi && (int)threadIdx.x < pages_per_tile) first_page = table_entry(ti_lo);
+  // FUSE: one new token per request at position q_start; its tile is patched by the workgroup that walks it.
+  // The heads to process are numbered vi: the G query heads, then the new key, then the new value;
+  // wave w takes vi = w, w + 4, ...  The operands of its first head are loaded before the tile loads start.
+  const int p_new = sm.q_start;
+  const int tile_new = p_new / kTileKeys;
+  const bool owner = FUSE && fz.write_kv && tile_new >= ti_lo && tile_new < ti_hi;
+  const int n_vec = owner ? G + 2 : G;
+  const T* new_row = q + (long)sm.q_off * ldq;
+  const bool rotated = FUSE && fz.cos_table != nullptr;
+  long page_new = -1;
+  HeadVec hv;
+  auto head_src = [&](int vi) -> const T* {
+    return new_row + (long)(vi < G ? kvh * G + vi : vi == G ? fz.nq + kvh : fz.nq + nkv + kvh) * D;
+  };
+  auto head_fetch = [&](int vi) {
+    if (vi <= G)
+      head_load<T>(hv, head_src(vi), D, vi < G ? fz.q_weight : fz.k_weight, fz.cos_table, fz.sin_table, p_new,
+                   fz.rot, lane);
+    else
+      head_load<T>(hv, head_src(vi), D, nullptr, nullptr, nullptr, 0, 0, lane);
+  };
+  if (FUSE) {
+    if (owner) page_new = tbl[p_new >> page_shift];
+    if (wave < n_vec) head_fetch(wave);
+  }
+  if (ti_lo < ti_hi && (int)threadIdx.x < pages_per_tile) tile_pages[(ti_lo & 1) * 16 + threadIdx.x] = first_page;
+  __syncthreads();
   if (ti_lo < ti_hi) {
-    if ((int)threadIdx.x < pages_per_tile) tile_pages[(ti_lo & 1) * 16 + threadIdx.x] = table_entry(ti_lo);
-    __syncthreads();
     issue(ti_lo);
     if (ti_lo + 1 < ti_hi && (int)threadIdx.x < pages_per_tile) held = table_entry(ti_lo + 1);
+  }
+  if (FUSE) {
+    float* ystage = reinterpret_cast<float*>(prob) + wave * D;               // the exchange buffers are free until the loop
+    T* qrot = reinterpret_cast<T*>(reinterpret_cast<float*>(prob) + 4 * D);  // [16][D]
+    const int slot_new = p_new & (page_size - 1);
+    for (int vi = wave; vi < n_vec; vi += 4) {  // uniform for the wave
+      if (vi != wave) head_fetch(vi);
+      if (vi < G) {
+        head_finish<T>(hv, D, fz.q_weight != nullptr, fz.eps, rotated, fz.rot, ystage, lane,
+                       [&](int e, T v) { qrot[vi * D + e] = v; });
+      } else if (vi == G) {
+        T* dst = fz.k_out + ((max(page_new, 0L) * nkv + kvh) * page_size + slot_new) * D;
+        head_finish<T>(hv, D, fz.k_weight != nullptr, fz.eps, rotated, fz.rot, ystage, lane, [&](int e, T v) {
+          knew[e] = v;
+          if (page_new >= 0) dst[e] = v;
+        });
+      } else {
+        T* dst = fz.v_out + ((max(page_new, 0L) * nkv + kvh) * D) * page_size + slot_new;
+        head_finish<T>(hv, D, false, 0.f, false, 0, ystage, lane, [&](int e, T v) {
+          vnew[e] = v;
+          if (page_new >= 0) dst[(long)e * page_size] = v;
+        });
+      }
+    }
+    __syncthreads();
+    const T* qr = qrot;
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+      const int col = c * A::KCHUNK + g * VEC;
+      qv[c] = (row_ok && col < D) ? *reinterpret_cast<const vec_t*>(qr + row16 * D + min(col, D - VEC)) : A::zero();
+    }
   }
   for (int ti = ti_lo; ti < ti_hi; ++ti) {
     const int t0 = ti * kTileKeys;
@@ -1374,14 +1458,27 @@ __global__ __launch_bounds__(256) void attention_coop_dma_kernel(
     __asm__ volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this thread's pieces of the tile have landed
     if (ti + 1 < ti_hi && (int)threadIdx.x < pages_per_tile) tile_pages[((ti + 1) & 1) * 16 + threadIdx.x] = held;
     __syncthreads();  // the tile is complete (and the other buffer has been read by every wave)
-    if (t0 + kTileKeys > sm.kv_len || t0 < lo_valid) {  // uniform: clean the values of keys that are not held
+    const bool patch = owner && ti == tile_new;  // the new key and value go into this tile
+    if (t0 + kTileKeys > sm.kv_len || t0 < lo_valid || patch) {  // uniform: clean the values of keys that are not held
 #pragma unroll
       for (int i = 0; i < PER; ++i) {
         const int p = i * NT + (int)threadIdx.x;
         if (PER * NT != TOTAL && p >= TOTAL) break;
         const int key0 = t0 + (p / D) * VEC;
         vec_t* at = reinterpret_cast<vec_t*>(v_lds + p * 16);
-        *at = mask_keys(*at, lo_valid - key0, sm.kv_len - key0);
+        vec_t v = mask_keys(*at, lo_valid - key0, sm.kv_len - key0);
+        if (FUSE && patch) {
+          const T fresh = vnew[p % D];
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) v[e] = key0 + e == p_new ? fresh : v[e];
+          const int row = p / KPIECES;
+          if (t0 + row == p_new) {
+            const int piece = (p % KPIECES - row % KPIECES + KPIECES) % KPIECES;
+            *reinterpret_cast<vec_t*>(const_cast<unsigned char*>(k_lds) + p * 16) =
+                *reinterpret_cast<const vec_t*>(knew + piece * VEC);
+          }
+        }
+        *at = v;
       }
       __syncthreads();
     }
@@ -1648,7 +1745,7 @@ static bool coop_supported(int dtype) {
 
 // The streamed cooperative kernel: one or two buffers of a K and a V tile,
 // two rows of page ids and the exchange buffers of the cooperative kernel.
-constexpr size_t kDmaExtra = 2 * 16 * sizeof(int) + kCoopExtra;
+constexpr size_t kDmaExtra = 2 * 16 * sizeof(int) + kCoopExtra + 2 * D * 4;  // + new key and value (FUSE)
 constexpr int coop_dma_bufs(size_t elem) {
   return 2 * (2 * kTileKeys * D * elem) + kDmaExtra <= kLdsLimit ? 2 : 1;
 }
@@ -1666,9 +1763,9 @@ static bool coop_dma_supported(int dtype) {
   int& st = state[dtype == kF32 ? 0 : 1];
   if (st == 0) {
     hipError_t e = dtype == kF32
-        ? hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_coop_dma_kernel<float, kDmaBufsF32>),
+        ? hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_coop_dma_kernel<float, kDmaBufsF32, false>),
                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes)
-        : hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_coop_dma_kernel<bf16_t, kDmaBufsBF16>),
+        : hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_coop_dma_kernel<bf16_t, kDmaBufsBF16, false>),
                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
     if (e != hipSuccess) (void)hipGetLastError();
     st = e == hipSuccess ? 1 : -1;
@@ -1677,6 +1774,81 @@ static bool coop_dma_supported(int dtype) {
 }
 // 1 if the streamed cooperative kernel (variant 5) can run for this dtype.
 extern "C" int ls_attn_coop_dma_supported(int dtype) { return coop_dma_supported(dtype) ? 1 : 0; }
+
+// The fused decode step (FUSE) stages the rotated query heads in the exchange
+// buffers before the loop needs them: 4 rows of D floats and 16 rows of D elements.
+static bool decode_fused_supported(int dtype) {
+  const size_t elem = dtype == kF32 ? 4 : 2;
+  if (4 * D * 4 + 16 * D * elem > (size_t)NB * 64 * 16) return false;
+  const size_t bytes = coop_dma_lds_bytes(dtype);
+  if (bytes > kLdsLimit) return false;
+  if (bytes <= 64 * 1024) return true;
+  static int state[2] = {0, 0};
+  int& st = state[dtype == kF32 ? 0 : 1];
+  if (st == 0) {
+    hipError_t e = dtype == kF32
+        ? hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_coop_dma_kernel<float, kDmaBufsF32, true>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes)
+        : hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_coop_dma_kernel<bf16_t, kDmaBufsBF16, true>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+    if (e != hipSuccess) (void)hipGetLastError();
+    st = e == hipSuccess ? 1 : -1;
+  }
+  return st == 1;
+}
+// 1 if ls_attention_decode can run for this dtype.
+extern "C" int ls_attn_decode_fused_supported(int dtype) { return decode_fused_supported(dtype) ? 1 : 0; }
+
+// A step of single decoded tokens, with the per-head norm, the rotation and
+// the cache write of qk_rope_kv fused in.  qkv [tokens, ld]: the raw fused
+// projection (nq query heads, then nkv key heads, then nkv value heads); every
+// request of `seqs` that the items name brings exactly one token.  The items
+// are those of the cooperative variants.  cos/sin [table_positions][rot/2];
+// max_pos is the largest position of the step.
+extern "C" int ls_attention_decode(int dtype, const void* qkv, long ld, void* k_pages, void* v_pages, int nq, int nkv,
+                                   int page_size, const int* table, int table_stride, const void* seqs,
+                                   const void* items, int n_items, void* out, long ldo, float* part_acc,
+                                   float* part_ml, float scale, int window, const float* q_weight,
+                                   const float* k_weight, float eps, const float* cos_table, const float* sin_table,
+                                   int rot, int table_positions, int max_pos, int write_kv, void* stream) {
+  LS_REQUIRE(n_items > 0 && nkv > 0 && nq > 0 && nq % nkv == 0, "decode attention: bad sizes");
+  const int G = nq / nkv;
+  LS_REQUIRE(G <= 16, "decode attention: %d query heads per kv head, at most 16 fit a work item", G);
+  LS_REQUIRE(page_size >= 8 && kTileKeys % page_size == 0 && (page_size & (page_size - 1)) == 0,
+             "decode attention: page size %d must be a power of two from 8 that divides the key tile %d", page_size,
+             kTileKeys);
+  LS_REQUIRE(ld % 8 == 0 && ldo % 4 == 0 && ld >= (long)(nq + 2 * nkv) * D && ldo >= (long)nq * D,
+             "decode attention: row strides ld=%ld ldo=%ld do not fit the heads", ld, ldo);
+  LS_REQUIRE(reinterpret_cast<uintptr_t>(qkv) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0 &&
+                 reinterpret_cast<uintptr_t>(k_pages) % 16 == 0 && reinterpret_cast<uintptr_t>(v_pages) % 16 == 0,
+             "decode attention: operands must be 16-byte aligned");
+  LS_REQUIRE(rot >= 0 && rot <= D && rot % 2 == 0, "decode attention: rotary_dim %d must be even and at most %d", rot, D);
+  LS_REQUIRE(!cos_table || (sin_table && table_positions > max_pos),
+             "decode attention: rotation tables hold %d positions, the step reaches %d", table_positions, max_pos);
+  LS_REQUIRE(decode_fused_supported(dtype), "decode attention: the fused kernel does not fit into LDS for this head size");
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  dim3 grid(n_items, nkv);
+  int page_shift = 0;
+  while ((1 << page_shift) < page_size) ++page_shift;
+  const size_t bytes = coop_dma_lds_bytes(dtype);
+  if (dtype == kF32) {
+    DecodeFuse<float> fz{q_weight, k_weight, eps, cos_table, sin_table, rot, nq, write_kv, (float*)k_pages, (float*)v_pages};
+    hipLaunchKernelGGL((attention_coop_dma_kernel<float, kDmaBufsF32, true>), grid, dim3(256), bytes, s,
+                       (const float*)qkv, ld, (const float*)k_pages, (const float*)v_pages, nkv, page_size, page_shift,
+                       table, table_stride, (const SeqMeta*)seqs, (const AttnItem*)items, (float*)out, ldo, part_acc,
+                       part_ml, G, scale, window, fz);
+  } else if (dtype == kBF16) {
+    DecodeFuse<bf16_t> fz{q_weight, k_weight, eps, cos_table, sin_table, rot, nq, write_kv, (bf16_t*)k_pages,
+                          (bf16_t*)v_pages};
+    hipLaunchKernelGGL((attention_coop_dma_kernel<bf16_t, kDmaBufsBF16, true>), grid, dim3(256), bytes, s,
+                       (const bf16_t*)qkv, ld, (const bf16_t*)k_pages, (const bf16_t*)v_pages, nkv, page_size,
+                       page_shift, table, table_stride, (const SeqMeta*)seqs, (const AttnItem*)items, (bf16_t*)out, ldo,
+                       part_acc, part_ml, G, scale, window, fz);
+  } else {
+    return fail("decode attention: unknown dtype %d", dtype);
+  }
+  return check_launch("attention (decode, fused)");
+}
 
 // The wide kernel: two buffers of a K and a V tile, and two rows of page ids.
 constexpr int kWideWaves = 8;
@@ -1755,15 +1927,15 @@ extern "C" int ls_attention(int dtype, const void* q, long ldq, const void* k_pa
     LS_REQUIRE(page_size >= 8, "attention: the streamed variants need pages of at least 8 keys, got %d", page_size);
     const size_t bytes = coop_dma_lds_bytes(dtype);
     if (dtype == kF32)
-      hipLaunchKernelGGL((attention_coop_dma_kernel<float, kDmaBufsF32>), grid, dim3(256), bytes, s, (const float*)q,
-                         ldq, (const float*)k_pages, (const float*)v_pages, nkv, page_size, page_shift, table,
-                         table_stride, (const SeqMeta*)seqs, (const AttnItem*)items, (float*)out, ldo, part_acc,
-                         part_ml, G, scale, window);
+      hipLaunchKernelGGL((attention_coop_dma_kernel<float, kDmaBufsF32, false>), grid, dim3(256), bytes, s,
+                         (const float*)q, ldq, (const float*)k_pages, (const float*)v_pages, nkv, page_size,
+                         page_shift, table, table_stride, (const SeqMeta*)seqs, (const AttnItem*)items, (float*)out,
+                         ldo, part_acc, part_ml, G, scale, window, DecodeFuse<float>{});
     else if (dtype == kBF16)
-      hipLaunchKernelGGL((attention_coop_dma_kernel<bf16_t, kDmaBufsBF16>), grid, dim3(256), bytes, s,
+      hipLaunchKernelGGL((attention_coop_dma_kernel<bf16_t, kDmaBufsBF16, false>), grid, dim3(256), bytes, s,
                          (const bf16_t*)q, ldq, (const bf16_t*)k_pages, (const bf16_t*)v_pages, nkv, page_size,
                          page_shift, table, table_stride, (const SeqMeta*)seqs, (const AttnItem*)items, (bf16_t*)out,
-                         ldo, part_acc, part_ml, G, scale, window);
+                         ldo, part_acc, part_ml, G, scale, window, DecodeFuse<bf16_t>{});
     else
       return fail("attention: unknown dtype %d", dtype);
     return check_launch("attention (cooperative, streamed)");

@@ -142,6 +142,89 @@ __device__ __forceinline__ float row_sumsq_part(const float* __restrict__ src, i
   return part;
 }
 
+// One head of one token: optional RMSNorm over the head (weight != nullptr),
+// then the half-split rotation of its first `rot` elements.  One wave runs it
+// in two phases, so that a caller can put other loads between them:
+// head_load brings the lane's elements (e = lane, lane + 64, ...), their norm
+// weights and rotation factors into registers; head_finish does the
+// arithmetic and hands the results to `dst(e, value)`.  `y` is an LDS row of
+// d floats private to the wave.  The sum of squares: lane l adds x[l]^2,
+// x[l+64]^2, ... ascending, then a butterfly over the wave.  Every kernel
+// that normalises a head goes through these two, so a head has the same bits
+// wherever it is processed.
+constexpr int kMaxHeadDim = 256;
+constexpr int kHeadPerLane = kMaxHeadDim / 64;
+struct HeadVec {
+  float x[kHeadPerLane], w[kHeadPerLane], c[kHeadPerLane], s[kHeadPerLane];
+};
+
+template <typename T>
+__device__ __forceinline__ void head_load(HeadVec& h, const T* src, int d, const float* __restrict__ weight,
+                                          const float* __restrict__ cos_table, const float* __restrict__ sin_table,
+                                          int pos, int rot, int lane) {
+  const int half = rot / 2;
+#pragma unroll
+  for (int i = 0; i < kHeadPerLane; ++i) {
+    const int e = lane + 64 * i;
+    const bool in = e < d;
+    h.x[i] = in ? to_f32(src[e]) : 0.f;
+    h.w[i] = (weight && in) ? weight[e] : 1.f;
+    h.c[i] = 1.f;
+    h.s[i] = 0.f;
+    if (cos_table && e < rot) {
+      const int idx = e < half ? e : e - half;
+      h.c[i] = cos_table[(long)pos * half + idx];
+      h.s[i] = sin_table[(long)pos * half + idx];
+    }
+  }
+}
+
+template <typename T, typename Dst>
+__device__ __forceinline__ void head_finish(const HeadVec& h, int d, bool normed, float eps, bool rotated, int rot,
+                                            float* __restrict__ y, int lane, Dst dst) {
+  float part = 0.f;
+#pragma unroll
+  for (int i = 0; i < kHeadPerLane; ++i) {
+    const int e = lane + 64 * i;
+    if (e < d) {
+      y[e] = h.x[i];
+      part = part + h.x[i] * h.x[i];
+    }
+  }
+  if (normed) {
+    const float total = wave_sum(part);
+    const float scale = 1.0f / sqrtf(total / (float)d + eps);
+#pragma unroll
+    for (int i = 0; i < kHeadPerLane; ++i) {
+      const int e = lane + 64 * i;
+      if (e < d) y[e] = (h.x[i] * scale) * h.w[i];
+    }
+  }
+  // The staging row is private to this wave: order its writes before the
+  // reads of other lanes without a workgroup barrier.
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  const int half = rot / 2;
+#pragma unroll
+  for (int i = 0; i < kHeadPerLane; ++i) {
+    const int e = lane + 64 * i;
+    if (e >= d) continue;
+    float v = y[e];
+    if (rotated && e < rot) {
+      const int idx = e < half ? e : e - half;
+      const float lo = y[idx];
+      const float hi = y[idx + half];
+      v = e < half ? lo * h.c[i] - hi * h.s[i] : hi * h.c[i] + lo * h.s[i];
+    }
+    dst(e, from_f32<T>(v));
+  }
+  // the row may be reused by the caller for its next head
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
 }  // namespace ls
 
 // Error reporting across the C interface: every entry point returns 0 or a

@@ -61,7 +61,6 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ 
 // One wave per (token, head); sums of squares: lane i adds x[i]^2,
 // x[i+64]^2, ... ascending, then a butterfly over the wave.
 // ---------------------------------------------------------------------------
-constexpr int kMaxHeadDim = 256;
 
 struct SeqMeta {  // one per sequence of the step (all int32)
   int q_off;      // first packed row
@@ -109,39 +108,11 @@ __global__ __launch_bounds__(256) void qk_rope_kv_kernel(
   }
 
   const float* weight = is_q ? q_weight : k_weight;
-  float* y = stage[wave];
-  float part = 0.f;
-  for (int e = lane; e < d; e += 64) {
-    const float v = to_f32(src[e]);
-    y[e] = v;
-    part = part + v * v;
-  }
-  if (weight) {
-    const float total = wave_sum(part);
-    const float scale = 1.0f / sqrtf(total / (float)d + eps);
-    for (int e = lane; e < d; e += 64) y[e] = (y[e] * scale) * weight[e];
-  }
-  // The staging row is private to this wave: order its writes before the
-  // reads of other lanes without a workgroup barrier (waves of other heads
-  // may have left already).
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-  __builtin_amdgcn_wave_barrier();
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-
   T* dst = is_q ? src : k_pages + ((page * nkv + (head - nq)) * page_size + slot) * d;
-  const int half = rot / 2;
-  for (int e = lane; e < d; e += 64) {
-    float v = y[e];
-    if (cos_table && e < rot) {
-      const int i = e < half ? e : e - half;
-      const float c = cos_table[(long)pos * half + i];
-      const float s = sin_table[(long)pos * half + i];
-      const float lo = y[i];
-      const float hi = y[i + half];
-      v = e < half ? lo * c - hi * s : hi * c + lo * s;
-    }
-    dst[e] = from_f32<T>(v);
-  }
+  HeadVec hv;
+  head_load<T>(hv, src, d, weight, cos_table, sin_table, pos, rot, lane);
+  head_finish<T>(hv, d, weight != nullptr, eps, cos_table != nullptr, rot, stage[wave], lane,
+                 [&](int e, T v) { dst[e] = v; });
 }
 
 // ---------------------------------------------------------------------------

@@ -97,6 +97,11 @@ class Kernels:
         lib = self.attention_lib(head_dim)
         return page_size >= 8 and bool(lib.ls_attn_coop_dma_supported(c_int(DTYPE_CODE[dtype])))
 
+    def decode_fused_supported(self, head_dim: int, dtype: torch.dtype, page_size: int) -> bool:
+        """Whether ``attention_decode`` (norm, rotation and cache write inside the attention kernel) can run."""
+        lib = self.attention_lib(head_dim)
+        return page_size >= 8 and bool(lib.ls_attn_decode_fused_supported(c_int(DTYPE_CODE[dtype])))
+
     def wide_supported(self, head_dim: int, dtype: torch.dtype, page_size: int) -> bool:
         """Whether the wide attention kernel (variant 4, for prompt portions) can run."""
         return page_size >= 8 and bool(self.attention_lib(head_dim).ls_attn_wide_supported(c_int(DTYPE_CODE[dtype])))
@@ -284,6 +289,43 @@ class Kernels:
             c_int(page_size), _ptr(table), c_int(table.shape[1]), _ptr(seqs), _ptr(items), c_int(n_items),
             _ptr(out), c_long(out.stride(0)), _ptr(part_acc), _ptr(part_ml), c_int(nq // nkv), c_float(scale),
             c_int(window), c_int(variant), c_int(max_rows), _stream())
+        self._check(lib, code)
+
+    def attention_decode(self, qkv: torch.Tensor, nq: int, nkv: int, d: int, k_pages, v_pages, page_size: int,
+                         table, seqs, items, n_items: int, out: torch.Tensor, part_acc, part_ml, scale: float,
+                         window: int, q_weight, k_weight, eps: float, cos, sin, rot: int, max_pos: int,
+                         write_kv: bool) -> None:
+        """A step of single decoded tokens: what ``qk_rope_kv`` and ``attention`` (cooperative items) do,
+        in one launch.  ``qkv`` is the raw fused projection; every request brings exactly one token."""
+        lib = self.attention_lib(d)
+        _rows_ok(qkv, "attention_decode qkv"); _rows_ok(out, "attention_decode out")
+        _need(qkv.dtype in DTYPE_CODE and out.dtype == qkv.dtype, "attention_decode qkv/out dtype")
+        _need(nq % nkv == 0, f"{nq} query heads are not a multiple of {nkv} kv heads")
+        heads = nq + 2 * nkv if write_kv else nq
+        _need(qkv.shape[1] >= heads * d and out.shape[1] >= nq * d, "attention_decode rows are too short")
+        _need(k_pages.dtype == qkv.dtype and v_pages.dtype == qkv.dtype and k_pages.is_contiguous()
+              and v_pages.is_contiguous() and k_pages.shape[1:] == (nkv, page_size, d)
+              and v_pages.shape[1:] == (nkv, d, page_size), "attention cache pages have the wrong layout or dtype")
+        _need(table.dtype == torch.int32 and table.dim() == 2 and table.is_contiguous(), "attention block table")
+        _need(items.dtype == torch.int32 and items.is_contiguous() and items.numel() >= 8 * n_items,
+              "attention items must hold 8 int32 each")
+        for w in (q_weight, k_weight):
+            _need(w is None or (w.dtype == torch.float32 and w.is_contiguous() and w.numel() == d),
+                  "per-head norm weights must be float32 [head_dim]")
+        positions = 0
+        if cos is not None:
+            _need(sin is not None and cos.dtype == torch.float32 and sin.dtype == torch.float32
+                  and cos.is_contiguous() and sin.is_contiguous() and cos.shape == sin.shape
+                  and cos.shape[1] == rot // 2, "rotation tables must be float32 [positions, rot/2]")
+            positions = cos.shape[0]
+        if n_items == 0:
+            return
+        code = lib.ls_attention_decode(
+            c_int(DTYPE_CODE[qkv.dtype]), _ptr(qkv), c_long(qkv.stride(0)), _ptr(k_pages), _ptr(v_pages), c_int(nq),
+            c_int(nkv), c_int(page_size), _ptr(table), c_int(table.shape[1]), _ptr(seqs), _ptr(items),
+            c_int(n_items), _ptr(out), c_long(out.stride(0)), _ptr(part_acc), _ptr(part_ml), c_float(scale),
+            c_int(window), _ptr(q_weight), _ptr(k_weight), c_float(eps), _ptr(cos), _ptr(sin), c_int(rot),
+            c_int(positions), c_int(max_pos), c_int(1 if write_kv else 0), _stream())
         self._check(lib, code)
 
     def attention_combine(self, d: int, seqs, items, n_items: int, nq: int, nkv: int, part_acc, part_ml,

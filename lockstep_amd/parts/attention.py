@@ -21,6 +21,12 @@ from ..config.base import PartSpec
 from ..ops import ADD_F32, STORE_F32
 from .base import Mixer, PagedKVSpec, WeightSpec, build_part, register_part
 
+import os
+
+# Steps of single decoded tokens run norm, rotation and cache write inside the
+# attention kernel (one launch less per layer); "0" keeps the separate kernel.
+FUSE_DECODE = os.environ.get("LOCKSTEP_FUSE_DECODE", "1") not in ("", "0")
+
 
 @register_part("attention")
 class Attention(Mixer):
@@ -109,12 +115,23 @@ class Attention(Mixer):
             k.gemm(x, self.w_qkv, qkv, **fused)
         else:
             k.gemm(x, self.w_q, qkv[:, : nq * d], **fused)
-        k.qk_rope_kv(qkv, t, nq, nkv, d, self.q_norm, self.k_norm, self.norm_eps, self.position.cos,
-                     self.position.sin, self.position.rotary_dim, ctx.tok_seq, ctx.tok_pos, ctx.seqs,
-                     ctx.max_position, group.table, key_pages, value_pages, group.page_size, run.writes_cache)
         attn = ctx.buf("attention.out", (t, nq * d), rt.dtype)
         window = int(self.window) if self.window is not None else 0
         plan = ctx.attention_plan(nq // nkv, nkv, d, window)
+        if plan.decode_fused and FUSE_DECODE:
+            # single decoded tokens: norm, rotation and cache write happen inside the attention kernel
+            k.attention_decode(qkv, nq, nkv, d, key_pages, value_pages, group.page_size, group.table, ctx.seqs,
+                               plan.coop_items, plan.n_coop, attn, plan.part_acc, plan.part_ml, self.scale, window,
+                               self.q_norm, self.k_norm, self.norm_eps, self.position.cos, self.position.sin,
+                               self.position.rotary_dim, ctx.max_position, run.writes_cache)
+            if plan.n_combine:
+                k.attention_combine(d, ctx.seqs, plan.combine_items, plan.n_combine, nq, nkv, plan.part_acc,
+                                    plan.part_ml, attn)
+            k.gemm(attn, self.w_o, out, ADD_F32 if accumulate else STORE_F32)
+            return
+        k.qk_rope_kv(qkv, t, nq, nkv, d, self.q_norm, self.k_norm, self.norm_eps, self.position.cos,
+                     self.position.sin, self.position.rotary_dim, ctx.tok_seq, ctx.tok_pos, ctx.seqs,
+                     ctx.max_position, group.table, key_pages, value_pages, group.page_size, run.writes_cache)
         if plan.n_items:
             k.attention(qkv, nq, nkv, d, key_pages, value_pages, group.page_size, group.table, ctx.seqs,
                         plan.items, plan.n_items, attn, plan.part_acc, plan.part_ml, self.scale, window)

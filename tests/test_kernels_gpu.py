@@ -447,6 +447,70 @@ def test_decode_attention_is_the_same_in_every_kernel(dtype, nq, nkv, d, ps):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nq,nkv,d,ps,rot,normed,window", [
+    (16, 8, 128, 16, 128, True, 0), (8, 1, 64, 32, 64, True, 0), (4, 4, 16, 8, 16, True, 0),
+    (6, 2, 48, 16, 32, False, 0), (4, 2, 32, 8, 0, True, 0), (4, 2, 64, 16, 64, True, 200)])
+def test_fused_decode_attention_equals_the_separate_kernels(dtype, nq, nkv, d, ps, rot, normed, window):
+    """A decoded token through qk_rope_kv + cooperative attention, and through the one fused launch:
+    the same output bits and the same cache contents, at the edges of pages, tiles and splits."""
+    if not K().decode_fused_supported(d, dtype, ps):
+        pytest.skip("the fused decode kernel does not fit into LDS for this head size")
+    from lockstep_amd.ops import kernels
+
+    g = torch.Generator().manual_seed(d + nq)
+    total = 530
+    qkv = (torch.randn(total, (nq + 2 * nkv) * d, generator=g) * 2).to(dtype).cuda()
+    qw = (1 + 0.3 * torch.randn(d, generator=g)).cuda() if normed else None
+    kw = (1 + 0.3 * torch.randn(d, generator=g)).cuda() if normed else None
+    cos = sin = None
+    if rot:
+        inv = 1.0 / (1e4 ** (torch.arange(0, rot // 2, dtype=torch.float64) * 2 / rot))
+        ang = torch.arange(total, dtype=torch.float64)[:, None] * inv[None, :]
+        cos, sin = ang.cos().float().cuda(), ang.sin().float().cuda()
+    eps = 1e-5
+    tile, split = kernels().attention_geometry(d)
+    for p in (0, 1, ps - 1, ps, 127, 128, 255, 256, 257, 300, 511, 512, 529):
+        base = PagedCase(dtype, nq, nkv, d, ps, p + 1, shuffle_seed=p)
+        if p:
+            ctx_rows = qkv[:p].clone()
+            base.write(ctx_rows, 0, qw, kw, eps, cos, sin, rot)
+        first_needed = max(0, p - window + 1) // ps if window else 0
+        base.table[1, :first_needed] = -1
+        k0, v0 = base.k_pages.clone(), base.v_pages.clone()
+        # separate kernels
+        row = qkv[p:p + 1].clone()
+        base.write(row, p, qw, kw, eps, cos, sin, rot)
+        want = base.attend(row, p, d ** -0.5, window=window, variant=5)
+        k_want, v_want = base.k_pages.clone(), base.v_pages.clone()
+        for use_split in (True, False):
+            base.k_pages.copy_(k0); base.v_pages.copy_(v0)
+            lo = max(0, p - window + 1) if window else 0
+            split_lo = lo // split
+            n_splits = p // split + 1 - split_lo
+            if use_split:
+                items = [v for s_ in range(split_lo, split_lo + n_splits) for v in (0, 0, s_, s_ + 1, 0, n_splits, split_lo, 0)]
+                combine = [0, 0, 0, n_splits]
+            else:
+                items, combine = [0, 0, split_lo, p // split + 1, -1, 0, 0, 0], []
+            part_rows = max(nkv * (nq // nkv) * n_splits, 1)
+            part_acc = torch.full((part_rows, d), float("nan"), dtype=torch.float32, device="cuda")
+            part_ml = torch.full((part_rows, 2), float("nan"), dtype=torch.float32, device="cuda")
+            out = torch.full((1, nq * d), float("nan"), dtype=dtype, device="cuda")
+            items_t = torch.tensor(items, dtype=torch.int32).cuda()
+            raw = qkv[p:p + 1].clone()
+            K().attention_decode(raw, nq, nkv, d, base.k_pages, base.v_pages, ps, base.table, base.seqs(p, 1), items_t,
+                                 len(items) // 8, out, part_acc, part_ml, d ** -0.5, window, qw, kw, eps, cos, sin, rot,
+                                 p, True)
+            if combine:
+                K().attention_combine(d, base.seqs(p, 1), torch.tensor(combine, dtype=torch.int32).cuda(), 1, nq, nkv,
+                                      part_acc, part_ml, out)
+            assert torch.equal(out.view(1, nq, d), want), f"position {p}, split={use_split}"
+            same_k = (base.k_pages == k_want) | ((base.k_pages != base.k_pages) & (k_want != k_want))
+            same_v = (base.v_pages == v_want) | ((base.v_pages != base.v_pages) & (v_want != v_want))
+            assert bool(same_k.all()) and bool(same_v.all()), f"cache after position {p}, split={use_split}"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("m", [1, 9, 16, 40, 200])
 @pytest.mark.parametrize("inter,k", [(136, 96), (3072, 1024), (48, 260)])
 def test_gemm_with_swiglu_epilogue(dtype, m, inter, k):
