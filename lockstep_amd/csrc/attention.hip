@@ -744,35 +744,42 @@ __global__ __launch_bounds__(64 * NW) void attention_wide_kernel(
     const int key = min(ti * kTileKeys + ((int)threadIdx.x << page_shift), sm.kv_len - 1);
     return tbl[key >> page_shift];
   };
-  // Start the loads of a tile into its buffer.  Every address is clamped to a
-  // held key of a held page, so nothing outside the cache is touched.
+  // Start the loads of a tile into its buffer.  What does not depend on the
+  // tile is computed once: the offset of each of the thread's pieces inside
+  // its page.  Keys past the request's end need no clamp of their own: the
+  // page id of their page is that of the last held page (table_entry clamps),
+  // so the loads stay inside the cache, and what they bring is masked.
+  const long page_stride = (long)nkv * page_size * D;  // elements of one page, K or V
+  int k_off[PER], v_off[PER];
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    const int p = i * NT + (int)threadIdx.x;
+    const int row = p / KPIECES;
+    const int slot = p % KPIECES;
+    const int piece = (slot - row % KPIECES + KPIECES) % KPIECES;
+    k_off[i] = (kvh * page_size + (row & (page_size - 1))) * D + piece * VEC;
+    const int c = p / D;
+    const int d = p % D;
+    v_off[i] = ((kvh * D + d) << page_shift) + ((c * VEC) & (page_size - 1));
+  }
   auto issue = [&](int ti) {
-    const int t0 = ti * kTileKeys;
     const int* pages = tile_pages + (ti & 1) * 16;
     unsigned char* k_buf = lds + (ti & 1) * BUF_BYTES;
     unsigned char* v_buf = k_buf + TILE_BYTES;
-    const int last_key = sm.kv_len - 1;
+    int k_page[PER], v_page[PER];
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {  // all page ids first: their LDS reads overlap
+      const int p = i * NT + (int)threadIdx.x;
+      k_page[i] = pages[min((p / KPIECES) >> page_shift, 15)];
+      v_page[i] = pages[min(((p / D) * VEC) >> page_shift, 15)];
+    }
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
-      const int p = i * NT + (int)threadIdx.x;
       if (PER * NT != TOTAL && i * NT + wave * 64 >= TOTAL) break;  // uniform for the wave
-      {
-        const int row = p / KPIECES;
-        const int slot = p % KPIECES;
-        const int piece = (slot - row % KPIECES + KPIECES) % KPIECES;
-        const int key = min(t0 + row, last_key);
-        const int page = max(pages[(key - t0) >> page_shift], 0);
-        const T* src = k_pages + (((long)page * nkv + kvh) * page_size + (key & (page_size - 1))) * D + piece * VEC;
-        __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(k_buf + (i * NT + wave * 64) * 16), 16, 0, 0);
-      }
-      {
-        const int c = p / D;
-        const int d = p % D;
-        const int key = min(t0 + c * VEC, last_key & ~(VEC - 1));
-        const int page = max(pages[(key - t0) >> page_shift], 0);
-        const T* src = v_pages + ((((long)page * nkv + kvh) * D + d) << page_shift) + (key & (page_size - 1));
-        __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(v_buf + (i * NT + wave * 64) * 16), 16, 0, 0);
-      }
+      const T* k_src = k_pages + (long)max(k_page[i], 0) * page_stride + k_off[i];
+      __builtin_amdgcn_global_load_lds((gptr_t)k_src, (lptr_t)(k_buf + (i * NT + wave * 64) * 16), 16, 0, 0);
+      const T* v_src = v_pages + (long)max(v_page[i], 0) * page_stride + v_off[i];
+      __builtin_amdgcn_global_load_lds((gptr_t)v_src, (lptr_t)(v_buf + (i * NT + wave * 64) * 16), 16, 0, 0);
     }
   };
 
@@ -962,298 +969,13 @@ __global__ __launch_bounds__(64 * NW) void attention_wide_kernel(
 
 
 // Variant 3, "cooperative": for work items with at most 16 rows (one decoded
-// token per request and up to 16 query heads per kv head), where the staged
-// kernel would leave three of its four waves idle.  All four waves hold the
-// same 16 rows.  Wave w computes the score blocks 2w and 2w+1 of a tile and
-// the output columns of the blocks w, w+4, ...; row maxima, per-block sums and
+// token per request and up to 16 query heads per kv head), where the other
+// kernels would leave most of their waves idle.  All four waves hold the same
+// 16 rows.  Wave w computes the score blocks 2w and 2w+1 of a tile and the
+// output columns of the blocks w, w+4, ...; row maxima, per-block sums and
 // probabilities meet in LDS.  Every number is produced by the same
 // instruction sequence as in the other variants, so the bits are the same.
-// STAGE tiles (a whole split when it fits) are fetched at once.
-template <typename T, int STAGE>
-__global__ __launch_bounds__(256) void attention_coop_kernel(
-    const T* __restrict__ q, long ldq, const T* __restrict__ k_pages, const T* __restrict__ v_pages, int nkv,
-    int page_size, int page_shift, const int* __restrict__ table, int table_stride,
-    const SeqMeta* __restrict__ seqs, const AttnItem* __restrict__ items, T* __restrict__ out, long ldo,
-    float* __restrict__ part_acc, float* __restrict__ part_ml, int G, float scale, int window) {
-  typedef Atom<T> A;
-  typedef typename A::vec_t vec_t;
-  constexpr int SZ = sizeof(T);
-  constexpr int NC = (D + A::KCHUNK - 1) / A::KCHUNK;
-  constexpr int KROW = D * SZ;
-  constexpr int KPIECES = KROW / 16;
-  constexpr int VROW = kTileKeys * SZ;
-  constexpr int VPIECES = VROW / 16;
-  constexpr int TOTAL = kTileKeys * KPIECES;
-  constexpr int PER = (TOTAL + 255) / 256;
-  constexpr int TILES_PER_SPLIT = kSplitKeys / kTileKeys;
-  constexpr int LOG_VEC = (A::VEC == 8) ? 3 : 2;
-  constexpr int TILE_BYTES = 2 * kTileKeys * KROW;  // K tile + V tile
-  constexpr int MYDB = (DB + 3) / 4;                 // output blocks of one wave
-
-  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
-  float* wmax = reinterpret_cast<float*>(lds + STAGE * TILE_BYTES);  // [4][16]
-  float* psum = wmax + 64;                                            // [NB][64]
-  f32x4* prob = reinterpret_cast<f32x4*>(psum + NB * 64);             // [NB][64]
-
-  const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
-  const AttnItem item = items[blockIdx.x];
-  const SeqMeta sm = seqs[item.seq];
-  const int kvh = blockIdx.y;
-  const int rows_total = sm.q_len * G;  // <= 16, checked on the host
-  const int row16 = lane & 15;
-  const int g = lane >> 4;
-  const int r = row16;
-  const bool row_ok = r < rows_total;
-  const int qi = row_ok ? r / G : 0;
-  const int head = kvh * G + (row_ok ? r % G : 0);
-  const int q_pos = sm.q_start + qi;
-  // this row sees the keys key_lo <= key <= key_hi (none if the row does not exist)
-  const int key_hi = row_ok ? q_pos : -1;
-  const int key_lo = window > 0 ? q_pos - window + 1 : 0;
-  const int first_pos = sm.q_start;
-  const int last_pos = sm.q_start + (rows_total - 1) / G;
-  const int lo_valid = window > 0 ? max(0, sm.q_start - window + 1) : 0;
-  const int* __restrict__ tbl = table + (long)sm.table_row * table_stride;
-  const bool direct = item.part_base < 0;
-  const int vshift = page_shift - LOG_VEC;
-
-  vec_t qv[NC];
-#pragma unroll
-  for (int c = 0; c < NC; ++c)
-    qv[c] = load_vec<T>(q + (long)head * D, sm.q_off + qi, c * A::KCHUNK + g * A::VEC, D, ldq, row_ok, true);
-
-  int ti_lo = item.split_begin * TILES_PER_SPLIT;
-  if (window > 0) ti_lo = max(ti_lo, max(0, first_pos - window + 1) / kTileKeys);
-  const int ti_hi = min(item.split_end * TILES_PER_SPLIT, last_pos / kTileKeys + 1);
-
-  // a wave keeps only its own output blocks: block j of the arrays is column block wave + 4j
-  f32x4 cur_acc[MYDB], run_acc[MYDB];
-  float cur_m = kNegSentinel, cur_l = 0.f, run_m = kNegSentinel, run_l = 0.f;
-#pragma unroll
-  for (int j = 0; j < MYDB; ++j) {
-    cur_acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
-    run_acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
-  }
-
-  for (int tb = ti_lo; tb < ti_hi; tb += STAGE) {
-    // ---- fetch STAGE tiles: all page ids, then all data, then LDS ------------
-    int kpage[STAGE][PER], vpage[STAGE][PER];
-#pragma unroll
-    for (int st = 0; st < STAGE; ++st) {
-      const int t0 = (tb + st) * kTileKeys;
-#pragma unroll
-      for (int i = 0; i < PER; ++i) {
-        const int p = threadIdx.x + 256 * i;
-        const int key = t0 + p / KPIECES;
-        kpage[st][i] = tbl[min(key, sm.kv_len - 1) >> page_shift];
-        const int q1 = p >> vshift;
-        const int key0 = t0 + ((q1 / D) << page_shift) + ((p & ((1 << vshift) - 1)) << LOG_VEC);
-        vpage[st][i] = tbl[min(key0, sm.kv_len - 1) >> page_shift];
-      }
-    }
-    __builtin_amdgcn_sched_barrier(0);  // every page id is requested before the first data load is built from one
-    vec_t kreg[STAGE][PER], vreg[STAGE][PER];
-#pragma unroll
-    for (int st = 0; st < STAGE; ++st) {  // loads only, from clamped addresses
-      const int t0 = (tb + st) * kTileKeys;
-#pragma unroll
-      for (int i = 0; i < PER; ++i) {
-        const int p = threadIdx.x + 256 * i;
-        {
-          const int key = min(t0 + p / KPIECES, sm.kv_len - 1);
-          const int page = max(kpage[st][i], 0);
-          const T* src = k_pages + (((long)page * nkv + kvh) * page_size + (key & (page_size - 1))) * D +
-                         (p % KPIECES) * A::VEC;
-          kreg[st][i] = *reinterpret_cast<const vec_t*>(src);
-        }
-        {
-          const int q1 = p >> vshift;
-          const int kp = p & ((1 << vshift) - 1);
-          const int page = max(vpage[st][i], 0);
-          const T* src = v_pages + ((((long)page * nkv + kvh) * D + q1 % D) << page_shift) + (kp << LOG_VEC);
-          vreg[st][i] = *reinterpret_cast<const vec_t*>(src);
-        }
-      }
-    }
-    __builtin_amdgcn_sched_barrier(0);  // ... and every data load is issued before the first one is waited for
-    __syncthreads();  // the previous stage has been consumed
-#pragma unroll
-    for (int st = 0; st < STAGE; ++st) {  // zero what is not a held key, write to LDS
-      unsigned char* k_lds = lds + st * TILE_BYTES;
-      unsigned char* v_lds = k_lds + kTileKeys * KROW;
-      const int t0 = (tb + st) * kTileKeys;
-      const bool tile_in = tb + st < ti_hi;
-#pragma unroll
-      for (int i = 0; i < PER; ++i) {
-        const int p = threadIdx.x + 256 * i;
-        const int kt = p / KPIECES;
-        const int piece = p % KPIECES;
-        const int key = t0 + kt;
-        const bool k_ok = tile_in && key < sm.kv_len && key >= lo_valid && kpage[st][i] >= 0;
-        *reinterpret_cast<vec_t*>(k_lds + kt * KROW + ((piece + kt) % KPIECES) * 16) =
-            k_ok ? kreg[st][i] : A::zero();
-        const int q1 = p >> vshift;
-        const int kp = p & ((1 << vshift) - 1);
-        const int pg = q1 / D;
-        const int d = q1 % D;
-        const int key0 = t0 + (pg << page_shift) + (kp << LOG_VEC);
-        const int n_hi = (tile_in && vpage[st][i] >= 0) ? sm.kv_len - key0 : 0;
-        const int vpiece = (pg << vshift) + kp;
-        *reinterpret_cast<vec_t*>(v_lds + d * VROW + ((vpiece + d) % VPIECES) * 16) =
-            mask_keys(vreg[st][i], lo_valid - key0, n_hi);
-      }
-    }
-    __syncthreads();
-
-    // ---- the tiles of this stage ------------------------------------------------
-    for (int st = 0; st < STAGE; ++st) {
-      const int ti = tb + st;
-      if (ti >= ti_hi) break;
-      const int t0 = ti * kTileKeys;
-      const unsigned char* k_lds = lds + st * TILE_BYTES;
-      const unsigned char* v_lds = k_lds + kTileKeys * KROW;
-
-      // score blocks 2w and 2w+1
-      f32x4 s[2];
-      float my_max = kNegSentinel;
-#pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        const int kb = 2 * wave + j;
-        s[j] = f32x4{0.f, 0.f, 0.f, 0.f};
-        const int row = kb * 16 + row16;
-#pragma unroll
-        for (int c = 0; c < NC; ++c) {
-          const int piece = c * 4 + g;
-          vec_t kv = A::zero();
-          if (piece < KPIECES)
-            kv = *reinterpret_cast<const vec_t*>(k_lds + row * KROW + ((piece + row) % KPIECES) * 16);
-          A::mma(s[j], kv, qv[c]);
-        }
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int key = t0 + kb * 16 + 4 * g + e;
-          const float v = ((key <= key_hi) & (key >= key_lo)) ? s[j][e] * scale : kMasked;
-          s[j][e] = v;
-          my_max = fmaxf(my_max, v);
-        }
-      }
-      my_max = quad16_max(my_max);
-      if (g == 0) wmax[wave * 16 + row16] = my_max;
-      __syncthreads();
-      const float tile_max = fmaxf(fmaxf(wmax[row16], wmax[16 + row16]), fmaxf(wmax[32 + row16], wmax[48 + row16]));
-      const float m_new = fmaxf(cur_m, tile_max);
-      const float alpha = softmax_exp<T>(cur_m - m_new);
-#pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        const int kb = 2 * wave + j;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) s[j][e] = softmax_exp<T>(s[j][e] - m_new);  // masked: exp(-inf) = 0
-        psum[kb * 64 + lane] = (s[j][0] + s[j][1]) + (s[j][2] + s[j][3]);
-        prob[kb * 64 + lane] = s[j];
-      }
-      __syncthreads();
-      float p_sum = 0.f;
-#pragma unroll
-      for (int kb = 0; kb < NB; ++kb) p_sum = p_sum + psum[kb * 64 + lane];
-      p_sum = quad16_sum(p_sum);
-      cur_l = cur_l * alpha + p_sum;
-      cur_m = m_new;
-#pragma unroll
-      for (int j = 0; j < MYDB; ++j)
-#pragma unroll
-        for (int e = 0; e < 4; ++e) cur_acc[j][e] = cur_acc[j][e] * alpha;
-      constexpr int KB16 = A::VEC / 4;
-#pragma unroll
-      for (int kb = 0; kb < NB; kb += KB16) {
-        vec_t pv;
-#pragma unroll
-        for (int h = 0; h < KB16; ++h) {
-          const f32x4 four = prob[(kb + h) * 64 + lane];
-#pragma unroll
-          for (int e = 0; e < 4; ++e) pv[h * 4 + e] = from_f32<T>(four[e]);
-        }
-#pragma unroll
-        for (int j = 0; j < MYDB; ++j) {
-          const int blk = wave + 4 * j;
-          if (blk >= DB) continue;
-          const int d = blk * 16 + row16;
-          vec_t vv;
-#pragma unroll
-          for (int h = 0; h < KB16; ++h) {
-            const int byte = ((kb + h) * 16 + 4 * g) * SZ;
-            const unsigned char* src = v_lds + d * VROW + (((byte >> 4) + d) % VPIECES) * 16 + (byte & 15);
-            if (SZ == 2) {
-              bf16x4 four = *reinterpret_cast<const bf16x4*>(src);
-#pragma unroll
-              for (int e = 0; e < 4; ++e) vv[h * 4 + e] = four[e];
-            } else {
-              f32x4 four = *reinterpret_cast<const f32x4*>(src);
-#pragma unroll
-              for (int e = 0; e < 4; ++e) vv[h * 4 + e] = four[e];
-            }
-          }
-          A::mma(cur_acc[j], vv, pv);
-        }
-      }
-      if (direct && ((ti + 1) % TILES_PER_SPLIT == 0 || ti + 1 == ti_hi)) {
-        if (cur_l > 0.f) {  // the fold of fold_split, on this wave's blocks
-          const float m_fold = fmaxf(run_m, cur_m);
-          const float fa = softmax_exp<T>(run_m - m_fold);
-          const float fb = softmax_exp<T>(cur_m - m_fold);
-#pragma unroll
-          for (int j = 0; j < MYDB; ++j)
-#pragma unroll
-            for (int e = 0; e < 4; ++e) run_acc[j][e] = run_acc[j][e] * fa + cur_acc[j][e] * fb;
-          run_l = run_l * fa + cur_l * fb;
-          run_m = m_fold;
-        }
-#pragma unroll
-        for (int j = 0; j < MYDB; ++j) cur_acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
-        cur_m = kNegSentinel;
-        cur_l = 0.f;
-      }
-    }
-  }
-
-  if (!row_ok) return;
-  if (direct) {
-    T* dst = out + (long)(sm.q_off + qi) * ldo + (long)head * D;
-    const float l = run_l;
-#pragma unroll
-    for (int j = 0; j < MYDB; ++j) {
-      const int blk = wave + 4 * j;
-      if (blk >= DB) continue;
-      float o[4];
-#pragma unroll
-      for (int e = 0; e < 4; ++e) o[e] = l > 0.f ? run_acc[j][e] / l : 0.f;
-      T* p = dst + blk * 16 + 4 * g;
-      if (SZ == 2) {
-        bf16x4 v;
-        v[0] = (bf16_t)o[0]; v[1] = (bf16_t)o[1]; v[2] = (bf16_t)o[2]; v[3] = (bf16_t)o[3];
-        *reinterpret_cast<bf16x4*>(p) = v;
-      } else {
-        *reinterpret_cast<f32x4*>(p) = f32x4{o[0], o[1], o[2], o[3]};
-      }
-    }
-  } else {
-    const int split = item.split_begin;
-    const long pr = item.part_base + ((long)kvh * rows_total + r) * item.n_splits + (split - item.split_lo);
-    float* pa = part_acc + pr * D;
-#pragma unroll
-    for (int j = 0; j < MYDB; ++j) {
-      const int blk = wave + 4 * j;
-      if (blk < DB) *reinterpret_cast<f32x4*>(pa + blk * 16 + 4 * g) = cur_acc[j];
-    }
-    if (wave == 0 && g == 0) {
-      part_ml[pr * 2] = cur_m;
-      part_ml[pr * 2 + 1] = cur_l;
-    }
-  }
-}
-
-// Variant 5, "cooperative, streamed": the cooperative kernel's arithmetic with
-// the wide kernel's data path.  The K and V tiles go from global memory
+// The data path is the wide kernel's: the K and V tiles go from global memory
 // straight into LDS; with NBUF == 2 the next tile is in flight while the four
 // waves work on the current one, with NBUF == 1 (large heads) a tile is loaded
 // after the previous one has been consumed.
@@ -1280,7 +1002,7 @@ struct DecodeFuse {
 };
 
 template <typename T, int NBUF, bool FUSE>
-__global__ __launch_bounds__(256) void attention_coop_dma_kernel(
+__global__ __launch_bounds__(256) void attention_coop_kernel(
     const T* __restrict__ q, long ldq, const T* __restrict__ k_pages, const T* __restrict__ v_pages, int nkv,
     int page_size, int page_shift, const int* __restrict__ table, int table_stride,
     const SeqMeta* __restrict__ seqs, const AttnItem* __restrict__ items, T* __restrict__ out, long ldo,
@@ -1310,6 +1032,12 @@ __global__ __launch_bounds__(256) void attention_coop_dma_kernel(
   T* knew = reinterpret_cast<T*>(prob + NB * 64);                        // FUSE: [D] new key, [D] new value
   T* vnew = knew + D;
 
+#ifdef LS_ATTN_PROBE
+  long long pr_t[16];
+  for (int i = 0; i < 16; ++i) pr_t[i] = 0;
+  long long pr_last = clock64();
+  const long long pr_begin = pr_last;
+#endif
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const AttnItem item = items[blockIdx.x];
@@ -1331,6 +1059,8 @@ __global__ __launch_bounds__(256) void attention_coop_dma_kernel(
   const int* __restrict__ tbl = table + (long)sm.table_row * table_stride;
   const bool direct = item.part_base < 0;
   const int pages_per_tile = kTileKeys >> page_shift;
+  if (sm.kv_len < 0) return;
+  PROBE(0)
 
   vec_t qv[NC];
   if (!FUSE) {
@@ -1347,33 +1077,37 @@ __global__ __launch_bounds__(256) void attention_coop_dma_kernel(
     const int key = min(ti * kTileKeys + ((int)threadIdx.x << page_shift), sm.kv_len - 1);
     return tbl[key >> page_shift];
   };
+  const long page_stride = (long)nkv * page_size * D;  // elements of one page, K or V
+  int k_off[PER], v_off[PER];
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    const int p = i * NT + (int)threadIdx.x;
+    const int row = p / KPIECES;
+    const int slot = p % KPIECES;
+    const int piece = (slot - row % KPIECES + KPIECES) % KPIECES;
+    k_off[i] = (kvh * page_size + (row & (page_size - 1))) * D + piece * VEC;
+    const int c = p / D;
+    const int d = p % D;
+    v_off[i] = ((kvh * D + d) << page_shift) + ((c * VEC) & (page_size - 1));
+  }
   auto issue = [&](int ti) {
-    const int t0 = ti * kTileKeys;
     const int* pages = tile_pages + (ti & 1) * 16;
     unsigned char* k_buf = lds + (NBUF == 2 ? (ti & 1) : 0) * BUF_BYTES;
     unsigned char* v_buf = k_buf + TILE_BYTES;
-    const int last_key = sm.kv_len - 1;
+    int k_page[PER], v_page[PER];
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {  // all page ids first: their LDS reads overlap
+      const int p = i * NT + (int)threadIdx.x;
+      k_page[i] = pages[min((p / KPIECES) >> page_shift, 15)];
+      v_page[i] = pages[min(((p / D) * VEC) >> page_shift, 15)];
+    }
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
-      const int p = i * NT + (int)threadIdx.x;
       if (PER * NT != TOTAL && i * NT + wave * 64 >= TOTAL) break;  // uniform for the wave
-      {
-        const int row = p / KPIECES;
-        const int slot = p % KPIECES;
-        const int piece = (slot - row % KPIECES + KPIECES) % KPIECES;
-        const int key = min(t0 + row, last_key);
-        const int page = max(pages[(key - t0) >> page_shift], 0);
-        const T* src = k_pages + (((long)page * nkv + kvh) * page_size + (key & (page_size - 1))) * D + piece * VEC;
-        __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(k_buf + (i * NT + wave * 64) * 16), 16, 0, 0);
-      }
-      {
-        const int c = p / D;
-        const int d = p % D;
-        const int key = min(t0 + c * VEC, last_key & ~(VEC - 1));
-        const int page = max(pages[(key - t0) >> page_shift], 0);
-        const T* src = v_pages + ((((long)page * nkv + kvh) * D + d) << page_shift) + (key & (page_size - 1));
-        __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(v_buf + (i * NT + wave * 64) * 16), 16, 0, 0);
-      }
+      const T* k_src = k_pages + (long)max(k_page[i], 0) * page_stride + k_off[i];
+      __builtin_amdgcn_global_load_lds((gptr_t)k_src, (lptr_t)(k_buf + (i * NT + wave * 64) * 16), 16, 0, 0);
+      const T* v_src = v_pages + (long)max(v_page[i], 0) * page_stride + v_off[i];
+      __builtin_amdgcn_global_load_lds((gptr_t)v_src, (lptr_t)(v_buf + (i * NT + wave * 64) * 16), 16, 0, 0);
     }
   };
 
@@ -1416,10 +1150,12 @@ __global__ __launch_bounds__(256) void attention_coop_dma_kernel(
   }
   if (ti_lo < ti_hi && (int)threadIdx.x < pages_per_tile) tile_pages[(ti_lo & 1) * 16 + threadIdx.x] = first_page;
   __syncthreads();
+  PROBE(1)
   if (ti_lo < ti_hi) {
     issue(ti_lo);
     if (ti_lo + 1 < ti_hi && (int)threadIdx.x < pages_per_tile) held = table_entry(ti_lo + 1);
   }
+  PROBE(2)
   if (FUSE) {
     float* ystage = reinterpret_cast<float*>(prob) + wave * D;               // the exchange buffers are free until the loop
     T* qrot = reinterpret_cast<T*>(reinterpret_cast<float*>(prob) + 4 * D);  // [16][D]
@@ -1451,13 +1187,16 @@ __global__ __launch_bounds__(256) void attention_coop_dma_kernel(
       qv[c] = (row_ok && col < D) ? *reinterpret_cast<const vec_t*>(qr + row16 * D + min(col, D - VEC)) : A::zero();
     }
   }
+  PROBE(3)
   for (int ti = ti_lo; ti < ti_hi; ++ti) {
     const int t0 = ti * kTileKeys;
     const unsigned char* k_lds = lds + (NBUF == 2 ? (ti & 1) : 0) * BUF_BYTES;
     unsigned char* v_lds = lds + (NBUF == 2 ? (ti & 1) : 0) * BUF_BYTES + TILE_BYTES;
     __asm__ volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this thread's pieces of the tile have landed
+    PROBE(4)
     if (ti + 1 < ti_hi && (int)threadIdx.x < pages_per_tile) tile_pages[((ti + 1) & 1) * 16 + threadIdx.x] = held;
     __syncthreads();  // the tile is complete (and the other buffer has been read by every wave)
+    PROBE(5)
     const bool patch = owner && ti == tile_new;  // the new key and value go into this tile
     if (t0 + kTileKeys > sm.kv_len || t0 < lo_valid || patch) {  // uniform: clean the values of keys that are not held
 #pragma unroll
@@ -1488,6 +1227,7 @@ __global__ __launch_bounds__(256) void attention_coop_dma_kernel(
     }
 
     // score blocks 2w and 2w+1
+    PROBE(6)
     f32x4 s[2];
     float my_max = kNegSentinel;
     {
@@ -1521,7 +1261,9 @@ __global__ __launch_bounds__(256) void attention_coop_dma_kernel(
     }
     my_max = quad16_max(my_max);
     if (g == 0) wmax[wave * 16 + row16] = my_max;
+    PROBE(7)
     __syncthreads();
+    PROBE(8)
     const float tile_max = fmaxf(fmaxf(wmax[row16], wmax[16 + row16]), fmaxf(wmax[32 + row16], wmax[48 + row16]));
     const float m_new = fmaxf(cur_m, tile_max);
     const float alpha = softmax_exp<T>(cur_m - m_new);
@@ -1560,7 +1302,9 @@ __global__ __launch_bounds__(256) void attention_coop_dma_kernel(
         }
         vop[kp][j] = vv;
       }
+    PROBE(9)
     __syncthreads();
+    PROBE(10)
     float p_sum = 0.f;
 #pragma unroll
     for (int kb = 0; kb < NB; ++kb) p_sum = p_sum + psum[kb * 64 + lane];
@@ -1586,6 +1330,7 @@ __global__ __launch_bounds__(256) void attention_coop_dma_kernel(
         A::mma(cur_acc[j], vop[kp][j], pv);
       }
     }
+    PROBE(11)
     if (direct && ((ti + 1) % TILES_PER_SPLIT == 0 || ti + 1 == ti_hi)) {
       if (cur_l > 0.f) {  // the fold of fold_split, on this wave's blocks
         const float m_fold = fmaxf(run_m, cur_m);
@@ -1610,6 +1355,14 @@ __global__ __launch_bounds__(256) void attention_coop_dma_kernel(
     }
   }
 
+#ifdef LS_ATTN_PROBE
+  if (threadIdx.x == 0 && kvh == 0 && part_ml != nullptr) {
+    long long* dst = reinterpret_cast<long long*>(part_ml + (1 << 20)) + blockIdx.x * 16;
+    for (int i = 0; i < 12; ++i) dst[i] = pr_t[i];
+    dst[12] = clock64() - pr_begin;
+    dst[13] = ti_hi - ti_lo;
+  }
+#endif
   if (!row_ok) return;
   if (direct) {
     T* dst = out + (long)(sm.q_off + qi) * ldo + (long)head * D;
@@ -1690,10 +1443,6 @@ using namespace ls;
 extern "C" int ls_attn_head_dim() { return D; }
 extern "C" int ls_attn_tile_keys() { return kTileKeys; }
 extern "C" int ls_attn_split_keys() { return kSplitKeys; }
-static bool coop_supported(int dtype);
-// 1 if the cooperative kernel (work items of at most 16 rows) can run for this dtype.
-extern "C" int ls_attn_coop_supported(int dtype) { return coop_supported(dtype) ? 1 : 0; }
-
 // Whether the staged kernel can have `bytes` of LDS: up to 64 KB always; above
 // that the function attribute is raised once per kernel (the device offers
 // 160 KB per workgroup); if that is refused the direct kernel runs instead.
@@ -1714,16 +1463,20 @@ static bool staged_fits(int dtype, size_t bytes) {
   return st == 1;
 }
 
-// The cooperative kernel stages two tiles (a whole split) when they fit into
-// 160 KB together with its exchange buffers, else one.
-constexpr size_t kCoopExtra = 64 * 4 + NB * 64 * 4 + NB * 64 * 16;
+constexpr size_t kCoopExtra = 64 * 4 + NB * 64 * 4 + NB * 64 * 16;  // row maxima, block sums, probabilities
 constexpr size_t kLdsLimit = 160 * 1024;
-constexpr int coop_stage(size_t elem) { return 2 * (2 * kTileKeys * D * elem) + kCoopExtra <= kLdsLimit ? 2 : 1; }
-constexpr int kCoopStageF32 = coop_stage(4);
-constexpr int kCoopStageBF16 = coop_stage(2);
+
+// The cooperative kernel: one or two buffers of a K and a V tile,
+// two rows of page ids and the exchange buffers of the cooperative kernel.
+constexpr size_t kCoopLdsExtra = 2 * 16 * sizeof(int) + kCoopExtra + 2 * D * 4;  // + new key and value (FUSE)
+constexpr int coop_bufs(size_t elem) {
+  return 2 * (2 * kTileKeys * D * elem) + kCoopLdsExtra <= kLdsLimit ? 2 : 1;
+}
+constexpr int kCoopBufsF32 = coop_bufs(4);
+constexpr int kCoopBufsBF16 = coop_bufs(2);
 static size_t coop_lds_bytes(int dtype) {
   const size_t elem = dtype == kF32 ? 4 : 2;
-  return (dtype == kF32 ? kCoopStageF32 : kCoopStageBF16) * (2 * (size_t)kTileKeys * D * elem) + kCoopExtra;
+  return (dtype == kF32 ? kCoopBufsF32 : kCoopBufsBF16) * (2 * (size_t)kTileKeys * D * elem) + kCoopLdsExtra;
 }
 static bool coop_supported(int dtype) {
   const size_t bytes = coop_lds_bytes(dtype);
@@ -1733,63 +1486,33 @@ static bool coop_supported(int dtype) {
   int& st = state[dtype == kF32 ? 0 : 1];
   if (st == 0) {
     hipError_t e = dtype == kF32
-        ? hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_coop_kernel<float, kCoopStageF32>),
+        ? hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_coop_kernel<float, kCoopBufsF32, false>),
                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes)
-        : hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_coop_kernel<bf16_t, kCoopStageBF16>),
+        : hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_coop_kernel<bf16_t, kCoopBufsBF16, false>),
                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
     if (e != hipSuccess) (void)hipGetLastError();
     st = e == hipSuccess ? 1 : -1;
   }
   return st == 1;
 }
-
-// The streamed cooperative kernel: one or two buffers of a K and a V tile,
-// two rows of page ids and the exchange buffers of the cooperative kernel.
-constexpr size_t kDmaExtra = 2 * 16 * sizeof(int) + kCoopExtra + 2 * D * 4;  // + new key and value (FUSE)
-constexpr int coop_dma_bufs(size_t elem) {
-  return 2 * (2 * kTileKeys * D * elem) + kDmaExtra <= kLdsLimit ? 2 : 1;
-}
-constexpr int kDmaBufsF32 = coop_dma_bufs(4);
-constexpr int kDmaBufsBF16 = coop_dma_bufs(2);
-static size_t coop_dma_lds_bytes(int dtype) {
-  const size_t elem = dtype == kF32 ? 4 : 2;
-  return (dtype == kF32 ? kDmaBufsF32 : kDmaBufsBF16) * (2 * (size_t)kTileKeys * D * elem) + kDmaExtra;
-}
-static bool coop_dma_supported(int dtype) {
-  const size_t bytes = coop_dma_lds_bytes(dtype);
-  if (bytes > kLdsLimit) return false;
-  if (bytes <= 64 * 1024) return true;
-  static int state[2] = {0, 0};
-  int& st = state[dtype == kF32 ? 0 : 1];
-  if (st == 0) {
-    hipError_t e = dtype == kF32
-        ? hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_coop_dma_kernel<float, kDmaBufsF32, false>),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes)
-        : hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_coop_dma_kernel<bf16_t, kDmaBufsBF16, false>),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
-    if (e != hipSuccess) (void)hipGetLastError();
-    st = e == hipSuccess ? 1 : -1;
-  }
-  return st == 1;
-}
-// 1 if the streamed cooperative kernel (variant 5) can run for this dtype.
-extern "C" int ls_attn_coop_dma_supported(int dtype) { return coop_dma_supported(dtype) ? 1 : 0; }
+// 1 if the cooperative kernel (variant 3, work items of at most 16 rows) can run for this dtype.
+extern "C" int ls_attn_coop_supported(int dtype) { return coop_supported(dtype) ? 1 : 0; }
 
 // The fused decode step (FUSE) stages the rotated query heads in the exchange
 // buffers before the loop needs them: 4 rows of D floats and 16 rows of D elements.
 static bool decode_fused_supported(int dtype) {
   const size_t elem = dtype == kF32 ? 4 : 2;
   if (4 * D * 4 + 16 * D * elem > (size_t)NB * 64 * 16) return false;
-  const size_t bytes = coop_dma_lds_bytes(dtype);
+  const size_t bytes = coop_lds_bytes(dtype);
   if (bytes > kLdsLimit) return false;
   if (bytes <= 64 * 1024) return true;
   static int state[2] = {0, 0};
   int& st = state[dtype == kF32 ? 0 : 1];
   if (st == 0) {
     hipError_t e = dtype == kF32
-        ? hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_coop_dma_kernel<float, kDmaBufsF32, true>),
+        ? hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_coop_kernel<float, kCoopBufsF32, true>),
                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes)
-        : hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_coop_dma_kernel<bf16_t, kDmaBufsBF16, true>),
+        : hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_coop_kernel<bf16_t, kCoopBufsBF16, true>),
                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
     if (e != hipSuccess) (void)hipGetLastError();
     st = e == hipSuccess ? 1 : -1;
@@ -1830,17 +1553,17 @@ extern "C" int ls_attention_decode(int dtype, const void* qkv, long ld, void* k_
   dim3 grid(n_items, nkv);
   int page_shift = 0;
   while ((1 << page_shift) < page_size) ++page_shift;
-  const size_t bytes = coop_dma_lds_bytes(dtype);
+  const size_t bytes = coop_lds_bytes(dtype);
   if (dtype == kF32) {
     DecodeFuse<float> fz{q_weight, k_weight, eps, cos_table, sin_table, rot, nq, write_kv, (float*)k_pages, (float*)v_pages};
-    hipLaunchKernelGGL((attention_coop_dma_kernel<float, kDmaBufsF32, true>), grid, dim3(256), bytes, s,
+    hipLaunchKernelGGL((attention_coop_kernel<float, kCoopBufsF32, true>), grid, dim3(256), bytes, s,
                        (const float*)qkv, ld, (const float*)k_pages, (const float*)v_pages, nkv, page_size, page_shift,
                        table, table_stride, (const SeqMeta*)seqs, (const AttnItem*)items, (float*)out, ldo, part_acc,
                        part_ml, G, scale, window, fz);
   } else if (dtype == kBF16) {
     DecodeFuse<bf16_t> fz{q_weight, k_weight, eps, cos_table, sin_table, rot, nq, write_kv, (bf16_t*)k_pages,
                           (bf16_t*)v_pages};
-    hipLaunchKernelGGL((attention_coop_dma_kernel<bf16_t, kDmaBufsBF16, true>), grid, dim3(256), bytes, s,
+    hipLaunchKernelGGL((attention_coop_kernel<bf16_t, kCoopBufsBF16, true>), grid, dim3(256), bytes, s,
                        (const bf16_t*)qkv, ld, (const bf16_t*)k_pages, (const bf16_t*)v_pages, nkv, page_size,
                        page_shift, table, table_stride, (const SeqMeta*)seqs, (const AttnItem*)items, (bf16_t*)out, ldo,
                        part_acc, part_ml, G, scale, window, fz);
@@ -1902,43 +1625,24 @@ extern "C" int ls_attention(int dtype, const void* q, long ldq, const void* k_pa
   const size_t elem = dtype == kF32 ? 4 : 2;
   const size_t lds_bytes = 2 * (size_t)kTileKeys * D * elem;
   if (variant == 3) {
-    LS_REQUIRE(max_rows <= 16, "attention: the cooperative variant takes work items of at most 16 rows, got %d",
-               max_rows);
-    LS_REQUIRE(coop_supported(dtype), "attention: the cooperative variant does not fit into LDS for this head size");
-    const size_t bytes = coop_lds_bytes(dtype);
-    if (dtype == kF32)
-      hipLaunchKernelGGL((attention_coop_kernel<float, kCoopStageF32>), grid, dim3(256), bytes, s, (const float*)q,
-                         ldq, (const float*)k_pages, (const float*)v_pages, nkv, page_size, page_shift, table,
-                         table_stride, (const SeqMeta*)seqs, (const AttnItem*)items, (float*)out, ldo, part_acc,
-                         part_ml, G, scale, window);
-    else if (dtype == kBF16)
-      hipLaunchKernelGGL((attention_coop_kernel<bf16_t, kCoopStageBF16>), grid, dim3(256), bytes, s,
-                         (const bf16_t*)q, ldq, (const bf16_t*)k_pages, (const bf16_t*)v_pages, nkv, page_size,
-                         page_shift, table, table_stride, (const SeqMeta*)seqs, (const AttnItem*)items, (bf16_t*)out,
-                         ldo, part_acc, part_ml, G, scale, window);
-    else
-      return fail("attention: unknown dtype %d", dtype);
-    return check_launch("attention (cooperative)");
-  }
-  if (variant == 5) {
     LS_REQUIRE(max_rows <= 16, "attention: the cooperative variants take work items of at most 16 rows, got %d",
                max_rows);
-    LS_REQUIRE(coop_dma_supported(dtype), "attention: the streamed cooperative variant does not fit into LDS");
-    LS_REQUIRE(page_size >= 8, "attention: the streamed variants need pages of at least 8 keys, got %d", page_size);
-    const size_t bytes = coop_dma_lds_bytes(dtype);
+    LS_REQUIRE(coop_supported(dtype), "attention: the cooperative variant does not fit into LDS for this head size");
+    LS_REQUIRE(page_size >= 8, "attention: the cooperative variant needs pages of at least 8 keys, got %d", page_size);
+    const size_t bytes = coop_lds_bytes(dtype);
     if (dtype == kF32)
-      hipLaunchKernelGGL((attention_coop_dma_kernel<float, kDmaBufsF32, false>), grid, dim3(256), bytes, s,
+      hipLaunchKernelGGL((attention_coop_kernel<float, kCoopBufsF32, false>), grid, dim3(256), bytes, s,
                          (const float*)q, ldq, (const float*)k_pages, (const float*)v_pages, nkv, page_size,
                          page_shift, table, table_stride, (const SeqMeta*)seqs, (const AttnItem*)items, (float*)out,
                          ldo, part_acc, part_ml, G, scale, window, DecodeFuse<float>{});
     else if (dtype == kBF16)
-      hipLaunchKernelGGL((attention_coop_dma_kernel<bf16_t, kDmaBufsBF16, false>), grid, dim3(256), bytes, s,
+      hipLaunchKernelGGL((attention_coop_kernel<bf16_t, kCoopBufsBF16, false>), grid, dim3(256), bytes, s,
                          (const bf16_t*)q, ldq, (const bf16_t*)k_pages, (const bf16_t*)v_pages, nkv, page_size,
                          page_shift, table, table_stride, (const SeqMeta*)seqs, (const AttnItem*)items, (bf16_t*)out,
                          ldo, part_acc, part_ml, G, scale, window, DecodeFuse<bf16_t>{});
     else
       return fail("attention: unknown dtype %d", dtype);
-    return check_launch("attention (cooperative, streamed)");
+    return check_launch("attention (cooperative)");
   }
   if (variant == 4) {
     LS_REQUIRE(wide_supported(dtype), "attention: the wide variant does not fit into LDS for this head size");

@@ -38,7 +38,6 @@ class AttentionPlan:
     coop_items: torch.Tensor | None
     n_coop: int
     coop_max_rows: int
-    coop_variant: int
     decode_fused: bool        # every request brings one token and the fused decode kernel can take the step
     wide_items: torch.Tensor | None
     n_wide: int
@@ -121,11 +120,7 @@ class StepContext:
             return
         tile, split = self.rt.kernels.attention_geometry(head_dim)
         kernels = self.rt.kernels
-        # rows of decoded tokens: the streamed cooperative kernel, else the cooperative one
-        if kernels.coop_dma_supported(head_dim, self.rt.dtype, self.cache.page_size):
-            coop_ok, coop_variant = True, 5
-        else:
-            coop_ok, coop_variant = kernels.coop_supported(head_dim, self.rt.dtype), 3
+        coop_ok = kernels.coop_supported(head_dim, self.rt.dtype, self.cache.page_size)
         # with a workgroup per CU anyway, one workgroup walks all splits of a request itself
         whole_requests = self.n_seqs * nkv >= 256
         wide_ok = self.rt.kernels.wide_supported(head_dim, self.rt.dtype, self.cache.page_size)
@@ -168,21 +163,21 @@ class StepContext:
                     last_pos = q_start + min((block + 1) * block_rows - 1, rows - 1) // group_size
                     begin = (max(0, first_pos - window + 1) // split) if window > 0 else 0
                     target.append((i, block, begin, last_pos // split + 1, -1, 0, 0, 0))
-        decode_fused = (coop_variant == 5 and not items and not wide and bool((self.q_len == 1).all())
+        decode_fused = (coop_ok and not items and not wide and bool((self.q_len == 1).all())
                         and kernels.decode_fused_supported(head_dim, self.rt.dtype, self.cache.page_size))
         # the longest row blocks first: they decide when the launch ends
         wide.sort(key=lambda it: it[2] - it[3])
         self._plans[key] = (np.asarray(items, dtype=np.int64).reshape(-1),
                             np.asarray(combine, dtype=np.int64).reshape(-1), len(items), len(combine), part_rows,
                             np.asarray(coop, dtype=np.int64).reshape(-1), len(coop), coop_max_rows,
-                            np.asarray(wide, dtype=np.int64).reshape(-1), len(wide), coop_variant, decode_fused)
+                            np.asarray(wide, dtype=np.int64).reshape(-1), len(wide), decode_fused)
         self._plan_specs.append(key)
 
     def upload(self) -> None:
         """Copy all metadata to the device in one transfer."""
         parts = list(self._host_parts)
         for key in self._plan_specs:
-            items, combine, _, _, _, coop, _, _, wide, _, _, _ = self._plans[key]
+            items, combine, _, _, _, coop, _, _, wide, _, _ = self._plans[key]
             parts += [items, combine, coop, wide]
         flat = np.concatenate(parts).astype(np.int32)
         host = torch.from_numpy(flat)
@@ -203,7 +198,7 @@ class StepContext:
         self._device_plans: dict[tuple, AttentionPlan] = {}
         for key in self._plan_specs:
             (items, combine, n_items, n_combine, part_rows, coop, n_coop, coop_max_rows, wide, n_wide,
-             coop_variant, decode_fused) = self._plans[key]
+             decode_fused) = self._plans[key]
             head_dim = key[2]
             d_items, d_combine, d_coop = take(items.shape[0]), take(combine.shape[0]), take(coop.shape[0])
             d_wide = take(wide.shape[0])
@@ -212,7 +207,7 @@ class StepContext:
                 part_acc = self.workspace.get(f"attention.part_acc.{head_dim}", (part_rows, head_dim), torch.float32)
                 part_ml = self.workspace.get("attention.part_ml", (part_rows, 2), torch.float32)
             self._device_plans[key] = AttentionPlan(d_items, n_items, d_coop if n_coop else None, n_coop,
-                                                    coop_max_rows, coop_variant, decode_fused,
+                                                    coop_max_rows, decode_fused,
                                                     d_wide if n_wide else None, n_wide,
                                                     d_combine if n_combine else None,
                                                     n_combine, part_acc, part_ml)

@@ -88,14 +88,10 @@ class Kernels:
             self.attention_paths[head_dim] = str(path)
         return lib
 
-    def coop_supported(self, head_dim: int, dtype: torch.dtype) -> bool:
+    def coop_supported(self, head_dim: int, dtype: torch.dtype, page_size: int = 16) -> bool:
         """Whether the cooperative attention kernel can run (its tiles must fit into LDS)."""
-        return bool(self.attention_lib(head_dim).ls_attn_coop_supported(c_int(DTYPE_CODE[dtype])))
-
-    def coop_dma_supported(self, head_dim: int, dtype: torch.dtype, page_size: int) -> bool:
-        """Whether the streamed cooperative attention kernel (variant 5) can run."""
         lib = self.attention_lib(head_dim)
-        return page_size >= 8 and bool(lib.ls_attn_coop_dma_supported(c_int(DTYPE_CODE[dtype])))
+        return page_size >= 8 and bool(lib.ls_attn_coop_supported(c_int(DTYPE_CODE[dtype])))
 
     def decode_fused_supported(self, head_dim: int, dtype: torch.dtype, page_size: int) -> bool:
         """Whether ``attention_decode`` (norm, rotation and cache write inside the attention kernel) can run."""
@@ -269,8 +265,7 @@ class Kernels:
         """Launch the attention kernel over ``n_items`` work items (see attention.hip).
         ``variant``: 0 staged through LDS where it fits, 1 direct from global memory, 2 staged or
         error, 3 cooperative (every item has at most 16 rows; ``max_rows`` states the largest),
-        4 wide (tiles loaded straight into LDS; items count row blocks of ``attention_block_rows``),
-        5 cooperative with tiles loaded straight into LDS (same items as 3)."""
+        4 wide (prompt portions; items count row blocks of ``attention_block_rows``)."""
         lib = self.attention_lib(d)
         _rows_ok(q, "attention q"); _rows_ok(out, "attention out")
         _need(q.dtype in DTYPE_CODE and out.dtype == q.dtype, "attention q/out dtype")

@@ -138,7 +138,7 @@ class Attention(Mixer):
         if plan.n_coop:
             k.attention(qkv, nq, nkv, d, key_pages, value_pages, group.page_size, group.table, ctx.seqs,
                         plan.coop_items, plan.n_coop, attn, plan.part_acc, plan.part_ml, self.scale, window,
-                        variant=plan.coop_variant, max_rows=plan.coop_max_rows)
+                        variant=3, max_rows=plan.coop_max_rows)
         if plan.n_wide:
             k.attention(qkv, nq, nkv, d, key_pages, value_pages, group.page_size, group.table, ctx.seqs,
                         plan.wide_items, plan.n_wide, attn, plan.part_acc, plan.part_ml, self.scale, window,

@@ -316,14 +316,10 @@ def test_attention_row_is_the_same_alone_in_a_portion_and_in_the_whole_prompt(dt
         assert torch.equal(alone[0], full[p]), f"row {p} alone"
         alone = whole.attend(qkv[p:p + 1], p, d ** -0.5, variant=1)
         assert torch.equal(alone[0], full[p]), f"row {p} alone, loaded directly"
-        if K().coop_supported(d, dtype):
+        if K().coop_supported(d, dtype, ps):
             for split in (True, False):
                 alone = whole.attend(qkv[p:p + 1], p, d ** -0.5, variant=3, force_split=split)
                 assert torch.equal(alone[0], full[p]), f"row {p} alone, cooperative kernel, split={split}"
-        if K().coop_dma_supported(d, dtype, ps):
-            for split in (True, False):
-                alone = whole.attend(qkv[p:p + 1], p, d ** -0.5, variant=5, force_split=split)
-                assert torch.equal(alone[0], full[p]), f"row {p} alone, streamed cooperative kernel, split={split}"
         both = whole.attend(qkv[p:p + 1], p, d ** -0.5, force_split=False)
         assert torch.equal(both[0], full[p]), f"row {p} alone, direct"
     for lo, hi in ((250, 262), (0, 3), (500, 700), (255, 257), (690, 700)):
@@ -365,10 +361,6 @@ def test_attention_window(dtype, window):
         case.table.copy_(saved)
         assert torch.equal(alone[0], out[p]), f"row {p}"
         assert torch.equal(coop[0], out[p]), f"row {p}, cooperative kernel"
-        case.table[1, :first_needed] = -1
-        dma = case.attend(dev[p:p + 1], p, d ** -0.5, window=window, variant=5)
-        case.table.copy_(saved)
-        assert torch.equal(dma[0], out[p]), f"row {p}, streamed cooperative kernel"
         assert torch.equal(wide, out[lo:p + 1]), f"rows {lo}..{p}, wide kernel"
 
 
@@ -435,12 +427,10 @@ def test_decode_attention_is_the_same_in_every_kernel(dtype, nq, nkv, d, ps):
         ref = case.attend(dev[start:start + n], start, d ** -0.5, variant=1, force_split=False)
         assert rel_err(ref, want[start:start + n]) < ATT_TOL[dtype], (start, n)
         variants = [(0, True), (0, False), (1, True)]
-        if K().coop_supported(d, dtype):
+        if K().coop_supported(d, dtype, ps):
             variants += [(3, True), (3, False)]
         if K().wide_supported(d, dtype, ps):
             variants += [(4, True), (4, False)]
-        if K().coop_dma_supported(d, dtype, ps):
-            variants += [(5, True), (5, False)]
         for variant, split in variants:
             got = case.attend(dev[start:start + n], start, d ** -0.5, variant=variant, force_split=split)
             assert torch.equal(got, ref), f"start={start} n={n} variant={variant} split={split}"
@@ -480,7 +470,7 @@ def test_fused_decode_attention_equals_the_separate_kernels(dtype, nq, nkv, d, p
         # separate kernels
         row = qkv[p:p + 1].clone()
         base.write(row, p, qw, kw, eps, cos, sin, rot)
-        want = base.attend(row, p, d ** -0.5, window=window, variant=5)
+        want = base.attend(row, p, d ** -0.5, window=window, variant=3)
         k_want, v_want = base.k_pages.clone(), base.v_pages.clone()
         for use_split in (True, False):
             base.k_pages.copy_(k0); base.v_pages.copy_(v0)
