@@ -985,7 +985,7 @@ __global__ __launch_bounds__(64 * NW) void attention_wide_kernel(
 // key heads, value heads in a row); the workgroup normalises and rotates its
 // query heads into LDS, and the workgroup whose tiles hold the new position
 // does the same for the new key, writes key and value to the cache pages and
-// patches them into its LDS tile.  Each head goes through head_norm_rope, as
+// patches them into its LDS tile.  Each head goes through head16_finish, as
 // in the stand-alone kernel, so the bits are the same.
 template <typename T>
 struct DecodeFuse {
@@ -1132,62 +1132,69 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
   const int n_vec = owner ? G + 2 : G;
   const T* new_row = q + (long)sm.q_off * ldq;
   const bool rotated = FUSE && fz.cos_table != nullptr;
+  // Sixteen lanes a head (head16_finish): the workgroup's sixteen groups take the heads vi = group, group + 16.
+  constexpr int PASSES = D > 128 ? 2 : 1;
+  const int gl = threadIdx.x & 15;
+  const int grp = threadIdx.x >> 4;
   long page_new = -1;
-  HeadVec hv;
+  float hx[8 * PASSES];
+  HeadFactors<PASSES> hf;
   auto head_src = [&](int vi) -> const T* {
     return new_row + (long)(vi < G ? kvh * G + vi : vi == G ? fz.nq + kvh : fz.nq + nkv + kvh) * D;
   };
   auto head_fetch = [&](int vi) {
+    head16_load_values<T, PASSES>(hx, head_src(vi), D, gl);
     if (vi <= G)
-      head_load<T>(hv, head_src(vi), D, vi < G ? fz.q_weight : fz.k_weight, fz.cos_table, fz.sin_table, p_new,
-                   fz.rot, lane);
-    else
-      head_load<T>(hv, head_src(vi), D, nullptr, nullptr, nullptr, 0, 0, lane);
+      head16_load_factors<PASSES>(hf, D, vi < G ? fz.q_weight : fz.k_weight, fz.cos_table, fz.sin_table, p_new,
+                                  fz.rot, gl);
   };
   if (FUSE) {
     if (owner) page_new = tbl[p_new >> page_shift];
-    if (wave < n_vec) head_fetch(wave);
+    if (grp < n_vec) head_fetch(grp);
   }
   if (ti_lo < ti_hi && (int)threadIdx.x < pages_per_tile) tile_pages[(ti_lo & 1) * 16 + threadIdx.x] = first_page;
   __syncthreads();
-  PROBE(1)
   if (ti_lo < ti_hi) {
     issue(ti_lo);
     if (ti_lo + 1 < ti_hi && (int)threadIdx.x < pages_per_tile) held = table_entry(ti_lo + 1);
   }
-  PROBE(2)
   if (FUSE) {
-    float* ystage = reinterpret_cast<float*>(prob) + wave * D;               // the exchange buffers are free until the loop
-    T* qrot = reinterpret_cast<T*>(reinterpret_cast<float*>(prob) + 4 * D);  // [16][D]
+    T* qrot = reinterpret_cast<T*>(prob);  // [16][D]: the exchange buffers are free until the loop
     const int slot_new = p_new & (page_size - 1);
-    for (int vi = wave; vi < n_vec; vi += 4) {  // uniform for the wave
-      if (vi != wave) head_fetch(vi);
+    for (int vi = grp; vi < n_vec; vi += 16) {  // uniform for the group
+      if (vi != grp) head_fetch(vi);
       if (vi < G) {
-        head_finish<T>(hv, D, fz.q_weight != nullptr, fz.eps, rotated, fz.rot, ystage, lane,
-                       [&](int e, T v) { qrot[vi * D + e] = v; });
+        head16_finish<T, PASSES>(hx, hf, D, fz.q_weight != nullptr, fz.eps, rotated, fz.rot, gl,
+                                 [&](int e0, const T (&v)[8]) { store8<T>(qrot + vi * D + e0, v); });
       } else if (vi == G) {
         T* dst = fz.k_out + ((max(page_new, 0L) * nkv + kvh) * page_size + slot_new) * D;
-        head_finish<T>(hv, D, fz.k_weight != nullptr, fz.eps, rotated, fz.rot, ystage, lane, [&](int e, T v) {
-          knew[e] = v;
-          if (page_new >= 0) dst[e] = v;
-        });
+        head16_finish<T, PASSES>(hx, hf, D, fz.k_weight != nullptr, fz.eps, rotated, fz.rot, gl,
+                                 [&](int e0, const T (&v)[8]) {
+                                   store8<T>(knew + e0, v);
+                                   if (page_new >= 0) store8<T>(dst + e0, v);
+                                 });
       } else {
         T* dst = fz.v_out + ((max(page_new, 0L) * nkv + kvh) * D) * page_size + slot_new;
-        head_finish<T>(hv, D, false, 0.f, false, 0, ystage, lane, [&](int e, T v) {
-          vnew[e] = v;
-          if (page_new >= 0) dst[(long)e * page_size] = v;
-        });
+#pragma unroll
+        for (int p = 0; p < PASSES; ++p) {
+          const int e0 = 128 * p + 8 * gl;
+          if (e0 >= D) continue;
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            const T v = from_f32<T>(hx[8 * p + j]);
+            vnew[e0 + j] = v;
+            if (page_new >= 0) dst[(long)(e0 + j) * page_size] = v;
+          }
+        }
       }
     }
     __syncthreads();
-    const T* qr = qrot;
 #pragma unroll
     for (int c = 0; c < NC; ++c) {
       const int col = c * A::KCHUNK + g * VEC;
-      qv[c] = (row_ok && col < D) ? *reinterpret_cast<const vec_t*>(qr + row16 * D + min(col, D - VEC)) : A::zero();
+      qv[c] = (row_ok && col < D) ? *reinterpret_cast<const vec_t*>(qrot + row16 * D + min(col, D - VEC)) : A::zero();
     }
   }
-  PROBE(3)
   for (int ti = ti_lo; ti < ti_hi; ++ti) {
     const int t0 = ti * kTileKeys;
     const unsigned char* k_lds = lds + (NBUF == 2 ? (ti & 1) : 0) * BUF_BYTES;
@@ -1499,10 +1506,10 @@ static bool coop_supported(int dtype) {
 extern "C" int ls_attn_coop_supported(int dtype) { return coop_supported(dtype) ? 1 : 0; }
 
 // The fused decode step (FUSE) stages the rotated query heads in the exchange
-// buffers before the loop needs them: 4 rows of D floats and 16 rows of D elements.
+// buffers before the loop needs them: 16 rows of D elements.
 static bool decode_fused_supported(int dtype) {
   const size_t elem = dtype == kF32 ? 4 : 2;
-  if (4 * D * 4 + 16 * D * elem > (size_t)NB * 64 * 16) return false;
+  if (16 * D * elem > (size_t)NB * 64 * 16) return false;
   const size_t bytes = coop_lds_bytes(dtype);
   if (bytes > kLdsLimit) return false;
   if (bytes <= 64 * 1024) return true;
@@ -1545,7 +1552,13 @@ extern "C" int ls_attention_decode(int dtype, const void* qkv, long ld, void* k_
   LS_REQUIRE(reinterpret_cast<uintptr_t>(qkv) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0 &&
                  reinterpret_cast<uintptr_t>(k_pages) % 16 == 0 && reinterpret_cast<uintptr_t>(v_pages) % 16 == 0,
              "decode attention: operands must be 16-byte aligned");
-  LS_REQUIRE(rot >= 0 && rot <= D && rot % 2 == 0, "decode attention: rotary_dim %d must be even and at most %d", rot, D);
+  LS_REQUIRE(rot >= 0 && head16_supported(D, rot), "decode attention: rotary_dim %d must be even and at most %d",
+             rot, D);
+  LS_REQUIRE((!q_weight || reinterpret_cast<uintptr_t>(q_weight) % 16 == 0) &&
+                 (!k_weight || reinterpret_cast<uintptr_t>(k_weight) % 16 == 0) &&
+                 (!cos_table || (reinterpret_cast<uintptr_t>(cos_table) % 16 == 0 &&
+                                 reinterpret_cast<uintptr_t>(sin_table) % 16 == 0)),
+             "decode attention: norm weights and rotation tables must be 16-byte aligned");
   LS_REQUIRE(!cos_table || (sin_table && table_positions > max_pos),
              "decode attention: rotation tables hold %d positions, the step reaches %d", table_positions, max_pos);
   LS_REQUIRE(decode_fused_supported(dtype), "decode attention: the fused kernel does not fit into LDS for this head size");

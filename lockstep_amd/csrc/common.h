@@ -142,87 +142,174 @@ __device__ __forceinline__ float row_sumsq_part(const float* __restrict__ src, i
   return part;
 }
 
-// One head of one token: optional RMSNorm over the head (weight != nullptr),
-// then the half-split rotation of its first `rot` elements.  One wave runs it
-// in two phases, so that a caller can put other loads between them:
-// head_load brings the lane's elements (e = lane, lane + 64, ...), their norm
-// weights and rotation factors into registers; head_finish does the
-// arithmetic and hands the results to `dst(e, value)`.  `y` is an LDS row of
-// d floats private to the wave.  The sum of squares: lane l adds x[l]^2,
-// x[l+64]^2, ... ascending, then a butterfly over the wave.  Every kernel
-// that normalises a head goes through these two, so a head has the same bits
-// wherever it is processed.
+// One head of one token: optional RMSNorm over the head, then the half-split
+// rotation of its first `rot` elements.  Sixteen neighbouring lanes (a group)
+// process a head; lane i of the group holds the elements [8i, 8i + 8) and, for
+// heads of more than 128 elements (PASSES == 2), also [128 + 8i, 128 + 8i + 8),
+// so that values, weights and rotation factors move as 16-byte vectors and no
+// LDS is needed.  The sum of squares: a lane adds its squares in ascending
+// order of the element, then the group adds over the lanes i+8, i+4, i+2,
+// i+1 (mod 16), which leaves the same bits in all of its lanes.  The partner
+// of the rotation, half = rot/2 elements away, is fetched from its lane by a
+// shuffle (one per element where half is a multiple of 8, a slower gather
+// otherwise).  Every
+// kernel that normalises a head goes through these functions, so a head has
+// the same bits wherever it is processed.
 constexpr int kMaxHeadDim = 256;
-constexpr int kHeadPerLane = kMaxHeadDim / 64;
-struct HeadVec {
-  float x[kHeadPerLane], w[kHeadPerLane], c[kHeadPerLane], s[kHeadPerLane];
+
+__host__ __device__ inline bool head16_supported(int d, int rot) {
+  return d % 8 == 0 && d <= kMaxHeadDim && rot % 2 == 0 && rot <= d;
+}
+
+template <int PASSES>
+struct HeadFactors {  // what does not depend on the head's values
+  float w[8 * PASSES], c[8 * PASSES], s[8 * PASSES];
 };
 
-template <typename T>
-__device__ __forceinline__ void head_load(HeadVec& h, const T* src, int d, const float* __restrict__ weight,
-                                          const float* __restrict__ cos_table, const float* __restrict__ sin_table,
-                                          int pos, int rot, int lane) {
+template <int N>
+__device__ __forceinline__ void load_floats8(float* dst, const float* __restrict__ src, bool ok, float fill) {
+  if (ok) {
+    const f32x4 lo = *reinterpret_cast<const f32x4*>(src);
+    const f32x4 hi = *reinterpret_cast<const f32x4*>(src + 4);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      dst[j] = lo[j];
+      dst[4 + j] = hi[j];
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) dst[j] = fill;
+  }
+}
+
+// gl: the lane's index in its group of 16.  weight / tables may be nullptr.
+template <int PASSES>
+__device__ __forceinline__ void head16_load_factors(HeadFactors<PASSES>& f, int d, const float* __restrict__ weight,
+                                                    const float* __restrict__ cos_table,
+                                                    const float* __restrict__ sin_table, int pos, int rot, int gl) {
   const int half = rot / 2;
 #pragma unroll
-  for (int i = 0; i < kHeadPerLane; ++i) {
-    const int e = lane + 64 * i;
-    const bool in = e < d;
-    h.x[i] = in ? to_f32(src[e]) : 0.f;
-    h.w[i] = (weight && in) ? weight[e] : 1.f;
-    h.c[i] = 1.f;
-    h.s[i] = 0.f;
-    if (cos_table && e < rot) {
-      const int idx = e < half ? e : e - half;
-      h.c[i] = cos_table[(long)pos * half + idx];
-      h.s[i] = sin_table[(long)pos * half + idx];
+  for (int p = 0; p < PASSES; ++p) {
+    const int e0 = 128 * p + 8 * gl;
+    load_floats8<8>(f.w + 8 * p, weight + (weight ? e0 : 0), weight != nullptr && e0 < d, 1.f);
+    if ((half & 7) == 0) {  // uniform: a run of eight lies on one side of the half
+      const bool turn = cos_table != nullptr && e0 < rot;
+      const int idx = e0 < half ? e0 : e0 - half;
+      const long at = turn ? (long)pos * half + idx : 0;
+      load_floats8<8>(f.c + 8 * p, cos_table + at, turn, 1.f);
+      load_floats8<8>(f.s + 8 * p, sin_table + at, turn, 0.f);
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int e = e0 + j;
+        const bool turn = cos_table != nullptr && e < rot;
+        const long at = turn ? (long)pos * half + (e < half ? e : e - half) : 0;
+        f.c[8 * p + j] = turn ? cos_table[at] : 1.f;
+        f.s[8 * p + j] = turn ? sin_table[at] : 0.f;
+      }
     }
   }
 }
 
-template <typename T, typename Dst>
-__device__ __forceinline__ void head_finish(const HeadVec& h, int d, bool normed, float eps, bool rotated, int rot,
-                                            float* __restrict__ y, int lane, Dst dst) {
+// src: the head's first element; 16-byte aligned.
+template <typename T, int PASSES>
+__device__ __forceinline__ void head16_load_values(float (&x)[8 * PASSES], const T* src, int d, int gl) {
+#pragma unroll
+  for (int p = 0; p < PASSES; ++p) {
+    const int e0 = 128 * p + 8 * gl;
+    if (e0 < d) {
+      if (sizeof(T) == 2) {
+        const bf16x8 v = *reinterpret_cast<const bf16x8*>(src + e0);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) x[8 * p + j] = to_f32(v[j]);
+      } else {
+        load_floats8<8>(x + 8 * p, reinterpret_cast<const float*>(src) + e0, true, 0.f);
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) x[8 * p + j] = 0.f;
+    }
+  }
+}
+
+// Value of `v` in lane `from` (0..15) of the caller's group.
+__device__ __forceinline__ float group16_get(float v, int from) {
+  return __shfl(v, (threadIdx.x & 48) | from, kWave);
+}
+
+// dst(e0, vals): called for each run of eight finished elements [e0, e0 + 8) of the head.
+template <typename T, int PASSES, typename Dst>
+__device__ __forceinline__ void head16_finish(const float (&x)[8 * PASSES], const HeadFactors<PASSES>& f, int d,
+                                              bool normed, float eps, bool rotated, int rot, int gl, Dst dst) {
+  float y[8 * PASSES];
   float part = 0.f;
 #pragma unroll
-  for (int i = 0; i < kHeadPerLane; ++i) {
-    const int e = lane + 64 * i;
-    if (e < d) {
-      y[e] = h.x[i];
-      part = part + h.x[i] * h.x[i];
-    }
-  }
+  for (int i = 0; i < 8 * PASSES; ++i) part = part + x[i] * x[i];  // elements past d are zeros
   if (normed) {
-    const float total = wave_sum(part);
-    const float scale = 1.0f / sqrtf(total / (float)d + eps);
 #pragma unroll
-    for (int i = 0; i < kHeadPerLane; ++i) {
-      const int e = lane + 64 * i;
-      if (e < d) y[e] = (h.x[i] * scale) * h.w[i];
-    }
+    for (int k = 8; k > 0; k >>= 1) part = part + group16_get(part, (gl + k) & 15);
+    const float scale = 1.0f / sqrtf(part / (float)d + eps);
+#pragma unroll
+    for (int i = 0; i < 8 * PASSES; ++i) y[i] = (x[i] * scale) * f.w[i];
+  } else {
+#pragma unroll
+    for (int i = 0; i < 8 * PASSES; ++i) y[i] = x[i];
   }
-  // The staging row is private to this wave: order its writes before the
-  // reads of other lanes without a workgroup barrier.
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-  __builtin_amdgcn_wave_barrier();
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
   const int half = rot / 2;
+  const bool run_aligned = (half & 7) == 0;  // uniform
 #pragma unroll
-  for (int i = 0; i < kHeadPerLane; ++i) {
-    const int e = lane + 64 * i;
-    if (e >= d) continue;
-    float v = y[e];
-    if (rotated && e < rot) {
-      const int idx = e < half ? e : e - half;
-      const float lo = y[idx];
-      const float hi = y[idx + half];
-      v = e < half ? lo * h.c[i] - hi * h.s[i] : hi * h.c[i] + lo * h.s[i];
+  for (int p = 0; p < PASSES; ++p) {
+    const int e0 = 128 * p + 8 * gl;
+    T out[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int e = e0 + j;
+      float v = y[8 * p + j];
+      if (rotated) {  // uniform
+        // the partner lies half elements above (for the lower half) or below
+        const bool lower = e < half;
+        const int partner = lower ? e + half : e - half;
+        const int from_lane = (partner & 127) >> 3;
+        const int from_pass = e < rot ? partner >> 7 : 0;
+        float other = 0.f;
+        if (run_aligned) {  // the partner has the same place j in its lane's run
+          other = group16_get(y[j], from_lane);
+          if (PASSES == 2) {
+            const float other1 = group16_get(y[8 + j], from_lane);
+            other = from_pass ? other1 : other;
+          }
+        } else {
+#pragma unroll
+          for (int k = 0; k < 8 * PASSES; ++k) {
+            const float cand = group16_get(y[k], from_lane);
+            other = (k == 8 * from_pass + (partner & 7)) ? cand : other;
+          }
+        }
+        if (e < rot) {
+          const float lo = lower ? v : other;
+          const float hi = lower ? other : v;
+          v = lower ? lo * f.c[8 * p + j] - hi * f.s[8 * p + j] : hi * f.c[8 * p + j] + lo * f.s[8 * p + j];
+        }
+      }
+      out[j] = from_f32<T>(v);
     }
-    dst(e, from_f32<T>(v));
+    if (e0 < d) dst(e0, out);
   }
-  // the row may be reused by the caller for its next head
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-  __builtin_amdgcn_wave_barrier();
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// Store eight elements at a 16-byte aligned address.
+template <typename T>
+__device__ __forceinline__ void store8(T* at, const T (&v)[8]) {
+  if (sizeof(T) == 2) {
+    bf16x8 w;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) w[j] = v[j];
+    *reinterpret_cast<bf16x8*>(at) = w;
+  } else {
+    float* p = reinterpret_cast<float*>(at);
+    *reinterpret_cast<f32x4*>(p) = f32x4{(float)v[0], (float)v[1], (float)v[2], (float)v[3]};
+    *reinterpret_cast<f32x4*>(p + 4) = f32x4{(float)v[4], (float)v[5], (float)v[6], (float)v[7]};
+  }
 }
 
 }  // namespace ls

@@ -40,13 +40,57 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ 
   const int r_out = blockIdx.x;
   const long r_in = rows ? rows[r_out] : r_out;
   const float* src = x + r_in * ldx;
+  T* dst = out + (long)r_out * ld_out;
   const bool vec_ok = (ldx & 3) == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0;
+  // Rows of up to 4,096 elements stay in registers between the two passes, and their weights are
+  // requested before the reduction, so the kernel waits for memory once.  The sum is row_sumsq_part's.
+  constexpr int KEEP = 4;
+  const bool fast = vec_ok && width <= KEEP * 1024 && (width & 3) == 0 &&
+                    (reinterpret_cast<uintptr_t>(weight) & 15) == 0 && (ld_out & 3) == 0 &&
+                    (reinterpret_cast<uintptr_t>(out) & (4 * sizeof(T) - 1)) == 0;
+  if (fast) {
+    f32x4 v[KEEP], w[KEEP];
+    float part = 0.f;
+#pragma unroll
+    for (int c = 0; c < KEEP; ++c) {
+      const int base = 1024 * c + 4 * (int)threadIdx.x;
+      const bool in = base < width;
+      v[c] = in ? *reinterpret_cast<const f32x4*>(src + base) : f32x4{0.f, 0.f, 0.f, 0.f};
+      w[c] = in ? *reinterpret_cast<const f32x4*>(weight + base) : f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+#pragma unroll
+    for (int c = 0; c < KEEP; ++c)
+      if (1024 * c + 4 * (int)threadIdx.x < width) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) part = part + v[c][e] * v[c][e];
+      }
+    part = wave_sum(part);
+    if ((threadIdx.x & 63) == 0) wave_part[threadIdx.x >> 6] = part;
+    __syncthreads();
+    const float total = ((wave_part[0] + wave_part[1]) + wave_part[2]) + wave_part[3];
+    const float scale = 1.0f / sqrtf(total / (float)width + eps);
+#pragma unroll
+    for (int c = 0; c < KEEP; ++c) {
+      const int base = 1024 * c + 4 * (int)threadIdx.x;
+      if (base >= width) continue;
+      float o[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) o[e] = (v[c][e] * scale) * w[c][e];
+      if (sizeof(T) == 2) {
+        bf16x4 b;
+        b[0] = (bf16_t)o[0]; b[1] = (bf16_t)o[1]; b[2] = (bf16_t)o[2]; b[3] = (bf16_t)o[3];
+        *reinterpret_cast<bf16x4*>(dst + base) = b;
+      } else {
+        *reinterpret_cast<f32x4*>(dst + base) = f32x4{o[0], o[1], o[2], o[3]};
+      }
+    }
+    return;
+  }
   float part = wave_sum(row_sumsq_part(src, width, threadIdx.x, vec_ok));
   if ((threadIdx.x & 63) == 0) wave_part[threadIdx.x >> 6] = part;
   __syncthreads();
   const float total = ((wave_part[0] + wave_part[1]) + wave_part[2]) + wave_part[3];
   const float scale = 1.0f / sqrtf(total / (float)width + eps);
-  T* dst = out + (long)r_out * ld_out;
   for (int e = threadIdx.x; e < width; e += 256) dst[e] = from_f32<T>((src[e] * scale) * weight[e]);
 }
 
@@ -71,48 +115,67 @@ struct SeqMeta {  // one per sequence of the step (all int32)
   int reserved[3];
 };
 
-template <typename T>
+template <typename T, int PASSES>
 __global__ __launch_bounds__(256) void qk_rope_kv_kernel(
     T* __restrict__ qkv, long ld, int nq, int nkv, int d, const float* __restrict__ q_weight,
     const float* __restrict__ k_weight, float eps, const float* __restrict__ cos_table,
     const float* __restrict__ sin_table, int rot, const int* __restrict__ tok_seq, const int* __restrict__ tok_pos,
     const SeqMeta* __restrict__ seqs, const int* __restrict__ table, int table_stride, T* __restrict__ k_pages,
-    T* __restrict__ v_pages, int page_size, int write_kv) {
-  __shared__ float stage[4][kMaxHeadDim];
-  const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
-  const int t = blockIdx.x;
-  const int head = blockIdx.y * 4 + wave;
-  const int heads = write_kv ? nq + 2 * nkv : nq;
-  if (head >= heads) return;
-
-  T* src = qkv + (long)t * ld + (long)head * d;
-  const int pos = tok_pos[t];
-  const bool is_q = head < nq;
-  const bool is_k = !is_q && head < nq + nkv;
-
-  long page = 0;
-  int slot = 0;
-  if (!is_q) {
+    T* __restrict__ v_pages, int page_size, int write_kv, int n_tokens) {
+  const int head_blocks = (int)(((long)n_tokens * (write_kv ? nq + nkv : nq) + 15) / 16);
+  if ((int)blockIdx.x >= head_blocks) {
+    // Values: a workgroup copies 16 consecutive tokens of the batch.  Sixteen neighbouring lanes
+    // hold the same column of 16 tokens, so where the tokens are neighbours in a page their
+    // 2-byte elements leave as whole 32-byte runs of the transposed page.
+    // A workgroup takes 64 columns of its 16 tokens: four loads a thread, all in flight together.
+    const int width = nkv * d;  // the value heads of a token are contiguous; so are the rows of a page
+    const int col_blocks = (width + 63) / 64;
+    const int vb = (int)blockIdx.x - head_blocks;
+    const int j = threadIdx.x & 15;
+    const int t = (vb / col_blocks) * 16 + j;
+    if (t >= n_tokens) return;
+    const int pos = tok_pos[t];
     const SeqMeta sm = seqs[tok_seq[t]];
-    page = table[(long)sm.table_row * table_stride + pos / page_size];
-    slot = pos % page_size;
-    if (page < 0) return;  // the host never schedules a write to a page it does not hold
-  }
-
-  if (!is_q && !is_k) {
-    const int kvh = head - nq - nkv;
-    T* dst = v_pages + ((page * nkv + kvh) * d) * page_size + slot;
-    for (int e = lane; e < d; e += 64) dst[(long)e * page_size] = src[e];
+    const long page = table[(long)sm.table_row * table_stride + pos / page_size];
+    if (page < 0) return;
+    const int slot = pos % page_size;
+    const T* src = qkv + (long)t * ld + (long)(nq + nkv) * d;
+    T* dst = v_pages + page * nkv * d * page_size + slot;
+    const int c0 = (vb % col_blocks) * 64 + (threadIdx.x >> 4);
+    T v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) v[u] = src[min(c0 + 16 * u, width - 1)];
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (c0 + 16 * u < width) dst[(long)(c0 + 16 * u) * page_size] = v[u];
     return;
   }
-
+  // Query and key heads: sixteen lanes a head (see head16_finish), sixteen heads a workgroup.
+  const int heads = write_kv ? nq + nkv : nq;  // the value heads are copied by the workgroups above
+  const int gl = threadIdx.x & 15;
+  const long gid = (long)blockIdx.x * 16 + (threadIdx.x >> 4);
+  if (gid >= (long)n_tokens * heads) return;  // the whole group leaves
+  const int t = (int)(gid / heads);
+  const int head = (int)(gid % heads);
+  const bool is_q = head < nq;
+  T* src = qkv + (long)t * ld + (long)head * d;
+  const int pos = tok_pos[t];
+  T* dst = src;
+  bool held = true;
+  if (!is_q) {
+    const SeqMeta sm = seqs[tok_seq[t]];
+    const long page = table[(long)sm.table_row * table_stride + pos / page_size];
+    held = page >= 0;  // the host never schedules a write to a page it does not hold
+    dst = k_pages + ((max(page, 0L) * nkv + (head - nq)) * page_size + pos % page_size) * d;
+  }
   const float* weight = is_q ? q_weight : k_weight;
-  T* dst = is_q ? src : k_pages + ((page * nkv + (head - nq)) * page_size + slot) * d;
-  HeadVec hv;
-  head_load<T>(hv, src, d, weight, cos_table, sin_table, pos, rot, lane);
-  head_finish<T>(hv, d, weight != nullptr, eps, cos_table != nullptr, rot, stage[wave], lane,
-                 [&](int e, T v) { dst[e] = v; });
+  float x[8 * PASSES];
+  HeadFactors<PASSES> f;
+  head16_load_values<T, PASSES>(x, src, d, gl);
+  head16_load_factors<PASSES>(f, d, weight, cos_table, sin_table, pos, rot, gl);
+  head16_finish<T, PASSES>(x, f, d, weight != nullptr, eps, cos_table != nullptr, rot, gl, [&](int e0, const T (&v)[8]) {
+    if (held) store8<T>(dst + e0, v);
+  });
 }
 
 // ---------------------------------------------------------------------------
@@ -266,17 +329,32 @@ extern "C" int ls_qk_rope_kv(int dtype, void* qkv, long ld, int n_tokens, int nq
   LS_REQUIRE(ld >= (long)heads * d, "qk_rope_kv: row stride %ld shorter than %d heads of %d", ld, heads, d);
   LS_REQUIRE(!write_kv || (k_pages && v_pages && table && page_size > 0), "qk_rope_kv: cache operands missing");
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-  dim3 grid(n_tokens, (heads + 3) / 4);
-  if (dtype == kF32)
-    hipLaunchKernelGGL(qk_rope_kv_kernel<float>, grid, dim3(256), 0, s, (float*)qkv, ld, nq, nkv, d, q_weight,
-                       k_weight, eps, cos_table, sin_table, rot, tok_seq, tok_pos, (const SeqMeta*)seqs, table,
-                       table_stride, (float*)k_pages, (float*)v_pages, page_size, write_kv);
-  else if (dtype == kBF16)
-    hipLaunchKernelGGL(qk_rope_kv_kernel<bf16_t>, grid, dim3(256), 0, s, (bf16_t*)qkv, ld, nq, nkv, d, q_weight,
-                       k_weight, eps, cos_table, sin_table, rot, tok_seq, tok_pos, (const SeqMeta*)seqs, table,
-                       table_stride, (bf16_t*)k_pages, (bf16_t*)v_pages, page_size, write_kv);
-  else
+  LS_REQUIRE(head16_supported(d, rot), "qk_rope_kv: head_dim %d must be a multiple of 8 up to %d and rotary_dim %d even and "
+             "at most head_dim", d, kMaxHeadDim, rot);
+  const size_t elem = dtype == kF32 ? 4 : 2;
+  LS_REQUIRE(reinterpret_cast<uintptr_t>(qkv) % 16 == 0 && (ld * elem) % 16 == 0 && (d * elem) % 16 == 0 &&
+                 (!write_kv || reinterpret_cast<uintptr_t>(k_pages) % 16 == 0),
+             "qk_rope_kv: rows, heads and pages must be 16-byte aligned (ld=%ld, head_dim=%d)", ld, d);
+  LS_REQUIRE((!q_weight || reinterpret_cast<uintptr_t>(q_weight) % 16 == 0) &&
+                 (!k_weight || reinterpret_cast<uintptr_t>(k_weight) % 16 == 0) &&
+                 (!cos_table || (reinterpret_cast<uintptr_t>(cos_table) % 16 == 0 &&
+                                 reinterpret_cast<uintptr_t>(sin_table) % 16 == 0)),
+             "qk_rope_kv: norm weights and rotation tables must be 16-byte aligned");
+  const long head_blocks = ((long)n_tokens * (write_kv ? nq + nkv : nq) + 15) / 16;
+  const long value_blocks = write_kv ? (long)((n_tokens + 15) / 16) * (((long)nkv * d + 63) / 64) : 0;
+  dim3 grid((unsigned)(head_blocks + value_blocks));
+#define LS_ROPE(T_, P_)                                                                                            \
+  hipLaunchKernelGGL((qk_rope_kv_kernel<T_, P_>), grid, dim3(256), 0, s, (T_*)qkv, ld, nq, nkv, d, q_weight, k_weight, \
+                     eps, cos_table, sin_table, rot, tok_seq, tok_pos, (const SeqMeta*)seqs, table, table_stride,   \
+                     (T_*)k_pages, (T_*)v_pages, page_size, write_kv, n_tokens)
+  if (dtype == kF32) {
+    if (d > 128) LS_ROPE(float, 2); else LS_ROPE(float, 1);
+  } else if (dtype == kBF16) {
+    if (d > 128) LS_ROPE(bf16_t, 2); else LS_ROPE(bf16_t, 1);
+  } else {
     return fail("qk_rope_kv: unknown dtype %d", dtype);
+  }
+#undef LS_ROPE
   return check_launch("qk_rope_kv");
 }
 
