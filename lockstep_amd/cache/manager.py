@@ -230,7 +230,10 @@ class CacheManager:
         """
         request = self.requests[request_id]
         start = request.length if start is None else start
-        if -(-end // self.page_size) > self.max_pages_per_request:
+        needed_to = -(-end // self.page_size)
+        if all(len(mine.pages) >= needed_to for mine in request.groups):
+            return  # the last page still has room: nothing to take
+        if needed_to > self.max_pages_per_request:
             raise ValueError(f"{end} tokens exceed the {self.max_pages_per_request * self.page_size} "
                              "tokens a request may hold")
         need = self.pages_to_reserve(request_id, start, end)

@@ -66,14 +66,15 @@ constexpr int DB = D / 16;          // 16-column blocks of the head
 struct SeqMeta {
   int q_off, q_len, q_start, kv_len, table_row, reserved[3];
 };
-struct AttnItem {  // one workgroup column of the attention launch
+struct AttnItem {  // one workgroup column of the attention launch (16 ints)
   int seq;         // index into SeqMeta
-  int row_block;   // 64-row block of the sequence's rows
+  int row_block;   // row block of the sequence's rows
   int split_begin, split_end;
   int part_base;   // first partial row of the sequence, or -1: direct
   int n_splits;    // splits of the sequence that have a partial
   int split_lo;    // first of them (splits below lie behind the window)
   int reserved;
+  SeqMeta sm;      // a copy of seqs[seq], so that the kernel needs one load to know its work
 };
 
 // A masked score is minus infinity, so its probability exp(-inf - m) is an
@@ -165,7 +166,7 @@ __global__ __launch_bounds__(256) void attention_direct_kernel(
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const AttnItem item = items[blockIdx.x];
-  const SeqMeta sm = seqs[item.seq];
+  const SeqMeta sm = item.sm;
   const int kvh = blockIdx.y;
   const int rows_total = sm.q_len * G;
   const int r0 = item.row_block * 64 + wave * 16;
@@ -363,7 +364,7 @@ __global__ __launch_bounds__(256, LS_STAGED_MIN_BLOCKS) void attention_staged_ke
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const AttnItem item = items[blockIdx.x];
-  const SeqMeta sm = seqs[item.seq];
+  const SeqMeta sm = item.sm;
   const int kvh = blockIdx.y;
   const int rows_total = sm.q_len * G;
   const int block_r0 = item.row_block * 64;
@@ -704,7 +705,7 @@ __global__ __launch_bounds__(64 * NW) void attention_wide_kernel(
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const AttnItem item = items[blockIdx.x];
-  const SeqMeta sm = seqs[item.seq];
+  const SeqMeta sm = item.sm;
   const int kvh = blockIdx.y;
   const int rows_total = sm.q_len * G;
   const int block_r0 = item.row_block * ROWS;
@@ -1041,7 +1042,7 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const AttnItem item = items[blockIdx.x];
-  const SeqMeta sm = seqs[item.seq];
+  const SeqMeta sm = item.sm;
   const int kvh = blockIdx.y;
   const int rows_total = sm.q_len * G;  // <= 16, checked on the host
   const int row16 = lane & 15;
@@ -1406,8 +1407,10 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
   }
 }
 
-struct CombineItem {
+struct CombineItem {  // 8 ints
   int seq, row_block, part_base, n_splits;
+  int q_off, q_len;  // of seqs[seq]
+  int reserved[2];
 };
 
 template <typename T>
@@ -1419,9 +1422,8 @@ __global__ __launch_bounds__(256) void combine_kernel(const SeqMeta* __restrict_
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const CombineItem item = items[blockIdx.x];
-  const SeqMeta sm = seqs[item.seq];
   const int kvh = blockIdx.y;
-  const int rows_total = sm.q_len * G;
+  const int rows_total = item.q_len * G;
   const int r = item.row_block * 64 + wave * 16 + (lane & 15);
   if (r >= rows_total) return;
   const int g = lane >> 4;
@@ -1438,7 +1440,7 @@ __global__ __launch_bounds__(256) void combine_kernel(const SeqMeta* __restrict_
     for (int blk = 0; blk < DB; ++blk) acc[blk] = *reinterpret_cast<const f32x4*>(part_acc + pr * D + blk * 16 + 4 * g);
     fold_split<T>(run, acc, part_ml[pr * 2], part_ml[pr * 2 + 1]);
   }
-  store_output<T>(run, out + (long)(sm.q_off + qi) * ldo + (long)head * D, g);
+  store_output<T>(run, out + (long)(item.q_off + qi) * ldo + (long)head * D, g);
 }
 
 }  // namespace ls
@@ -1617,7 +1619,7 @@ extern "C" int ls_attn_block_rows(int variant) { return variant == 4 ? 16 * kWid
 // direct one elsewhere, 1 forces the direct kernel, 2 the staged one.
 // q [tokens, ldq]: head h of a token at columns [h*D, (h+1)*D).  out likewise
 // with ldo.  k_pages [pages][nkv][page_size][D], v_pages [pages][nkv][D][page_size].
-// table [rows][table_stride] int32 (page id or -1).  items: n_items AttnItem.
+// table [rows][table_stride] int32 (page id or -1).  items: n_items AttnItem (16 ints each).
 extern "C" int ls_attention(int dtype, const void* q, long ldq, const void* k_pages, const void* v_pages, int nkv,
                             int page_size, const int* table, int table_stride, const void* seqs, const void* items,
                             int n_items, void* out, long ldo, float* part_acc, float* part_ml, int G, float scale,

@@ -39,9 +39,11 @@ enum Epilogue : int {
 
 __host__ __device__ inline int kslice_for(int K) { return 256 * ((K + 4095) / 4096); }
 
+// `old`: for kAddF32 with vector stores, the four values the element's owner
+// has already read from C (nullptr: read them here).
 template <typename T, int EPI>
 __device__ __forceinline__ void epilogue4(void* __restrict__ C, long ldc, int m, int n, int M, int N,
-                                          const float total[4], bool vec_ok) {
+                                          const float total[4], bool vec_ok, const f32x4* old_vals = nullptr) {
   if (m >= M || n >= N) return;
   if (EPI == kStore) {
     T* row = reinterpret_cast<T*>(C) + (long)m * ldc;
@@ -65,7 +67,7 @@ __device__ __forceinline__ void epilogue4(void* __restrict__ C, long ldc, int m,
       f32x4* p = reinterpret_cast<f32x4*>(row + n);
       f32x4 v = f32x4{total[0], total[1], total[2], total[3]};
       if (EPI == kAddF32) {
-        f32x4 old = *p;
+        const f32x4 old = old_vals ? *old_vals : *p;
         v = f32x4{old[0] + v[0], old[1] + v[1], old[2] + v[2], old[3] + v[3]};
       }
       *p = v;
@@ -176,6 +178,14 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const void* __rest
   }
   const bool norm_vec = NORM && aligned && ldx % 4 == 0 && reinterpret_cast<uintptr_t>(norm_w) % 16 == 0;
 
+  // kAddF32: the owner of an output element reads its old value now, not after the products
+  f32x4 old_vals = f32x4{0.f, 0.f, 0.f, 0.f};
+  const bool preload = EPI == kAddF32 && vec_ok && (int)threadIdx.x < MT * 64 &&
+                       (int)(threadIdx.x >> 6) * 16 + row16 < M && n0 + g * 4 + 3 < N;
+  if (preload)
+    old_vals = *reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(C) +
+                                               (long)((threadIdx.x >> 6) * 16 + row16) * ldc + n0 + g * 4);
+
   for (int s = wave; s < nslices; s += NW) {
     f32x4 acc[NT][MT];
 #pragma unroll
@@ -261,7 +271,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const void* __rest
     if (EPI == kSwiGLU)
       epilogue_swiglu4<T>(C, ldc, m, blockIdx.x * 16 + (l >> 4) * 4, M, out_cols, total[0], total[NT - 1], vec_ok);
     else
-      epilogue4<T, EPI>(C, ldc, m, n0 + (l >> 4) * 4, M, N, total[0], vec_ok);
+      epilogue4<T, EPI>(C, ldc, m, n0 + (l >> 4) * 4, M, N, total[0], vec_ok,
+                        (preload && idx == (int)threadIdx.x) ? &old_vals : nullptr);
   }
 }
 

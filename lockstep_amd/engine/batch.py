@@ -21,6 +21,8 @@ from typing import Hashable, Sequence
 import numpy as np
 import torch
 
+from ..ops.kernels import pack_attention_items, pack_combine_items
+
 
 @dataclass
 class StepEntry:
@@ -56,6 +58,23 @@ class Workspace:
         self.device = device
         self._buffers: dict[tuple, torch.Tensor] = {}
         self.version = 0
+        self.plan_templates: dict[tuple, tuple] = {}   # work lists of decode steps by shape
+        self._stage = None                             # pinned host buffer of the metadata upload
+        self._stage_np = None
+        self._stage_done = None
+
+    def staging(self, n: int):
+        """A pinned int32 host buffer of at least ``n`` elements as a numpy view, free to be
+        overwritten (its last copy to the device has finished)."""
+        if self._stage is None or self._stage.shape[0] < n:
+            if self._stage_done is not None:
+                self._stage_done.synchronize()
+            self._stage = torch.empty(max(2 * n, 4096), dtype=torch.int32, pin_memory=True)
+            self._stage_np = self._stage.numpy()
+            self._stage_done = torch.cuda.Event()
+        elif self._stage_done is not None:
+            self._stage_done.synchronize()
+        return self._stage, self._stage_np, self._stage_done
 
     def get(self, name: str, shape, dtype) -> torch.Tensor:
         shape = tuple(int(s) for s in shape)
@@ -88,28 +107,38 @@ class StepContext:
         lengths = [len(e.tokens) for e in self.entries]
         self.n_seqs = len(self.entries)
         self.n_tokens = int(sum(lengths))
+        self._single_tokens = self.n_tokens == self.n_seqs
         # host-side views, also for parts written in plain torch (tests)
-        self.q_len = np.asarray(lengths, dtype=np.int64)
-        self.q_off = np.concatenate([[0], np.cumsum(self.q_len)[:-1]]).astype(np.int64)
-        self.q_start = np.asarray([cache.length(e.request) for e in self.entries], dtype=np.int64)
-        self.kv_len = self.q_start + self.q_len
-        self.slots = np.asarray([cache.slot(e.request) for e in self.entries], dtype=np.int64)
+        starts = [cache.length(e.request) for e in self.entries]
+        offsets = [0] * self.n_seqs
+        for i in range(1, self.n_seqs):
+            offsets[i] = offsets[i - 1] + lengths[i - 1]
+        seqs = np.zeros((self.n_seqs, 8), dtype=np.int64)
+        seqs[:, 0], seqs[:, 1], seqs[:, 2] = offsets, lengths, starts
+        seqs[:, 3] = seqs[:, 1] + seqs[:, 2]
+        seqs[:, 4] = [cache.slot(e.request) for e in self.entries]
+        self.q_off, self.q_len, self.q_start, self.kv_len, self.slots = (seqs[:, c] for c in range(5))
         self.max_position = int(self.kv_len.max()) - 1
 
-        tokens = np.concatenate([np.asarray(e.tokens, dtype=np.int64) for e in self.entries])
-        tok_seq = np.repeat(np.arange(self.n_seqs), self.q_len)
-        tok_pos = np.concatenate([np.arange(s, s + n) for s, n in zip(self.q_start, self.q_len)])
-        seqs = np.zeros((self.n_seqs, 8), dtype=np.int64)
-        seqs[:, 0], seqs[:, 1], seqs[:, 2], seqs[:, 3], seqs[:, 4] = (
-            self.q_off, self.q_len, self.q_start, self.kv_len, self.slots)
-        want = [int(self.q_off[i]) + int(w) for i, e in enumerate(self.entries) for w in e.want]
+        if self._single_tokens:
+            tokens = np.asarray([e.tokens[0] for e in self.entries], dtype=np.int64)
+            tok_seq = np.arange(self.n_seqs)
+            tok_pos = self.q_start
+            want = [i for i, e in enumerate(self.entries) for w in e.want]
+        else:
+            tokens = np.concatenate([np.asarray(e.tokens, dtype=np.int64) for e in self.entries])
+            tok_seq = np.repeat(np.arange(self.n_seqs), self.q_len)
+            tok_pos = np.concatenate([np.arange(s, s + n) for s, n in zip(starts, lengths)])
+            want = [offsets[i] + int(w) for i, e in enumerate(self.entries) for w in e.want]
         self.n_want = len(want)
+        self._seq_rows = seqs
         self._host_parts: list[np.ndarray] = [tokens, tok_seq, tok_pos, seqs.reshape(-1),
                                               np.asarray(want, dtype=np.int64)]
         self._plans: dict[tuple, tuple] = {}
         self._plan_specs: list[tuple] = []
         self._uploaded = False
-        self.token_ids = self.tok_seq = self.tok_pos = self.seqs = self.want_rows = None
+        self._meta = None
+        self._views = None
         self.host_tokens = tokens
 
     # -- attention work lists -----------------------------------------------------
@@ -130,10 +159,34 @@ class StepContext:
         part_rows = 0
         bucket = 0
         if self.fixed_shape:
-            longest = max((int(k) - 1) // split + 1 for k in self.kv_len)
+            longest = (int(self.kv_len.max()) - 1) // split + 1
             bucket = 1
             while bucket < longest:
                 bucket = bucket * 2 if bucket < 8 else bucket + 8
+            if coop_ok and group_size <= 16 and self._single_tokens:
+                # a decode step: the lists depend on its shape only, the requests' rows are appended
+                shape = (self.n_seqs, group_size, nkv, bucket, whole_requests)
+                made = self.workspace.plan_templates.get(shape)
+                if made is None:
+                    for i in range(self.n_seqs):
+                        if whole_requests:
+                            coop.append((i, 0, 0, bucket, -1, 0, 0, 0))
+                        else:
+                            base = part_rows
+                            part_rows += nkv * group_size * bucket
+                            coop += [(i, 0, s, s + 1, base, bucket, 0, 0) for s in range(bucket)]
+                            combine.append((i, 0, base, bucket))
+                    made = (np.asarray(coop, dtype=np.int64).reshape(-1, 8),
+                            np.asarray(combine, dtype=np.int64).reshape(-1, 4), part_rows)
+                    self.workspace.plan_templates[shape] = made
+                coop_t, combine_t, part_rows = made
+                empty = np.zeros(0, dtype=np.int64)
+                decode_fused = kernels.decode_fused_supported(head_dim, self.rt.dtype, self.cache.page_size)
+                self._plans[key] = (empty, pack_combine_items(combine_t, self._seq_rows), 0, len(combine_t), part_rows,
+                                    pack_attention_items(coop_t, self._seq_rows), len(coop_t), group_size,
+                                    empty, 0, decode_fused)
+                self._plan_specs.append(key)
+                return
         for i in range(self.n_seqs):
             q_len, q_start, kv_len = int(self.q_len[i]), int(self.q_start[i]), int(self.kv_len[i])
             rows = q_len * group_size
@@ -167,22 +220,38 @@ class StepContext:
                         and kernels.decode_fused_supported(head_dim, self.rt.dtype, self.cache.page_size))
         # the longest row blocks first: they decide when the launch ends
         wide.sort(key=lambda it: it[2] - it[3])
-        self._plans[key] = (np.asarray(items, dtype=np.int64).reshape(-1),
-                            np.asarray(combine, dtype=np.int64).reshape(-1), len(items), len(combine), part_rows,
-                            np.asarray(coop, dtype=np.int64).reshape(-1), len(coop), coop_max_rows,
-                            np.asarray(wide, dtype=np.int64).reshape(-1), len(wide), decode_fused)
+        self._plans[key] = (pack_attention_items(items, self._seq_rows),
+                            pack_combine_items(combine, self._seq_rows), len(items), len(combine), part_rows,
+                            pack_attention_items(coop, self._seq_rows), len(coop), coop_max_rows,
+                            pack_attention_items(wide, self._seq_rows), len(wide), decode_fused)
         self._plan_specs.append(key)
 
     def upload(self) -> None:
-        """Copy all metadata to the device in one transfer."""
+        """Copy all metadata to the device in one transfer (from a pinned buffer, asynchronously)."""
         parts = list(self._host_parts)
         for key in self._plan_specs:
             items, combine, _, _, _, coop, _, _, wide, _, _ = self._plans[key]
             parts += [items, combine, coop, wide]
-        flat = np.concatenate(parts).astype(np.int32)
-        host = torch.from_numpy(flat)
-        dev = self.workspace.get("step.meta", (flat.shape[0],), torch.int32)
-        dev.copy_(host, non_blocking=False)
+        total = sum(p.shape[0] for p in parts)
+        stage, view, done = self.workspace.staging(total)
+        at = 0
+        for p in parts:
+            n = p.shape[0]
+            if n:
+                view[at:at + n] = p
+                at += n
+        dev = self.workspace.get("step.meta", (total,), torch.int32)
+        dev.copy_(stage[:total], non_blocking=True)
+        done.record()
+        self._meta = dev
+        self._views = None
+        self._uploaded = True
+
+    def _materialize(self) -> dict:
+        """Device views of the uploaded metadata (made when a part first asks: a replayed graph never does)."""
+        if self._views is not None:
+            return self._views
+        dev = self._meta
         offset = 0
 
         def take(n):
@@ -192,10 +261,8 @@ class StepContext:
             return out
 
         t, s = self.n_tokens, self.n_seqs
-        self.token_ids, self.tok_seq, self.tok_pos = take(t), take(t), take(t)
-        self.seqs = take(8 * s)
-        self.want_rows = take(self.n_want)
-        self._device_plans: dict[tuple, AttentionPlan] = {}
+        views = {"token_ids": take(t), "tok_seq": take(t), "tok_pos": take(t), "seqs": take(8 * s),
+                 "want_rows": take(self.n_want), "plans": {}}
         for key in self._plan_specs:
             (items, combine, n_items, n_combine, part_rows, coop, n_coop, coop_max_rows, wide, n_wide,
              decode_fused) = self._plans[key]
@@ -206,12 +273,19 @@ class StepContext:
             if part_rows:
                 part_acc = self.workspace.get(f"attention.part_acc.{head_dim}", (part_rows, head_dim), torch.float32)
                 part_ml = self.workspace.get("attention.part_ml", (part_rows, 2), torch.float32)
-            self._device_plans[key] = AttentionPlan(d_items, n_items, d_coop if n_coop else None, n_coop,
-                                                    coop_max_rows, decode_fused,
-                                                    d_wide if n_wide else None, n_wide,
-                                                    d_combine if n_combine else None,
-                                                    n_combine, part_acc, part_ml)
-        self._uploaded = True
+            views["plans"][key] = AttentionPlan(d_items, n_items, d_coop if n_coop else None, n_coop,
+                                                coop_max_rows, decode_fused,
+                                                d_wide if n_wide else None, n_wide,
+                                                d_combine if n_combine else None,
+                                                n_combine, part_acc, part_ml)
+        self._views = views
+        return views
+
+    token_ids = property(lambda self: self._materialize()["token_ids"])
+    tok_seq = property(lambda self: self._materialize()["tok_seq"])
+    tok_pos = property(lambda self: self._materialize()["tok_pos"])
+    seqs = property(lambda self: self._materialize()["seqs"])
+    want_rows = property(lambda self: self._materialize()["want_rows"])
 
     def plan_signature(self) -> tuple:
         """Sizes of the work lists: equal signatures mean an equal device layout."""
@@ -220,7 +294,7 @@ class StepContext:
                      for key in self._plan_specs) + (self.n_tokens, self.n_want)
 
     def attention_plan(self, group_size: int, nkv: int, head_dim: int, window: int) -> AttentionPlan:
-        return self._device_plans[(group_size, nkv, head_dim, window)]
+        return self._materialize()["plans"][(group_size, nkv, head_dim, window)]
 
     def buf(self, name: str, shape, dtype) -> torch.Tensor:
         return self.workspace.get(name, shape, dtype)

@@ -21,6 +21,7 @@ import torch
 from ..cache import CacheManager
 from ..config import ModelConfig, ModelSpec, config_from_dir
 from ..parts import WeightSpec, build_part, part_class
+from ..parts.base import device_epoch
 from ..weights.store import load_weights, weights_from_dict
 from .batch import StepContext, StepEntry, Workspace
 from .runtime import Runtime
@@ -66,6 +67,14 @@ class Model:
         self.workspace = Workspace(rt.device)
         self.use_graphs = os.environ.get("LOCKSTEP_NO_GRAPHS", "") in ("", "0")
         self._graph_safe = all(layer.mixer.graph_safe for layer in self.layers)
+        # one mixer of each group of equal ones is asked to prepare a step
+        seen, self._preparers = set(), []
+        for layer in self.layers:
+            group = layer.mixer.prepare_group()
+            if group is None or group not in seen:
+                self._preparers.append(layer.mixer)
+                if group is not None:
+                    seen.add(group)
         self.graph_replays = 0
 
     # -- weights --------------------------------------------------------------
@@ -105,8 +114,12 @@ class Model:
             if e.request in seen:
                 raise ValueError(f"request {e.request!r} appears twice in one step")
             seen.add(e.request)
-            ids = np.asarray(e.tokens)
-            if ids.min() < 0 or ids.max() >= vocab:
+            if len(e.tokens) == 1:
+                inside = 0 <= int(e.tokens[0]) < vocab
+            else:
+                ids = np.asarray(e.tokens)
+                inside = ids.min() >= 0 and ids.max() < vocab
+            if not inside:
                 raise ValueError(f"request {e.request!r} brings a token id outside [0, {vocab})")
             for w in e.want:
                 if not 0 <= w < len(e.tokens):
@@ -114,8 +127,8 @@ class Model:
         for e in entries:
             start = cache.length(e.request)
             cache.reserve(e.request, start + len(e.tokens))
-            for gi, group in enumerate(cache.groups):
-                if cache.ever_shared:
+            if cache.ever_shared:
+                for gi in range(len(cache.groups)):
                     for logical in range(start // cache.page_size, -(-(start + len(e.tokens)) // cache.page_size)):
                         cache.assert_exclusive(e.request, gi, logical)
         cache.sync_tables()
@@ -125,8 +138,8 @@ class Model:
         graphed = (self.use_graphs and self._graph_safe
                    and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries))
         ctx = StepContext(self.rt, cache, self.workspace, entries, fixed_shape=graphed)
-        for layer in self.layers:
-            layer.mixer.prepare(ctx)
+        for mixer in self._preparers:
+            mixer.prepare(ctx)
         ctx.upload()
         logits = self._forward_graphed(ctx, cache) if graphed else self._forward(ctx)
         for e, end in zip(entries, ctx.kv_len):
@@ -148,10 +161,7 @@ class Model:
         return logits
 
     def _graph_key(self, ctx: StepContext) -> tuple:
-        tables = tuple((t.data_ptr(), t.shape[0]) for t in
-                       (getattr(getattr(layer.mixer, "position", None), "cos", None) for layer in self.layers)
-                       if t is not None)
-        return (self.serial, ctx.n_seqs, ctx.plan_signature(), self.workspace.version, tables)
+        return (self.serial, ctx.n_seqs, ctx.plan_signature(), self.workspace.version, device_epoch())
 
     def _forward_graphed(self, ctx: StepContext, cache):
         """Replay the captured graph of this step shape, capturing it first if

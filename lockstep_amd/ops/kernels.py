@@ -70,6 +70,7 @@ class Kernels:
         self._attention: dict[int, ctypes.CDLL] = {}
         self.attention_paths: dict[int, str] = {}
         self._argmax_scratch: dict = {}
+        self._capabilities: dict = {}
 
     # -- helpers ------------------------------------------------------------
     @staticmethod
@@ -88,28 +89,37 @@ class Kernels:
             self.attention_paths[head_dim] = str(path)
         return lib
 
+    def _memo(self, key, compute):
+        """Capability queries do not change while the process runs: ask the library once."""
+        have = self._capabilities.get(key)
+        if have is None:
+            have = self._capabilities[key] = compute()
+        return have
+
     def coop_supported(self, head_dim: int, dtype: torch.dtype, page_size: int = 16) -> bool:
         """Whether the cooperative attention kernel can run (its tiles must fit into LDS)."""
-        lib = self.attention_lib(head_dim)
-        return page_size >= 8 and bool(lib.ls_attn_coop_supported(c_int(DTYPE_CODE[dtype])))
+        return self._memo(("coop", head_dim, dtype, page_size), lambda: page_size >= 8 and bool(
+            self.attention_lib(head_dim).ls_attn_coop_supported(c_int(DTYPE_CODE[dtype]))))
 
     def decode_fused_supported(self, head_dim: int, dtype: torch.dtype, page_size: int) -> bool:
         """Whether ``attention_decode`` (norm, rotation and cache write inside the attention kernel) can run."""
-        lib = self.attention_lib(head_dim)
-        return page_size >= 8 and bool(lib.ls_attn_decode_fused_supported(c_int(DTYPE_CODE[dtype])))
+        return self._memo(("decode_fused", head_dim, dtype, page_size), lambda: page_size >= 8 and bool(
+            self.attention_lib(head_dim).ls_attn_decode_fused_supported(c_int(DTYPE_CODE[dtype]))))
 
     def wide_supported(self, head_dim: int, dtype: torch.dtype, page_size: int) -> bool:
         """Whether the wide attention kernel (variant 4, for prompt portions) can run."""
-        return page_size >= 8 and bool(self.attention_lib(head_dim).ls_attn_wide_supported(c_int(DTYPE_CODE[dtype])))
+        return self._memo(("wide", head_dim, dtype, page_size), lambda: page_size >= 8 and bool(
+            self.attention_lib(head_dim).ls_attn_wide_supported(c_int(DTYPE_CODE[dtype]))))
 
     def attention_block_rows(self, head_dim: int, variant: int) -> int:
         """Rows of the row blocks that work items of this variant count in."""
-        return int(self.attention_lib(head_dim).ls_attn_block_rows(c_int(variant)))
+        return self._memo(("block_rows", head_dim, variant),
+                          lambda: int(self.attention_lib(head_dim).ls_attn_block_rows(c_int(variant))))
 
     def attention_geometry(self, head_dim: int) -> tuple[int, int]:
         """(keys per tile, keys per split) of the attention kernels."""
-        lib = self.attention_lib(head_dim)
-        return lib.ls_attn_tile_keys(), lib.ls_attn_split_keys()
+        return self._memo(("geometry", head_dim), lambda: (self.attention_lib(head_dim).ls_attn_tile_keys(),
+                                                           self.attention_lib(head_dim).ls_attn_split_keys()))
 
     # -- matrix product -------------------------------------------------------
     def gemm(self, x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, epilogue: int = STORE,
@@ -275,8 +285,8 @@ class Kernels:
               and v_pages.is_contiguous() and k_pages.shape[1:] == (nkv, page_size, d)
               and v_pages.shape[1:] == (nkv, d, page_size), "attention cache pages have the wrong layout or dtype")
         _need(table.dtype == torch.int32 and table.dim() == 2 and table.is_contiguous(), "attention block table")
-        _need(items.dtype == torch.int32 and items.is_contiguous() and items.numel() >= 8 * n_items,
-              "attention items must hold 8 int32 each")
+        _need(items.dtype == torch.int32 and items.is_contiguous() and items.numel() >= ATTENTION_ITEM_INTS * n_items,
+              "attention items must hold 16 int32 each (see pack_attention_items)")
         if n_items == 0:
             return
         code = lib.ls_attention(
@@ -302,8 +312,8 @@ class Kernels:
               and v_pages.is_contiguous() and k_pages.shape[1:] == (nkv, page_size, d)
               and v_pages.shape[1:] == (nkv, d, page_size), "attention cache pages have the wrong layout or dtype")
         _need(table.dtype == torch.int32 and table.dim() == 2 and table.is_contiguous(), "attention block table")
-        _need(items.dtype == torch.int32 and items.is_contiguous() and items.numel() >= 8 * n_items,
-              "attention items must hold 8 int32 each")
+        _need(items.dtype == torch.int32 and items.is_contiguous() and items.numel() >= ATTENTION_ITEM_INTS * n_items,
+              "attention items must hold 16 int32 each (see pack_attention_items)")
         for w in (q_weight, k_weight):
             _need(w is None or (w.dtype == torch.float32 and w.is_contiguous() and w.numel() == d),
                   "per-head norm weights must be float32 [head_dim]")
@@ -328,14 +338,45 @@ class Kernels:
         lib = self.attention_lib(d)
         _rows_ok(out, "combine out")
         _need(out.dtype in DTYPE_CODE and out.shape[1] >= nq * d, "combine out rows are too short")
-        _need(items.dtype == torch.int32 and items.is_contiguous() and items.numel() >= 4 * n_items,
-              "combine items must hold 4 int32 each")
+        _need(items.dtype == torch.int32 and items.is_contiguous() and items.numel() >= COMBINE_ITEM_INTS * n_items,
+              "combine items must hold 8 int32 each (see pack_combine_items)")
         if n_items == 0:
             return
         code = lib.ls_attention_combine(c_int(DTYPE_CODE[out.dtype]), _ptr(seqs), _ptr(items), c_int(n_items),
                                         c_int(nkv), _ptr(part_acc), _ptr(part_ml), _ptr(out),
                                         c_long(out.stride(0)), c_int(nq // nkv), _stream())
         self._check(lib, code)
+
+
+ATTENTION_ITEM_INTS = 16
+COMBINE_ITEM_INTS = 8
+
+
+def pack_attention_items(items, seqs) -> "np.ndarray":
+    """Work items of the attention kernels as the device wants them.  ``items``:
+    rows of (seq, row_block, split_begin, split_end, part_base, n_splits,
+    split_lo, 0); ``seqs``: the step's rows of (q_off, q_len, q_start, kv_len,
+    table_row, 0, 0, 0).  Each item gets a copy of its request's row appended, so
+    that a workgroup learns its work from one load."""
+    import numpy as np
+
+    items = np.asarray(items, dtype=np.int64).reshape(-1, 8)
+    seqs = np.asarray(seqs, dtype=np.int64).reshape(-1, 8)
+    if not len(items):
+        return np.zeros(0, dtype=np.int64)
+    return np.concatenate([items, seqs[items[:, 0]]], axis=1).reshape(-1)
+
+
+def pack_combine_items(items, seqs) -> "np.ndarray":
+    """Combine items (seq, row_block, part_base, n_splits) with q_off and q_len of their request appended."""
+    import numpy as np
+
+    items = np.asarray(items, dtype=np.int64).reshape(-1, 4)
+    seqs = np.asarray(seqs, dtype=np.int64).reshape(-1, 8)
+    if not len(items):
+        return np.zeros(0, dtype=np.int64)
+    pad = np.zeros((len(items), 2), dtype=np.int64)
+    return np.concatenate([items, seqs[items[:, 0], :2], pad], axis=1).reshape(-1)
 
 
 _INSTANCE: Kernels | None = None

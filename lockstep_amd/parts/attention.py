@@ -95,6 +95,14 @@ class Attention(Mixer):
             self.q_norm = rt.vector(weights.get(f"{self.prefix}.q_norm.weight"))
             self.k_norm = rt.vector(weights.get(f"{self.prefix}.k_norm.weight"))
         rt.kernels.attention_lib(self.d)
+        if hasattr(self.position, "bind"):
+            self.position.bind(rt)      # layers with equal constants share their tables
+
+    def prepare_group(self):
+        share = getattr(self.position, "share_key", None)
+        if share is None:
+            return None
+        return ("attention", self.nq, self.nkv, self.d, self.window, share())
 
     def prepare(self, ctx) -> None:
         self.position.ensure(ctx.max_position + 1, ctx.rt)

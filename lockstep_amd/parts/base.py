@@ -119,6 +119,11 @@ class Mixer(Part):
     def prepare(self, ctx) -> None:
         """Declare per-step needs (work lists) before the step's metadata is uploaded."""
 
+    def prepare_group(self):
+        """Mixers that return the same hashable value here need ``prepare`` only once a step
+        (one of them is called); None: always call this one."""
+        return None
+
     def forward(self, ctx, run, x, out, accumulate: bool) -> None:
         raise NotImplementedError
 
@@ -182,3 +187,18 @@ def part_class(kind: str) -> type:
 
 def build_part(spec: PartSpec, prefix: str = "", **extra: Any) -> Part:
     return part_class(spec.kind)(spec, prefix, **extra)
+
+
+# Captured graphs hold the addresses of device tensors that parts own (tables that grow with
+# the longest position, for instance).  A part that replaces such a tensor bumps the epoch;
+# the model keys its graphs on it.
+_DEVICE_EPOCH = 0
+
+
+def device_epoch() -> int:
+    return _DEVICE_EPOCH
+
+
+def bump_device_epoch() -> None:
+    global _DEVICE_EPOCH
+    _DEVICE_EPOCH += 1

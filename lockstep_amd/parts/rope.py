@@ -9,7 +9,10 @@ from __future__ import annotations
 import torch
 
 from ..config.base import PartSpec
-from .base import PositionEncoding, register_part
+from .base import PositionEncoding, bump_device_epoch, register_part
+
+# Layers with the same constants share one pair of tables per device.
+_TABLES: dict[tuple, list] = {}
 
 
 @register_part("rope_half")
@@ -22,8 +25,18 @@ class RotaryHalf(PositionEncoding):
         self.theta = float(spec["theta"])
         if self.rotary_dim % 2 or self.rotary_dim <= 0:
             raise ValueError(f"rotary_dim {self.rotary_dim} must be a positive even number")
-        self.cos = None
-        self.sin = None
+        self._store = None
+
+    @property
+    def cos(self):
+        return None if self._store is None else self._store[0]
+
+    @property
+    def sin(self):
+        return None if self._store is None else self._store[1]
+
+    def share_key(self):
+        return (self.rotary_dim, self.theta)
 
     def tables(self, positions: torch.Tensor):
         half = self.rotary_dim // 2
@@ -32,14 +45,21 @@ class RotaryHalf(PositionEncoding):
         angles = positions.to(torch.float64)[:, None] * inv_freq[None, :]
         return angles.cos().to(torch.float32), angles.sin().to(torch.float32)
 
+    def bind(self, rt) -> None:
+        """Attach to the tables that all layers with these constants share on this device."""
+        self._store = _TABLES.setdefault((self.rotary_dim, self.theta, str(rt.device)), [None, None])
+
     def ensure(self, max_position: int, rt) -> None:
-        have = 0 if self.cos is None else self.cos.shape[0]
+        if self._store is None:
+            self.bind(rt)
+        have = 0 if self._store[0] is None else self._store[0].shape[0]
         if max_position <= have:
             return
         size = max(max_position, 2 * have, 256)
         cos, sin = self.tables(torch.arange(size))
-        self.cos = cos.to(rt.device).contiguous()
-        self.sin = sin.to(rt.device).contiguous()
+        self._store[0] = cos.to(rt.device).contiguous()
+        self._store[1] = sin.to(rt.device).contiguous()
+        bump_device_epoch()
 
 
 @register_part("no_position")
@@ -49,3 +69,6 @@ class NoPosition(PositionEncoding):
     rotary_dim = 0
     cos = None
     sin = None
+
+    def share_key(self):
+        return ("none",)

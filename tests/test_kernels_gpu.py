@@ -239,15 +239,19 @@ class PagedCase:
                 last = q_start + min(b * br + br - 1, rows - 1) // g
                 begin = (max(0, first - window + 1) // split) if window else 0
                 items += [0, b, begin, last // split + 1, -1, 0, 0, 0]
-        items_t = torch.tensor(items, dtype=torch.int32).cuda()
+        from lockstep_amd.ops import pack_attention_items, pack_combine_items
+
+        seq_row = self.seqs(q_start, t).cpu().numpy()
+        n_items = len(items) // 8
+        items_t = torch.from_numpy(pack_attention_items(items, seq_row)).to(torch.int32).cuda()
         out = torch.full((t, self.nq * self.d), float("nan"), dtype=self.dtype, device="cuda")
         part_acc = torch.full((max(part_rows, 1), self.d), float("nan"), dtype=torch.float32, device="cuda")
         part_ml = torch.full((max(part_rows, 1), 2), float("nan"), dtype=torch.float32, device="cuda")
         K().attention(qkv, self.nq, self.nkv, self.d, self.k_pages, self.v_pages, self.ps, self.table,
-                      self.seqs(q_start, t), items_t, len(items) // 8, out, part_acc, part_ml, scale, window,
+                      self.seqs(q_start, t), items_t, n_items, out, part_acc, part_ml, scale, window,
                       variant, rows)
         if combine:
-            comb = torch.tensor(combine, dtype=torch.int32).cuda()
+            comb = torch.from_numpy(pack_combine_items(combine, seq_row)).to(torch.int32).cuda()
             K().attention_combine(self.d, self.seqs(q_start, t), comb, len(combine) // 4, self.nq, self.nkv,
                                   part_acc, part_ml, out)
         return out.view(t, self.nq, self.d)
@@ -486,14 +490,17 @@ def test_fused_decode_attention_equals_the_separate_kernels(dtype, nq, nkv, d, p
             part_acc = torch.full((part_rows, d), float("nan"), dtype=torch.float32, device="cuda")
             part_ml = torch.full((part_rows, 2), float("nan"), dtype=torch.float32, device="cuda")
             out = torch.full((1, nq * d), float("nan"), dtype=dtype, device="cuda")
-            items_t = torch.tensor(items, dtype=torch.int32).cuda()
+            from lockstep_amd.ops import pack_attention_items, pack_combine_items
+
+            seq_row = base.seqs(p, 1).cpu().numpy()
+            items_t = torch.from_numpy(pack_attention_items(items, seq_row)).to(torch.int32).cuda()
             raw = qkv[p:p + 1].clone()
             K().attention_decode(raw, nq, nkv, d, base.k_pages, base.v_pages, ps, base.table, base.seqs(p, 1), items_t,
                                  len(items) // 8, out, part_acc, part_ml, d ** -0.5, window, qw, kw, eps, cos, sin, rot,
                                  p, True)
             if combine:
-                K().attention_combine(d, base.seqs(p, 1), torch.tensor(combine, dtype=torch.int32).cuda(), 1, nq, nkv,
-                                      part_acc, part_ml, out)
+                comb = torch.from_numpy(pack_combine_items(combine, seq_row)).to(torch.int32).cuda()
+                K().attention_combine(d, base.seqs(p, 1), comb, 1, nq, nkv, part_acc, part_ml, out)
             assert torch.equal(out.view(1, nq, d), want), f"position {p}, split={use_split}"
             same_k = (base.k_pages == k_want) | ((base.k_pages != base.k_pages) & (k_want != k_want))
             same_v = (base.v_pages == v_want) | ((base.v_pages != base.v_pages) & (v_want != v_want))
