@@ -264,3 +264,27 @@ def test_a_large_decode_batch_gives_each_request_the_bits_it_gets_alone(plain_lo
         want = feed(model, alone, "x", prompts[i], [lengths[i]] + [1] * n_decode)[lengths[i]:]
         got = torch.stack([t[i] for t in together])
         assert torch.equal(got, want), f"request {i} (context {lengths[i]})"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name,page_size", [("A", 16), ("B", 8)])
+def test_the_first_tokens_of_a_sequence(plain_logits, dtype, name, page_size):
+    """A sequence decoded one by one from its very first token (position 0 has one key, the first
+    page and the first tile are being filled): right against the plain implementation, and the
+    same bits as the whole prompt in one step."""
+    folder, seqs = for_plain(plain_logits, name, dtype)
+    tokens, want = seqs[40]
+    model = load(folder, dtype)
+    cache = model.make_cache(num_pages=16, page_size=page_size, poison_on_free=True)
+    whole = feed(model, cache, "whole", tokens, [])
+    cache.close("whole")
+    stepwise = feed(model, cache, "steps", tokens, [1] * len(tokens))
+    cache.close("steps")
+    pair = feed(model, cache, "pair", tokens, [2, 1, 1, 2])
+    assert rel_err(stepwise[:3], want[:3]) < TOL[dtype]
+    assert rel_err(stepwise, want) < TOL[dtype]
+    assert torch.equal(stepwise, whole) and torch.equal(pair, whole)
+    one_folder, one_seqs = for_plain(plain_logits, name, dtype)
+    single, single_want = one_seqs[1]
+    cache.close("pair")
+    assert rel_err(feed(model, cache, "one", single, []), single_want) < TOL[dtype]
