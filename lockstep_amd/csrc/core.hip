@@ -196,6 +196,65 @@ __global__ __launch_bounds__(256) void swiglu_kernel(const T* __restrict__ gu, T
 }
 
 // ---------------------------------------------------------------------------
+// Residual add of a product left as slice sums, then RMSNorm of the new row:
+//   h[row] += (P[0][row] + P[1][row] + ...)   (slices ascending, from +0)
+//   out[r] = rmsnorm(h[row]) * weight         (skipped when out == nullptr)
+// `row` = rows[r] when a row list is given (then only the listed rows are
+// touched).  The sums and the norm are those of the separate kernels
+// (skinny product's fold and epilogue, rmsnorm_kernel), bit for bit.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void add_rmsnorm_kernel(float* __restrict__ h, const float* __restrict__ P,
+                                                          int slices, int p_rows, const float* __restrict__ weight,
+                                                          T* __restrict__ out, const int* __restrict__ rows, int width,
+                                                          long ldh, long ld_out, float eps) {
+  __shared__ float wave_part[4];
+  const int r_out = blockIdx.x;
+  const long row = rows ? rows[r_out] : r_out;
+  float* hrow = h + row * ldh;
+  // requirements checked on the host: width % 4 == 0, 16-byte aligned rows; any width
+  f32x4 w_first = f32x4{0.f, 0.f, 0.f, 0.f};  // the weights of the thread's first run, requested before the sums
+  if (out != nullptr && 4 * (int)threadIdx.x < width) w_first = *reinterpret_cast<const f32x4*>(weight + 4 * threadIdx.x);
+  float part = 0.f;
+  constexpr int BATCH = 16;  // slice sums requested together
+  for (int base = 4 * threadIdx.x; base < width; base += 1024) {
+    f32x4 total = f32x4{0.f, 0.f, 0.f, 0.f};
+    const f32x4 old = *reinterpret_cast<const f32x4*>(hrow + base);
+    for (int s0 = 0; s0 < slices; s0 += BATCH) {
+      f32x4 p[BATCH];
+#pragma unroll
+      for (int u = 0; u < BATCH; ++u)  // clamped: all loads are issued before the first is needed
+        p[u] = *reinterpret_cast<const f32x4*>(P + ((long)min(s0 + u, slices - 1) * p_rows + row) * width + base);
+#pragma unroll
+      for (int u = 0; u < BATCH; ++u)
+        if (s0 + u < slices) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) total[e] = total[e] + p[u][e];
+        }
+    }
+    f32x4 fresh;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) fresh[e] = old[e] + total[e];
+    *reinterpret_cast<f32x4*>(hrow + base) = fresh;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) part = part + fresh[e] * fresh[e];
+  }
+  if (out == nullptr) return;
+  part = wave_sum(part);
+  if ((threadIdx.x & 63) == 0) wave_part[threadIdx.x >> 6] = part;
+  __syncthreads();
+  const float total = ((wave_part[0] + wave_part[1]) + wave_part[2]) + wave_part[3];
+  const float scale = 1.0f / sqrtf(total / (float)width + eps);
+  T* dst = out + (long)r_out * ld_out;
+  for (int base = 4 * threadIdx.x; base < width; base += 1024) {
+    const f32x4 v = *reinterpret_cast<const f32x4*>(hrow + base);  // this thread wrote it above
+    const f32x4 w = base == 4 * (int)threadIdx.x ? w_first : *reinterpret_cast<const f32x4*>(weight + base);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) dst[base + e] = from_f32<T>((v[e] * scale) * w[e]);
+  }
+}
+
+// ---------------------------------------------------------------------------
 // Arg-max of float rows with the lowest index among equal maxima (NaN never
 // wins; a row without a winner gives 0).  A row is cut into chunks of
 // kArgmaxChunk elements, one workgroup each, whose winners a second small
@@ -313,6 +372,30 @@ extern "C" int ls_rmsnorm(int dtype, const float* x, const float* weight, void* 
   else
     return fail("rmsnorm: unknown dtype %d", dtype);
   return check_launch("rmsnorm");
+}
+
+// h [*, ldh] float: rows (all n_rows first rows, or the listed ones) get the slice sums P [slices][p_rows][width]
+// added (ascending), then out [n_rows, ld_out] = rmsnorm of the new rows; out == nullptr: add only.
+extern "C" int ls_add_rmsnorm(int dtype, float* h, const float* P, int slices, int p_rows, const float* weight,
+                              void* out, const int* rows, int n_rows, int width, long ldh, long ld_out, float eps,
+                              void* stream) {
+  LS_REQUIRE(n_rows > 0 && width > 0 && slices > 0 && p_rows > 0 && ldh >= width, "add_rmsnorm: bad sizes");
+  LS_REQUIRE(width % 4 == 0 && ldh % 4 == 0 && reinterpret_cast<uintptr_t>(h) % 16 == 0 &&
+                 reinterpret_cast<uintptr_t>(P) % 16 == 0,
+             "add_rmsnorm: rows must be 16-byte aligned and a multiple of 4 wide (width %d, ldh %ld)", width, ldh);
+  LS_REQUIRE(out == nullptr || (weight != nullptr && ld_out >= width && reinterpret_cast<uintptr_t>(weight) % 16 == 0),
+             "add_rmsnorm: the norm needs an aligned weight and an output row of %d elements", width);
+  LS_REQUIRE(rows != nullptr || n_rows <= p_rows, "add_rmsnorm: %d rows, the slice sums hold %d", n_rows, p_rows);
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  if (dtype == kF32)
+    hipLaunchKernelGGL(add_rmsnorm_kernel<float>, dim3(n_rows), dim3(256), 0, s, h, P, slices, p_rows, weight,
+                       (float*)out, rows, width, ldh, ld_out, eps);
+  else if (dtype == kBF16)
+    hipLaunchKernelGGL(add_rmsnorm_kernel<bf16_t>, dim3(n_rows), dim3(256), 0, s, h, P, slices, p_rows, weight,
+                       (bf16_t*)out, rows, width, ldh, ld_out, eps);
+  else
+    return fail("add_rmsnorm: unknown dtype %d", dtype);
+  return check_launch("add_rmsnorm");
 }
 
 extern "C" int ls_qk_rope_kv(int dtype, void* qkv, long ld, int n_tokens, int nq, int nkv, int d,

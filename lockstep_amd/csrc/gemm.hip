@@ -277,6 +277,64 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const void* __rest
 }
 
 // ---------------------------------------------------------------------------
+// Slice kernel (at most 16 rows): the skinny kernel's slice sums, left
+// unfolded.  A workgroup takes 16 output columns and a few consecutive K
+// slices, one per wave, and writes each slice's sums to P [slices][M][N]
+// (float); whoever consumes P adds the slices in ascending order, which is
+// the order every other kernel uses.  Cutting K over workgroups puts a
+// product with few output columns on all CUs (a CU alone streams its weights
+// slowly), at the price of the fold, which the consumer (add_rmsnorm_kernel)
+// does on the way.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void gemm_slices_kernel(const T* __restrict__ X, const T* __restrict__ W,
+                                                          float* __restrict__ P, int M, int N, int K, long ldx,
+                                                          int kslice, int aligned, int slices_per_group) {
+  typedef Atom<T> A;
+  typedef typename A::vec_t vec_t;
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int n0 = blockIdx.x * 16;
+  const int row16 = lane & 15;
+  const int g = lane >> 4;
+  const int nslices = (K + kslice - 1) / kslice;
+  const int s = blockIdx.y * slices_per_group + wave;
+  if (wave >= slices_per_group || s >= nslices) return;
+
+  f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+  const int k_begin = s * kslice;
+  const int k_end = min(K, k_begin + kslice);
+  constexpr int UNR = 8;
+  for (int k0 = k_begin; k0 < k_end; k0 += UNR * A::KCHUNK) {
+    vec_t w[UNR], x[UNR];
+#pragma unroll
+    for (int u = 0; u < UNR; ++u) {
+      const int k = k0 + u * A::KCHUNK + g * A::VEC;
+      const bool in = k0 + u * A::KCHUNK < k_end;
+      w[u] = load_vec<T>(W, n0 + row16, k, K, K, n0 + row16 < N && in, aligned);
+      x[u] = load_vec<T>(X, row16, k, K, ldx, row16 < M && in, aligned);
+    }
+#pragma unroll
+    for (int u = 0; u < UNR; ++u) {
+      if (k0 + u * A::KCHUNK >= k_end) break;  // uniform: a chunk is visited iff it starts inside the slice
+      A::mma(acc, w[u], x[u]);
+    }
+  }
+  // lane: row m = row16 of X, columns n0 + 4g .. n0 + 4g + 3
+  const int n = n0 + g * 4;
+  if (row16 < M && n < N) {
+    float* dst = P + ((long)s * M + row16) * N + n;
+    if (n + 3 < N && (N & 3) == 0) {
+      *reinterpret_cast<f32x4*>(dst) = acc;
+    } else {
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        if (n + r < N) dst[r] = acc[r];
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
 // Tiled kernel: BM x BN outputs per workgroup, four waves in a 2 x 2 grid,
 // each (BM/2) x (BN/2).  Both operands go through LDS in stages of 128 bytes
 // of K per row, double buffered: while stage i is multiplied, stage i+1 is
@@ -519,3 +577,44 @@ extern "C" int ls_gemm(int dtype, int epilogue, const void* X, const void* W, vo
 }
 
 extern "C" int ls_gemm_kslice(int K) { return ls::kslice_for(K); }
+
+// Number of K slices of a product over K (the first dimension of the partial sums of ls_gemm_slices).
+extern "C" int ls_gemm_slices_count(int K) {
+  const int kslice = ls::kslice_for(K);
+  return (K + kslice - 1) / kslice;
+}
+
+// Slice sums of X [M,K] @ W [N,K]^T for M <= 16: P [slices][M][N] float, P[s] = the sum over K slice s.
+// The product is P[0] + P[1] + ... added in this order, starting from +0.
+extern "C" int ls_gemm_slices(int dtype, const void* X, const void* W, float* P, int M, int N, int K, long ldx,
+                              void* stream) {
+  using namespace ls;
+  LS_REQUIRE(M > 0 && M <= 16 && N > 0 && K > 0, "gemm_slices: takes 1 to 16 rows, got M=%d N=%d K=%d", M, N, K);
+  LS_REQUIRE(ldx >= K && X && W && P, "gemm_slices: bad operands");
+  LS_REQUIRE(reinterpret_cast<uintptr_t>(P) % 16 == 0, "gemm_slices: the partial sums must be 16-byte aligned");
+  const int kslice = kslice_for(K);
+  const int nslices = (K + kslice - 1) / kslice;
+  const int col_blocks = (N + 15) / 16;
+  // enough groups of slices to fill the GPU, at most four slices (waves) a workgroup
+  int groups = (256 + col_blocks - 1) / col_blocks;
+  if (groups > nslices) groups = nslices;
+  if (groups < (nslices + 3) / 4) groups = (nslices + 3) / 4;
+  const int per_group = (nslices + groups - 1) / groups;
+  groups = (nslices + per_group - 1) / per_group;
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  dim3 grid(col_blocks, groups);
+  const size_t elem = dtype == kF32 ? 4 : 2;
+  const int vec = dtype == kF32 ? 4 : 8;
+  const int aligned = (K % vec == 0) && (ldx % vec == 0) && (reinterpret_cast<uintptr_t>(X) % 16 == 0) &&
+                      (reinterpret_cast<uintptr_t>(W) % 16 == 0);
+  (void)elem;
+  if (dtype == kF32)
+    hipLaunchKernelGGL(gemm_slices_kernel<float>, grid, dim3(64 * per_group), 0, s, (const float*)X, (const float*)W, P,
+                       M, N, K, ldx, kslice, aligned, per_group);
+  else if (dtype == kBF16)
+    hipLaunchKernelGGL(gemm_slices_kernel<bf16_t>, grid, dim3(64 * per_group), 0, s, (const bf16_t*)X,
+                       (const bf16_t*)W, P, M, N, K, ldx, kslice, aligned, per_group);
+  else
+    return fail("gemm_slices: unknown dtype %d", dtype);
+  return check_launch("gemm_slices");
+}

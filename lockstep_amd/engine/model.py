@@ -21,7 +21,7 @@ import torch
 from ..cache import CacheManager
 from ..config import ModelConfig, ModelSpec, config_from_dir
 from ..parts import WeightSpec, build_part, part_class
-from ..parts.base import device_epoch
+from ..parts.base import device_epoch, takes
 from ..weights.store import load_weights, weights_from_dict
 from .batch import StepContext, StepEntry, Workspace
 from .runtime import Runtime
@@ -67,6 +67,9 @@ class Model:
         self.workspace = Workspace(rt.device)
         self.use_graphs = os.environ.get("LOCKSTEP_NO_GRAPHS", "") in ("", "0")
         self._graph_safe = all(layer.mixer.graph_safe for layer in self.layers)
+        # which arrangements, and the final norm, take over an addition the previous layer left open
+        self._layer_takes_pending = [takes(layer.forward, "pending") for layer in self.layers]
+        self._final_takes_pending = takes(self.final_norm.forward, "pending")
         # one mixer of each group of equal ones is asked to prepare a step
         seen, self._preparers = set(), []
         for layer in self.layers:
@@ -150,11 +153,24 @@ class Model:
         """Launch the step's kernels on the current stream."""
         h = ctx.buf("residual", (ctx.n_tokens, self.spec.hidden_size), torch.float32)
         self.embedding.forward(ctx, ctx.token_ids, h)
+        pending = None          # an addition to h that a layer left to the next reader of h
         for run in self.schedule:
-            self.layers[run.layer].forward(ctx, run, h)
+            layer = self.layers[run.layer]
+            if self._layer_takes_pending[run.layer]:
+                pending = layer.forward(ctx, run, h, pending=pending)
+            else:
+                if pending is not None:
+                    pending.flush(ctx, h)
+                pending = None
+                layer.forward(ctx, run, h)
         if ctx.n_want:
             x = ctx.buf("final.normed", (ctx.n_want, self.spec.hidden_size), self.rt.dtype)
-            self.final_norm.forward(ctx, h, x, rows=ctx.want_rows)
+            if pending is not None and self._final_takes_pending:
+                self.final_norm.forward(ctx, h, x, rows=ctx.want_rows, pending=pending)
+            else:
+                if pending is not None:
+                    pending.flush(ctx, h)
+                self.final_norm.forward(ctx, h, x, rows=ctx.want_rows)
             if logits is None:
                 logits = torch.empty((ctx.n_want, self.spec.vocab_size), dtype=torch.float32, device=self.rt.device)
             self.head.forward(ctx, x, logits)

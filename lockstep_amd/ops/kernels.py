@@ -157,6 +157,51 @@ class Kernels:
                                  _ptr(norm_weight), c_float(eps), c_int(cols), _stream())
         self._check(self.core, code)
 
+    def gemm_slices_count(self, k: int) -> int:
+        """K slices of a product over ``k`` (first dimension of ``gemm_slices``'s output)."""
+        return self._memo(("slices", k), lambda: int(self.core.ls_gemm_slices_count(c_int(k))))
+
+    def gemm_slices(self, x: torch.Tensor, w: torch.Tensor, partials: torch.Tensor) -> None:
+        """Slice sums of ``x @ w.T`` for at most 16 rows: ``partials [slices, M, N]`` float32, to be added
+        in ascending order by the consumer (``add_rmsnorm``).  The work is cut over K as well as over N."""
+        _rows_ok(x, "gemm_slices x")
+        m, k = x.shape
+        n = w.shape[0]
+        _need(w.is_cuda and w.dim() == 2 and w.is_contiguous() and w.shape[1] == k and w.dtype == x.dtype
+              and w.dtype in DTYPE_CODE, "gemm_slices w must be [N, K] contiguous in the dtype of x")
+        _need(partials.is_cuda and partials.dtype == torch.float32 and partials.is_contiguous()
+              and partials.shape == (self.gemm_slices_count(k), m, n),
+              f"gemm_slices partials must be float32 [{self.gemm_slices_count(k)}, {m}, {n}]")
+        code = self.core.ls_gemm_slices(c_int(DTYPE_CODE[w.dtype]), _ptr(x), _ptr(w), _ptr(partials), c_int(m),
+                                        c_int(n), c_int(k), c_long(x.stride(0)), _stream())
+        self._check(self.core, code)
+
+    def add_rmsnorm(self, h: torch.Tensor, partials: torch.Tensor, weight, out, eps: float = 0.0,
+                    rows: torch.Tensor | None = None) -> None:
+        """``h[row] += partials[0][row] + partials[1][row] + ...``; then, unless ``out`` is None,
+        ``out = rmsnorm(h[row]) * weight`` as ``rmsnorm`` computes it.  ``rows`` selects rows of ``h``."""
+        _rows_ok(h, "add_rmsnorm h")
+        _need(h.dtype == torch.float32, "add_rmsnorm works on the float32 residual stream")
+        _need(partials.is_cuda and partials.dtype == torch.float32 and partials.is_contiguous()
+              and partials.dim() == 3 and partials.shape[2] == h.shape[1], "add_rmsnorm partials [slices, rows, width]")
+        n_rows = h.shape[0] if rows is None else rows.shape[0]
+        if rows is not None:
+            _need(rows.is_cuda and rows.dtype == torch.int32 and rows.is_contiguous(), "add_rmsnorm rows: int32 on the GPU")
+        dtype = torch.float32
+        ld_out = 0
+        if out is not None:
+            _rows_ok(out, "add_rmsnorm out")
+            _need(out.dtype in DTYPE_CODE and out.shape == (n_rows, h.shape[1]), "add_rmsnorm out shape or dtype")
+            _need(weight is not None and weight.dtype == torch.float32 and weight.is_contiguous()
+                  and weight.numel() == h.shape[1], "add_rmsnorm weight must be float32 [width]")
+            dtype, ld_out = out.dtype, out.stride(0)
+        if n_rows == 0:
+            return
+        code = self.core.ls_add_rmsnorm(c_int(DTYPE_CODE[dtype]), _ptr(h), _ptr(partials), c_int(partials.shape[0]),
+                                        c_int(partials.shape[1]), _ptr(weight), _ptr(out), _ptr(rows), c_int(n_rows),
+                                        c_int(h.shape[1]), c_long(h.stride(0)), c_long(ld_out), c_float(eps), _stream())
+        self._check(self.core, code)
+
     # -- rows -------------------------------------------------------------------
     def embed(self, tokens: torch.Tensor, table: torch.Tensor, out: torch.Tensor) -> None:
         _need(tokens.is_cuda and tokens.dtype == torch.int32 and tokens.dim() == 1 and tokens.is_contiguous(),

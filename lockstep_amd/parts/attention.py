@@ -19,7 +19,7 @@ import torch
 
 from ..config.base import PartSpec
 from ..ops import ADD_F32, STORE_F32
-from .base import Mixer, PagedKVSpec, WeightSpec, build_part, register_part
+from .base import DEFER_ADD_ROWS, Mixer, PagedKVSpec, PendingAdd, WeightSpec, build_part, register_part
 
 import os
 
@@ -108,9 +108,11 @@ class Attention(Mixer):
         self.position.ensure(ctx.max_position + 1, ctx.rt)
         ctx.plan_attention(self.nq // self.nkv, self.nkv, self.d, int(self.window) if self.window is not None else 0)
 
-    def forward(self, ctx, run, x, out, accumulate: bool, norm=None) -> None:
+    def forward(self, ctx, run, x, out, accumulate: bool, norm=None, defer: bool = False):
         """``norm``: when given, ``x`` is the float32 residual stream and ``norm``
-        (an RMSNorm part) is applied inside the projection."""
+        (an RMSNorm part) is applied inside the projection.  ``defer``: the addition
+        of the output projection to ``out`` may be left to the caller (a ``PendingAdd``
+        is returned)."""
         rt = ctx.rt
         k = rt.kernels
         t = ctx.n_tokens
@@ -135,8 +137,7 @@ class Attention(Mixer):
             if plan.n_combine:
                 k.attention_combine(d, ctx.seqs, plan.combine_items, plan.n_combine, nq, nkv, plan.part_acc,
                                     plan.part_ml, attn)
-            k.gemm(attn, self.w_o, out, ADD_F32 if accumulate else STORE_F32)
-            return
+            return self._project_out(ctx, attn, out, accumulate, defer)
         k.qk_rope_kv(qkv, t, nq, nkv, d, self.q_norm, self.k_norm, self.norm_eps, self.position.cos,
                      self.position.sin, self.position.rotary_dim, ctx.tok_seq, ctx.tok_pos, ctx.seqs,
                      ctx.max_position, group.table, key_pages, value_pages, group.page_size, run.writes_cache)
@@ -154,4 +155,15 @@ class Attention(Mixer):
         if plan.n_combine:
             k.attention_combine(d, ctx.seqs, plan.combine_items, plan.n_combine, nq, nkv, plan.part_acc,
                                 plan.part_ml, attn)
+        return self._project_out(ctx, attn, out, accumulate, defer)
+
+    def _project_out(self, ctx, attn, out, accumulate: bool, defer: bool):
+        k = ctx.rt.kernels
+        if defer and accumulate and 0 < ctx.n_tokens <= DEFER_ADD_ROWS:
+            slices = k.gemm_slices_count(self.nq * self.d)
+            partials = ctx.buf("attention.out_slices", (slices * ctx.n_tokens, out.shape[1]), torch.float32)
+            partials = partials.view(slices, ctx.n_tokens, out.shape[1])
+            k.gemm_slices(attn, self.w_o, partials)
+            return PendingAdd(partials)
         k.gemm(attn, self.w_o, out, ADD_F32 if accumulate else STORE_F32)
+        return None

@@ -189,6 +189,31 @@ def build_part(spec: PartSpec, prefix: str = "", **extra: Any) -> Part:
     return part_class(spec.kind)(spec, prefix, **extra)
 
 
+class PendingAdd:
+    """A matrix product that still has to be added to the residual stream, left as the sums of
+    its K slices: ``stream += partials[0] + partials[1] + ...`` (in this order).  A part that is
+    called with ``defer=True`` may return one instead of adding itself; the next reader of the
+    stream (a norm that takes ``pending``, or ``flush``) does the addition on its way."""
+
+    def __init__(self, partials):
+        self.partials = partials        # [slices, rows, width] float32
+
+    def flush(self, ctx, stream, rows=None) -> None:
+        ctx.rt.kernels.add_rmsnorm(stream, self.partials, None, None, 0.0, rows)
+
+
+#: steps of at most this many tokens leave the residual additions of the output products to the
+#: following norm (their work is then cut over K as well, which fills the GPU); 0 switches it off
+DEFER_ADD_ROWS = int(__import__("os").environ.get("LOCKSTEP_DEFER_ADD_ROWS", "16"))
+
+
+def takes(function, name: str) -> bool:
+    """Whether a part's method accepts the optional keyword ``name``."""
+    import inspect
+
+    return name in inspect.signature(function).parameters
+
+
 # Captured graphs hold the addresses of device tensors that parts own (tables that grow with
 # the longest position, for instance).  A part that replaces such a tensor bumps the epoch;
 # the model keys its graphs on it.

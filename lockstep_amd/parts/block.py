@@ -2,7 +2,7 @@
 
 from __future__ import annotations
 
-from .base import Arrangement, build_part, register_part
+from .base import Arrangement, PendingAdd, build_part, register_part, takes
 
 
 @register_part("prenorm_residual")
@@ -26,6 +26,11 @@ class PreNormResidual(Arrangement):
         self.feed_forward = build_part(layer_spec.feed_forward, self.join(base, p["feed_forward_prefix"]))
         self._fuse_mixer = self._fuses(self._mixer, self.mixer_norm)
         self._fuse_ff = self._fuses(self.feed_forward, self.feed_forward_norm)
+        # parts that can leave their residual addition to the next norm (see PendingAdd)
+        self._defer_mixer = takes(self._mixer.forward, "defer")
+        self._defer_ff = takes(self.feed_forward.forward, "defer")
+        self._norm1_pending = takes(self.mixer_norm.forward, "pending")
+        self._norm2_pending = takes(self.feed_forward_norm.forward, "pending")
 
     @classmethod
     def weight_specs(cls, layer_spec, prefix: str = ""):
@@ -65,18 +70,40 @@ class PreNormResidual(Arrangement):
         return (getattr(norm, "kind", "") == "rmsnorm"
                 and "norm" in inspect.signature(part.forward).parameters)
 
-    def forward(self, ctx, run, h) -> None:
+    def forward(self, ctx, run, h, pending=None):
+        """``pending``: an addition to ``h`` that the previous layer left to its reader.  Returns
+        the one this layer leaves (or None)."""
         rt = ctx.rt
         small = ctx.n_tokens <= self.FUSE_NORM_ROWS
+        if pending is not None and (small and self._fuse_mixer or not self._norm1_pending):
+            pending.flush(ctx, h)
+            pending = None
         if small and self._fuse_mixer:
-            self._mixer.forward(ctx, run, h, h, accumulate=True, norm=self.mixer_norm)
+            mixed = self._mixer.forward(ctx, run, h, h, accumulate=True, norm=self.mixer_norm)
         else:
             x = ctx.buf("block.normed", (ctx.n_tokens, h.shape[1]), rt.dtype)
-            self.mixer_norm.forward(ctx, h, x)
-            self._mixer.forward(ctx, run, x, h, accumulate=True)
+            if pending is not None:
+                self.mixer_norm.forward(ctx, h, x, pending=pending)
+            else:
+                self.mixer_norm.forward(ctx, h, x)
+            if self._defer_mixer:
+                mixed = self._mixer.forward(ctx, run, x, h, accumulate=True, defer=True)
+            else:
+                mixed = self._mixer.forward(ctx, run, x, h, accumulate=True)
+        mixed = mixed if isinstance(mixed, PendingAdd) else None
+        if mixed is not None and (small and self._fuse_ff or not self._norm2_pending):
+            mixed.flush(ctx, h)
+            mixed = None
         if small and self._fuse_ff:
-            self.feed_forward.forward(ctx, h, h, accumulate=True, norm=self.feed_forward_norm)
+            left = self.feed_forward.forward(ctx, h, h, accumulate=True, norm=self.feed_forward_norm)
         else:
             x = ctx.buf("block.normed", (ctx.n_tokens, h.shape[1]), rt.dtype)
-            self.feed_forward_norm.forward(ctx, h, x)
-            self.feed_forward.forward(ctx, x, h, accumulate=True)
+            if mixed is not None:
+                self.feed_forward_norm.forward(ctx, h, x, pending=mixed)
+            else:
+                self.feed_forward_norm.forward(ctx, h, x)
+            if self._defer_ff:
+                left = self.feed_forward.forward(ctx, x, h, accumulate=True, defer=True)
+            else:
+                left = self.feed_forward.forward(ctx, x, h, accumulate=True)
+        return left if isinstance(left, PendingAdd) else None

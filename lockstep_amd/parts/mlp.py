@@ -11,7 +11,7 @@ import torch
 
 from ..config.base import PartSpec
 from ..ops import ADD_F32, STORE_F32, SWIGLU, interleave_gate_up
-from .base import FeedForward, WeightSpec, register_part
+from .base import DEFER_ADD_ROWS, FeedForward, PendingAdd, WeightSpec, register_part
 
 
 @register_part("gated_mlp")
@@ -41,13 +41,21 @@ class GatedMLP(FeedForward):
         self.w_gate_up = rt.matrix(interleave_gate_up(gate, up))
         self.w_down = rt.matrix(weights.get(f"{self.prefix}.down_proj.weight"))
 
-    def forward(self, ctx, x, out, accumulate: bool, norm=None) -> None:
+    def forward(self, ctx, x, out, accumulate: bool, norm=None, defer: bool = False):
         """``norm``: when given, ``x`` is the float32 residual stream and ``norm``
-        (an RMSNorm part) is applied inside the first matrix product."""
+        (an RMSNorm part) is applied inside the first matrix product.  ``defer``: the
+        addition to ``out`` may be left to the caller (a ``PendingAdd`` is returned)."""
         rt = ctx.rt
         act = ctx.buf("mlp.act", (ctx.n_tokens, self.inter), rt.dtype)
         if norm is None:
             rt.kernels.gemm(x, self.w_gate_up, act, SWIGLU)
         else:
             rt.kernels.gemm(x, self.w_gate_up, act, SWIGLU, norm_weight=norm.weight, eps=norm.eps)
+        if defer and accumulate and 0 < ctx.n_tokens <= DEFER_ADD_ROWS:
+            slices = rt.kernels.gemm_slices_count(self.inter)
+            partials = ctx.buf("mlp.down_slices", (slices * ctx.n_tokens, out.shape[1]), torch.float32)
+            partials = partials.view(slices, ctx.n_tokens, out.shape[1])
+            rt.kernels.gemm_slices(act, self.w_down, partials)
+            return PendingAdd(partials)
         rt.kernels.gemm(act, self.w_down, out, ADD_F32 if accumulate else STORE_F32)
+        return None

@@ -28,5 +28,9 @@ class RMSNorm(Norm):
     def load(self, weights, rt) -> None:
         self.weight = rt.vector(weights.get(self.tensor_name(self.spec, self.prefix)))
 
-    def forward(self, ctx, x, out, rows=None) -> None:
-        ctx.rt.kernels.rmsnorm(x, self.weight, out, self.eps, rows)
+    def forward(self, ctx, x, out, rows=None, pending=None) -> None:
+        """``pending`` (a ``PendingAdd``): added to ``x`` first, in the same launch."""
+        if pending is not None:
+            ctx.rt.kernels.add_rmsnorm(x, pending.partials, self.weight, out, self.eps, rows)
+        else:
+            ctx.rt.kernels.rmsnorm(x, self.weight, out, self.eps, rows)

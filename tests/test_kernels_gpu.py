@@ -561,3 +561,42 @@ def test_gemm_with_fused_norm_equals_norm_then_gemm(dtype, m, n, k):
     with pytest.raises(KernelError):
         K().gemm(torch.zeros(17, k, device="cuda"), w, torch.empty(17, n, dtype=dtype, device="cuda"), STORE,
                  norm_weight=nw, eps=eps)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("m", [1, 8, 16])
+@pytest.mark.parametrize("n,k", [(1024, 3072), (96, 520), (1024, 2048), (40, 64)])
+def test_slice_sums_and_fused_add_norm_equal_the_separate_kernels(dtype, m, n, k):
+    """gemm_slices + add_rmsnorm give the bits of gemm(ADD_F32) + rmsnorm: the residual row and the
+    normalised row; also for a list of rows and for the plain addition."""
+    from lockstep_amd.ops import ADD_F32
+
+    g = torch.Generator().manual_seed(n + k + m)
+    x = torch.randn(m, k, generator=g).to(dtype).cuda()
+    w = (torch.randn(n, k, generator=g) * 0.1).to(dtype).cuda()
+    h0 = torch.randn(m, n, generator=g).cuda()
+    weight = (1 + 0.1 * torch.randn(n, generator=g)).cuda()
+    eps = 1e-5
+    h_ref = h0.clone()
+    K().gemm(x, w, h_ref, ADD_F32)
+    y_ref = torch.empty(m, n, dtype=dtype, device="cuda")
+    K().rmsnorm(h_ref, weight, y_ref, eps)
+    slices = K().gemm_slices_count(k)
+    partials = torch.full((slices, m, n), float("nan"), device="cuda")
+    K().gemm_slices(x, w, partials)
+    assert not torch.isnan(partials).any()
+    h = h0.clone()
+    y = torch.empty(m, n, dtype=dtype, device="cuda")
+    K().add_rmsnorm(h, partials, weight, y, eps)
+    assert torch.equal(h, h_ref) and torch.equal(y, y_ref)
+    want = (h0.double() + x.double() @ w.double().T)
+    assert rel_err(h, want) < (1e-5 if dtype is torch.float32 else 2e-2)
+    h = h0.clone()
+    K().add_rmsnorm(h, partials, None, None)
+    assert torch.equal(h, h_ref)
+    rows = torch.tensor([m - 1, 0][: min(2, m)], dtype=torch.int32).cuda()
+    h = h0.clone()
+    y = torch.empty(rows.shape[0], n, dtype=dtype, device="cuda")
+    K().add_rmsnorm(h, partials, weight, y, eps, rows)
+    assert torch.equal(y, y_ref[rows.long()])
+    assert torch.equal(h[rows.long()], h_ref[rows.long()])
