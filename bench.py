@@ -189,7 +189,7 @@ def main(argv=None) -> int:
     achieved = bytes_step / (elapsed / args.steps)
 
     record = {
-        "metric": "decode tok/s at batch 8 (Qwen3-0.6B sizes, 512-token prompts, greedy)",
+        "metric": f"decode tok/s at batch {args.batch} (Qwen3-0.6B sizes, {args.prompt_len}-token prompts, greedy)",
         "value": round(value, 1),
         "unit": "tokens/s",
         "n_gpus": 1,

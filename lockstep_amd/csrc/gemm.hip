@@ -277,7 +277,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const void* __rest
 }
 
 // ---------------------------------------------------------------------------
-// Slice kernel (at most 16 rows): the skinny kernel's slice sums, left
+// Slice kernel (at most 64 rows): the skinny kernel's slice sums, left
 // unfolded.  A workgroup takes 16 output columns and a few consecutive K
 // slices, one per wave, and writes each slice's sums to P [slices][M][N]
 // (float); whoever consumes P adds the slices in ascending order, which is
@@ -286,7 +286,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const void* __rest
 // slowly), at the price of the fold, which the consumer (add_rmsnorm_kernel)
 // does on the way.
 // ---------------------------------------------------------------------------
-template <typename T>
+template <typename T, int MT>
 __global__ __launch_bounds__(256) void gemm_slices_kernel(const T* __restrict__ X, const T* __restrict__ W,
                                                           float* __restrict__ P, int M, int N, int K, long ldx,
                                                           int kslice, int aligned, int slices_per_group) {
@@ -301,35 +301,43 @@ __global__ __launch_bounds__(256) void gemm_slices_kernel(const T* __restrict__ 
   const int s = blockIdx.y * slices_per_group + wave;
   if (wave >= slices_per_group || s >= nslices) return;
 
-  f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+  f32x4 acc[MT];
+#pragma unroll
+  for (int j = 0; j < MT; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
   const int k_begin = s * kslice;
   const int k_end = min(K, k_begin + kslice);
-  constexpr int UNR = 8;
+  constexpr int UNR = MT == 1 ? 8 : 4;
   for (int k0 = k_begin; k0 < k_end; k0 += UNR * A::KCHUNK) {
-    vec_t w[UNR], x[UNR];
+    vec_t w[UNR], x[MT][UNR];
 #pragma unroll
     for (int u = 0; u < UNR; ++u) {
       const int k = k0 + u * A::KCHUNK + g * A::VEC;
       const bool in = k0 + u * A::KCHUNK < k_end;
       w[u] = load_vec<T>(W, n0 + row16, k, K, K, n0 + row16 < N && in, aligned);
-      x[u] = load_vec<T>(X, row16, k, K, ldx, row16 < M && in, aligned);
+#pragma unroll
+      for (int j = 0; j < MT; ++j)
+        x[j][u] = load_vec<T>(X, j * 16 + row16, k, K, ldx, j * 16 + row16 < M && in, aligned);
     }
 #pragma unroll
     for (int u = 0; u < UNR; ++u) {
       if (k0 + u * A::KCHUNK >= k_end) break;  // uniform: a chunk is visited iff it starts inside the slice
-      A::mma(acc, w[u], x[u]);
+#pragma unroll
+      for (int j = 0; j < MT; ++j) A::mma(acc[j], w[u], x[j][u]);
     }
   }
-  // lane: row m = row16 of X, columns n0 + 4g .. n0 + 4g + 3
+  // lane: rows j * 16 + row16 of X, columns n0 + 4g .. n0 + 4g + 3
   const int n = n0 + g * 4;
-  if (row16 < M && n < N) {
-    float* dst = P + ((long)s * M + row16) * N + n;
+#pragma unroll
+  for (int j = 0; j < MT; ++j) {
+    const int m = j * 16 + row16;
+    if (m >= M || n >= N) continue;
+    float* dst = P + ((long)s * M + m) * N + n;
     if (n + 3 < N && (N & 3) == 0) {
-      *reinterpret_cast<f32x4*>(dst) = acc;
+      *reinterpret_cast<f32x4*>(dst) = acc[j];
     } else {
 #pragma unroll
       for (int r = 0; r < 4; ++r)
-        if (n + r < N) dst[r] = acc[r];
+        if (n + r < N) dst[r] = acc[j][r];
     }
   }
 }
@@ -584,12 +592,12 @@ extern "C" int ls_gemm_slices_count(int K) {
   return (K + kslice - 1) / kslice;
 }
 
-// Slice sums of X [M,K] @ W [N,K]^T for M <= 16: P [slices][M][N] float, P[s] = the sum over K slice s.
+// Slice sums of X [M,K] @ W [N,K]^T for M <= 64: P [slices][M][N] float, P[s] = the sum over K slice s.
 // The product is P[0] + P[1] + ... added in this order, starting from +0.
 extern "C" int ls_gemm_slices(int dtype, const void* X, const void* W, float* P, int M, int N, int K, long ldx,
                               void* stream) {
   using namespace ls;
-  LS_REQUIRE(M > 0 && M <= 16 && N > 0 && K > 0, "gemm_slices: takes 1 to 16 rows, got M=%d N=%d K=%d", M, N, K);
+  LS_REQUIRE(M > 0 && M <= 64 && N > 0 && K > 0, "gemm_slices: takes 1 to 64 rows, got M=%d N=%d K=%d", M, N, K);
   LS_REQUIRE(ldx >= K && X && W && P, "gemm_slices: bad operands");
   LS_REQUIRE(reinterpret_cast<uintptr_t>(P) % 16 == 0, "gemm_slices: the partial sums must be 16-byte aligned");
   const int kslice = kslice_for(K);
@@ -608,13 +616,21 @@ extern "C" int ls_gemm_slices(int dtype, const void* X, const void* W, float* P,
   const int aligned = (K % vec == 0) && (ldx % vec == 0) && (reinterpret_cast<uintptr_t>(X) % 16 == 0) &&
                       (reinterpret_cast<uintptr_t>(W) % 16 == 0);
   (void)elem;
-  if (dtype == kF32)
-    hipLaunchKernelGGL(gemm_slices_kernel<float>, grid, dim3(64 * per_group), 0, s, (const float*)X, (const float*)W, P,
-                       M, N, K, ldx, kslice, aligned, per_group);
-  else if (dtype == kBF16)
-    hipLaunchKernelGGL(gemm_slices_kernel<bf16_t>, grid, dim3(64 * per_group), 0, s, (const bf16_t*)X,
-                       (const bf16_t*)W, P, M, N, K, ldx, kslice, aligned, per_group);
-  else
+  const int mt = (M + 15) / 16;
+#define LS_SLICES(T_, MT_)                                                                                       \
+  hipLaunchKernelGGL((gemm_slices_kernel<T_, MT_>), grid, dim3(64 * per_group), 0, s, (const T_*)X, (const T_*)W, P, M, \
+                     N, K, ldx, kslice, aligned, per_group)
+#define LS_SLICES_MT(T_)                                              \
+  if (mt == 1) LS_SLICES(T_, 1); else if (mt == 2) LS_SLICES(T_, 2); \
+  else if (mt == 3) LS_SLICES(T_, 3); else LS_SLICES(T_, 4)
+  if (dtype == kF32) {
+    LS_SLICES_MT(float);
+  } else if (dtype == kBF16) {
+    LS_SLICES_MT(bf16_t);
+  } else {
     return fail("gemm_slices: unknown dtype %d", dtype);
+  }
+#undef LS_SLICES_MT
+#undef LS_SLICES
   return check_launch("gemm_slices");
 }

@@ -162,7 +162,7 @@ class Kernels:
         return self._memo(("slices", k), lambda: int(self.core.ls_gemm_slices_count(c_int(k))))
 
     def gemm_slices(self, x: torch.Tensor, w: torch.Tensor, partials: torch.Tensor) -> None:
-        """Slice sums of ``x @ w.T`` for at most 16 rows: ``partials [slices, M, N]`` float32, to be added
+        """Slice sums of ``x @ w.T`` for at most 64 rows: ``partials [slices, M, N]`` float32, to be added
         in ascending order by the consumer (``add_rmsnorm``).  The work is cut over K as well as over N."""
         _rows_ok(x, "gemm_slices x")
         m, k = x.shape

@@ -204,7 +204,7 @@ class PendingAdd:
 
 #: steps of at most this many tokens leave the residual additions of the output products to the
 #: following norm (their work is then cut over K as well, which fills the GPU); 0 switches it off
-DEFER_ADD_ROWS = int(__import__("os").environ.get("LOCKSTEP_DEFER_ADD_ROWS", "16"))
+DEFER_ADD_ROWS = int(__import__("os").environ.get("LOCKSTEP_DEFER_ADD_ROWS", "64"))
 
 
 def takes(function, name: str) -> bool:

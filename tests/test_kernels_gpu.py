@@ -564,7 +564,7 @@ def test_gemm_with_fused_norm_equals_norm_then_gemm(dtype, m, n, k):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("m", [1, 8, 16])
+@pytest.mark.parametrize("m", [1, 8, 16, 17, 40, 64])
 @pytest.mark.parametrize("n,k", [(1024, 3072), (96, 520), (1024, 2048), (40, 64)])
 def test_slice_sums_and_fused_add_norm_equal_the_separate_kernels(dtype, m, n, k):
     """gemm_slices + add_rmsnorm give the bits of gemm(ADD_F32) + rmsnorm: the residual row and the
