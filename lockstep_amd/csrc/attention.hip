@@ -1481,28 +1481,56 @@ constexpr size_t kCoopLdsExtra = 2 * 16 * sizeof(int) + kCoopExtra + 2 * D * 4; 
 constexpr int coop_bufs(size_t elem) {
   return 2 * (2 * kTileKeys * D * elem) + kCoopLdsExtra <= kLdsLimit ? 2 : 1;
 }
-constexpr int kCoopBufsF32 = coop_bufs(4);
-constexpr int kCoopBufsBF16 = coop_bufs(2);
-static size_t coop_lds_bytes(int dtype) {
-  const size_t elem = dtype == kF32 ? 4 : 2;
-  return (dtype == kF32 ? kCoopBufsF32 : kCoopBufsBF16) * (2 * (size_t)kTileKeys * D * elem) + kCoopLdsExtra;
-}
-static bool coop_supported(int dtype) {
-  const size_t bytes = coop_lds_bytes(dtype);
+template <typename T, int NBUF>
+constexpr size_t coop_kernel_lds() { return NBUF * (2 * (size_t)kTileKeys * D * sizeof(T)) + kCoopLdsExtra; }
+
+// Whether this instantiation can be launched (its LDS fits; above 64 KB the
+// function attribute is raised once).
+template <typename T, int NBUF, bool FUSE>
+static bool coop_kernel_ready() {
+  constexpr size_t bytes = coop_kernel_lds<T, NBUF>();
   if (bytes > kLdsLimit) return false;
   if (bytes <= 64 * 1024) return true;
-  static int state[2] = {0, 0};
-  int& st = state[dtype == kF32 ? 0 : 1];
-  if (st == 0) {
-    hipError_t e = dtype == kF32
-        ? hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_coop_kernel<float, kCoopBufsF32, false>),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes)
-        : hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_coop_kernel<bf16_t, kCoopBufsBF16, false>),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+  static int state = 0;  // 0 unknown, 1 granted, -1 refused
+  if (state == 0) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_coop_kernel<T, NBUF, FUSE>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
     if (e != hipSuccess) (void)hipGetLastError();
-    st = e == hipSuccess ? 1 : -1;
+    state = e == hipSuccess ? 1 : -1;
   }
-  return st == 1;
+  return state == 1;
+}
+
+// Launch with two buffers (the next tile in flight while one is worked on)
+// where they fit; when the grid brings at least two workgroups per CU, with
+// one buffer instead, so that two workgroups share a CU and overlap each
+// other's loads.
+template <typename T, bool FUSE>
+static int launch_coop(dim3 grid, hipStream_t s, const void* q, long ldq, const void* k_pages, const void* v_pages,
+                       int nkv, int page_size, int page_shift, const int* table, int table_stride, const void* seqs,
+                       const void* items, void* out, long ldo, float* part_acc, float* part_ml, int G, float scale,
+                       int window, DecodeFuse<T> fz) {
+  constexpr int BUFS = coop_bufs(sizeof(T));
+  const bool crowded = (long)grid.x * grid.y >= 512;
+#define LS_COOP(NBUF_)                                                                                              \
+  hipLaunchKernelGGL((attention_coop_kernel<T, NBUF_, FUSE>), grid, dim3(256), (coop_kernel_lds<T, NBUF_>()), s,       \
+                     (const T*)q, ldq, (const T*)k_pages, (const T*)v_pages, nkv, page_size, page_shift, table,        \
+                     table_stride, (const SeqMeta*)seqs, (const AttnItem*)items, (T*)out, ldo, part_acc, part_ml, G,   \
+                     scale, window, fz)
+  if (BUFS == 2 && !(crowded && coop_kernel_ready<T, 1, FUSE>())) {
+    if (!coop_kernel_ready<T, 2, FUSE>()) return fail("attention: the cooperative kernel does not fit into LDS");
+    LS_COOP(2);
+  } else {
+    if (!coop_kernel_ready<T, 1, FUSE>()) return fail("attention: the cooperative kernel does not fit into LDS");
+    LS_COOP(1);
+  }
+#undef LS_COOP
+  return 0;
+}
+
+static bool coop_supported(int dtype) {
+  return dtype == kF32 ? coop_kernel_ready<float, coop_bufs(4), false>()
+                       : coop_kernel_ready<bf16_t, coop_bufs(2), false>();
 }
 // 1 if the cooperative kernel (variant 3, work items of at most 16 rows) can run for this dtype.
 extern "C" int ls_attn_coop_supported(int dtype) { return coop_supported(dtype) ? 1 : 0; }
@@ -1512,21 +1540,8 @@ extern "C" int ls_attn_coop_supported(int dtype) { return coop_supported(dtype) 
 static bool decode_fused_supported(int dtype) {
   const size_t elem = dtype == kF32 ? 4 : 2;
   if (16 * D * elem > (size_t)NB * 64 * 16) return false;
-  const size_t bytes = coop_lds_bytes(dtype);
-  if (bytes > kLdsLimit) return false;
-  if (bytes <= 64 * 1024) return true;
-  static int state[2] = {0, 0};
-  int& st = state[dtype == kF32 ? 0 : 1];
-  if (st == 0) {
-    hipError_t e = dtype == kF32
-        ? hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_coop_kernel<float, kCoopBufsF32, true>),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes)
-        : hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_coop_kernel<bf16_t, kCoopBufsBF16, true>),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
-    if (e != hipSuccess) (void)hipGetLastError();
-    st = e == hipSuccess ? 1 : -1;
-  }
-  return st == 1;
+  return dtype == kF32 ? coop_kernel_ready<float, coop_bufs(4), true>()
+                       : coop_kernel_ready<bf16_t, coop_bufs(2), true>();
 }
 // 1 if ls_attention_decode can run for this dtype.
 extern "C" int ls_attn_decode_fused_supported(int dtype) { return decode_fused_supported(dtype) ? 1 : 0; }
@@ -1568,23 +1583,20 @@ extern "C" int ls_attention_decode(int dtype, const void* qkv, long ld, void* k_
   dim3 grid(n_items, nkv);
   int page_shift = 0;
   while ((1 << page_shift) < page_size) ++page_shift;
-  const size_t bytes = coop_lds_bytes(dtype);
+  int rc = 0;
   if (dtype == kF32) {
     DecodeFuse<float> fz{q_weight, k_weight, eps, cos_table, sin_table, rot, nq, write_kv, (float*)k_pages, (float*)v_pages};
-    hipLaunchKernelGGL((attention_coop_kernel<float, kCoopBufsF32, true>), grid, dim3(256), bytes, s,
-                       (const float*)qkv, ld, (const float*)k_pages, (const float*)v_pages, nkv, page_size, page_shift,
-                       table, table_stride, (const SeqMeta*)seqs, (const AttnItem*)items, (float*)out, ldo, part_acc,
-                       part_ml, G, scale, window, fz);
+    rc = launch_coop<float, true>(grid, s, qkv, ld, k_pages, v_pages, nkv, page_size, page_shift, table, table_stride,
+                                  seqs, items, out, ldo, part_acc, part_ml, G, scale, window, fz);
   } else if (dtype == kBF16) {
     DecodeFuse<bf16_t> fz{q_weight, k_weight, eps, cos_table, sin_table, rot, nq, write_kv, (bf16_t*)k_pages,
                           (bf16_t*)v_pages};
-    hipLaunchKernelGGL((attention_coop_kernel<bf16_t, kCoopBufsBF16, true>), grid, dim3(256), bytes, s,
-                       (const bf16_t*)qkv, ld, (const bf16_t*)k_pages, (const bf16_t*)v_pages, nkv, page_size,
-                       page_shift, table, table_stride, (const SeqMeta*)seqs, (const AttnItem*)items, (bf16_t*)out, ldo,
-                       part_acc, part_ml, G, scale, window, fz);
+    rc = launch_coop<bf16_t, true>(grid, s, qkv, ld, k_pages, v_pages, nkv, page_size, page_shift, table, table_stride,
+                                   seqs, items, out, ldo, part_acc, part_ml, G, scale, window, fz);
   } else {
     return fail("decode attention: unknown dtype %d", dtype);
   }
+  if (rc != 0) return rc;
   return check_launch("attention (decode, fused)");
 }
 
@@ -1644,19 +1656,17 @@ extern "C" int ls_attention(int dtype, const void* q, long ldq, const void* k_pa
                max_rows);
     LS_REQUIRE(coop_supported(dtype), "attention: the cooperative variant does not fit into LDS for this head size");
     LS_REQUIRE(page_size >= 8, "attention: the cooperative variant needs pages of at least 8 keys, got %d", page_size);
-    const size_t bytes = coop_lds_bytes(dtype);
+    int rc = 0;
     if (dtype == kF32)
-      hipLaunchKernelGGL((attention_coop_kernel<float, kCoopBufsF32, false>), grid, dim3(256), bytes, s,
-                         (const float*)q, ldq, (const float*)k_pages, (const float*)v_pages, nkv, page_size,
-                         page_shift, table, table_stride, (const SeqMeta*)seqs, (const AttnItem*)items, (float*)out,
-                         ldo, part_acc, part_ml, G, scale, window, DecodeFuse<float>{});
+      rc = launch_coop<float, false>(grid, s, q, ldq, k_pages, v_pages, nkv, page_size, page_shift, table, table_stride,
+                                     seqs, items, out, ldo, part_acc, part_ml, G, scale, window, DecodeFuse<float>{});
     else if (dtype == kBF16)
-      hipLaunchKernelGGL((attention_coop_kernel<bf16_t, kCoopBufsBF16, false>), grid, dim3(256), bytes, s,
-                         (const bf16_t*)q, ldq, (const bf16_t*)k_pages, (const bf16_t*)v_pages, nkv, page_size,
-                         page_shift, table, table_stride, (const SeqMeta*)seqs, (const AttnItem*)items, (bf16_t*)out,
-                         ldo, part_acc, part_ml, G, scale, window, DecodeFuse<bf16_t>{});
+      rc = launch_coop<bf16_t, false>(grid, s, q, ldq, k_pages, v_pages, nkv, page_size, page_shift, table,
+                                      table_stride, seqs, items, out, ldo, part_acc, part_ml, G, scale, window,
+                                      DecodeFuse<bf16_t>{});
     else
       return fail("attention: unknown dtype %d", dtype);
+    if (rc != 0) return rc;
     return check_launch("attention (cooperative)");
   }
   if (variant == 4) {
