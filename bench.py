@@ -6,7 +6,10 @@ prompt, with random weights at the Qwen3-0.6B layer sizes.
 
 A "step" is one decode step of the whole batch: the engine's step function
 followed by greedy sampling of every request's next token, which is fed back
-in the next step.  Requests start from 512-token random prompts (prefilled
+in the next step.  By default the pick is fed back on the device
+(``Model.decode_greedy``: the captured step is launched K times and the host
+reads the tokens once at the end); ``--host-sampling`` brings every step's
+logits to the ``Sampler`` on the host instead.  Requests start from 512-token random prompts (prefilled
 outside the timed region); K timed steps follow W untimed ones, bracketed by
 device synchronisation.  One JSON line is printed.  The reference publishes no
 tokens-a-second figure (it states ratios only), so ``vs_baseline`` is null.
@@ -79,7 +82,8 @@ def random_prompts(n: int, length: int, vocab: int, seed: int):
     return [torch.randint(0, vocab, (length,), generator=g).tolist() for _ in range(n)]
 
 
-def measure_decode(model, cfg, batch: int, prompt_len: int, steps: int, warmup: int, page_size: int):
+def measure_decode(model, cfg, batch: int, prompt_len: int, steps: int, warmup: int, page_size: int,
+                   device_loop: bool = True):
     """(seconds of the timed steps, mean context length during them)."""
     import torch
 
@@ -106,6 +110,12 @@ def measure_decode(model, cfg, batch: int, prompt_len: int, steps: int, warmup: 
         return tokens
 
     def decode(tokens, n):
+        if n <= 0:
+            return tokens
+        if device_loop:
+            # the greedy pick of every step is fed back on the device; the host reads the tokens at the end
+            picked = model.decode_greedy(cache, [r.uid for r in requests], tokens, n)
+            return picked[-1].tolist()
         for _ in range(n):
             logits = model.step(cache, [StepEntry(r.uid, [t], [0]) for r, t in zip(requests, tokens)])
             tokens = sampler.sample(logits, requests)
@@ -162,6 +172,8 @@ def main(argv=None) -> int:
     p.add_argument("--page-size", type=int, default=16)
     p.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     p.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points and the prefill")
+    p.add_argument("--host-sampling", action="store_true",
+                   help="pick every step's tokens on the host (Model.step + Sampler) instead of the device-side loop")
     p.add_argument("--only-prefill", action="store_true",
                    help="run the prefill measurement alone and print its record (for profiling)")
     args = p.parse_args(argv)
@@ -182,7 +194,7 @@ def main(argv=None) -> int:
         return 0
 
     elapsed, context = measure_decode(model, cfg, args.batch, args.prompt_len, args.steps, args.warmup,
-                                      args.page_size)
+                                      args.page_size, not args.host_sampling)
     ms_per_step = 1e3 * elapsed / args.steps
     value = args.batch * args.steps / elapsed
     bytes_step = decode_bytes(cfg, args.batch, context, element)
@@ -209,6 +221,7 @@ def main(argv=None) -> int:
             "global_batch": args.batch, "prompt_len": args.prompt_len, "new_tokens": args.steps,
             "seq_len": args.prompt_len + args.steps, "max_context": 4096, "page_size": args.page_size,
             "prefill_len": args.prefill_len, "parallelism": "single GPU", "hip_graphs": bool(model.use_graphs),
+            "token_feedback": "host" if args.host_sampling else "device",
         },
         "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": PEAK_HBM / 1e9,
                      "unit": "GB/s", "frac": round(achieved / PEAK_HBM, 4)},
@@ -222,7 +235,8 @@ def main(argv=None) -> int:
                              "frac": round(flops / seconds / PEAK_FLOPS[args.dtype], 4)}
         points = {}
         for batch, steps in ((1, min(args.steps, 128)), (64, min(args.steps, 64))):
-            t, _ = measure_decode(model, cfg, batch, args.prompt_len, steps, min(args.warmup, 4), args.page_size)
+            t, _ = measure_decode(model, cfg, batch, args.prompt_len, steps, min(args.warmup, 4), args.page_size,
+                                  not args.host_sampling)
             points[f"decode_b{batch}"] = round(batch * steps / t, 1)
         record["points"] = points
     torch.cuda.synchronize()

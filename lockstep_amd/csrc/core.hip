@@ -338,6 +338,46 @@ __global__ __launch_bounds__(256) void argmax_final_kernel(const float* __restri
   if (threadIdx.x == 0) out[blockIdx.x] = bi == 0x7fffffff ? 0 : bi;
 }
 
+// ---------------------------------------------------------------------------
+// Between two decode steps that run without the host: every request takes the
+// token that was picked for it as its next input, at the next position.  The
+// step's metadata (see the engine's upload) is advanced in place: token ids,
+// token positions, the requests' rows (q_start, kv_len) and the copies of those
+// rows inside the attention work items.  The picked tokens are also appended
+// to a ring the host reads later: ring[step][request], step = *counter, which
+// is incremented.
+// ---------------------------------------------------------------------------
+struct AdvanceLists {
+  int offset[4];  // first int of a list of 16-int attention items inside meta
+  int count[4];   // items in it
+};
+
+__global__ __launch_bounds__(256) void advance_decode_kernel(int* __restrict__ meta, int n_seqs, int off_tokens,
+                                                             int off_positions, int off_seqs,
+                                                             const int* __restrict__ picked, int* __restrict__ ring,
+                                                             int* __restrict__ counter, AdvanceLists lists) {
+  // one workgroup, so that the counter can be read by all of it before one thread moves it on
+  const int tid = threadIdx.x;
+  const int stride = blockDim.x;
+  const int step = *counter;
+  for (int i = tid; i < n_seqs; i += stride) {
+    const int token = picked[i];
+    meta[off_tokens + i] = token;
+    meta[off_positions + i] += 1;
+    meta[off_seqs + 8 * i + 2] += 1;  // q_start
+    meta[off_seqs + 8 * i + 3] += 1;  // kv_len
+    ring[(long)step * n_seqs + i] = token;
+  }
+#pragma unroll
+  for (int l = 0; l < 4; ++l)
+    for (int i = tid; i < lists.count[l]; i += stride) {
+      meta[lists.offset[l] + 16 * i + 10] += 1;  // AttnItem.sm.q_start
+      meta[lists.offset[l] + 16 * i + 11] += 1;  // AttnItem.sm.kv_len
+    }
+  __syncthreads();
+  if (tid == 0) *counter = step + 1;
+}
+
 }  // namespace ls
 
 LS_DEFINE_ERROR_API
@@ -474,4 +514,23 @@ extern "C" int ls_argmax(const float* x, int* out, int rows, int width, long ld,
                      chunks);
   if (chunks > 1) hipLaunchKernelGGL(argmax_final_kernel, dim3(rows), dim3(256), 0, s, part_v, part_i, out, chunks);
   return check_launch("argmax");
+}
+
+// meta: the step's uploaded metadata; picked [n_seqs]: the tokens chosen for the requests; ring
+// [steps][n_seqs] and counter: where the loop's output goes.  lists: up to four (offset, count) pairs of
+// attention work-item lists inside meta (offset in ints; unused pairs have count 0).
+extern "C" int ls_advance_decode(int* meta, int n_seqs, int off_tokens, int off_positions, int off_seqs,
+                                 const int* picked, int* ring, int* counter, const int* list_offsets,
+                                 const int* list_counts, int n_lists, void* stream) {
+  LS_REQUIRE(meta && picked && ring && counter && n_seqs > 0, "advance_decode: bad operands");
+  LS_REQUIRE(n_lists >= 0 && n_lists <= 4, "advance_decode: at most four item lists, got %d", n_lists);
+  AdvanceLists lists;
+  for (int l = 0; l < 4; ++l) {
+    lists.offset[l] = l < n_lists ? list_offsets[l] : 0;
+    lists.count[l] = l < n_lists ? list_counts[l] : 0;
+  }
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  hipLaunchKernelGGL(advance_decode_kernel, dim3(1), dim3(256), 0, s, meta, n_seqs, off_tokens, off_positions,
+                     off_seqs, picked, ring, counter, lists);
+  return check_launch("advance_decode");
 }

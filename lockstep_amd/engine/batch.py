@@ -92,14 +92,18 @@ class Workspace:
 class StepContext:
     """Everything a part may read about the step (see module docstring)."""
 
-    def __init__(self, rt, cache, workspace: Workspace, entries: Sequence[StepEntry], fixed_shape: bool = False):
+    def __init__(self, rt, cache, workspace: Workspace, entries: Sequence[StepEntry], fixed_shape: bool = False,
+                 horizon: int = 0):
         """``fixed_shape`` lays the attention work out so that its size depends
         only on the number of requests and on a bucket of the longest context:
         every request gets one work item per split up to the bucket (items past a
         request's own length produce empty partial results, which the combine
         step skips, so the bits do not change).  A captured graph of the step
-        then stays valid from one decode step to the next."""
+        then stays valid from one decode step to the next.  ``horizon``: the
+        layout (and the position tables) must also hold when every request has grown
+        by this many more tokens (decode steps that run without the host)."""
         self.fixed_shape = fixed_shape
+        self.horizon = int(horizon)
         self.rt = rt
         self.cache = cache
         self.workspace = workspace
@@ -118,7 +122,7 @@ class StepContext:
         seqs[:, 3] = seqs[:, 1] + seqs[:, 2]
         seqs[:, 4] = [cache.slot(e.request) for e in self.entries]
         self.q_off, self.q_len, self.q_start, self.kv_len, self.slots = (seqs[:, c] for c in range(5))
-        self.max_position = int(self.kv_len.max()) - 1
+        self.max_position = int(self.kv_len.max()) - 1 + self.horizon
 
         if self._single_tokens:
             tokens = np.asarray([e.tokens[0] for e in self.entries], dtype=np.int64)
@@ -159,7 +163,7 @@ class StepContext:
         part_rows = 0
         bucket = 0
         if self.fixed_shape:
-            longest = (int(self.kv_len.max()) - 1) // split + 1
+            longest = (int(self.kv_len.max()) + self.horizon - 1) // split + 1
             bucket = 1
             while bucket < longest:
                 bucket = bucket * 2 if bucket < 8 else bucket + 8
@@ -246,6 +250,25 @@ class StepContext:
         self._meta = dev
         self._views = None
         self._uploaded = True
+
+    def meta_layout(self) -> dict:
+        """Where things lie inside the uploaded metadata (offsets in ints): ``tokens``, ``positions``,
+        ``seqs`` and ``item_lists``, the (offset, count) of every list of attention work items."""
+        t, s = self.n_tokens, self.n_seqs
+        at = 3 * t + 8 * s + self.n_want
+        lists = []
+        for key in self._plan_specs:
+            items, combine, n_items, _, _, coop, n_coop, _, wide, n_wide, _ = self._plans[key]
+            if n_items:
+                lists.append((at, n_items))
+            at += items.shape[0] + combine.shape[0]
+            if n_coop:
+                lists.append((at, n_coop))
+            at += coop.shape[0]
+            if n_wide:
+                lists.append((at, n_wide))
+            at += wide.shape[0]
+        return {"tokens": 0, "positions": 2 * t, "seqs": 3 * t, "item_lists": lists, "meta": self._meta}
 
     def _materialize(self) -> dict:
         """Device views of the uploaded metadata (made when a part first asks: a replayed graph never does)."""

@@ -208,6 +208,104 @@ class Model:
         return result
 
 
+    # -- decode steps without the host ---------------------------------------------------
+    LOOP_CAPACITY = 256           # steps one call of the device loop may run
+
+    def decode_greedy(self, cache: CacheManager, requests: Sequence, tokens: Sequence[int], n_steps: int):
+        """``n_steps`` decode steps of ``requests`` (ids of open requests whose next input tokens are
+        ``tokens``) with the greedy pick of each step fed back on the device: the host launches the
+        captured step ``n_steps`` times and reads the picked tokens once at the end.  Returns them as
+        an int array ``[n_steps, len(requests)]``.  Logits are those of ``step`` (same kernels, same
+        bits), so the tokens equal those of step-by-step greedy decoding."""
+        n = len(requests)
+        if n == 0 or n_steps <= 0:
+            return np.zeros((0, n), dtype=np.int64)
+        if len(set(requests)) != n:
+            raise ValueError("a request appears twice")
+        vocab = self.spec.vocab_size
+        if any(not 0 <= int(t) < vocab for t in tokens):
+            raise ValueError(f"a token id lies outside [0, {vocab})")
+        if not (self.use_graphs and self._graph_safe):
+            return self._decode_greedy_stepwise(cache, requests, tokens, n_steps)
+        out = []
+        tokens = [int(t) for t in tokens]
+        while n_steps > 0:
+            chunk = min(n_steps, self.LOOP_CAPACITY)
+            picked = self._decode_loop(cache, requests, tokens, chunk)
+            if picked is None:
+                return np.concatenate(out + [self._decode_greedy_stepwise(cache, requests, tokens, n_steps)])
+            out.append(picked)
+            tokens = picked[-1].tolist()
+            n_steps -= chunk
+        return np.concatenate(out)
+
+    def _decode_greedy_stepwise(self, cache, requests, tokens, n_steps):
+        picked = torch.empty(len(requests), dtype=torch.int32, device=self.rt.device)
+        out = np.zeros((n_steps, len(requests)), dtype=np.int64)
+        tokens = [int(t) for t in tokens]
+        for i in range(n_steps):
+            logits = self.step(cache, [StepEntry(r, [t], [0]) for r, t in zip(requests, tokens)])
+            self.rt.kernels.argmax(logits, picked)
+            tokens = picked.cpu().tolist()
+            out[i] = tokens
+        return out
+
+    def _decode_loop(self, cache, requests, tokens, n_steps):
+        n = len(requests)
+        starts = [cache.length(r) for r in requests]
+        for r, start in zip(requests, starts):
+            cache.reserve(r, start + n_steps)          # every page the loop will write, now
+            if cache.ever_shared:
+                for gi in range(len(cache.groups)):
+                    for logical in range(start // cache.page_size, -(-(start + n_steps) // cache.page_size)):
+                        cache.assert_exclusive(r, gi, logical)
+        cache.sync_tables()
+        entries = [StepEntry(r, [t], [0]) for r, t in zip(requests, tokens)]
+        ctx = StepContext(self.rt, cache, self.workspace, entries, fixed_shape=True, horizon=n_steps - 1)
+        for mixer in self._preparers:
+            mixer.prepare(ctx)
+        ctx.upload()
+        layout = ctx.meta_layout()
+        if len(layout["item_lists"]) > 4:
+            return None                                   # more work lists than the advance kernel takes
+        kernels = self.rt.kernels
+        ring = self.workspace.get("loop.ring", (self.LOOP_CAPACITY * max(n, 64),), torch.int32)
+        counter = self.workspace.get("loop.counter", (1,), torch.int32)
+        picked = self.workspace.get("loop.picked", (max(n, 64),), torch.int32)
+        counter.zero_()
+
+        def one_step(logits):
+            self._forward(ctx, logits)
+            kernels.argmax(logits, picked[:n])
+            kernels.advance_decode(layout["meta"], n, layout["tokens"], layout["positions"], layout["seqs"], picked,
+                                   ring, counter, layout["item_lists"])
+
+        graphs = cache.__dict__.setdefault("_step_graphs", {})
+        key = ("loop",) + self._graph_key(ctx)
+        held = graphs.get(key)
+        done = 0
+        if held is None:
+            logits = torch.empty((n, self.spec.vocab_size), dtype=torch.float32, device=self.rt.device)
+            one_step(logits)                              # sizes the workspace; it is the loop's first step
+            done = 1
+            key = ("loop",) + self._graph_key(ctx)
+            if len(graphs) >= 32:
+                graphs.clear()
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                one_step(logits)
+            graphs[key] = held = (graph, logits)
+        graph = held[0]
+        for _ in range(n_steps - done):
+            graph.replay()
+        self.graph_replays += n_steps - done
+        out = ring[: n_steps * n].cpu().numpy().reshape(n_steps, n).astype(np.int64)
+        for r, start in zip(requests, starts):
+            cache.commit(r, start + n_steps)
+        return out
+
+
 def load_model(model_dir, dtype="bfloat16", device="cuda:0") -> Model:
     """Open a folder with config.json and model.safetensors; the class of the
     configuration, and with it the architecture, is chosen by config.json."""

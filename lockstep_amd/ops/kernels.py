@@ -265,6 +265,24 @@ class Kernels:
                                    c_long(logits.stride(0)), _ptr(scratch), c_long(scratch.numel()), _stream())
         self._check(self.core, code)
 
+    def advance_decode(self, meta: torch.Tensor, n_seqs: int, off_tokens: int, off_positions: int, off_seqs: int,
+                       picked: torch.Tensor, ring: torch.Tensor, counter: torch.Tensor, lists) -> None:
+        """Between two decode steps that run without the host: the picked tokens become the next
+        inputs, positions and lengths inside the uploaded metadata ``meta`` move on by one, and the
+        tokens are appended to ``ring[counter]``.  ``lists``: (offset, count) of the attention
+        work-item lists inside ``meta`` (16 ints an item)."""
+        for t in (meta, picked, ring, counter):
+            _need(t.is_cuda and t.dtype == torch.int32 and t.is_contiguous(), "advance_decode works on int32 GPU tensors")
+        _need(picked.numel() >= n_seqs and len(lists) <= 4, "advance_decode: picked too short or more than four lists")
+        offsets = (ctypes.c_int * 4)(*([o for o, _ in lists] + [0] * (4 - len(lists))))
+        counts = (ctypes.c_int * 4)(*([c for _, c in lists] + [0] * (4 - len(lists))))
+        for o, c in lists:
+            _need(0 <= o and o + 16 * c <= meta.numel(), "advance_decode: an item list lies outside the metadata")
+        code = self.core.ls_advance_decode(_ptr(meta), c_int(n_seqs), c_int(off_tokens), c_int(off_positions),
+                                           c_int(off_seqs), _ptr(picked), _ptr(ring), _ptr(counter), offsets, counts,
+                                           c_int(len(lists)), _stream())
+        self._check(self.core, code)
+
     # -- attention ----------------------------------------------------------------
     def qk_rope_kv(self, qkv: torch.Tensor, n_tokens: int, nq: int, nkv: int, d: int, q_weight, k_weight,
                    eps: float, cos, sin, rot: int, tok_seq, tok_pos, seqs, max_pos: int, table, k_pages,

@@ -288,3 +288,42 @@ def test_the_first_tokens_of_a_sequence(plain_logits, dtype, name, page_size):
     single, single_want = one_seqs[1]
     cache.close("pair")
     assert rel_err(feed(model, cache, "one", single, []), single_want) < TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name,page_size", [("A", 16), ("B", 8)])
+def test_the_device_side_decode_loop_picks_the_tokens_of_stepwise_greedy_decoding(plain_logits, dtype, name, page_size):
+    """Decode steps whose greedy picks are fed back on the device (no host in between) give the
+    tokens of step-by-step decoding, leave the same cache behind, and can be called again;
+    contexts cross pages, tiles and a split of the keys on the way."""
+    from lockstep_amd.engine.batch import StepEntry
+
+    folder = plain_logits["gen"][name]
+    model = load(folder, dtype)
+    vocab = model.spec.vocab_size
+    prompts = [random_tokens(n, vocab, seed=900 + n) for n in (3, 120, 250)]
+    steps = 140
+
+    def prefill(cache):
+        first = []
+        for i, p in enumerate(prompts):
+            cache.open(f"r{i}")
+            logits = model.step(cache, [StepEntry(f"r{i}", p, [len(p) - 1])])
+            first.append(int(logits[0].argmax()))
+        return first
+
+    ids = [f"r{i}" for i in range(len(prompts))]
+    stepwise_cache = model.make_cache(num_pages=200, page_size=page_size)
+    tokens = prefill(stepwise_cache)
+    want = model._decode_greedy_stepwise(stepwise_cache, ids, tokens, steps)
+
+    loop_cache = model.make_cache(num_pages=200, page_size=page_size)
+    tokens = prefill(loop_cache)
+    got_a = model.decode_greedy(loop_cache, ids, tokens, 60)
+    got_b = model.decode_greedy(loop_cache, ids, got_a[-1].tolist(), steps - 60)       # the captured loop again
+    got = torch.cat([torch.as_tensor(got_a), torch.as_tensor(got_b)])
+    assert torch.equal(got, torch.as_tensor(want))
+    assert [loop_cache.length(r) for r in ids] == [stepwise_cache.length(r) for r in ids]
+    probe = [StepEntry(r, [int(t)], [0]) for r, t in zip(ids, want[-1])]
+    assert torch.equal(model.step(loop_cache, probe), model.step(stepwise_cache, probe))
+    loop_cache.audit(); stepwise_cache.audit()
