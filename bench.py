@@ -201,7 +201,7 @@ def main(argv=None) -> int:
     achieved = bytes_step / (elapsed / args.steps)
 
     record = {
-        "metric": f"decode tok/s at batch {args.batch} (Qwen3-0.6B sizes, {args.prompt_len}-token prompts, greedy)",
+        "metric": f"decode tok/s at batch {args.batch} ({args.model} layer sizes, {args.prompt_len}-token prompts, greedy)",
         "value": round(value, 1),
         "unit": "tokens/s",
         "n_gpus": 1,
