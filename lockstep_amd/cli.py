@@ -55,6 +55,8 @@ def cmd_run(argv) -> int:
     p.add_argument("--enable-prefix-cache", action="store_true")
     p.add_argument("--reserve", default="full", choices=["full", "lazy"],
                    help="take a request's pages at admission (full) or step by step (lazy)")
+    p.add_argument("--decode-burst", type=int, default=32,
+                   help="up to this many greedy decode steps run on the GPU without the host in between (1: none)")
     args = p.parse_args(argv)
 
     import tempfile
@@ -89,7 +91,7 @@ def cmd_run(argv) -> int:
         llm = LLM(folder, dtype=args.dtype, num_pages=args.num_blocks, page_size=args.block_size,
                   max_batched_tokens=args.max_batched_tokens, prefill_chunk=args.prefill_chunk,
                   max_running=args.max_running, enable_prefix_cache=args.enable_prefix_cache,
-                  eos_token_ids=args.eos, reserve=args.reserve)
+                  eos_token_ids=args.eos, reserve=args.reserve, decode_burst=args.decode_burst)
         outputs = llm.generate(requests)
     for uid in sorted(outputs):
         print(json.dumps({"uid": uid, "tokens": outputs[uid]}))

@@ -54,11 +54,12 @@ class LLM:
     def __init__(self, model_dir, dtype: str = "bfloat16", device: str = "cuda:0", num_pages: int = 512,
                  page_size: int = 16, max_batched_tokens: int | None = None, prefill_chunk: int | None = None,
                  max_running: int = 64, enable_prefix_cache: bool = False, eos_token_ids=None,
-                 reserve: str = "full", audit: bool = False, max_tokens_per_request: int | None = None):
+                 reserve: str = "full", audit: bool = False, max_tokens_per_request: int | None = None,
+                 decode_burst: int = 32):
         self.model = load_model(model_dir, dtype=dtype, device=device)
         self.options = dict(num_blocks=num_pages, block_size=page_size, max_batched_tokens=max_batched_tokens,
                             enable_prefix_cache=enable_prefix_cache, eos_token_ids=eos_token_ids, reserve=reserve,
-                            audit=audit, max_tokens_per_request=max_tokens_per_request)
+                            audit=audit, max_tokens_per_request=max_tokens_per_request, decode_burst=decode_burst)
         self.prefill_chunk = prefill_chunk
         self.max_running = max_running
 

@@ -67,9 +67,14 @@ class Scheduler:
     def __init__(self, model, num_blocks: int, policy: Policy | None = None, eos_token_ids=None,
                  audit: bool = True, block_size: int = 16, enable_prefix_cache: bool = False, *,
                  max_batched_tokens: int | None = None, reserve: str = "full", max_requests: int | None = None,
-                 max_tokens_per_request: int | None = None, sampler=None, cache=None, keep_logits: bool = False):
+                 max_tokens_per_request: int | None = None, sampler=None, cache=None, keep_logits: bool = False,
+                 decode_burst: int = 1):
         """``num_blocks`` pages of ``block_size`` tokens (the reference's names).
-        ``max_batched_tokens`` bounds the tokens of one step (None: no bound)."""
+        ``max_batched_tokens`` bounds the tokens of one step (None: no bound).
+        ``decode_burst`` > 1: while nothing waits, every running request is decoding greedily and no
+        decision could differ from step to step (default policy, pages reserved in full, no
+        end-of-sequence ids, no audit), up to that many decode steps run as one call of the model's
+        device-side loop (``decode_greedy``); the tokens are those of single steps."""
         if reserve not in ("full", "lazy"):
             raise ValueError("reserve must be 'full' or 'lazy'")
         self.model = model
@@ -79,6 +84,7 @@ class Scheduler:
         self.reserve_mode = reserve
         self.max_batched_tokens = max_batched_tokens
         self.keep_logits = keep_logits
+        self.decode_burst = max(1, int(decode_burst))
         self.counters = Counters()
         self.lifecycle: dict[str, list] = {}
         max_running = getattr(self.policy, "max_running", 64)
@@ -313,6 +319,12 @@ class Scheduler:
                 (self.cache.state_digest(), self.prefix.state_digest() if self.prefix else ()))
             self.cache.audit()
 
+        self._retire_finished()
+
+        self.step_index += 1
+        return True
+
+    def _retire_finished(self) -> None:
         for request in list(self.running):
             if not request.generated:
                 continue
@@ -330,11 +342,38 @@ class Scheduler:
                         self.counters.hit("cache_insert", created)
                 self.cache.close(request.uid)
 
-        self.step_index += 1
+    def _burst(self, max_steps: int) -> bool:
+        """Several decode steps in one call of the model's device-side loop, when every decision of
+        those steps is known in advance (see ``decode_burst``).  Returns whether it ran."""
+        if self.decode_burst <= 1 or self.waiting or not self.running or self.eos or self.audit_enabled:
+            return False
+        if self.keep_logits or self.reserve_mode != "full" or type(self.policy) is not DefaultPolicy:
+            return False
+        if not hasattr(self.model, "decode_greedy"):
+            return False
+        if self.max_batched_tokens is not None and self.max_batched_tokens < len(self.running):
+            return False
+        for r in self.running:
+            if r.temperature > 0 or not r.generated or r.total_tokens() - r.kv_len != 1:
+                return False
+        steps = min(self.decode_burst, max_steps - self.step_index,
+                    min(r.max_new_tokens - len(r.generated) for r in self.running))
+        if steps <= 1:
+            return False
+        uids = [r.uid for r in self.running]
+        picked = self.model.decode_greedy(self.cache, uids, [r.generated[-1] for r in self.running], steps)
+        for row in picked:
+            for request, token in zip(self.running, row):
+                request.generated.append(int(token))
+                request.kv_len += 1
+                self.counters.hit("decode_step")
+                self._event(request.uid, Event.DECODE)
+            self.step_index += 1
+        self._retire_finished()
         return True
 
     def run(self, max_steps: int = 1 << 20) -> dict:
-        while self.step() and self.step_index < max_steps:
+        while (self._burst(max_steps) or self.step()) and self.step_index < max_steps:
             pass
         if self.audit_enabled:
             self.cache.audit()

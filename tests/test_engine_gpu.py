@@ -169,6 +169,14 @@ def test_greedy_generation_through_the_entry_points(plain_logits, name, page_siz
     half.options["max_batched_tokens"] = 20
     assert half.generate(requests(), policy=FixedChunkPolicy(5)) == base
     assert half.generate(requests()[1:2]) == {"r1": base["r1"]}
+    # decode steps in bursts on the GPU (no audit, default policy): the same tokens, float32 and bfloat16
+    for dtype, tokens in (("float32", want), ("bfloat16", base)):
+        fast = LLM(folder, dtype=dtype, num_pages=64, page_size=page_size, audit=False, decode_burst=7)
+        scheduler = fast.scheduler()
+        for r in requests():
+            scheduler.submit(r)
+        assert scheduler.run() == tokens
+        assert fast.model.graph_replays > 0 and scheduler.counters["decode_step"] == len(prompts) * (new - 1)
 
 
 def test_sampled_generation_follows_the_plain_sampler(plain_logits):

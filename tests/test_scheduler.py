@@ -55,6 +55,19 @@ class StandInModel:
         self.batches.append(batch)
         return torch.stack(rows) if rows else None
 
+    def decode_greedy(self, cache, requests, tokens, n_steps):
+        """What the engine's device-side loop does, step by step."""
+        import numpy as np
+        from lockstep_amd.engine.batch import StepEntry
+
+        self.bursts = getattr(self, "bursts", []) + [n_steps]
+        out = []
+        for _ in range(n_steps):
+            logits = self.step(cache, [StepEntry(r, [t], [0]) for r, t in zip(requests, tokens)])
+            tokens = [greedy(row) for row in logits]
+            out.append(tokens)
+        return np.asarray(out)
+
 
 def expected_greedy(prompt, n, eos=()):
     context, out = list(prompt), []
@@ -263,3 +276,30 @@ def test_lifecycle_follows_the_state_machine():
     c = run(reqs(ps, n=8), policy=FixedChunkPolicy(7))[1].trajectory
     assert a.hexdigest() == b.hexdigest() and a.first_divergence(b) is None
     assert a.hexdigest() != c.hexdigest() and a.first_divergence(c) == 0
+
+
+def test_decode_bursts_change_neither_tokens_nor_counts():
+    """With decode_burst > 1 runs of decode steps go through the model's device-side loop: same
+    tokens, same counters, same number of steps, same life cycle; a burst never runs past a
+    request's last token, and not while something waits, samples, or may stop at an end token."""
+    ps = prompts(3, 20, 41)
+    lengths = (5, 9, 14)
+
+    def build():
+        return [Request(uid=f"r{i}", prompt=p, max_new_tokens=n) for i, (p, n) in enumerate(zip(ps, lengths))]
+
+    single, s1, m1 = run(build(), audit=False)
+    burst, s2, m2 = run(build(), audit=False, decode_burst=4)
+    assert burst == single == {f"r{i}": expected_greedy(p, n) for i, (p, n) in enumerate(zip(ps, lengths))}
+    assert getattr(m2, "bursts", []) and max(m2.bursts) <= 4
+    assert not hasattr(m1, "bursts")
+    assert s1.counters.counts == s2.counters.counts
+    assert s1.step_index == s2.step_index and s1.lifecycle == s2.lifecycle
+    # conditions that keep single steps: audit on, an end token, sampling, a waiting request
+    for kw, requests in (({"audit": True}, build()), ({"audit": False, "eos_token_ids": [7]}, build()),
+                         ({"audit": False}, [Request(uid="t", prompt=ps[0], max_new_tokens=6, temperature=0.8, seed=3)])):
+        _, _, m = run(requests, decode_burst=4, **kw)
+        assert not hasattr(m, "bursts"), kw
+    many = [Request(uid=f"w{i}", prompt=ps[0], max_new_tokens=8) for i in range(3)]
+    out, s3, m3 = run(many, audit=False, decode_burst=16, policy=None, num_blocks=2)   # pages for two at a time
+    assert out == {f"w{i}": expected_greedy(ps[0], 8) for i in range(3)}
