@@ -323,7 +323,10 @@ def test_the_device_side_decode_loop_picks_the_tokens_of_stepwise_greedy_decodin
     ids = [f"r{i}" for i in range(len(prompts))]
     stepwise_cache = model.make_cache(num_pages=200, page_size=page_size)
     tokens = prefill(stepwise_cache)
-    want = model._decode_greedy_stepwise(stepwise_cache, ids, tokens, steps)
+    model.use_graphs = False                      # the reference: eager steps, picks read by the host
+    want = model.decode_greedy(stepwise_cache, ids, tokens, steps)
+    model.use_graphs = True
+    assert model.graph_replays == 0
 
     loop_cache = model.make_cache(num_pages=200, page_size=page_size)
     tokens = prefill(loop_cache)
