@@ -513,7 +513,9 @@ int launch_gemm(const void* X, const void* W, void* C, int M, int N, int K, long
   const int vec_ok = (ldc % 4 == 0) && (reinterpret_cast<uintptr_t>(C) % (4 * out_size) == 0);
   const T* w = reinterpret_cast<const T*>(W);
   if (norm_w && M > 16) return fail("gemm: the fused norm prologue takes at most 16 rows, got %d", M);
-  if (M <= 64) {
+  // Up to 64 rows the skinny kernel; but with more than 16 rows and very many columns (the logits
+  // head) its workgroups re-read all rows of X for 16 columns each, and the tiled kernel reads less.
+  if (M <= 64 && !(M > 16 && N >= 32768)) {
     const int mt = (M + 15) / 16;
     // 16 waves leave 128 registers a lane: only for one or two row tiles
     const int nw = (nslices > 8 && mt * NT <= 2) ? 16 : (nslices > 4 ? 8 : 4);
