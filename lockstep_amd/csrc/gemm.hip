@@ -15,6 +15,8 @@
 // so a lane ends with four consecutive n of one row m and stores them as one
 // vector.
 
+#include <type_traits>
+
 #include "common.h"
 
 namespace ls {
@@ -24,6 +26,9 @@ namespace ls {
 #endif
 #ifndef LS_GEMM_PD_BIG
 #define LS_GEMM_PD_BIG 1      // register prefetch depth (stages) of the 128 x 128 kernel
+#endif
+#ifndef LS_GEMM_STREAM
+#define LS_GEMM_STREAM 1      // 0: never the streaming kernel
 #endif
 #ifndef LS_GEMM_PD_SMALL
 #define LS_GEMM_PD_SMALL 2    // ... and of the 64 x 64 kernel
@@ -277,6 +282,140 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const void* __rest
 }
 
 // ---------------------------------------------------------------------------
+// Streaming kernel (at most 32 rows, many output columns): the skinny kernel's
+// arithmetic with another walk.  A workgroup has one wave per K slice and
+// takes the column blocks b = blockIdx.x, blockIdx.x + gridDim.x, ...  A wave
+// keeps its slice of X in registers for the whole walk, so the rows of X are
+// read once per workgroup instead of once per 16 columns (with 8 rows that is
+// half as much again as the weights themselves), and the weights of its next
+// unit (UC chunks of a tile) are always in flight while it multiplies the
+// current one, also across column blocks and across the two barriers of the
+// fold.  Slice sums meet in LDS and are folded in ascending order, as in the
+// skinny kernel.
+// ---------------------------------------------------------------------------
+template <typename T, int MT, int EPI, int XC>
+__global__ __launch_bounds__(1024) void gemm_stream_kernel(const T* __restrict__ X, const T* __restrict__ W,
+                                                           void* __restrict__ C, int M, int N, int K, long ldx,
+                                                           long ldc, int kslice, int aligned, int vec_ok,
+                                                           int out_cols, int blocks) {
+  typedef Atom<T> A;
+  typedef typename A::vec_t vec_t;
+  constexpr int NT = (EPI == kSwiGLU) ? 2 : 1;  // weight tiles per column block
+  constexpr int UC = 4;                          // chunks per unit
+  constexpr int UQ = XC / UC;                    // units per tile
+  constexpr int UNITS = NT * UQ;                 // units per column block
+  constexpr int RING = (MT * XC <= 8) ? 4 : 2;   // unit buffers in registers: one in use, the others in flight
+  constexpr int AHEAD = RING - 1;
+  static_assert(XC % UC == 0, "a tile is a whole number of units");
+  extern __shared__ float part[];  // [2][waves][NT][MT][256]
+
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int nw = blockDim.x >> 6;  // = number of K slices
+  const int row16 = lane & 15;
+  const int g = lane >> 4;
+  const int k_begin = wave * kslice;
+  const int k_end = min(K, k_begin + kslice);
+
+  auto fetch = [&](int b, int t, int q, vec_t (&dst)[UC]) {
+    const int n = (b * NT + t) * 16 + row16;
+#pragma unroll
+    for (int c = 0; c < UC; ++c) {
+      const int kc = k_begin + (q * UC + c) * A::KCHUNK;
+      dst[c] = load_vec<T>(W, n, kc + g * A::VEC, K, K, n < N && kc < k_end, aligned);
+    }
+  };
+
+  // Units are numbered through the walk: unit u of the workgroup is unit u % UNITS of its block u / UNITS
+  // and lives in buffer u % RING.
+  vec_t wbuf[RING][UC];
+  int b = blockIdx.x;
+#pragma unroll
+  for (int u = 0; u < AHEAD; ++u) {
+    const int bu = b + (u / UNITS) * (int)gridDim.x;
+    if (bu < blocks) fetch(bu, (u % UNITS) / UQ, (u % UNITS) % UQ, wbuf[u % RING]);
+  }
+
+  vec_t xs[MT][XC];
+#pragma unroll
+  for (int j = 0; j < MT; ++j)
+#pragma unroll
+    for (int c = 0; c < XC; ++c) {
+      const int kc = k_begin + c * A::KCHUNK;
+      xs[j][c] = load_vec<T>(X, j * 16 + row16, kc + g * A::VEC, K, ldx, j * 16 + row16 < M && kc < k_end, aligned);
+    }
+
+  // One column block; `par` is the buffer that holds the block's first unit (static, so that the
+  // register buffers are addressed statically).
+  static_assert(UNITS % RING == 0 || (2 * UNITS) % RING == 0, "the buffer of a block's first unit has period two");
+  auto block_step = [&](auto par, int it) {
+    constexpr int P = decltype(par)::value;
+    float* mine = part + (it & 1) * (nw * NT * MT * 256);
+    f32x4 acc[NT][MT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int j = 0; j < MT; ++j) acc[t][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int idx = 0; idx < UNITS; ++idx) {
+      const int t = idx / UQ;
+      const int q = idx % UQ;
+      const int far_block = b + ((idx + AHEAD) / UNITS) * (int)gridDim.x;  // the block of the unit AHEAD units on
+      if (far_block < blocks)
+        fetch(far_block, ((idx + AHEAD) % UNITS) / UQ, ((idx + AHEAD) % UNITS) % UQ, wbuf[(P + idx + AHEAD) % RING]);
+#pragma unroll
+      for (int c = 0; c < UC; ++c) {
+        if (k_begin + (q * UC + c) * A::KCHUNK >= k_end) break;  // uniform: a chunk is visited iff it starts inside the slice
+#pragma unroll
+        for (int j = 0; j < MT; ++j) A::mma(acc[t][j], wbuf[(P + idx) % RING][c], xs[j][q * UC + c]);
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int j = 0; j < MT; ++j)
+        *reinterpret_cast<f32x4*>(&mine[(((wave * NT + t) * MT + j) * 64 + lane) * 4]) = acc[t][j];
+    // One barrier a block: the next block's sums go to the other half of `part`, and the half
+    // written now is written again only after the next barrier, which the folding wave reaches
+    // after its fold.
+    __syncthreads();
+    // row tile j of this block is folded by wave (it * MT + j) % nw, so the duty goes round
+    const int j = (wave + nw - (it * MT) % nw) % nw;
+    if (j < MT) {
+      float total[NT][4];
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) total[t][r] = 0.f;
+        for (int s = 0; s < nw; ++s) {
+          const f32x4 p = *reinterpret_cast<const f32x4*>(&mine[(((s * NT + t) * MT + j) * 64 + lane) * 4]);
+#pragma unroll
+          for (int r = 0; r < 4; ++r) total[t][r] = total[t][r] + p[r];
+        }
+      }
+      const int m = j * 16 + row16;
+      if (EPI == kSwiGLU)
+        epilogue_swiglu4<T>(C, ldc, m, b * 16 + g * 4, M, out_cols, total[0], total[NT - 1], vec_ok);
+      else
+        epilogue4<T, EPI>(C, ldc, m, b * 16 + g * 4, M, N, total[0], vec_ok);
+    }
+  };
+
+  // the first buffer of a block advances by UNITS % RING from block to block
+  for (int it = 0; b < blocks;) {
+    block_step(std::integral_constant<int, 0>{}, it);
+    b += gridDim.x;
+    ++it;
+    if (UNITS % RING != 0) {  // UNITS = 2, RING = 4: every other block starts in buffer 2
+      if (b >= blocks) break;
+      block_step(std::integral_constant<int, UNITS % RING>{}, it);
+      b += gridDim.x;
+      ++it;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
 // Slice kernel (at most 64 rows): the skinny kernel's slice sums, left
 // unfolded.  A workgroup takes 16 output columns and a few consecutive K
 // slices, one per wave, and writes each slice's sums to P [slices][M][N]
@@ -500,6 +639,19 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const T* __restrict__ X
     }
 }
 
+// Compute units of the current device (asked once per device).
+inline int compute_units() {
+  static int cached[64] = {0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (cached[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cached[dev] = n;
+  }
+  return cached[dev];
+}
+
 template <typename T, int EPI>
 int launch_gemm(const void* X, const void* W, void* C, int M, int N, int K, long ldx, long ldc, const float* norm_w,
                 float eps, int out_cols, hipStream_t stream) {
@@ -515,6 +667,29 @@ int launch_gemm(const void* X, const void* W, void* C, int M, int N, int K, long
   if (norm_w && M > 16) return fail("gemm: the fused norm prologue takes at most 16 rows, got %d", M);
   // Up to 64 rows the skinny kernel; but with more than 16 rows and very many columns (the logits
   // head) its workgroups re-read all rows of X for 16 columns each, and the tiled kernel reads less.
+  const int mt_rows = (M + 15) / 16;
+  const int col_blocks = (N + 16 * NT - 1) / (16 * NT);
+  const int xc = kslice / Atom<T>::KCHUNK;  // chunks per slice
+  // The streaming kernel where a workgroup would get more than one column block: a CU holds 16 waves
+  // of it (one per K slice), so 16 / nslices workgroups.
+  const int stream_wgs = compute_units() * (16 / nslices > 0 ? 16 / nslices : 1);
+  const size_t stream_lds = 2 * (size_t)nslices * NT * mt_rows * 256 * sizeof(float);  // two sets of slice sums
+  if (!norm_w && mt_rows <= 2 && xc % 4 == 0 && xc * mt_rows <= 16 && nslices <= 16 && col_blocks > stream_wgs &&
+      stream_lds <= 64 * 1024 && LS_GEMM_STREAM) {
+    const int rounds = (col_blocks + stream_wgs - 1) / stream_wgs;
+    dim3 grid((col_blocks + rounds - 1) / rounds);
+    const size_t lds = stream_lds;
+#define LS_STREAM(MT_, XC_)                                                                                        \
+  hipLaunchKernelGGL((gemm_stream_kernel<T, MT_, EPI, XC_>), grid, dim3(nslices * 64), lds, stream,                \
+                     reinterpret_cast<const T*>(X), w, C, M, N, K, ldx, ldc, kslice, aligned, vec_ok, out_cols,   \
+                     col_blocks)
+    if (mt_rows == 1 && xc == 8) LS_STREAM(1, 8);
+    else if (mt_rows == 1 && xc == 16) LS_STREAM(1, 16);
+    else if (mt_rows == 2 && xc == 8) LS_STREAM(2, 8);
+    else return fail("gemm: no streaming kernel for %d chunks a slice and %d row tiles", xc, mt_rows);
+#undef LS_STREAM
+    return check_launch("gemm");
+  }
   if (M <= 64 && !(M > 16 && N >= 32768)) {
     const int mt = (M + 15) / 16;
     // 16 waves leave 128 registers a lane: only for one or two row tiles

@@ -76,6 +76,59 @@ def test_gemm_row_does_not_depend_on_the_batch(dtype):
             assert torch.equal(one[0], full[i]), f"row {i} k={k} n={n}"
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("k,n", [(4096, 4096 + 24), (1000, 16384 + 24), (5120, 4096 + 104), (260, 32768 + 40),
+                                 (2048, 8192 + 8)])
+def test_gemm_with_few_rows_and_many_columns_has_the_same_bits(dtype, k, n):
+    """With up to 32 rows and more column blocks than the GPU holds workgroups, a workgroup walks
+    several column blocks with its rows of X in registers (the streaming kernel).  Every row has
+    the bits it has in a large batch, with every epilogue; a row of the sums equals the double
+    precision product."""
+    from lockstep_amd.ops import ADD_F32, STORE, STORE_F32
+
+    g = torch.Generator().manual_seed(k + n)
+    x = torch.randn(200, k, generator=g).to(dtype).cuda()
+    w = (torch.randn(n, k, generator=g) * 0.1).to(dtype).cuda()
+    full = torch.empty(200, n, dtype=torch.float32, device="cuda")
+    K().gemm(x, w, full, STORE_F32)
+    want = x[:3].double().cpu() @ w.double().cpu().T
+    assert rel_err(full[:3], want) < 2e-5
+    base = torch.randn(32, n, generator=g).cuda()
+    for rows in (1, 8, 16, 17, 32):
+        part = torch.empty(rows, n, dtype=torch.float32, device="cuda")
+        K().gemm(x[:rows], w, part, STORE_F32)
+        assert torch.equal(part, full[:rows]), f"rows={rows}"
+        stored = torch.empty(rows, n, dtype=dtype, device="cuda")
+        K().gemm(x[:rows], w, stored, STORE)
+        assert torch.equal(stored, full[:rows].to(dtype)), f"rows={rows}, stored in {dtype}"
+        acc = base[:rows].clone()
+        K().gemm(x[:rows], w, acc, ADD_F32)
+        assert torch.equal(acc, base[:rows] + full[:rows]), f"rows={rows}, added"
+    one = torch.empty(1, n, dtype=torch.float32, device="cuda")
+    K().gemm(x[31:32], w, one, STORE_F32)
+    assert torch.equal(one[0], full[31])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("inter,k", [(4096 + 40, 4096), (16384 + 72, 1024)])
+def test_swiglu_with_few_rows_and_many_columns_has_the_same_bits(dtype, inter, k):
+    from lockstep_amd.ops import SWIGLU, interleave_gate_up
+
+    g = torch.Generator().manual_seed(inter + k)
+    x = torch.randn(150, k, generator=g).to(dtype).cuda()
+    gate = (torch.randn(inter, k, generator=g) * 0.05).to(dtype)
+    up = (torch.randn(inter, k, generator=g) * 0.05).to(dtype)
+    w = interleave_gate_up(gate, up).cuda()
+    full = torch.empty(150, inter, dtype=dtype, device="cuda")
+    K().gemm(x, w, full, SWIGLU)
+    want = torch.nn.functional.silu(x[:2].double().cpu() @ gate.double().T) * (x[:2].double().cpu() @ up.double().T)
+    assert rel_err(full[:2], want) < TOL[dtype]
+    for rows in (1, 8, 16, 20, 32):
+        part = torch.empty(rows, inter, dtype=dtype, device="cuda")
+        K().gemm(x[:rows], w, part, SWIGLU)
+        assert torch.equal(part, full[:rows]), f"rows={rows}"
+
+
 def test_gemm_refuses_mismatched_operands():
     from lockstep_amd.ops import KernelError
 
