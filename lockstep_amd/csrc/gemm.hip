@@ -297,7 +297,7 @@ template <typename T, int MT, int EPI, int XC>
 __global__ __launch_bounds__(1024) void gemm_stream_kernel(const T* __restrict__ X, const T* __restrict__ W,
                                                            void* __restrict__ C, int M, int N, int K, long ldx,
                                                            long ldc, int kslice, int aligned, int vec_ok,
-                                                           int out_cols, int blocks) {
+                                                           int out_cols, int blocks, int row_groups) {
   typedef Atom<T> A;
   typedef typename A::vec_t vec_t;
   constexpr int NT = (EPI == kSwiGLU) ? 2 : 1;  // weight tiles per column block
@@ -316,6 +316,15 @@ __global__ __launch_bounds__(1024) void gemm_stream_kernel(const T* __restrict__
   const int g = lane >> 4;
   const int k_begin = wave * kslice;
   const int k_end = min(K, k_begin + kslice);
+  // With more than 16 * MT rows the rows are cut into groups of 16 * MT, each with workgroups of its own
+  // that walk the same column blocks.  Workgroup ids go round the XCDs, so the ids 8i .. 8i + 7 of one group
+  // and the next eight ids of the other group sit pairwise on the same XCD and walk in step: what one of
+  // them has fetched, the other finds in that XCD's L2.
+  const int id = blockIdx.x;
+  const int row_group = row_groups > 1 ? (id >> 3) % row_groups : 0;
+  const int walker = row_groups > 1 ? (id / (8 * row_groups)) * 8 + (id & 7) : id;
+  const int walkers = gridDim.x / row_groups;
+  const int m_base = row_group * MT * 16;
 
   auto fetch = [&](int b, int t, int q, vec_t (&dst)[UC]) {
     const int n = (b * NT + t) * 16 + row16;
@@ -329,10 +338,10 @@ __global__ __launch_bounds__(1024) void gemm_stream_kernel(const T* __restrict__
   // Units are numbered through the walk: unit u of the workgroup is unit u % UNITS of its block u / UNITS
   // and lives in buffer u % RING.
   vec_t wbuf[RING][UC];
-  int b = blockIdx.x;
+  int b = walker;
 #pragma unroll
   for (int u = 0; u < AHEAD; ++u) {
-    const int bu = b + (u / UNITS) * (int)gridDim.x;
+    const int bu = b + (u / UNITS) * walkers;
     if (bu < blocks) fetch(bu, (u % UNITS) / UQ, (u % UNITS) % UQ, wbuf[u % RING]);
   }
 
@@ -342,7 +351,8 @@ __global__ __launch_bounds__(1024) void gemm_stream_kernel(const T* __restrict__
 #pragma unroll
     for (int c = 0; c < XC; ++c) {
       const int kc = k_begin + c * A::KCHUNK;
-      xs[j][c] = load_vec<T>(X, j * 16 + row16, kc + g * A::VEC, K, ldx, j * 16 + row16 < M && kc < k_end, aligned);
+      xs[j][c] = load_vec<T>(X, m_base + j * 16 + row16, kc + g * A::VEC, K, ldx,
+                             m_base + j * 16 + row16 < M && kc < k_end, aligned);
     }
 
   // One column block; `par` is the buffer that holds the block's first unit (static, so that the
@@ -351,37 +361,38 @@ __global__ __launch_bounds__(1024) void gemm_stream_kernel(const T* __restrict__
   auto block_step = [&](auto par, int it) {
     constexpr int P = decltype(par)::value;
     float* mine = part + (it & 1) * (nw * NT * MT * 256);
-    f32x4 acc[NT][MT];
-#pragma unroll
-    for (int t = 0; t < NT; ++t)
-#pragma unroll
-      for (int j = 0; j < MT; ++j) acc[t][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+    f32x4 acc[MT];  // of the tile in work; a finished tile's sums go to LDS at once
 #pragma unroll
     for (int idx = 0; idx < UNITS; ++idx) {
       const int t = idx / UQ;
       const int q = idx % UQ;
-      const int far_block = b + ((idx + AHEAD) / UNITS) * (int)gridDim.x;  // the block of the unit AHEAD units on
+      if (q == 0) {
+#pragma unroll
+        for (int j = 0; j < MT; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+      }
+      const int far_block = b + ((idx + AHEAD) / UNITS) * walkers;  // the block of the unit AHEAD units on
       if (far_block < blocks)
         fetch(far_block, ((idx + AHEAD) % UNITS) / UQ, ((idx + AHEAD) % UNITS) % UQ, wbuf[(P + idx + AHEAD) % RING]);
 #pragma unroll
       for (int c = 0; c < UC; ++c) {
         if (k_begin + (q * UC + c) * A::KCHUNK >= k_end) break;  // uniform: a chunk is visited iff it starts inside the slice
 #pragma unroll
-        for (int j = 0; j < MT; ++j) A::mma(acc[t][j], wbuf[(P + idx) % RING][c], xs[j][q * UC + c]);
+        for (int j = 0; j < MT; ++j) A::mma(acc[j], wbuf[(P + idx) % RING][c], xs[j][q * UC + c]);
+      }
+      if (q == UQ - 1) {
+#pragma unroll
+        for (int j = 0; j < MT; ++j)
+          *reinterpret_cast<f32x4*>(&mine[(((wave * NT + t) * MT + j) * 64 + lane) * 4]) = acc[j];
       }
     }
-#pragma unroll
-    for (int t = 0; t < NT; ++t)
-#pragma unroll
-      for (int j = 0; j < MT; ++j)
-        *reinterpret_cast<f32x4*>(&mine[(((wave * NT + t) * MT + j) * 64 + lane) * 4]) = acc[t][j];
     // One barrier a block: the next block's sums go to the other half of `part`, and the half
     // written now is written again only after the next barrier, which the folding wave reaches
     // after its fold.
     __syncthreads();
     // row tile j of this block is folded by wave (it * MT + j) % nw, so the duty goes round
-    const int j = (wave + nw - (it * MT) % nw) % nw;
-    if (j < MT) {
+#pragma unroll
+    for (int j = 0; j < MT; ++j) {
+      if ((it * MT + j) % nw != wave) continue;  // uniform for the wave
       float total[NT][4];
 #pragma unroll
       for (int t = 0; t < NT; ++t) {
@@ -393,7 +404,7 @@ __global__ __launch_bounds__(1024) void gemm_stream_kernel(const T* __restrict__
           for (int r = 0; r < 4; ++r) total[t][r] = total[t][r] + p[r];
         }
       }
-      const int m = j * 16 + row16;
+      const int m = m_base + j * 16 + row16;
       if (EPI == kSwiGLU)
         epilogue_swiglu4<T>(C, ldc, m, b * 16 + g * 4, M, out_cols, total[0], total[NT - 1], vec_ok);
       else
@@ -404,15 +415,30 @@ __global__ __launch_bounds__(1024) void gemm_stream_kernel(const T* __restrict__
   // the first buffer of a block advances by UNITS % RING from block to block
   for (int it = 0; b < blocks;) {
     block_step(std::integral_constant<int, 0>{}, it);
-    b += gridDim.x;
+    b += walkers;
     ++it;
     if (UNITS % RING != 0) {  // UNITS = 2, RING = 4: every other block starts in buffer 2
       if (b >= blocks) break;
       block_step(std::integral_constant<int, UNITS % RING>{}, it);
-      b += gridDim.x;
+      b += walkers;
       ++it;
     }
   }
+}
+
+// Dynamic LDS beyond 64 KB has to be granted per kernel (once).
+template <typename T, int MT, int EPI, int XC>
+static bool stream_lds_ready(size_t bytes) {
+  if (bytes <= 64 * 1024) return true;
+  if (bytes > 128 * 1024) return false;
+  static int state = 0;  // 0 unknown, 1 granted, -1 refused
+  if (state == 0) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_stream_kernel<T, MT, EPI, XC>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
+    if (e != hipSuccess) (void)hipGetLastError();
+    state = e == hipSuccess ? 1 : -1;
+  }
+  return state == 1;
 }
 
 // ---------------------------------------------------------------------------
@@ -673,22 +699,34 @@ int launch_gemm(const void* X, const void* W, void* C, int M, int N, int K, long
   // The streaming kernel where a workgroup would get more than one column block: a CU holds 16 waves
   // of it (one per K slice), so 16 / nslices workgroups.
   const int stream_wgs = compute_units() * (16 / nslices > 0 ? 16 / nslices : 1);
-  const size_t stream_lds = 2 * (size_t)nslices * NT * mt_rows * 256 * sizeof(float);  // two sets of slice sums
-  if (!norm_w && mt_rows <= 2 && xc % 4 == 0 && xc * mt_rows <= 16 && nslices <= 16 && col_blocks > stream_wgs &&
-      stream_lds <= 64 * 1024 && LS_GEMM_STREAM) {
-    const int rounds = (col_blocks + stream_wgs - 1) / stream_wgs;
-    dim3 grid((col_blocks + rounds - 1) / rounds);
-    const size_t lds = stream_lds;
-#define LS_STREAM(MT_, XC_)                                                                                        \
-  hipLaunchKernelGGL((gemm_stream_kernel<T, MT_, EPI, XC_>), grid, dim3(nslices * 64), lds, stream,                \
-                     reinterpret_cast<const T*>(X), w, C, M, N, K, ldx, ldc, kslice, aligned, vec_ok, out_cols,   \
-                     col_blocks)
-    if (mt_rows == 1 && xc == 8) LS_STREAM(1, 8);
-    else if (mt_rows == 1 && xc == 16) LS_STREAM(1, 16);
-    else if (mt_rows == 2 && xc == 8) LS_STREAM(2, 8);
-    else return fail("gemm: no streaming kernel for %d chunks a slice and %d row tiles", xc, mt_rows);
+  // up to 32 rows one group of rows; up to 64 two groups of 32 that share the weights through L2
+  const int row_groups = mt_rows <= 2 ? 1 : 2;
+  const int group_tiles = mt_rows <= 2 ? mt_rows : 2;
+  const size_t stream_lds = 2 * (size_t)nslices * NT * group_tiles * 256 * sizeof(float);  // two sets of slice sums
+  // (two groups read the weights twice, the second time rarely from L2 in practice: with very many
+  // columns, where the tiled kernel does well, they are not worth it)
+  if (!norm_w && mt_rows <= 4 && xc % 4 == 0 && xc * group_tiles <= 16 && nslices <= 16 &&
+      col_blocks * row_groups > stream_wgs && stream_lds <= 128 * 1024 && !(row_groups > 1 && N >= 32768) &&
+      LS_GEMM_STREAM) {
+    int walkers = stream_wgs / row_groups;
+    const int rounds = (col_blocks + walkers - 1) / walkers;
+    walkers = (col_blocks + rounds - 1) / rounds;
+    if (row_groups > 1) walkers = (walkers + 7) / 8 * 8;  // whole rounds of the XCDs, see the kernel
+    dim3 grid(walkers * row_groups);
+    bool launched = true;
+#define LS_STREAM(MT_, XC_)                                                                                       \
+  if (stream_lds_ready<T, MT_, EPI, XC_>(stream_lds))                                                             \
+    hipLaunchKernelGGL((gemm_stream_kernel<T, MT_, EPI, XC_>), grid, dim3(nslices * 64), stream_lds, stream,      \
+                       reinterpret_cast<const T*>(X), w, C, M, N, K, ldx, ldc, kslice, aligned, vec_ok, out_cols, \
+                       col_blocks, row_groups);                                                                   \
+  else                                                                                                            \
+    launched = false
+    if (group_tiles == 1 && xc == 8) LS_STREAM(1, 8);
+    else if (group_tiles == 1 && xc == 16) LS_STREAM(1, 16);
+    else if (group_tiles == 2 && xc == 8) LS_STREAM(2, 8);
+    else launched = false;
 #undef LS_STREAM
-    return check_launch("gemm");
+    if (launched) return check_launch("gemm");
   }
   if (M <= 64 && !(M > 16 && N >= 32768)) {
     const int mt = (M + 15) / 16;

@@ -78,12 +78,12 @@ def test_gemm_row_does_not_depend_on_the_batch(dtype):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("k,n", [(4096, 4096 + 24), (1000, 16384 + 24), (5120, 4096 + 104), (260, 32768 + 40),
-                                 (2048, 8192 + 8)])
+                                 (2048, 8192 + 8), (96, 65536 + 48)])
 def test_gemm_with_few_rows_and_many_columns_has_the_same_bits(dtype, k, n):
-    """With up to 32 rows and more column blocks than the GPU holds workgroups, a workgroup walks
-    several column blocks with its rows of X in registers (the streaming kernel).  Every row has
-    the bits it has in a large batch, with every epilogue; a row of the sums equals the double
-    precision product."""
+    """With up to 64 rows and more column blocks than the GPU holds workgroups, a workgroup walks
+    several column blocks with its rows of X in registers (the streaming kernel; beyond 32 rows two
+    groups of workgroups take 32 rows each).  Every row has the bits it has in a large batch, with
+    every epilogue; a row of the sums equals the double precision product."""
     from lockstep_amd.ops import ADD_F32, STORE, STORE_F32
 
     g = torch.Generator().manual_seed(k + n)
@@ -93,8 +93,8 @@ def test_gemm_with_few_rows_and_many_columns_has_the_same_bits(dtype, k, n):
     K().gemm(x, w, full, STORE_F32)
     want = x[:3].double().cpu() @ w.double().cpu().T
     assert rel_err(full[:3], want) < 2e-5
-    base = torch.randn(32, n, generator=g).cuda()
-    for rows in (1, 8, 16, 17, 32):
+    base = torch.randn(64, n, generator=g).cuda()
+    for rows in (1, 8, 16, 17, 32, 33, 50, 64):
         part = torch.empty(rows, n, dtype=torch.float32, device="cuda")
         K().gemm(x[:rows], w, part, STORE_F32)
         assert torch.equal(part, full[:rows]), f"rows={rows}"
@@ -123,7 +123,7 @@ def test_swiglu_with_few_rows_and_many_columns_has_the_same_bits(dtype, inter, k
     K().gemm(x, w, full, SWIGLU)
     want = torch.nn.functional.silu(x[:2].double().cpu() @ gate.double().T) * (x[:2].double().cpu() @ up.double().T)
     assert rel_err(full[:2], want) < TOL[dtype]
-    for rows in (1, 8, 16, 20, 32):
+    for rows in (1, 8, 16, 20, 32, 40, 64):
         part = torch.empty(rows, inter, dtype=dtype, device="cuda")
         K().gemm(x[:rows], w, part, SWIGLU)
         assert torch.equal(part, full[:rows]), f"rows={rows}"
