@@ -6,10 +6,12 @@
 //   ascending 64-byte chunks of K, starting from zero;
 //   the slice sums are added in ascending order to a total that starts at +0.
 // The skinny kernel (M <= 64, decode) gives each slice to a wave, so the
-// weights stream from HBM with many waves in flight; the tiled kernel
-// (prefill) walks the slices one after the other with both operands staged
-// in LDS.  Both produce the same bits for a row, so a token's projections do
-// not depend on how many tokens share its step.
+// weights stream from HBM with many waves in flight; the streaming kernel
+// does the same for products with many columns, one workgroup walking many
+// column blocks; the slice kernel leaves the slice sums to its consumer; the
+// tiled kernel (prefill) walks the slices one after the other with both
+// operands staged in LDS.  All produce the same bits for a row, so a token's
+// projections do not depend on how many tokens share its step.
 //
 // The MFMA runs "swapped": W rows are the first operand, X rows the second,
 // so a lane ends with four consecutive n of one row m and stores them as one
