@@ -254,6 +254,72 @@ __global__ __launch_bounds__(256) void add_rmsnorm_kernel(float* __restrict__ h,
   }
 }
 
+// The same for rows of more than 1,024 elements: 1,024 threads, so that the
+// slice sums of a whole row of up to 4,096 elements are requested at once
+// (a row is one workgroup's work, and with few rows the kernel's time is that
+// of one row).  Thread (c0, t) = (tid / 256, tid % 256) forms the new values
+// of the runs 1024 c + 4 t, c = c0, c0 + 4, ...; the squares are then added by
+// the threads t of the first four waves over c = 0, 1, ... from LDS, which is
+// row_sumsq_part's order.
+template <typename T>
+__global__ __launch_bounds__(1024) void add_rmsnorm_wide_kernel(float* __restrict__ h, const float* __restrict__ P,
+                                                                int slices, int p_rows,
+                                                                const float* __restrict__ weight, T* __restrict__ out,
+                                                                const int* __restrict__ rows, int width, long ldh,
+                                                                long ld_out, float eps) {
+  extern __shared__ __attribute__((aligned(16))) float fresh_lds[];  // the new row
+  __shared__ float wave_part[4];
+  const int r_out = blockIdx.x;
+  const long row = rows ? rows[r_out] : r_out;
+  float* hrow = h + row * ldh;
+  const int t = threadIdx.x & 255;
+  const int c0 = threadIdx.x >> 8;
+  constexpr int BATCH = 16;  // slice sums requested together
+  for (int base = 1024 * c0 + 4 * t; base < width; base += 4096) {
+    f32x4 total = f32x4{0.f, 0.f, 0.f, 0.f};
+    const f32x4 old = *reinterpret_cast<const f32x4*>(hrow + base);
+    for (int s0 = 0; s0 < slices; s0 += BATCH) {
+      f32x4 p[BATCH];
+#pragma unroll
+      for (int u = 0; u < BATCH; ++u)  // clamped: all loads are issued before the first is needed
+        p[u] = *reinterpret_cast<const f32x4*>(P + ((long)min(s0 + u, slices - 1) * p_rows + row) * width + base);
+#pragma unroll
+      for (int u = 0; u < BATCH; ++u)
+        if (s0 + u < slices) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) total[e] = total[e] + p[u][e];
+        }
+    }
+    f32x4 fresh;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) fresh[e] = old[e] + total[e];
+    *reinterpret_cast<f32x4*>(hrow + base) = fresh;
+    *reinterpret_cast<f32x4*>(fresh_lds + base) = fresh;
+  }
+  if (out == nullptr) return;
+  __syncthreads();
+  if (c0 == 0) {
+    float part = 0.f;
+    for (int base = 4 * t; base < width; base += 1024) {
+      const f32x4 v = *reinterpret_cast<const f32x4*>(fresh_lds + base);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) part = part + v[e] * v[e];
+    }
+    part = wave_sum(part);
+    if ((threadIdx.x & 63) == 0) wave_part[threadIdx.x >> 6] = part;
+  }
+  __syncthreads();
+  const float total = ((wave_part[0] + wave_part[1]) + wave_part[2]) + wave_part[3];
+  const float scale = 1.0f / sqrtf(total / (float)width + eps);
+  T* dst = out + (long)r_out * ld_out;
+  for (int base = 1024 * c0 + 4 * t; base < width; base += 4096) {
+    const f32x4 v = *reinterpret_cast<const f32x4*>(fresh_lds + base);
+    const f32x4 w = *reinterpret_cast<const f32x4*>(weight + base);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) dst[base + e] = from_f32<T>((v[e] * scale) * w[e]);
+  }
+}
+
 // ---------------------------------------------------------------------------
 // Arg-max of float rows with the lowest index among equal maxima (NaN never
 // wins; a row without a winner gives 0).  A row is cut into chunks of
@@ -427,14 +493,24 @@ extern "C" int ls_add_rmsnorm(int dtype, float* h, const float* P, int slices, i
              "add_rmsnorm: the norm needs an aligned weight and an output row of %d elements", width);
   LS_REQUIRE(rows != nullptr || n_rows <= p_rows, "add_rmsnorm: %d rows, the slice sums hold %d", n_rows, p_rows);
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  if (dtype != kF32 && dtype != kBF16) return fail("add_rmsnorm: unknown dtype %d", dtype);
+  // wide rows (few of them: the time of the kernel is the time of one row): four times the threads
+  const size_t row_bytes = (size_t)width * sizeof(float);
+  if (width > 1024 && row_bytes <= 64 * 1024) {
+    if (dtype == kF32)
+      hipLaunchKernelGGL(add_rmsnorm_wide_kernel<float>, dim3(n_rows), dim3(1024), row_bytes, s, h, P, slices, p_rows,
+                         weight, (float*)out, rows, width, ldh, ld_out, eps);
+    else
+      hipLaunchKernelGGL(add_rmsnorm_wide_kernel<bf16_t>, dim3(n_rows), dim3(1024), row_bytes, s, h, P, slices,
+                         p_rows, weight, (bf16_t*)out, rows, width, ldh, ld_out, eps);
+    return check_launch("add_rmsnorm");
+  }
   if (dtype == kF32)
     hipLaunchKernelGGL(add_rmsnorm_kernel<float>, dim3(n_rows), dim3(256), 0, s, h, P, slices, p_rows, weight,
                        (float*)out, rows, width, ldh, ld_out, eps);
-  else if (dtype == kBF16)
+  else
     hipLaunchKernelGGL(add_rmsnorm_kernel<bf16_t>, dim3(n_rows), dim3(256), 0, s, h, P, slices, p_rows, weight,
                        (bf16_t*)out, rows, width, ldh, ld_out, eps);
-  else
-    return fail("add_rmsnorm: unknown dtype %d", dtype);
   return check_launch("add_rmsnorm");
 }
 
