@@ -1102,21 +1102,13 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
       k_page[i] = pages[min((p / KPIECES) >> page_shift, 15)];
       v_page[i] = pages[min(((p / D) * VEC) >> page_shift, 15)];
     }
-    // Keys from kv_len on are not fetched: their scores are masked whatever the key rows hold, and their
-    // values are set to zero in LDS before use (the tile that holds kv_len is always cleaned).
-    const int live = sm.kv_len - ti * kTileKeys;
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
-      const int first = i * NT + wave * 64;  // the wave's first piece: the tests below are uniform for the wave
-      if (PER * NT != TOTAL && first >= TOTAL) break;
-      if (first / KPIECES < live) {
-        const T* k_src = k_pages + (long)max(k_page[i], 0) * page_stride + k_off[i];
-        __builtin_amdgcn_global_load_lds((gptr_t)k_src, (lptr_t)(k_buf + first * 16), 16, 0, 0);
-      }
-      if ((first / D) * VEC < live) {
-        const T* v_src = v_pages + (long)max(v_page[i], 0) * page_stride + v_off[i];
-        __builtin_amdgcn_global_load_lds((gptr_t)v_src, (lptr_t)(v_buf + first * 16), 16, 0, 0);
-      }
+      if (PER * NT != TOTAL && i * NT + wave * 64 >= TOTAL) break;  // uniform for the wave
+      const T* k_src = k_pages + (long)max(k_page[i], 0) * page_stride + k_off[i];
+      __builtin_amdgcn_global_load_lds((gptr_t)k_src, (lptr_t)(k_buf + (i * NT + wave * 64) * 16), 16, 0, 0);
+      const T* v_src = v_pages + (long)max(v_page[i], 0) * page_stride + v_off[i];
+      __builtin_amdgcn_global_load_lds((gptr_t)v_src, (lptr_t)(v_buf + (i * NT + wave * 64) * 16), 16, 0, 0);
     }
   };
 

@@ -17,6 +17,7 @@
 // so a lane ends with four consecutive n of one row m and stores them as one
 // vector.
 
+#include <algorithm>
 #include <type_traits>
 
 #include "common.h"
@@ -509,6 +510,102 @@ __global__ __launch_bounds__(256) void gemm_slices_kernel(const T* __restrict__ 
   }
 }
 
+// The slice kernel as a walk (products with many K slices and enough column
+// blocks that workgroups can take several): wave = slice, its rows of X stay
+// in registers, the weights of the next units are in flight across column
+// blocks as in the streaming kernel.  The waves share nothing, so there is no
+// barrier.
+template <typename T, int MT, int XC>
+__global__ __launch_bounds__(256) void gemm_slices_stream_kernel(const T* __restrict__ X, const T* __restrict__ W,
+                                                                 float* __restrict__ P, int M, int N, int K, long ldx,
+                                                                 int kslice, int aligned, int slices_per_group,
+                                                                 int blocks) {
+  typedef Atom<T> A;
+  typedef typename A::vec_t vec_t;
+  constexpr int UC = 4;                          // chunks per unit
+  constexpr int UNITS = XC / UC;                 // units per column block
+  constexpr int RING = (MT * XC <= 24) ? 4 : 2;  // unit buffers in registers
+  constexpr int AHEAD = RING - 1;
+  static_assert(XC % UC == 0 && (UNITS % RING == 0 || (2 * UNITS) % RING == 0), "units and ring");
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int row16 = lane & 15;
+  const int g = lane >> 4;
+  const int nslices = (K + kslice - 1) / kslice;
+  const int s = blockIdx.y * slices_per_group + wave;
+  if (wave >= slices_per_group || s >= nslices) return;
+  const int k_begin = s * kslice;
+  const int k_end = min(K, k_begin + kslice);
+  const int walkers = gridDim.x;
+  const int m_base = blockIdx.z * MT * 16;  // more than 16 * MT rows: groups of rows, each with workgroups of its own
+
+  auto fetch = [&](int b, int q, vec_t (&dst)[UC]) {
+    const int n = b * 16 + row16;
+#pragma unroll
+    for (int c = 0; c < UC; ++c) {
+      const int kc = k_begin + (q * UC + c) * A::KCHUNK;
+      dst[c] = load_vec<T>(W, n, kc + g * A::VEC, K, K, n < N && kc < k_end, aligned);
+    }
+  };
+  vec_t wbuf[RING][UC];
+  int b = blockIdx.x;
+#pragma unroll
+  for (int u = 0; u < AHEAD; ++u) {
+    const int bu = b + (u / UNITS) * walkers;
+    if (bu < blocks) fetch(bu, u % UNITS, wbuf[u % RING]);
+  }
+  vec_t xs[MT][XC];
+#pragma unroll
+  for (int j = 0; j < MT; ++j)
+#pragma unroll
+    for (int c = 0; c < XC; ++c) {
+      const int kc = k_begin + c * A::KCHUNK;
+      xs[j][c] = load_vec<T>(X, m_base + j * 16 + row16, kc + g * A::VEC, K, ldx,
+                             m_base + j * 16 + row16 < M && kc < k_end, aligned);
+    }
+
+  auto block_step = [&](auto par) {
+    constexpr int P0 = decltype(par)::value;
+    f32x4 acc[MT];
+#pragma unroll
+    for (int j = 0; j < MT; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int idx = 0; idx < UNITS; ++idx) {
+      const int far_block = b + ((idx + AHEAD) / UNITS) * walkers;
+      if (far_block < blocks) fetch(far_block, (idx + AHEAD) % UNITS, wbuf[(P0 + idx + AHEAD) % RING]);
+#pragma unroll
+      for (int c = 0; c < UC; ++c) {
+        if (k_begin + (idx * UC + c) * A::KCHUNK >= k_end) break;  // uniform: a chunk is visited iff it starts inside the slice
+#pragma unroll
+        for (int j = 0; j < MT; ++j) A::mma(acc[j], wbuf[(P0 + idx) % RING][c], xs[j][idx * UC + c]);
+      }
+    }
+    const int n = b * 16 + g * 4;
+#pragma unroll
+    for (int j = 0; j < MT; ++j) {
+      const int m = m_base + j * 16 + row16;
+      if (m >= M || n >= N) continue;
+      float* dst = P + ((long)s * M + m) * N + n;
+      if (n + 3 < N && (N & 3) == 0) {
+        *reinterpret_cast<f32x4*>(dst) = acc[j];
+      } else {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          if (n + r < N) dst[r] = acc[j][r];
+      }
+    }
+  };
+  while (b < blocks) {
+    block_step(std::integral_constant<int, 0>{});
+    b += walkers;
+    if (UNITS % RING != 0) {
+      if (b >= blocks) break;
+      block_step(std::integral_constant<int, UNITS % RING>{});
+      b += walkers;
+    }
+  }
+}
+
 // ---------------------------------------------------------------------------
 // Tiled kernel: BM x BN outputs per workgroup, four waves in a 2 x 2 grid,
 // each (BM/2) x (BN/2).  Both operands go through LDS in stages of 128 bytes
@@ -707,7 +804,8 @@ int launch_gemm(const void* X, const void* W, void* C, int M, int N, int K, long
   const size_t stream_lds = 2 * (size_t)nslices * NT * group_tiles * 256 * sizeof(float);  // two sets of slice sums
   // (two groups read the weights twice, the second time rarely from L2 in practice: with very many
   // columns, where the tiled kernel does well, they are not worth it)
-  if (!norm_w && mt_rows <= 4 && xc % 4 == 0 && xc * group_tiles <= 16 && nslices <= 16 &&
+  // (with fewer than eight slices the skinny kernel's small workgroups, several a CU, do as well or better)
+  if (!norm_w && mt_rows <= 4 && xc % 4 == 0 && xc * group_tiles <= 16 && nslices >= 8 && nslices <= 16 &&
       col_blocks * row_groups > stream_wgs && stream_lds <= 128 * 1024 && !(row_groups > 1 && N >= 32768) &&
       LS_GEMM_STREAM) {
     int walkers = stream_wgs / row_groups;
@@ -828,12 +926,39 @@ extern "C" int ls_gemm_slices(int dtype, const void* X, const void* W, float* P,
   groups = (nslices + per_group - 1) / per_group;
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   dim3 grid(col_blocks, groups);
-  const size_t elem = dtype == kF32 ? 4 : 2;
   const int vec = dtype == kF32 ? 4 : 8;
   const int aligned = (K % vec == 0) && (ldx % vec == 0) && (reinterpret_cast<uintptr_t>(X) % 16 == 0) &&
                       (reinterpret_cast<uintptr_t>(W) % 16 == 0);
-  (void)elem;
   const int mt = (M + 15) / 16;
+  // With more than 16 rows, where the rows of X outweigh the weights of a column block, and at least four
+  // workgroups a CU, workgroups walk two or more column blocks each with X in registers (the walk keeps
+  // two workgroups a CU).  Up to 16 rows the walk measured no faster: fewer waves, less in flight.
+  const int xc = kslice / (dtype == kF32 ? 16 : 32);  // 64-byte chunks per slice
+  // row tiles a workgroup holds in registers (xs: 4 * xc registers a tile); more rows go to further groups
+  // (24 chunks a slice with two tiles need 268 registers: one wave a SIMD, measured slower than the plain kernel)
+  const int group_tiles = xc <= 8 ? std::min(mt, 4) : (xc <= 16 ? std::min(mt, 2) : 0);
+  const int row_groups = group_tiles > 0 ? (mt + group_tiles - 1) / group_tiles : 0;
+  const int rounds =
+      (int)std::min<long>(4, (long)col_blocks * groups * std::max(row_groups, 1) / (2L * compute_units()));
+  if (rounds >= 2 && mt >= 2 && group_tiles > 0 && xc % 4 == 0 && LS_GEMM_STREAM) {
+    int walkers = (col_blocks + rounds - 1) / rounds;
+    if (row_groups > 1) walkers = (walkers + 7) / 8 * 8;  // the groups' workgroups of a walk sit on the same XCD
+    dim3 walk_grid(walkers, groups, row_groups);
+    bool launched = true;
+#define LS_WALK(T_, MT_, XC_)                                                                                     \
+  hipLaunchKernelGGL((gemm_slices_stream_kernel<T_, MT_, XC_>), walk_grid, dim3(64 * per_group), 0, s, (const T_*)X, \
+                     (const T_*)W, P, M, N, K, ldx, kslice, aligned, per_group, col_blocks)
+#define LS_WALK_T(T_)                                                          \
+  if (group_tiles == 2 && xc == 8) LS_WALK(T_, 2, 8);                          \
+  else if (group_tiles == 3 && xc == 8) LS_WALK(T_, 3, 8);                     \
+  else if (group_tiles == 4 && xc == 8) LS_WALK(T_, 4, 8);                     \
+  else if (group_tiles == 2 && xc == 16) LS_WALK(T_, 2, 16);                   \
+  else launched = false
+    if (dtype == kF32) { LS_WALK_T(float); } else if (dtype == kBF16) { LS_WALK_T(bf16_t); } else launched = false;
+#undef LS_WALK_T
+#undef LS_WALK
+    if (launched) return check_launch("gemm_slices");
+  }
 #define LS_SLICES(T_, MT_)                                                                                       \
   hipLaunchKernelGGL((gemm_slices_kernel<T_, MT_>), grid, dim3(64 * per_group), 0, s, (const T_*)X, (const T_*)W, P, M, \
                      N, K, ldx, kslice, aligned, per_group)
