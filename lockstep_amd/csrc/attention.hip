@@ -1433,12 +1433,24 @@ __global__ __launch_bounds__(256) void combine_kernel(const SeqMeta* __restrict_
   RowState run;
   run.reset();
   const long pr0 = item.part_base + ((long)kvh * rows_total + r) * item.n_splits;
-  for (int s = 0; s < item.n_splits; ++s) {
-    const long pr = pr0 + s;
-    f32x4 acc[DB];
+  // The partial results of several splits are requested together (a request far away has many splits and
+  // the fold of each waits for its loads); they are folded in ascending order all the same.
+  constexpr int BATCH = DB <= 8 ? 4 : 2;
+  for (int s0 = 0; s0 < item.n_splits; s0 += BATCH) {
+    f32x4 acc[BATCH][DB];
+    float m[BATCH], l[BATCH];
 #pragma unroll
-    for (int blk = 0; blk < DB; ++blk) acc[blk] = *reinterpret_cast<const f32x4*>(part_acc + pr * D + blk * 16 + 4 * g);
-    fold_split<T>(run, acc, part_ml[pr * 2], part_ml[pr * 2 + 1]);
+    for (int u = 0; u < BATCH; ++u) {
+      const long pr = pr0 + min(s0 + u, item.n_splits - 1);  // clamped: loaded, not used
+#pragma unroll
+      for (int blk = 0; blk < DB; ++blk)
+        acc[u][blk] = *reinterpret_cast<const f32x4*>(part_acc + pr * D + blk * 16 + 4 * g);
+      m[u] = part_ml[pr * 2];
+      l[u] = part_ml[pr * 2 + 1];
+    }
+#pragma unroll
+    for (int u = 0; u < BATCH; ++u)
+      if (s0 + u < item.n_splits) fold_split<T>(run, acc[u], m[u], l[u]);
   }
   store_output<T>(run, out + (long)(item.q_off + qi) * ldo + (long)head * D, g);
 }
