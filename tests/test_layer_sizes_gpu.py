@@ -1,0 +1,165 @@
+"""The engine at the layer sizes of real models (one or two layers of them):
+head size 128, widths of 1,024 to 4,096, K cut into 4 to 16 slices.  These
+sizes take other kernels and other paths inside the kernels than the tiny
+configurations do (128 x 128 tiles, the streaming and the walking products,
+the cooperative and the wide attention kernel at their full tile sizes), so
+the cuttings are compared bit for bit here as well, and the 32-bit path with
+the plain implementation."""
+
+from __future__ import annotations
+
+import json
+
+import pytest
+import torch
+
+from helpers import BF16_TOL, FP32_TOL, feed, random_tokens, rel_err
+
+pytestmark = pytest.mark.gpu
+
+# width, query heads, kv heads, feed-forward width, layers, vocabulary (not a multiple of 16), tied head
+SIZES = {
+    "0.6b-like": dict(hidden_size=1024, num_attention_heads=16, num_key_value_heads=8, head_dim=128,
+                      intermediate_size=3072, num_hidden_layers=2, vocab_size=4099, tie_word_embeddings=True,
+                      rms_norm_eps=1e-6, rope_theta=1000000.0, max_position_embeddings=2048),
+    "8b-like": dict(hidden_size=4096, num_attention_heads=32, num_key_value_heads=8, head_dim=128,
+                    intermediate_size=12288, num_hidden_layers=1, vocab_size=5003, tie_word_embeddings=False,
+                    rms_norm_eps=1e-6, rope_theta=1000000.0, max_position_embeddings=2048),
+}
+
+
+@pytest.fixture(scope="module")
+def models(tmp_path_factory):
+    """name -> (folder, config); weights as a real checkpoint has them in size (std 0.02), norm
+    weights spread around one."""
+    from lockstep_amd.config import Qwen3Config
+    from lockstep_amd.weights import write_random_model
+
+    out = {}
+    for name, raw in SIZES.items():
+        config = Qwen3Config.from_dict(raw)
+        folder = tmp_path_factory.mktemp(name.replace(".", "_"))
+        write_random_model(config, folder, seed=11, std=0.02, norm_std=0.1)
+        out[name] = (folder, config)
+    return out
+
+
+def load(folder, dtype):
+    from lockstep_amd.engine.model import load_model
+
+    return load_model(folder, dtype=dtype)
+
+
+@pytest.mark.parametrize("name", list(SIZES))
+def test_cuttings_give_the_same_bits_at_real_layer_sizes(models, name):
+    """bfloat16: a request whole; most of it in one step and the last 32 tokens one by one; in
+    portions of changing size; and the tail decoded beside other requests, from the captured graph."""
+    from lockstep_amd.engine.batch import StepEntry
+
+    folder, config = models[name]
+    model = load(folder, "bfloat16")
+    vocab = config.vocab_size
+    n = 620                                                       # three splits, the last tile partly filled
+    tokens = random_tokens(n, vocab, seed=1)
+    cache = model.make_cache(num_pages=3 * 48 + 8, page_size=16, max_requests=8)
+    whole = feed(model, cache, "whole", tokens, [n])
+    assert torch.isfinite(whole).all()
+    cache.close("whole")
+    tail = feed(model, cache, "tail", tokens, [n - 32] + [1] * 32)
+    assert torch.equal(tail, whole), "prefix in one step, the last 32 tokens one by one"
+    cache.close("tail")
+    cut = feed(model, cache, "cut", tokens, [2, 37, 128, 3, 255, 64, 2, 100])
+    assert torch.equal(cut, whole), "portions of changing size"
+    cache.close("cut")
+
+    # the last 24 tokens beside two other requests that decode too (different lengths), then beside a prompt portion
+    others = {"o1": random_tokens(300, vocab, seed=2), "o2": random_tokens(77, vocab, seed=3)}
+    for rid, toks in others.items():
+        cache.open(rid)
+        model.step(cache, [StepEntry(rid, toks[:-30], [])])
+    cache.open("mix")
+    model.step(cache, [StepEntry("mix", tokens[:n - 24], [])])
+    rows = []
+    for k in range(24):
+        entries = [StepEntry("mix", [tokens[n - 24 + k]], [0])]
+        for rid, toks in others.items():
+            entries.append(StepEntry(rid, [toks[len(toks) - 30 + k]], []))
+        if k == 20:                                               # a prompt portion joins the decode step
+            cache.open("late")
+            entries.append(StepEntry("late", random_tokens(50, vocab, seed=4), []))
+        rows.append(model.step(cache, entries).cpu())
+    assert torch.equal(torch.cat(rows), whole[n - 24:]), "decoded beside other requests"
+    assert model.graph_replays > 10
+
+
+@pytest.mark.parametrize("name", list(SIZES))
+def test_many_requests_decode_with_the_bits_of_one(models, name):
+    """40 requests in a decode step (three row tiles in the products, more than 256 (request, kv
+    head) pairs in attention) against each of them alone."""
+    from lockstep_amd.engine.batch import StepEntry
+
+    folder, config = models[name]
+    model = load(folder, "bfloat16")
+    vocab = config.vocab_size
+    n_req, n_decode = 40, 3
+    lengths = [5 + (61 * i) % 400 for i in range(n_req)]
+    prompts = [random_tokens(m + n_decode, vocab, seed=50 + i) for i, m in enumerate(lengths)]
+    cache = model.make_cache(num_pages=sum(-(-(m + n_decode) // 16) for m in lengths) + 4, page_size=16,
+                             max_requests=n_req + 1)
+    for lo in range(0, n_req, 4):
+        group = range(lo, min(lo + 4, n_req))
+        for i in group:
+            cache.open(f"r{i}")
+        model.step(cache, [StepEntry(f"r{i}", prompts[i][:lengths[i]], []) for i in group])
+    together = [model.step(cache, [StepEntry(f"r{i}", [prompts[i][lengths[i] + k]], [0]) for i in range(n_req)]).cpu()
+                for k in range(n_decode)]
+    for i in (0, 13, 39):
+        alone = model.make_cache(num_pages=32, page_size=16)
+        want = feed(model, alone, "x", prompts[i], [lengths[i]] + [1] * n_decode)[lengths[i]:]
+        assert torch.equal(torch.stack([t[i] for t in together]), want), f"request {i} (context {lengths[i]})"
+
+
+def test_the_32_bit_path_matches_plain_at_real_layer_sizes(models):
+    """float32 against the plain float64 implementation, and bfloat16 within its tolerance, on the
+    two-layer configuration (whole prompt and decoded tail)."""
+    from plain.qwen3_plain import PlainModel
+
+    folder, config = models["0.6b-like"]
+    tokens = random_tokens(300, config.vocab_size, seed=9)
+    want = PlainModel(folder).logits(tokens)
+    for dtype, tol in (("float32", FP32_TOL), ("bfloat16", BF16_TOL)):
+        model = load(folder, dtype)
+        cache = model.make_cache(num_pages=40, page_size=16)
+        got = feed(model, cache, "a", tokens, [270] + [1] * 30)
+        err = rel_err(got, want)
+        print(f"0.6b-like {dtype}: rel err {err:.3e}")
+        assert err < tol
+
+
+def test_the_device_side_loop_at_real_layer_sizes(models):
+    """Greedy tokens from the device-side loop equal those of step-by-step decoding (logits well
+    apart are not guaranteed with these weights, so the comparison is between the engine's two ways,
+    which share every kernel)."""
+    from lockstep_amd.engine.batch import StepEntry
+
+    folder, config = models["0.6b-like"]
+    model = load(folder, "bfloat16")
+    prompts = {f"r{i}": random_tokens(40 + 90 * i, config.vocab_size, seed=70 + i) for i in range(3)}
+    picked = {}
+    for way in ("loop", "steps"):
+        cache = model.make_cache(num_pages=96, page_size=16, max_requests=4)
+        first = []
+        for rid, toks in prompts.items():
+            cache.open(rid)
+            logits = model.step(cache, [StepEntry(rid, toks, [len(toks) - 1])])
+            first.append(int(logits[0].argmax()))
+        if way == "loop":
+            picked[way] = model.decode_greedy(cache, list(prompts), first, 12).tolist()
+        else:
+            rows, cur = [], first
+            for _ in range(12):
+                logits = model.step(cache, [StepEntry(rid, [t], [0]) for rid, t in zip(prompts, cur)])
+                cur = [int(row.argmax()) for row in logits]
+                rows.append(cur)
+            picked[way] = rows
+    assert picked["loop"] == picked["steps"]
