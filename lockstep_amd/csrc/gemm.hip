@@ -33,6 +33,9 @@ namespace ls {
 #ifndef LS_GEMM_STREAM
 #define LS_GEMM_STREAM 1      // 0: never the streaming kernel
 #endif
+#ifndef LS_GEMM_GROUP_M
+#define LS_GEMM_GROUP_M 4     // row tiles per band of the tile numbering (0: column-major numbering)
+#endif
 #ifndef LS_GEMM_PD_SMALL
 #define LS_GEMM_PD_SMALL 2    // ... and of the 64 x 64 kernel
 #endif
@@ -634,12 +637,22 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const T* __restrict__ X
   constexpr int STAGE_BYTES = (BM + BN) * kRowStride;
   __shared__ __attribute__((aligned(16))) unsigned char lds[2 * STAGE_BYTES];
 
-  // XCD-aware numbering: consecutive ids on one XCD walk the row tiles of one weight tile
+  // XCD-aware numbering: workgroup ids go round the eight XCDs; give each XCD a contiguous run of tiles
   int id = blockIdx.x;
   const int total_tiles = tiles_m * tiles_n;
   if (total_tiles % 8 == 0) id = (id % 8) * (total_tiles / 8) + id / 8;
+#if LS_GEMM_GROUP_M > 0
+  // ... and inside bands of LS_GEMM_GROUP_M row tiles, so that the workgroups that run together on an XCD
+  // form a block of tiles with few distinct operand tiles (those stay in the XCD's L2)
+  const int band = id / (LS_GEMM_GROUP_M * tiles_n);
+  const int in_band = id % (LS_GEMM_GROUP_M * tiles_n);
+  const int band_rows = min(LS_GEMM_GROUP_M, tiles_m - band * LS_GEMM_GROUP_M);
+  const int tile_m = band * LS_GEMM_GROUP_M + in_band % band_rows;
+  const int tile_n = in_band / band_rows;
+#else
   const int tile_m = id % tiles_m;
   const int tile_n = id / tiles_m;
+#endif
   const int m_base = tile_m * BM;
   const int n_base = tile_n * BN;
 
