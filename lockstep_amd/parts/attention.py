@@ -26,6 +26,9 @@ import os
 # Steps of single decoded tokens run norm, rotation and cache write inside the
 # attention kernel (one launch less per layer); "0" keeps the separate kernel.
 FUSE_DECODE = os.environ.get("LOCKSTEP_FUSE_DECODE", "1") not in ("", "0")
+# From this many attention workgroups on (two a CU: the kernel is then bound by the cache it streams) the
+# prologue of the fused kernel costs more than the separate norm/rotation launch; measured +2 % at batch 64.
+FUSE_DECODE_BELOW = int(os.environ.get("LOCKSTEP_FUSE_DECODE_BELOW", "512"))
 
 
 @register_part("attention")
@@ -128,7 +131,7 @@ class Attention(Mixer):
         attn = ctx.buf("attention.out", (t, nq * d), rt.dtype)
         window = int(self.window) if self.window is not None else 0
         plan = ctx.attention_plan(nq // nkv, nkv, d, window)
-        if plan.decode_fused and FUSE_DECODE:
+        if plan.decode_fused and FUSE_DECODE and plan.n_coop * nkv < FUSE_DECODE_BELOW:
             # single decoded tokens: norm, rotation and cache write happen inside the attention kernel
             k.attention_decode(qkv, nq, nkv, d, key_pages, value_pages, group.page_size, group.table, ctx.seqs,
                                plan.coop_items, plan.n_coop, attn, plan.part_acc, plan.part_ml, self.scale, window,

@@ -94,14 +94,16 @@ def test_cuttings_give_the_same_bits_at_real_layer_sizes(models, name):
 
 @pytest.mark.parametrize("name", list(SIZES))
 def test_many_requests_decode_with_the_bits_of_one(models, name):
-    """40 requests in a decode step (three row tiles in the products, more than 256 (request, kv
-    head) pairs in attention) against each of them alone."""
+    """Many requests in a decode step against each of them alone: 40 (three row tiles in the
+    products, more than 256 (request, kv head) pairs in attention: one workgroup a pair, norm and
+    rotation inside the attention kernel) and 66 (five row tiles, more than 512 pairs: norm and
+    rotation as a launch of their own)."""
     from lockstep_amd.engine.batch import StepEntry
 
     folder, config = models[name]
     model = load(folder, "bfloat16")
     vocab = config.vocab_size
-    n_req, n_decode = 40, 3
+    n_req, n_decode = {"0.6b-like": 66, "8b-like": 40}[name], 3
     lengths = [5 + (61 * i) % 400 for i in range(n_req)]
     prompts = [random_tokens(m + n_decode, vocab, seed=50 + i) for i, m in enumerate(lengths)]
     cache = model.make_cache(num_pages=sum(-(-(m + n_decode) // 16) for m in lengths) + 4, page_size=16,
@@ -113,7 +115,7 @@ def test_many_requests_decode_with_the_bits_of_one(models, name):
         model.step(cache, [StepEntry(f"r{i}", prompts[i][:lengths[i]], []) for i in group])
     together = [model.step(cache, [StepEntry(f"r{i}", [prompts[i][lengths[i] + k]], [0]) for i in range(n_req)]).cpu()
                 for k in range(n_decode)]
-    for i in (0, 13, 39):
+    for i in (0, 13, n_req - 1):
         alone = model.make_cache(num_pages=32, page_size=16)
         want = feed(model, alone, "x", prompts[i], [lengths[i]] + [1] * n_decode)[lengths[i]:]
         assert torch.equal(torch.stack([t[i] for t in together]), want), f"request {i} (context {lengths[i]})"
