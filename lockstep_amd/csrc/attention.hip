@@ -1612,32 +1612,37 @@ extern "C" int ls_attention_decode(int dtype, const void* qkv, long ld, void* k_
   return check_launch("attention (decode, fused)");
 }
 
-// The wide kernel: two buffers of a K and a V tile, and two rows of page ids.
+// The wide kernel: two buffers of a K and a V tile, and two rows of page ids.  Eight waves (row blocks of
+// 128) or, for steps with so few rows that 128-row blocks would leave CUs without work, four (blocks of 64).
 constexpr int kWideWaves = 8;
+constexpr int kNarrowWaves = 4;
 static size_t wide_lds_bytes(int dtype) { return 4 * (size_t)kTileKeys * D * (dtype == kF32 ? 4 : 2) + 2 * 16 * sizeof(int); }
+template <typename T, int NW>
+static bool wide_kernel_ready(size_t bytes) {
+  static int state = 0;  // 0 unknown, 1 granted, -1 refused
+  if (state == 0) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_wide_kernel<T, NW>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+    if (e != hipSuccess) (void)hipGetLastError();
+    state = e == hipSuccess ? 1 : -1;
+  }
+  return state == 1;
+}
 static bool wide_supported(int dtype) {
   const size_t bytes = wide_lds_bytes(dtype);
   if (bytes > kLdsLimit) return false;
   if (bytes <= 64 * 1024) return true;
-  static int state[2] = {0, 0};
-  int& st = state[dtype == kF32 ? 0 : 1];
-  if (st == 0) {
-    hipError_t e = dtype == kF32
-        ? hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_wide_kernel<float, kWideWaves>),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes)
-        : hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_wide_kernel<bf16_t, kWideWaves>),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
-    if (e != hipSuccess) (void)hipGetLastError();
-    st = e == hipSuccess ? 1 : -1;
-  }
-  return st == 1;
+  return dtype == kF32 ? (wide_kernel_ready<float, kWideWaves>(bytes) && wide_kernel_ready<float, kNarrowWaves>(bytes))
+                       : (wide_kernel_ready<bf16_t, kWideWaves>(bytes) && wide_kernel_ready<bf16_t, kNarrowWaves>(bytes));
 }
-// 1 if the wide kernel (variant 4) can run for this dtype.
+// 1 if the wide kernel (variants 4 and 5) can run for this dtype.
 extern "C" int ls_attn_wide_supported(int dtype) { return wide_supported(dtype) ? 1 : 0; }
 // Rows of one work item's row block: AttnItem.row_block counts blocks of this many rows.
-extern "C" int ls_attn_block_rows(int variant) { return variant == 4 ? 16 * kWideWaves : 64; }
+extern "C" int ls_attn_block_rows(int variant) {
+  return variant == 4 ? 16 * kWideWaves : variant == 5 ? 16 * kNarrowWaves : 64;
+}
 
-// variant: 4 runs the wide kernel (row blocks of ls_attn_block_rows(4) rows);
+// variant: 4 and 5 run the wide kernel (row blocks of ls_attn_block_rows(variant) rows: 128 and 64);
 // variant: 3 runs the cooperative kernel (all items must have at most 16 rows);
 // variant: 0 picks the staged kernel where its tiles fit into LDS and the
 // direct one elsewhere, 1 forces the direct kernel, 2 the staged one.
@@ -1681,22 +1686,21 @@ extern "C" int ls_attention(int dtype, const void* q, long ldq, const void* k_pa
     if (rc != 0) return rc;
     return check_launch("attention (cooperative)");
   }
-  if (variant == 4) {
+  if (variant == 4 || variant == 5) {
     LS_REQUIRE(wide_supported(dtype), "attention: the wide variant does not fit into LDS for this head size");
     LS_REQUIRE(page_size >= 8, "attention: the wide variant needs pages of at least 8 keys, got %d", page_size);
+    LS_REQUIRE(dtype == kF32 || dtype == kBF16, "attention: unknown dtype %d", dtype);
     const size_t bytes = wide_lds_bytes(dtype);
-    if (dtype == kF32)
-      hipLaunchKernelGGL((attention_wide_kernel<float, kWideWaves>), grid, dim3(64 * kWideWaves), bytes, s,
-                         (const float*)q, ldq, (const float*)k_pages, (const float*)v_pages, nkv, page_size,
-                         page_shift, table, table_stride, (const SeqMeta*)seqs, (const AttnItem*)items, (float*)out,
-                         ldo, part_acc, part_ml, G, scale, window);
-    else if (dtype == kBF16)
-      hipLaunchKernelGGL((attention_wide_kernel<bf16_t, kWideWaves>), grid, dim3(64 * kWideWaves), bytes, s,
-                         (const bf16_t*)q, ldq, (const bf16_t*)k_pages, (const bf16_t*)v_pages, nkv, page_size,
-                         page_shift, table, table_stride, (const SeqMeta*)seqs, (const AttnItem*)items, (bf16_t*)out,
-                         ldo, part_acc, part_ml, G, scale, window);
-    else
-      return fail("attention: unknown dtype %d", dtype);
+#define LS_WIDE(T_, NW_)                                                                                          \
+  hipLaunchKernelGGL((attention_wide_kernel<T_, NW_>), grid, dim3(64 * NW_), bytes, s, (const T_*)q, ldq,          \
+                     (const T_*)k_pages, (const T_*)v_pages, nkv, page_size, page_shift, table, table_stride,       \
+                     (const SeqMeta*)seqs, (const AttnItem*)items, (T_*)out, ldo, part_acc, part_ml, G, scale, window)
+    if (dtype == kF32) {
+      if (variant == 4) LS_WIDE(float, kWideWaves); else LS_WIDE(float, kNarrowWaves);
+    } else {
+      if (variant == 4) LS_WIDE(bf16_t, kWideWaves); else LS_WIDE(bf16_t, kNarrowWaves);
+    }
+#undef LS_WIDE
     return check_launch("attention (wide)");
   }
   const bool staged = variant != 1 && staged_fits(dtype, lds_bytes);

@@ -47,6 +47,7 @@ class AttentionPlan:
     n_combine: int
     part_acc: torch.Tensor | None
     part_ml: torch.Tensor | None
+    wide_variant: int = 4     # 4: row blocks of 128 rows, 5: of 64
 
 
 class Workspace:
@@ -140,6 +141,7 @@ class StepContext:
                                               np.asarray(want, dtype=np.int64)]
         self._plans: dict[tuple, tuple] = {}
         self._plan_specs: list[tuple] = []
+        self._wide_variants: dict[tuple, int] = {}
         self._uploaded = False
         self._meta = None
         self._views = None
@@ -157,7 +159,12 @@ class StepContext:
         # with a workgroup per CU anyway, one workgroup walks all splits of a request itself
         whole_requests = self.n_seqs * nkv >= 256
         wide_ok = self.rt.kernels.wide_supported(head_dim, self.rt.dtype, self.cache.page_size)
-        wide_rows = self.rt.kernels.attention_block_rows(head_dim, 4)
+        wide_variant, wide_rows = 4, self.rt.kernels.attention_block_rows(head_dim, 4)
+        if wide_ok:
+            # so few rows that the large row blocks would leave half of the CUs without a workgroup: smaller blocks
+            blocks = sum(-(-(int(q) * group_size) // wide_rows) for q in self.q_len if int(q) * group_size > 64)
+            if 0 < blocks * nkv <= kernels.compute_units() // 2:
+                wide_variant, wide_rows = 5, self.rt.kernels.attention_block_rows(head_dim, 5)
         items, coop, wide, combine = [], [], [], []
         coop_max_rows = 0
         part_rows = 0
@@ -228,6 +235,7 @@ class StepContext:
                             pack_combine_items(combine, self._seq_rows), len(items), len(combine), part_rows,
                             pack_attention_items(coop, self._seq_rows), len(coop), coop_max_rows,
                             pack_attention_items(wide, self._seq_rows), len(wide), decode_fused)
+        self._wide_variants[key] = wide_variant
         self._plan_specs.append(key)
 
     def upload(self) -> None:
@@ -300,7 +308,7 @@ class StepContext:
                                                 coop_max_rows, decode_fused,
                                                 d_wide if n_wide else None, n_wide,
                                                 d_combine if n_combine else None,
-                                                n_combine, part_acc, part_ml)
+                                                n_combine, part_acc, part_ml, self._wide_variants.get(key, 4))
         self._views = views
         return views
 

@@ -106,6 +106,11 @@ class Kernels:
         return self._memo(("decode_fused", head_dim, dtype, page_size), lambda: page_size >= 8 and bool(
             self.attention_lib(head_dim).ls_attn_decode_fused_supported(c_int(DTYPE_CODE[dtype]))))
 
+    def compute_units(self) -> int:
+        """Compute units of the current device."""
+        return self._memo(("compute_units",), lambda: int(
+            torch.cuda.get_device_properties(torch.cuda.current_device()).multi_processor_count))
+
     def wide_supported(self, head_dim: int, dtype: torch.dtype, page_size: int) -> bool:
         """Whether the wide attention kernel (variant 4, for prompt portions) can run."""
         return self._memo(("wide", head_dim, dtype, page_size), lambda: page_size >= 8 and bool(
@@ -338,7 +343,8 @@ class Kernels:
         """Launch the attention kernel over ``n_items`` work items (see attention.hip).
         ``variant``: 0 staged through LDS where it fits, 1 direct from global memory, 2 staged or
         error, 3 cooperative (every item has at most 16 rows; ``max_rows`` states the largest),
-        4 wide (prompt portions; items count row blocks of ``attention_block_rows``)."""
+        4 wide (prompt portions; items count row blocks of ``attention_block_rows``), 5 the same
+        with half the rows a block (for steps with few rows)."""
         lib = self.attention_lib(d)
         _rows_ok(q, "attention q"); _rows_ok(out, "attention out")
         _need(q.dtype in DTYPE_CODE and out.dtype == q.dtype, "attention q/out dtype")

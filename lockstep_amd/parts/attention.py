@@ -154,7 +154,7 @@ class Attention(Mixer):
         if plan.n_wide:
             k.attention(qkv, nq, nkv, d, key_pages, value_pages, group.page_size, group.table, ctx.seqs,
                         plan.wide_items, plan.n_wide, attn, plan.part_acc, plan.part_ml, self.scale, window,
-                        variant=4)
+                        variant=plan.wide_variant)
         if plan.n_combine:
             k.attention_combine(d, ctx.seqs, plan.combine_items, plan.n_combine, nq, nkv, plan.part_acc,
                                 plan.part_ml, attn)

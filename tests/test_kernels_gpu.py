@@ -352,6 +352,7 @@ def test_prefill_attention_matches_naive(dtype, nq, nkv, d, ps, kv_len):
     assert torch.equal(case.attend(dev, 0, d ** -0.5, variant=1), out)
     if K().wide_supported(d, dtype, ps):
         assert torch.equal(case.attend(dev, 0, d ** -0.5, variant=4), out), "wide kernel"
+        assert torch.equal(case.attend(dev, 0, d ** -0.5, variant=5), out), "wide kernel, row blocks of 64"
     if kv_len == 1:
         assert torch.equal(out.cpu().float()[0], v.float()[0].repeat_interleave(nq // nkv, dim=0))
 
@@ -386,9 +387,10 @@ def test_attention_row_is_the_same_alone_in_a_portion_and_in_the_whole_prompt(dt
         part = whole.attend(qkv[lo:hi], lo, d ** -0.5, force_split=True)
         assert torch.equal(part, full[lo:hi]), f"portion {lo}:{hi} split"
         if K().wide_supported(d, dtype, ps):
-            for split in (False, True):
-                part = whole.attend(qkv[lo:hi], lo, d ** -0.5, variant=4, force_split=split)
-                assert torch.equal(part, full[lo:hi]), f"portion {lo}:{hi}, wide kernel, split={split}"
+            for variant in (4, 5):
+                for split in (False, True):
+                    part = whole.attend(qkv[lo:hi], lo, d ** -0.5, variant=variant, force_split=split)
+                    assert torch.equal(part, full[lo:hi]), f"portion {lo}:{hi}, wide kernel {variant}, split={split}"
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -405,6 +407,7 @@ def test_attention_window(dtype, window):
     assert rel_err(out, want) < ATT_TOL[dtype]
     assert torch.equal(case.attend(dev, 0, d ** -0.5, window=window, variant=1), out)
     assert torch.equal(case.attend(dev, 0, d ** -0.5, window=window, variant=4), out)
+    assert torch.equal(case.attend(dev, 0, d ** -0.5, window=window, variant=5), out)
     # pages behind the window may be gone: mark them released and decode the last rows
     for p in (kv_len - 1, 300, 130):
         first_needed = max(0, p - window + 1) // ps
