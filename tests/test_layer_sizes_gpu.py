@@ -165,3 +165,47 @@ def test_the_device_side_loop_at_real_layer_sizes(models):
                 rows.append(cur)
             picked[way] = rows
     assert picked["loop"] == picked["steps"]
+
+
+@pytest.mark.parametrize("name", list(SIZES))
+def test_random_mixes_at_real_layer_sizes(models, name):
+    """Random mixes of one to five requests (lengths on both sides of the tile, split and row-block
+    edges), cut into portions of changing size beside decoded tokens, with a pool so small that
+    pages are used again: every position has the bits of its request run whole and alone."""
+    import random
+
+    from helpers import make_mixed_trace
+    from lockstep_amd.engine.batch import StepEntry
+
+    folder, config = models[name]
+    model = load(folder, "bfloat16")
+    rng = random.Random(7)
+    lengths = [2, 3, 17, 63, 64, 65, 127, 128, 129, 255, 256, 257, 300, 511, 640, 1000, 1300]
+    for it in range(25):
+        n_req = rng.randint(1, 5)
+        requests = {f"q{it}_{i}": random_tokens(rng.choice(lengths) + rng.randint(0, 40), config.vocab_size,
+                                                seed=it * 10 + i) for i in range(n_req)}
+        alone = model.make_cache(num_pages=96, page_size=16, max_requests=2)
+        want = {}
+        for rid, toks in requests.items():
+            want[rid] = feed(model, alone, rid, toks, [len(toks)])
+            alone.close(rid)
+        steps = make_mixed_trace(requests, seed=it, max_live=4, decode_tail=rng.choice([0, 1, 8, 33]),
+                                 max_portion=rng.choice([19, 64, 130, 700]))
+        pages = [-(-len(t) // 16) for t in requests.values()]
+        cache = model.make_cache(num_pages=max(sum(pages) * 2 // 3, max(pages) * min(4, n_req)) + 4, page_size=16,
+                                 max_requests=5)
+        got = {rid: [] for rid in requests}
+        for st in steps:
+            for e in st["entries"]:
+                if e["id"] not in cache.requests:
+                    cache.open(e["id"])
+            logits = model.step(cache, [StepEntry(e["id"], e["tokens"], e["want"]) for e in st["entries"]]).cpu()
+            at = 0
+            for e in st["entries"]:
+                got[e["id"]].append(logits[at:at + len(e["want"])])
+                at += len(e["want"])
+            for rid in st["end"]:
+                cache.close(rid)
+        for rid in requests:
+            assert torch.equal(torch.cat(got[rid]), want[rid]), f"mix {it}, request {rid} ({len(requests[rid])} tokens)"
