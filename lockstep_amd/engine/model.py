@@ -12,7 +12,6 @@ from __future__ import annotations
 
 import itertools
 import os
-from pathlib import Path
 from typing import Sequence
 
 import numpy as np

@@ -14,7 +14,7 @@ import json
 import mmap
 import struct
 from pathlib import Path
-from typing import Iterable, Mapping
+from typing import Mapping
 
 import numpy as np
 import torch

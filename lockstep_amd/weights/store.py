@@ -17,7 +17,7 @@ then aliases the embedding.
 
 from __future__ import annotations
 
-from typing import Iterable, Mapping, Sequence
+from typing import Mapping, Sequence
 
 import torch
 

@@ -8,7 +8,7 @@ import pytest
 import torch
 
 from conftest import TINY_A, TINY_B
-from lockstep_amd.config import (ConfigError, ModelConfig, PartSpec, Qwen3Config, config_from_dict, config_from_dir,
+from lockstep_amd.config import (ConfigError, ModelConfig, Qwen3Config, config_from_dict, config_from_dir,
                                  known_architectures, register_architecture, unregister_architecture)
 from lockstep_amd.engine.model import collect_ties, collect_weight_specs
 from lockstep_amd.weights import (SafetensorsFile, WeightError, load_weights, random_tensors, save_file,

@@ -3,8 +3,6 @@ operation, at sizes other than the engine's, in float32 and in bfloat16."""
 
 from __future__ import annotations
 
-import math
-
 import pytest
 import torch
 

@@ -8,8 +8,6 @@ the plain implementation."""
 
 from __future__ import annotations
 
-import json
-
 import pytest
 import torch
 

@@ -10,7 +10,7 @@ from dataclasses import dataclass
 import pytest
 import torch
 
-from helpers import FP32_TOL, feed, random_tokens, rel_err
+from helpers import feed, random_tokens, rel_err
 from plain import qwen3_plain as P
 
 pytestmark = pytest.mark.gpu

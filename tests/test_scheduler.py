@@ -13,7 +13,7 @@ from lockstep_amd.engine.policy import (DefaultPolicy, Event, FixedChunkPolicy, 
                                         PreemptAtStepsPolicy, ScriptedPolicy)
 from lockstep_amd.engine.scheduler import OversizedRequest, Request, Scheduler
 from lockstep_amd.parts import PagedKVSpec
-from lockstep_amd.sampling import Sampler, greedy, top_p
+from lockstep_amd.sampling import greedy, top_p
 
 VOCAB = 40
 

@@ -11,7 +11,6 @@ from pathlib import Path
 
 import numpy as np
 import pytest
-import torch
 
 from helpers import BF16_TOL, FP32_TOL, make_mixed_trace, max_live_tokens, random_tokens, rel_err
 
