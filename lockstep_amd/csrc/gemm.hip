@@ -165,7 +165,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const void* __rest
   const float* H = reinterpret_cast<const float*>(Xv);
   // UNR chunks at a time: all their loads are issued before the first MFMA
   // needs one, so a wave keeps several kilobytes in flight.
-  constexpr int UNR = (NT * MT == 1 && !NORM) ? 8 : 4;
+  // as many chunks as the registers of a wave allow (512 / (NW / 4) a lane), so that a slice of 256 elements is one round
+  constexpr int UNR = ((NT + MT) * 8 * 4 + NT * MT * 4 + 32 <= 2048 / NW && !NORM) ? 8 : 4;
   auto load_w = [&](int k0, int k_end, vec_t (&w)[NT][UNR]) {
 #pragma unroll
     for (int u = 0; u < UNR; ++u) {
@@ -477,7 +478,7 @@ __global__ __launch_bounds__(256) void gemm_slices_kernel(const T* __restrict__ 
   for (int j = 0; j < MT; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
   const int k_begin = s * kslice;
   const int k_end = min(K, k_begin + kslice);
-  constexpr int UNR = MT == 1 ? 8 : 4;
+  constexpr int UNR = 8;  // a slice of 256 elements in one round of loads
   for (int k0 = k_begin; k0 < k_end; k0 += UNR * A::KCHUNK) {
     vec_t w[UNR], x[MT][UNR];
 #pragma unroll
