@@ -55,6 +55,7 @@ constexpr int kSplitKeys = 256;
 #define LS_ATTN_RING 8
 #endif
 constexpr int kRing = LS_ATTN_RING;  // LDS operand reads kept in flight ahead of the MFMAs
+constexpr int kPageWindow = 32;      // tiles whose page ids a workgroup of the streaming kernels holds in LDS at a time
 #ifdef LS_ATTN_PROBE
 #define PROBE(i) { long long now_ = clock64(); pr_t[i] += now_ - pr_last; pr_last = now_; }
 #else
@@ -81,6 +82,24 @@ struct AttnItem {  // one workgroup column of the attention launch (16 ints)
 // exact zero without a select; running maxima start at the finite -1e30, so
 // "m" never becomes infinite and no difference of infinities can arise.
 constexpr float kMasked = -__builtin_huge_valf();
+
+// One 16-byte piece per lane from global memory straight into LDS: the wave's 64 pieces land at
+// `lds_wave_base` + 16 * lane, each lane names its own source.  Written as the instruction itself
+// (M0 holds the wave's LDS address): after the compiler's own form of it
+// (__builtin_amdgcn_global_load_lds) every later LDS read and every barrier waits for all such
+// loads in flight, because they might be reading what the loads write, and the loads of the next
+// tile could not overlap the work on this one.  The kernels wait for a tile's loads themselves
+// (s_waitcnt vmcnt) before the barrier after which the tile is read.
+__device__ __forceinline__ void load_to_lds16(const void* src, __attribute__((address_space(3))) void* lds_wave_base) {
+  const unsigned base = __builtin_amdgcn_readfirstlane((unsigned)(unsigned long)lds_wave_base);
+  __asm__ volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(base) : "memory", "m0");
+}
+
+// A workgroup barrier that makes the waves' own LDS writes visible and nothing else.  __syncthreads() also
+// waits for every load that is still writing into LDS (global_load_lds), which would end the overlap of the
+// next tile's loads with the work on this one; where a tile has to be complete, the kernel waits for its own
+// loads explicitly (s_waitcnt vmcnt) before the barrier.
+__device__ __forceinline__ void lds_barrier() { __asm__ volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 template <typename T> __device__ __forceinline__ float softmax_exp(float x);
 template <> __device__ __forceinline__ float softmax_exp<float>(float x) { return expf(x); }
@@ -700,7 +719,7 @@ __global__ __launch_bounds__(64 * NW) void attention_wide_kernel(
   typedef __attribute__((address_space(3))) void* lptr_t;
 
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
-  int* tile_pages = reinterpret_cast<int*>(lds + 2 * BUF_BYTES);  // [2][16]
+  int* tile_pages = reinterpret_cast<int*>(lds + 2 * BUF_BYTES);  // [kPageWindow][16]
 
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -740,15 +759,23 @@ __global__ __launch_bounds__(64 * NW) void attention_wide_kernel(
   if (window > 0) ti_lo = max(ti_lo, max(0, block_first_pos - window + 1) / kTileKeys);
   const int ti_hi = min(item.split_end * TILES_PER_SPLIT, block_last_pos / kTileKeys + 1);
 
-  // page id of page `threadIdx.x` of a tile (for the first pages_per_tile threads)
-  auto table_entry = [&](int ti) -> int {
-    const int key = min(ti * kTileKeys + ((int)threadIdx.x << page_shift), sm.kv_len - 1);
-    return tbl[key >> page_shift];
+  // The page ids of kPageWindow tiles at a time go into LDS, by ordinary loads, while no tile load is in
+  // flight (the compiler's waits for ordinary loads do not know of the tile loads and would wait for them too).
+  auto fill_pages = [&](int first_tile) {
+    for (int idx = threadIdx.x; idx < kPageWindow * 16; idx += NT) {
+      const int t = first_tile + idx / 16;
+      const int pg = idx % 16;
+      if (t < ti_hi && pg < pages_per_tile) {
+        const int key = min(t * kTileKeys + (pg << page_shift), sm.kv_len - 1);
+        tile_pages[idx] = tbl[key >> page_shift];
+      }
+    }
   };
+  auto window_start = [&](int ti) -> bool { return (ti - ti_lo) % kPageWindow == 0; };  // tile ti opens a window of ids
   // Start the loads of a tile into its buffer.  What does not depend on the
   // tile is computed once: the offset of each of the thread's pieces inside
   // its page.  Keys past the request's end need no clamp of their own: the
-  // page id of their page is that of the last held page (table_entry clamps),
+  // page id of their page is that of the last held page (fill_pages clamps),
   // so the loads stay inside the cache, and what they bring is masked.
   const long page_stride = (long)nkv * page_size * D;  // elements of one page, K or V
   int k_off[PER], v_off[PER];
@@ -764,7 +791,7 @@ __global__ __launch_bounds__(64 * NW) void attention_wide_kernel(
     v_off[i] = ((kvh * D + d) << page_shift) + ((c * VEC) & (page_size - 1));
   }
   auto issue = [&](int ti) {
-    const int* pages = tile_pages + (ti & 1) * 16;
+    const int* pages = tile_pages + ((ti - ti_lo) % kPageWindow) * 16;
     unsigned char* k_buf = lds + (ti & 1) * BUF_BYTES;
     unsigned char* v_buf = k_buf + TILE_BYTES;
     int k_page[PER], v_page[PER];
@@ -778,9 +805,9 @@ __global__ __launch_bounds__(64 * NW) void attention_wide_kernel(
     for (int i = 0; i < PER; ++i) {
       if (PER * NT != TOTAL && i * NT + wave * 64 >= TOTAL) break;  // uniform for the wave
       const T* k_src = k_pages + (long)max(k_page[i], 0) * page_stride + k_off[i];
-      __builtin_amdgcn_global_load_lds((gptr_t)k_src, (lptr_t)(k_buf + (i * NT + wave * 64) * 16), 16, 0, 0);
+      load_to_lds16(k_src, (lptr_t)(k_buf + (i * NT + wave * 64) * 16));
       const T* v_src = v_pages + (long)max(v_page[i], 0) * page_stride + v_off[i];
-      __builtin_amdgcn_global_load_lds((gptr_t)v_src, (lptr_t)(v_buf + (i * NT + wave * 64) * 16), 16, 0, 0);
+      load_to_lds16(v_src, (lptr_t)(v_buf + (i * NT + wave * 64) * 16));
     }
   };
 
@@ -788,26 +815,31 @@ __global__ __launch_bounds__(64 * NW) void attention_wide_kernel(
   run.reset();
   cur.reset();
 
-  int held = 0;
   if (ti_lo < ti_hi) {
-    if ((int)threadIdx.x < pages_per_tile) tile_pages[(ti_lo & 1) * 16 + threadIdx.x] = table_entry(ti_lo);
+    fill_pages(ti_lo);
     __syncthreads();
     issue(ti_lo);
-    if (ti_lo + 1 < ti_hi && (int)threadIdx.x < pages_per_tile) held = table_entry(ti_lo + 1);
   }
 #ifdef LS_ATTN_PROBE
   long long pr_t[8] = {0, 0, 0, 0, 0, 0, 0, 0};
   long long pr_last = clock64();
   const long long pr_begin = pr_last;
 #endif
+#pragma unroll
+  for (int c = 0; c < NC; ++c) __asm__ volatile("" ::"v"(qv[c]));  // the query rows are awaited here, not inside the loop
   for (int ti = ti_lo; ti < ti_hi; ++ti) {
     const int t0 = ti * kTileKeys;
     const unsigned char* k_lds = lds + (ti & 1) * BUF_BYTES;
     unsigned char* v_lds = lds + (ti & 1) * BUF_BYTES + TILE_BYTES;
+    if (ti != ti_lo && window_start(ti)) {  // nothing is in flight: the previous tile did not request this one
+      lds_barrier();
+      fill_pages(ti);
+      lds_barrier();
+      issue(ti);
+    }
     __asm__ volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this thread's pieces of the tile have landed
-    if (ti + 1 < ti_hi && (int)threadIdx.x < pages_per_tile) tile_pages[((ti + 1) & 1) * 16 + threadIdx.x] = held;
     PROBE(0)
-    __syncthreads();  // the tile is complete, and the other buffer has been read by every wave
+    lds_barrier();  // the tile is complete, and the other buffer has been read by every wave
     PROBE(1)
     if (t0 + kTileKeys > sm.kv_len || t0 < lo_valid) {  // uniform: clean the values of keys that are not held
 #pragma unroll
@@ -818,12 +850,9 @@ __global__ __launch_bounds__(64 * NW) void attention_wide_kernel(
         vec_t* at = reinterpret_cast<vec_t*>(v_lds + p * 16);
         *at = mask_keys(*at, lo_valid - key0, sm.kv_len - key0);
       }
-      __syncthreads();
+      lds_barrier();
     }
-    if (ti + 1 < ti_hi) {
-      issue(ti + 1);
-      if (ti + 2 < ti_hi && (int)threadIdx.x < pages_per_tile) held = table_entry(ti + 2);
-    }
+    if (ti + 1 < ti_hi && !window_start(ti + 1)) issue(ti + 1);  // a tile that opens a window of page ids waits for them
 
     PROBE(2)
     const bool mine = wave_active && t0 <= wave_last_pos &&
@@ -978,8 +1007,9 @@ __global__ __launch_bounds__(64 * NW) void attention_wide_kernel(
 // instruction sequence as in the other variants, so the bits are the same.
 // The data path is the wide kernel's: the K and V tiles go from global memory
 // straight into LDS; with NBUF == 2 the next tile is in flight while the four
-// waves work on the current one, with NBUF == 1 (large heads) a tile is loaded
-// after the previous one has been consumed.
+// waves work on the current one, with NBUF == 1 (large heads, or two workgroups
+// a CU) the K half of the single buffer is refilled as soon as the scores exist
+// and the V half once the outputs are updated.
 //
 // With FUSE the kernel also does what qk_rope_kv_kernel does for a step of
 // single decoded tokens: `q` is then the raw fused projection (query heads,
@@ -1026,8 +1056,8 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
   typedef __attribute__((address_space(3))) void* lptr_t;
 
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
-  int* tile_pages = reinterpret_cast<int*>(lds + NBUF * BUF_BYTES);      // [2][16]
-  float* wmax = reinterpret_cast<float*>(tile_pages + 32);               // [4][16]
+  int* tile_pages = reinterpret_cast<int*>(lds + NBUF * BUF_BYTES);      // [kPageWindow][16]
+  float* wmax = reinterpret_cast<float*>(tile_pages + kPageWindow * 16); // [4][16]
   float* psum = wmax + 64;                                               // [NB][64]
   f32x4* prob = reinterpret_cast<f32x4*>(psum + NB * 64);                // [NB][64]
   T* knew = reinterpret_cast<T*>(prob + NB * 64);                        // FUSE: [D] new key, [D] new value
@@ -1074,10 +1104,20 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
   if (window > 0) ti_lo = max(ti_lo, max(0, first_pos - window + 1) / kTileKeys);
   const int ti_hi = min(item.split_end * TILES_PER_SPLIT, last_pos / kTileKeys + 1);
 
-  auto table_entry = [&](int ti) -> int {
-    const int key = min(ti * kTileKeys + ((int)threadIdx.x << page_shift), sm.kv_len - 1);
-    return tbl[key >> page_shift];
+  // The page ids of kPageWindow tiles at a time go into LDS, by ordinary loads, while no tile load is in
+  // flight (the compiler's waits for ordinary loads do not know of the tile loads and would wait for them too).
+  auto fill_pages = [&](int first_tile) {
+    for (int idx = threadIdx.x; idx < kPageWindow * 16; idx += NT) {
+      const int t = first_tile + idx / 16;
+      const int pg = idx % 16;
+      if (t < ti_hi && pg < pages_per_tile) {
+        const int key = min(t * kTileKeys + (pg << page_shift), sm.kv_len - 1);
+        tile_pages[idx] = tbl[key >> page_shift];
+      }
+    }
   };
+  auto pages_of = [&](int ti) -> const int* { return tile_pages + ((ti - ti_lo) % kPageWindow) * 16; };
+  auto window_start = [&](int ti) -> bool { return (ti - ti_lo) % kPageWindow == 0; };  // tile ti opens a window of ids
   const long page_stride = (long)nkv * page_size * D;  // elements of one page, K or V
   int k_off[PER], v_off[PER];
 #pragma unroll
@@ -1092,7 +1132,7 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
     v_off[i] = ((kvh * D + d) << page_shift) + ((c * VEC) & (page_size - 1));
   }
   auto issue = [&](int ti) {
-    const int* pages = tile_pages + (ti & 1) * 16;
+    const int* pages = pages_of(ti);
     unsigned char* k_buf = lds + (NBUF == 2 ? (ti & 1) : 0) * BUF_BYTES;
     unsigned char* v_buf = k_buf + TILE_BYTES;
     int k_page[PER], v_page[PER];
@@ -1106,9 +1146,37 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
     for (int i = 0; i < PER; ++i) {
       if (PER * NT != TOTAL && i * NT + wave * 64 >= TOTAL) break;  // uniform for the wave
       const T* k_src = k_pages + (long)max(k_page[i], 0) * page_stride + k_off[i];
-      __builtin_amdgcn_global_load_lds((gptr_t)k_src, (lptr_t)(k_buf + (i * NT + wave * 64) * 16), 16, 0, 0);
+      load_to_lds16(k_src, (lptr_t)(k_buf + (i * NT + wave * 64) * 16));
       const T* v_src = v_pages + (long)max(v_page[i], 0) * page_stride + v_off[i];
-      __builtin_amdgcn_global_load_lds((gptr_t)v_src, (lptr_t)(v_buf + (i * NT + wave * 64) * 16), 16, 0, 0);
+      load_to_lds16(v_src, (lptr_t)(v_buf + (i * NT + wave * 64) * 16));
+    }
+  };
+  // With one buffer the K tile and the V tile are loaded apart: the K tile of the next tile as soon as the
+  // scores of this one exist, its V tile once the outputs are updated, so a load is in flight most of the time.
+  // Each thread issues exactly PER loads for a K tile and PER for a V tile, in this order for a given tile,
+  // which is what the waits below count on (loads complete in the order of their issue).
+  static_assert(NBUF == 2 || PER * NT == TOTAL, "the split loads assume whole rounds");
+  auto issue_k = [&](int ti) {
+    const int* pages = pages_of(ti);
+    int k_page[PER];
+#pragma unroll
+    for (int i = 0; i < PER; ++i) k_page[i] = pages[min(((i * NT + (int)threadIdx.x) / KPIECES) >> page_shift, 15)];
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const T* k_src = k_pages + (long)max(k_page[i], 0) * page_stride + k_off[i];
+      load_to_lds16(k_src, (lptr_t)(lds + (i * NT + wave * 64) * 16));
+    }
+  };
+  auto issue_v = [&](int ti) {
+    const int* pages = pages_of(ti);
+    int v_page[PER];
+#pragma unroll
+    for (int i = 0; i < PER; ++i)
+      v_page[i] = pages[min((((i * NT + (int)threadIdx.x) / D) * VEC) >> page_shift, 15)];
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const T* v_src = v_pages + (long)max(v_page[i], 0) * page_stride + v_off[i];
+      load_to_lds16(v_src, (lptr_t)(lds + TILE_BYTES + (i * NT + wave * 64) * 16));
     }
   };
 
@@ -1121,9 +1189,6 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
     run_acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
 
-  int held = 0;
-  int first_page = 0;
-  if (ti_lo < ti_hi && (int)threadIdx.x < pages_per_tile) first_page = table_entry(ti_lo);
   // FUSE: one new token per request at position q_start; its tile is patched by the workgroup that walks it.
   // The heads to process are numbered vi: the G query heads, then the new key, then the new value;
   // wave w takes vi = w, w + 4, ...  The operands of its first head are loaded before the tile loads start.
@@ -1153,12 +1218,17 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
     if (owner) page_new = tbl[p_new >> page_shift];
     if (grp < n_vec) head_fetch(grp);
   }
-  if (ti_lo < ti_hi && (int)threadIdx.x < pages_per_tile) tile_pages[(ti_lo & 1) * 16 + threadIdx.x] = first_page;
+  if (ti_lo < ti_hi) fill_pages(ti_lo);
   __syncthreads();
-  if (ti_lo < ti_hi) {
-    issue(ti_lo);
-    if (ti_lo + 1 < ti_hi && (int)threadIdx.x < pages_per_tile) held = table_entry(ti_lo + 1);
-  }
+  auto issue_tile = [&](int ti) {
+    if (NBUF == 2) {
+      issue(ti);
+    } else {
+      issue_k(ti);
+      issue_v(ti);
+    }
+  };
+  if (ti_lo < ti_hi) issue_tile(ti_lo);
   if (FUSE) {
     T* qrot = reinterpret_cast<T*>(prob);  // [16][D]: the exchange buffers are free until the loop
     const int slot_new = p_new & (page_size - 1);
@@ -1189,24 +1259,54 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
         }
       }
     }
-    __syncthreads();
+    lds_barrier();
 #pragma unroll
     for (int c = 0; c < NC; ++c) {
       const int col = c * A::KCHUNK + g * VEC;
       qv[c] = (row_ok && col < D) ? *reinterpret_cast<const vec_t*>(qrot + row16 * D + min(col, D - VEC)) : A::zero();
     }
   }
+  if (!FUSE) {  // the query rows, loaded from global memory, are awaited here and not inside the loop
+#pragma unroll
+    for (int c = 0; c < NC; ++c) __asm__ volatile("" ::"v"(qv[c]));
+  }
   for (int ti = ti_lo; ti < ti_hi; ++ti) {
     const int t0 = ti * kTileKeys;
     const unsigned char* k_lds = lds + (NBUF == 2 ? (ti & 1) : 0) * BUF_BYTES;
     unsigned char* v_lds = lds + (NBUF == 2 ? (ti & 1) : 0) * BUF_BYTES + TILE_BYTES;
-    __asm__ volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this thread's pieces of the tile have landed
+    // the next tile is requested ahead unless it opens a new window of page ids
+    const bool ahead = ti + 1 < ti_hi && !window_start(ti + 1);
+    if (ti != ti_lo && window_start(ti)) {  // nothing is in flight: the previous tile did not request this one
+      lds_barrier();
+      fill_pages(ti);
+      lds_barrier();
+      issue_tile(ti);
+    }
+    if (NBUF == 2) {
+      __asm__ volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this thread's pieces of the tile have landed
+    } else {
+      // this thread's pieces of the K tile have landed; its PER loads of the V tile, issued later, may be in flight
+      __asm__ volatile("s_waitcnt vmcnt(%0)" ::"n"(PER) : "memory");
+    }
     PROBE(4)
-    if (ti + 1 < ti_hi && (int)threadIdx.x < pages_per_tile) tile_pages[((ti + 1) & 1) * 16 + threadIdx.x] = held;
-    __syncthreads();  // the tile is complete (and the other buffer has been read by every wave)
+    lds_barrier();  // the tile (one buffer: its K half) is complete (and the other buffer has been read by every wave)
     PROBE(5)
     const bool patch = owner && ti == tile_new;  // the new key and value go into this tile
-    if (t0 + kTileKeys > sm.kv_len || t0 < lo_valid || patch) {  // uniform: clean the values of keys that are not held
+    const bool clean = t0 + kTileKeys > sm.kv_len || t0 < lo_valid || patch;  // uniform
+    if (NBUF == 1 && FUSE && patch) {  // the new key goes into the K tile now, the V tile is dealt with when it is there
+#pragma unroll
+      for (int i = 0; i < PER; ++i) {
+        const int p = i * NT + (int)threadIdx.x;
+        const int row = p / KPIECES;
+        if (t0 + row == p_new) {
+          const int piece = (p % KPIECES - row % KPIECES + KPIECES) % KPIECES;
+          *reinterpret_cast<vec_t*>(const_cast<unsigned char*>(k_lds) + p * 16) =
+              *reinterpret_cast<const vec_t*>(knew + piece * VEC);
+        }
+      }
+      lds_barrier();
+    }
+    auto clean_values = [&](bool with_key) {  // clean the values of keys that are not held, place the new ones
 #pragma unroll
       for (int i = 0; i < PER; ++i) {
         const int p = i * NT + (int)threadIdx.x;
@@ -1219,7 +1319,7 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
 #pragma unroll
           for (int e = 0; e < VEC; ++e) v[e] = key0 + e == p_new ? fresh : v[e];
           const int row = p / KPIECES;
-          if (t0 + row == p_new) {
+          if (with_key && t0 + row == p_new) {
             const int piece = (p % KPIECES - row % KPIECES + KPIECES) % KPIECES;
             *reinterpret_cast<vec_t*>(const_cast<unsigned char*>(k_lds) + p * 16) =
                 *reinterpret_cast<const vec_t*>(knew + piece * VEC);
@@ -1227,12 +1327,10 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
         }
         *at = v;
       }
-      __syncthreads();
-    }
-    if (NBUF == 2 && ti + 1 < ti_hi) {
-      issue(ti + 1);
-      if (ti + 2 < ti_hi && (int)threadIdx.x < pages_per_tile) held = table_entry(ti + 2);
-    }
+      lds_barrier();
+    };
+    if (NBUF == 2 && clean) clean_values(true);
+    if (NBUF == 2 && ahead) issue(ti + 1);
 
     // score blocks 2w and 2w+1
     PROBE(6)
@@ -1270,8 +1368,9 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
     my_max = quad16_max(my_max);
     if (g == 0) wmax[wave * 16 + row16] = my_max;
     PROBE(7)
-    __syncthreads();
+    lds_barrier();
     PROBE(8)
+    if (NBUF == 1 && ahead) issue_k(ti + 1);  // every wave has its scores: the K half of the buffer is free
     const float tile_max = fmaxf(fmaxf(wmax[row16], wmax[16 + row16]), fmaxf(wmax[32 + row16], wmax[48 + row16]));
     const float m_new = fmaxf(cur_m, tile_max);
     const float alpha = softmax_exp<T>(cur_m - m_new);
@@ -1283,10 +1382,13 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
       psum[kb * 64 + lane] = (s[j][0] + s[j][1]) + (s[j][2] + s[j][3]);
       prob[kb * 64 + lane] = s[j];
     }
-    // this wave's value operands do not depend on the probabilities: read them before the barrier
+    // this wave's value operands do not depend on the probabilities: with two buffers they are read before the
+    // barrier; with one buffer the V tile is only now awaited (the K loads of the next tile, issued after it,
+    // may stay in flight), complete for every thread after the barrier, and cleaned then
     constexpr int KB16 = VEC / 4;
     constexpr int NPAIR = NB / KB16;
     vec_t vop[NPAIR][MYDB];
+    auto read_values = [&]() {
 #pragma unroll
     for (int kp = 0; kp < NPAIR; ++kp)
 #pragma unroll
@@ -1310,9 +1412,21 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
         }
         vop[kp][j] = vv;
       }
+    };
+    if (NBUF == 2) {
+      read_values();
+    } else if (ahead) {
+      __asm__ volatile("s_waitcnt vmcnt(%0)" ::"n"(PER) : "memory");
+    } else {
+      __asm__ volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
     PROBE(9)
-    __syncthreads();
+    lds_barrier();
     PROBE(10)
+    if (NBUF == 1) {
+      if (clean) clean_values(false);
+      read_values();
+    }
     float p_sum = 0.f;
 #pragma unroll
     for (int kb = 0; kb < NB; ++kb) p_sum = p_sum + psum[kb * 64 + lane];
@@ -1357,9 +1471,8 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
       cur_l = 0.f;
     }
     if (NBUF == 1 && ti + 1 < ti_hi) {
-      __syncthreads();  // every wave is done with the buffer
-      issue(ti + 1);
-      if (ti + 2 < ti_hi && (int)threadIdx.x < pages_per_tile) held = table_entry(ti + 2);
+      lds_barrier();  // every wave is done with the V half of the buffer
+      if (ahead) issue_v(ti + 1);
     }
   }
 
@@ -1489,7 +1602,7 @@ constexpr size_t kLdsLimit = 160 * 1024;
 
 // The cooperative kernel: one or two buffers of a K and a V tile,
 // two rows of page ids and the exchange buffers of the cooperative kernel.
-constexpr size_t kCoopLdsExtra = 2 * 16 * sizeof(int) + kCoopExtra + 2 * D * 4;  // + new key and value (FUSE)
+constexpr size_t kCoopLdsExtra = kPageWindow * 16 * sizeof(int) + kCoopExtra + 2 * D * 4;  // + new key and value (FUSE)
 constexpr int coop_bufs(size_t elem) {
   return 2 * (2 * kTileKeys * D * elem) + kCoopLdsExtra <= kLdsLimit ? 2 : 1;
 }
@@ -1616,7 +1729,7 @@ extern "C" int ls_attention_decode(int dtype, const void* qkv, long ld, void* k_
 // 128) or, for steps with so few rows that 128-row blocks would leave CUs without work, four (blocks of 64).
 constexpr int kWideWaves = 8;
 constexpr int kNarrowWaves = 4;
-static size_t wide_lds_bytes(int dtype) { return 4 * (size_t)kTileKeys * D * (dtype == kF32 ? 4 : 2) + 2 * 16 * sizeof(int); }
+static size_t wide_lds_bytes(int dtype) { return 4 * (size_t)kTileKeys * D * (dtype == kF32 ? 4 : 2) + kPageWindow * 16 * sizeof(int); }
 template <typename T, int NW>
 static bool wide_kernel_ready(size_t bytes) {
   static int state = 0;  // 0 unknown, 1 granted, -1 refused

@@ -264,7 +264,7 @@ class PagedCase:
         K().qk_rope_kv(qkv, t, self.nq, self.nkv, self.d, q_norm, k_norm, eps, cos, sin, rot, tok_seq, tok_pos,
                        self.seqs(q_start, t), q_start + t - 1, self.table, self.k_pages, self.v_pages, self.ps, True)
 
-    def attend(self, qkv, q_start, scale, window=0, force_split=None, variant=0):
+    def attend(self, qkv, q_start, scale, window=0, force_split=None, variant=0, repeat=1):
         from lockstep_amd.ops import kernels
 
         t = qkv.shape[0]
@@ -293,6 +293,7 @@ class PagedCase:
                 items += [0, b, begin, last // split + 1, -1, 0, 0, 0]
         from lockstep_amd.ops import pack_attention_items, pack_combine_items
 
+        items = items * repeat      # the same work many times over (same values to the same places): a full GPU
         seq_row = self.seqs(q_start, t).cpu().numpy()
         n_items = len(items) // 8
         items_t = torch.from_numpy(pack_attention_items(items, seq_row)).to(torch.int32).cuda()
@@ -353,6 +354,38 @@ def test_prefill_attention_matches_naive(dtype, nq, nkv, d, ps, kv_len):
         assert torch.equal(case.attend(dev, 0, d ** -0.5, variant=5), out), "wide kernel, row blocks of 64"
     if kv_len == 1:
         assert torch.equal(out.cpu().float()[0], v.float()[0].repeat_interleave(nq // nkv, dim=0))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nq,nkv,d,ps", [(4, 2, 128, 16), (2, 1, 64, 8), (8, 4, 32, 64)])
+def test_attention_over_more_keys_than_one_window_of_page_ids(dtype, nq, nkv, d, ps):
+    """A workgroup of the streaming kernels holds the page ids of 32 tiles (4,096 keys) at a time.
+    Contexts beyond that: a prompt in one step, late portions and decoded tokens, each walking all
+    splits in one workgroup or cut into splits and combined; same bits in every kernel, and the
+    32-bit result against the naive formula.  One far key is made to stand out."""
+    n = 4096 * 2 + 300
+    qkv = rand_qkv(n, nq, nkv, d, dtype, seed=n + d, sharp=(37,))
+    case = PagedCase(dtype, nq, nkv, d, ps, n, shuffle_seed=5)
+    dev = qkv.cuda()
+    case.write(dev, 0)
+    full = case.attend(dev, 0, d ** -0.5)                                  # staged or direct kernel, row blocks of 64
+    q, k, v = split_qkv(qkv.double(), nq, nkv, d)
+    tail = slice(n - 40, n)
+    want = naive_attention(q[tail], k, v, n - 40, d ** -0.5)
+    assert rel_err(full[tail], want) < ATT_TOL[dtype]
+    if K().wide_supported(d, dtype, ps):
+        for variant in (4, 5):
+            assert torch.equal(case.attend(dev, 0, d ** -0.5, variant=variant), full), f"wide kernel {variant}"
+            late = case.attend(dev[n - 200:], n - 200, d ** -0.5, variant=variant)
+            assert torch.equal(late, full[n - 200:]), f"late portion, wide kernel {variant}"
+    if K().coop_supported(d, dtype, ps):
+        for p in (4095, 4096, 4100, 8191, 8192, n - 1):
+            for split in (False, True):
+                one = case.attend(dev[p:p + 1], p, d ** -0.5, variant=3, force_split=split)
+                assert torch.equal(one, full[p:p + 1]), f"decoded token at {p}, split={split}"
+        # with two workgroups a CU the kernel works with one buffer, refilled half by half
+        crowd = case.attend(dev[n - 1:], n - 1, d ** -0.5, variant=3, force_split=False, repeat=-(-600 // nkv))
+        assert torch.equal(crowd, full[n - 1:]), "decoded token, crowded launch"
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
