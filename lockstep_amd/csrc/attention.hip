@@ -101,6 +101,24 @@ __device__ __forceinline__ void load_to_lds16(const void* src, __attribute__((ad
 // loads explicitly (s_waitcnt vmcnt) before the barrier.
 __device__ __forceinline__ void lds_barrier() { __asm__ volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
+// Which key of a tile row r (0..15) of the score block kb stands for.  The score MFMA leaves a lane with rows
+// 4g..4g+3 of each 16-key block, and the value MFMA of two such blocks (bfloat16: 32 keys an atom) wants the
+// lane's eight probabilities to belong to the eight keys of its value operand.  With the rows of a pair of
+// blocks dealt as 0-3, 8-11, 16-19, 24-27 | 4-7, 12-15, 20-23, 28-31 those are the consecutive keys
+// 8g..8g+7 of the pair: one 16-byte read of the value tile instead of two of 8 bytes.  float32 atoms take 4 keys
+// a lane, which are consecutive anyway.  Every kernel deals the keys through this function, so the sums of the
+// probabilities and the products run over the keys in one and the same order everywhere.
+template <typename T>
+__device__ __forceinline__ constexpr int key_of_row(int kb, int r) {
+  return sizeof(T) == 2 ? 32 * (kb >> 1) + 8 * (r >> 2) + 4 * (kb & 1) + (r & 3) : 16 * kb + r;
+}
+// The rotation of a key row's 16-byte pieces in the LDS tile: the sixteen rows that a score block reads
+// together start in sixteen different slots.
+template <typename T>
+__device__ __forceinline__ constexpr int row_rotation(int row) {
+  return sizeof(T) == 2 ? (row & 3) + 4 * ((row >> 3) & 3) : row;
+}
+
 template <typename T> __device__ __forceinline__ float softmax_exp(float x);
 template <> __device__ __forceinline__ float softmax_exp<float>(float x) { return expf(x); }
 template <> __device__ __forceinline__ float softmax_exp<bf16_t>(float x) { return __expf(x); }
@@ -229,7 +247,7 @@ __global__ __launch_bounds__(256) void attention_direct_kernel(
 #pragma unroll
       for (int kb = 0; kb < NB; ++kb) {
         s[kb] = f32x4{0.f, 0.f, 0.f, 0.f};
-        const int key = t0 + kb * 16 + row16;
+        const int key = t0 + key_of_row<T>(kb, row16);
         bool key_ok = key < sm.kv_len && key >= lo_valid && key <= wave_last_pos;
         long page = key_ok ? tbl[key / page_size] : -1;
         key_ok = key_ok && page >= 0;
@@ -260,7 +278,7 @@ __global__ __launch_bounds__(256) void attention_direct_kernel(
         for (int kb = 0; kb < NB; ++kb)
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
-            const int key = t0 + kb * 16 + 4 * g + e;
+            const int key = t0 + key_of_row<T>(kb, 4 * g + e);
             const float v = ((key <= key_hi) & (key >= key_lo)) ? s[kb][e] * scale : kMasked;
             s[kb][e] = v;
             tile_max = fmaxf(tile_max, v);
@@ -296,7 +314,7 @@ __global__ __launch_bounds__(256) void attention_direct_kernel(
         for (int h = 0; h < KB16; ++h) {
 #pragma unroll
           for (int e = 0; e < 4; ++e) pv[h * 4 + e] = from_f32<T>(s[kb + h][e]);
-          const int key = t0 + (kb + h) * 16 + 4 * g;
+          const int key = t0 + key_of_row<T>(kb + h, 4 * g);
           vkey[h] = key;
           const bool any = key < sm.kv_len && key + 3 >= lo_valid;
           const long page = any ? tbl[key / page_size] : -1;
@@ -486,7 +504,8 @@ __global__ __launch_bounds__(256, LS_STAGED_MIN_BLOCKS) void attention_staged_ke
       const int piece = p % KPIECES;
       const int key = t0 + kt;
       const bool k_ok = key < sm.kv_len && key >= lo_valid && kpage_held[i] >= 0;
-      *reinterpret_cast<vec_t*>(k_lds + kt * KROW + ((piece + kt) % KPIECES) * 16) = k_ok ? kreg[j] : A::zero();
+      *reinterpret_cast<vec_t*>(k_lds + kt * KROW + ((piece + row_rotation<T>(kt)) % KPIECES) * 16) =
+          k_ok ? kreg[j] : A::zero();
       const int q1 = p >> vshift;
       const int kp = p & ((1 << vshift) - 1);
       const int pg = q1 / D;
@@ -550,10 +569,10 @@ __global__ __launch_bounds__(256, LS_STAGED_MIN_BLOCKS) void attention_staged_ke
         constexpr int NS = NB * NC;
         constexpr int RING = NS < kRing ? NS : kRing;
         auto k_read = [&](int idx) -> vec_t {
-          const int row = (idx / NC) * 16 + row16;
+          const int row = key_of_row<T>(idx / NC, row16);
           const int piece = (idx % NC) * 4 + g;
           const int pc = (4 * NC == KPIECES) ? piece : min(piece, KPIECES - 1);
-          vec_t kv = *reinterpret_cast<const vec_t*>(k_lds + row * KROW + ((pc + row) % KPIECES) * 16);
+          vec_t kv = *reinterpret_cast<const vec_t*>(k_lds + row * KROW + ((pc + row_rotation<T>(row)) % KPIECES) * 16);
           if (4 * NC != KPIECES) kv = piece < KPIECES ? kv : A::zero();
           return kv;
         };
@@ -586,7 +605,7 @@ __global__ __launch_bounds__(256, LS_STAGED_MIN_BLOCKS) void attention_staged_ke
         for (int kb = 0; kb < NB; ++kb)
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
-            const int key = t0 + kb * 16 + 4 * g + e;
+            const int key = t0 + key_of_row<T>(kb, 4 * g + e);
             const float v = ((key <= key_hi) & (key >= key_lo)) ? s[kb][e] * scale : kMasked;
             s[kb][e] = v;
             tile_max = fmaxf(tile_max, v);
@@ -621,7 +640,7 @@ __global__ __launch_bounds__(256, LS_STAGED_MIN_BLOCKS) void attention_staged_ke
           vec_t vv;
 #pragma unroll
           for (int h = 0; h < KB16; ++h) {
-            const int byte = ((kb + h) * 16 + 4 * g) * SZ;  // offset of the lane's four keys in the column row
+            const int byte = key_of_row<T>(kb + h, 4 * g) * SZ;  // offset of the lane's four keys in the column row
             const unsigned char* src = v_lds + d * VROW + (((byte >> 4) + d) % VPIECES) * 16 + (byte & 15);
             if (SZ == 2) {
               bf16x4 four = *reinterpret_cast<const bf16x4*>(src);
@@ -784,7 +803,7 @@ __global__ __launch_bounds__(64 * NW) void attention_wide_kernel(
     const int p = i * NT + (int)threadIdx.x;
     const int row = p / KPIECES;
     const int slot = p % KPIECES;
-    const int piece = (slot - row % KPIECES + KPIECES) % KPIECES;
+    const int piece = (slot - row_rotation<T>(row) % KPIECES + KPIECES) % KPIECES;
     k_off[i] = (kvh * page_size + (row & (page_size - 1))) * D + piece * VEC;
     const int c = p / D;
     const int d = p % D;
@@ -864,10 +883,10 @@ __global__ __launch_bounds__(64 * NW) void attention_wide_kernel(
         constexpr int NS = NB * NC;
         constexpr int RING = NS < kRing ? NS : kRing;
         auto k_read = [&](int idx) -> vec_t {
-          const int row = (idx / NC) * 16 + row16;
+          const int row = key_of_row<T>(idx / NC, row16);
           const int piece = (idx % NC) * 4 + g;
           const int pc = (4 * NC == KPIECES) ? piece : min(piece, KPIECES - 1);
-          vec_t kv = *reinterpret_cast<const vec_t*>(k_lds + row * KROW + ((pc + row) % KPIECES) * 16);
+          vec_t kv = *reinterpret_cast<const vec_t*>(k_lds + row * KROW + ((pc + row_rotation<T>(row)) % KPIECES) * 16);
           if (4 * NC != KPIECES) kv = piece < KPIECES ? kv : A::zero();
           return kv;
         };
@@ -899,7 +918,7 @@ __global__ __launch_bounds__(64 * NW) void attention_wide_kernel(
         for (int kb = 0; kb < NB; ++kb)
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
-            const int key = t0 + kb * 16 + 4 * g + e;
+            const int key = t0 + key_of_row<T>(kb, 4 * g + e);
             const float v = ((key <= key_hi) & (key >= key_lo)) ? s[kb][e] * scale : kMasked;
             s[kb][e] = v;
             tile_max = fmaxf(tile_max, v);
@@ -934,7 +953,7 @@ __global__ __launch_bounds__(64 * NW) void attention_wide_kernel(
           vec_t vv;
 #pragma unroll
           for (int h = 0; h < KB16; ++h) {
-            const int key = (kb + h) * 16 + 4 * g;  // the lane's four keys inside the tile
+            const int key = key_of_row<T>(kb + h, 4 * g);  // the lane's four keys inside the tile
             const unsigned char* src = v_lds + ((key / VEC) * D + d) * 16 + (key % VEC) * SZ;
             if (SZ == 2) {
               bf16x4 four = *reinterpret_cast<const bf16x4*>(src);
@@ -1125,7 +1144,7 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
     const int p = i * NT + (int)threadIdx.x;
     const int row = p / KPIECES;
     const int slot = p % KPIECES;
-    const int piece = (slot - row % KPIECES + KPIECES) % KPIECES;
+    const int piece = (slot - row_rotation<T>(row) % KPIECES + KPIECES) % KPIECES;
     k_off[i] = (kvh * page_size + (row & (page_size - 1))) * D + piece * VEC;
     const int c = p / D;
     const int d = p % D;
@@ -1299,7 +1318,7 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
         const int p = i * NT + (int)threadIdx.x;
         const int row = p / KPIECES;
         if (t0 + row == p_new) {
-          const int piece = (p % KPIECES - row % KPIECES + KPIECES) % KPIECES;
+          const int piece = (p % KPIECES - row_rotation<T>(row) % KPIECES + KPIECES) % KPIECES;
           *reinterpret_cast<vec_t*>(const_cast<unsigned char*>(k_lds) + p * 16) =
               *reinterpret_cast<const vec_t*>(knew + piece * VEC);
         }
@@ -1320,7 +1339,7 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
           for (int e = 0; e < VEC; ++e) v[e] = key0 + e == p_new ? fresh : v[e];
           const int row = p / KPIECES;
           if (with_key && t0 + row == p_new) {
-            const int piece = (p % KPIECES - row % KPIECES + KPIECES) % KPIECES;
+            const int piece = (p % KPIECES - row_rotation<T>(row) % KPIECES + KPIECES) % KPIECES;
             *reinterpret_cast<vec_t*>(const_cast<unsigned char*>(k_lds) + p * 16) =
                 *reinterpret_cast<const vec_t*>(knew + piece * VEC);
           }
@@ -1340,12 +1359,12 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
       vec_t kop[2][NC];
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
-        const int row = (2 * wave + j) * 16 + row16;
+        const int row = key_of_row<T>(2 * wave + j, row16);
 #pragma unroll
         for (int c = 0; c < NC; ++c) {
           const int piece = c * 4 + g;
           const int pc = (4 * NC == KPIECES) ? piece : min(piece, KPIECES - 1);
-          vec_t kv = *reinterpret_cast<const vec_t*>(k_lds + row * KROW + ((pc + row) % KPIECES) * 16);
+          vec_t kv = *reinterpret_cast<const vec_t*>(k_lds + row * KROW + ((pc + row_rotation<T>(row)) % KPIECES) * 16);
           if (4 * NC != KPIECES) kv = piece < KPIECES ? kv : A::zero();
           kop[j][c] = kv;
         }
@@ -1358,7 +1377,7 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
         for (int c = 0; c < NC; ++c) A::mma(s[j], kop[j][c], qv[c]);
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          const int key = t0 + kb * 16 + 4 * g + e;
+          const int key = t0 + key_of_row<T>(kb, 4 * g + e);
           const float v = ((key <= key_hi) & (key >= key_lo)) ? s[j][e] * scale : kMasked;
           s[j][e] = v;
           my_max = fmaxf(my_max, v);
@@ -1398,7 +1417,7 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
         vec_t vv;
 #pragma unroll
         for (int h = 0; h < KB16; ++h) {
-          const int key = (kp * KB16 + h) * 16 + 4 * g;
+          const int key = key_of_row<T>(kp * KB16 + h, 4 * g);
           const unsigned char* src = v_lds + ((key / VEC) * D + d) * 16 + (key % VEC) * SZ;
           if (SZ == 2) {
             bf16x4 four = *reinterpret_cast<const bf16x4*>(src);
