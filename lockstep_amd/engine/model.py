@@ -20,7 +20,7 @@ import torch
 from ..cache import CacheManager
 from ..config import ModelConfig, ModelSpec, config_from_dir
 from ..parts import WeightSpec, build_part, part_class
-from ..parts.base import device_epoch, takes
+from ..parts.base import device_epoch, graph_safe_tree, takes
 from ..weights.store import load_weights, weights_from_dict
 from .batch import StepContext, StepEntry, Workspace
 from .runtime import Runtime
@@ -65,7 +65,8 @@ class Model:
                 raise ValueError(f"the schedule names layer {run.layer}, the model has {len(self.layers)}")
         self.workspace = Workspace(rt.device)
         self.use_graphs = os.environ.get("LOCKSTEP_NO_GRAPHS", "") in ("", "0")
-        self._graph_safe = all(layer.mixer.graph_safe for layer in self.layers)
+        self._graph_safe = all(graph_safe_tree(part)
+                               for part in (self.embedding, *self.layers, self.final_norm, self.head))
         # which arrangements, and the final norm, take over an addition the previous layer left open
         self._layer_takes_pending = [takes(layer.forward, "pending") for layer in self.layers]
         self._final_takes_pending = takes(self.final_norm.forward, "pending")

@@ -40,6 +40,9 @@ class Attention(Mixer):
 
     graph_safe = True
 
+    def parts(self):
+        return (self.position,)
+
     def __init__(self, spec: PartSpec, prefix: str = ""):
         super().__init__(spec, prefix)
         p = spec.params

@@ -79,9 +79,20 @@ class Part:
 
     kind: str = ""
 
+    #: True if the part's ``forward`` only launches kernels that read the step's metadata and its
+    #: data from device memory, so a decode step may be captured in a HIP graph and replayed with
+    #: new metadata.  A part that reads sizes, slots or values on the host while it runs (a state
+    #: update in Python, a routing decision fetched from the device) must leave this False; one
+    #: such part anywhere in the model switches the graphs off for the model.
+    graph_safe = False
+
     def __init__(self, spec: PartSpec, prefix: str = ""):
         self.spec = spec
         self.prefix = prefix
+
+    def parts(self) -> Sequence["Part"]:
+        """The parts this part is built from (none for a leaf)."""
+        return ()
 
     @classmethod
     def weight_specs(cls, spec: PartSpec, prefix: str) -> list[WeightSpec]:
@@ -101,17 +112,24 @@ class Norm(Part):
 
 
 class PositionEncoding(Part):
+    """What the attention mixer asks of a position encoding: ``rotary_dim`` (the leading
+    dimensions of a head that are rotated, 0 for none; dimension ``i`` is paired with
+    ``i + rotary_dim/2``) and ``cos`` / ``sin``, float32 device tables ``[positions,
+    rotary_dim/2]`` of the angle of each pair at each absolute position (None while
+    ``rotary_dim`` is 0).  The frequencies, and any scaling of the positions, are the
+    part's own business.  Optional: ``share_key()`` (layers with equal keys use one set of
+    tables and are prepared once a step) and ``bind(rt)`` (called at load)."""
+
+    rotary_dim = 0
+    cos = None
+    sin = None
+
     def ensure(self, max_position: int, rt) -> None:
-        """Make tables cover positions ``< max_position``."""
+        """Make the tables cover positions ``< max_position``; a part that replaces a table
+        a captured graph may hold calls ``bump_device_epoch()``."""
 
 
 class Mixer(Part):
-    #: True if ``forward`` only launches kernels that read the step's metadata
-    #: from device memory, so a decode step may be captured in a HIP graph and
-    #: replayed with new metadata.  A mixer that reads sizes or slots on the
-    #: host while it runs must leave this False.
-    graph_safe = False
-
     def cache_spec(self):
         """``PagedKVSpec``, ``StateSpec`` or ``None``."""
         return None
@@ -205,6 +223,11 @@ class PendingAdd:
 #: steps of at most this many tokens leave the residual additions of the output products to the
 #: following norm (their work is then cut over K as well, which fills the GPU); 0 switches it off
 DEFER_ADD_ROWS = int(__import__("os").environ.get("LOCKSTEP_DEFER_ADD_ROWS", "64"))
+
+
+def graph_safe_tree(part: Part) -> bool:
+    """Whether ``part`` and every part below it may run inside a captured graph."""
+    return bool(part.graph_safe) and all(graph_safe_tree(p) for p in part.parts())
 
 
 def takes(function, name: str) -> bool:

@@ -15,6 +15,8 @@ class PreNormResidual(Arrangement):
     ``feed_forward_norm_name``.
     """
 
+    graph_safe = True
+
     def __init__(self, layer_spec, prefix: str = ""):
         super().__init__(layer_spec, build_part)
         p = layer_spec.arrangement.params

@@ -12,6 +12,8 @@ class TokenEmbedding(Part):
     """``h[t] = E[token[t]]``, no scaling (reference engine/model/qwen3.py:319).
     Parameters: ``name``, ``vocab_size``, ``hidden_size``."""
 
+    graph_safe = True
+
     def __init__(self, spec: PartSpec, prefix: str = ""):
         super().__init__(spec, prefix)
         self.table = None
@@ -33,6 +35,8 @@ class LinearHead(Part):
     engine/model/qwen3.py:373).  Parameters: ``name``, ``tied_to`` (a tensor
     name the head aliases when the checkpoint does not hold its own, or None),
     ``vocab_size``, ``hidden_size``."""
+
+    graph_safe = True
 
     def __init__(self, spec: PartSpec, prefix: str = ""):
         super().__init__(spec, prefix)

@@ -18,6 +18,8 @@ from .base import DEFER_ADD_ROWS, FeedForward, PendingAdd, WeightSpec, register_
 class GatedMLP(FeedForward):
     """Parameters: ``hidden_size``, ``intermediate_size``, ``activation``."""
 
+    graph_safe = True
+
     def __init__(self, spec: PartSpec, prefix: str = ""):
         super().__init__(spec, prefix)
         self.hidden = int(spec["hidden_size"])

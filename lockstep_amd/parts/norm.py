@@ -11,6 +11,8 @@ from .base import Norm, WeightSpec, register_part
 class RMSNorm(Norm):
     """Parameters: ``size``, ``eps``; ``name`` overrides the tensor name."""
 
+    graph_safe = True
+
     def __init__(self, spec: PartSpec, prefix: str = ""):
         super().__init__(spec, prefix)
         self.size = int(spec["size"])

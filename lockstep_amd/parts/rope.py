@@ -19,6 +19,8 @@ _TABLES: dict[tuple, list] = {}
 class RotaryHalf(PositionEncoding):
     """Parameters: ``rotary_dim`` (even, at most the head size), ``theta``."""
 
+    graph_safe = True
+
     def __init__(self, spec: PartSpec, prefix: str = ""):
         super().__init__(spec, prefix)
         self.rotary_dim = int(spec["rotary_dim"])
@@ -65,6 +67,8 @@ class RotaryHalf(PositionEncoding):
 @register_part("no_position")
 class NoPosition(PositionEncoding):
     """Leaves queries and keys as they are."""
+
+    graph_safe = True
 
     rotary_dim = 0
     cos = None

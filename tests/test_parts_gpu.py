@@ -342,3 +342,181 @@ def test_toy_architecture_registers_builds_and_steps(tmp_path, schedule):
     finally:
         unregister_part("toy_decay")
         unregister_architecture(ToyConfig)
+
+
+# ---------------------------------------------------------------------------
+# a second toy architecture, defined here as well: a feed-forward that routes
+# every token to one of several experts (it fetches the routing decision, so
+# it may not run inside a captured graph), and a position encoding with
+# frequencies and a stretch of its own behind the attention mixer
+# ---------------------------------------------------------------------------
+
+def _register_routed_toy():
+    from lockstep_amd.config import (LayerSpec, ModelConfig, ModelSpec, PartSpec, ScheduleEntry,
+                                     register_architecture)
+    from lockstep_amd.parts import FeedForward, PositionEncoding, WeightSpec, bump_device_epoch, register_part
+
+    @register_part("toy_linear_angles")
+    class LinearAngles(PositionEncoding):
+        """Pair i at position p turns by (p / stretch) * (i + 1) * step."""
+
+        graph_safe = True
+
+        def __init__(self, spec, prefix=""):
+            super().__init__(spec, prefix)
+            self.rotary_dim = int(spec["rotary_dim"])
+            self.stretch, self.step = float(spec["stretch"]), float(spec["step"])
+            self.cos = self.sin = None
+
+        def ensure(self, max_position, rt):
+            if self.cos is not None and self.cos.shape[0] >= max_position:
+                return
+            angles = _linear_angles(torch.arange(max(max_position, 24)), self.rotary_dim, self.stretch, self.step)
+            self.cos = angles.cos().float().to(rt.device).contiguous()
+            self.sin = angles.sin().float().to(rt.device).contiguous()
+            bump_device_epoch()                      # a captured graph holds the old tables
+
+    @register_part("toy_top1_experts")
+    class Top1Experts(FeedForward):
+        """logits = x R^T in float32; a token goes to the expert with the largest logit and its
+        output is softmax(logits)[expert] * down_e(relu(up_e(x)))."""
+
+        def __init__(self, spec, prefix=""):
+            super().__init__(spec, prefix)
+            self.hidden, self.experts, self.inter = (int(spec[k]) for k in ("hidden_size", "experts", "expert_size"))
+
+        @classmethod
+        def weight_specs(cls, spec, prefix):
+            h, n, i = (int(spec[k]) for k in ("hidden_size", "experts", "expert_size"))
+            out = [WeightSpec(f"{prefix}.router.weight", (n, h))]
+            for e in range(n):
+                out += [WeightSpec(f"{prefix}.experts.{e}.up.weight", (i, h)),
+                        WeightSpec(f"{prefix}.experts.{e}.down.weight", (h, i))]
+            return out
+
+        def load(self, weights, rt):
+            self.router = rt.vector(weights.get(f"{self.prefix}.router.weight"))
+            self.up = [rt.vector(weights.get(f"{self.prefix}.experts.{e}.up.weight")) for e in range(self.experts)]
+            self.down = [rt.vector(weights.get(f"{self.prefix}.experts.{e}.down.weight")) for e in range(self.experts)]
+
+        def forward(self, ctx, x, out, accumulate):
+            xf = x.float()
+            logits = xf @ self.router.T
+            choice = logits.argmax(-1)
+            gate = torch.softmax(logits, -1).gather(1, choice[:, None])
+            y = torch.zeros_like(xf)
+            for e in choice.unique().tolist():       # read on the host
+                rows = (choice == e).nonzero()[:, 0]
+                y[rows] = torch.relu(xf[rows] @ self.up[e].T) @ self.down[e].T
+            y = y * gate
+            out[:] = out + y if accumulate else y
+
+    @register_architecture
+    @dataclass(frozen=True)
+    class RoutedToyConfig(ModelConfig):
+        hidden_size: int
+        vocab_size: int
+        experts: int
+        routed: bool
+        architecture_names = ("toy-routed",)
+
+        def model_spec(self):
+            h = self.hidden_size
+            norm = PartSpec("rmsnorm", {"size": h, "eps": 1e-5})
+            routed = PartSpec("toy_top1_experts", {"hidden_size": h, "experts": self.experts, "expert_size": 24})
+            dense = PartSpec("gated_mlp", {"hidden_size": h, "intermediate_size": 2 * h, "activation": "silu"})
+            arr = PartSpec("prenorm_residual", {"mixer_prefix": "mixer", "feed_forward_prefix": "ff",
+                                                "mixer_norm_name": "norm1", "feed_forward_norm_name": "norm2"})
+            attn = PartSpec("attention", {"hidden_size": h, "num_heads": 3, "num_kv_heads": 1, "head_dim": 16,
+                                          "qk_norm": None,
+                                          "position": PartSpec("toy_linear_angles",
+                                                               {"rotary_dim": 12, "stretch": 4.0, "step": 0.3}),
+                                          "window": None, "bias": False, "scale": 0.25})
+            # layer 0 is dense, layer 1 routed (when asked for): parts are chosen layer by layer
+            layers = (LayerSpec("layers.0", arr, attn, dense, norm, norm),
+                      LayerSpec("layers.1", arr, attn, routed if self.routed else dense, norm, norm))
+            return ModelSpec(
+                hidden_size=h, vocab_size=self.vocab_size,
+                embedding=PartSpec("token_embedding", {"name": "embed.weight", "vocab_size": self.vocab_size,
+                                                       "hidden_size": h}),
+                layers=layers, schedule=(ScheduleEntry(0, 0, True), ScheduleEntry(1, 1, True)),
+                final_norm=PartSpec("rmsnorm", {"size": h, "eps": 1e-5, "name": "final_norm.weight"}),
+                head=PartSpec("linear_head", {"name": "head.weight", "tied_to": None,
+                                              "vocab_size": self.vocab_size, "hidden_size": h}))
+
+    return RoutedToyConfig
+
+
+def _linear_angles(positions, rotary_dim, stretch, step):
+    pairs = torch.arange(1, rotary_dim // 2 + 1, dtype=torch.float64)
+    return (positions.to(torch.float64) / stretch)[:, None] * (pairs * step)[None, :]
+
+
+def _routed_toy_plain(w, tokens, hidden, experts, routed):
+    """Plain float64 forward, whole sequence; also the smallest margin between a token's two best experts."""
+    t = len(tokens)
+    h = w["embed.weight"][torch.tensor(tokens)]
+    angles = _linear_angles(torch.arange(t), 12, 4.0, 0.3)
+    cos, sin = angles.cos(), angles.sin()
+    margin = float("inf")
+    for layer in range(2):
+        p = f"layers.{layer}"
+        x = P.rmsnorm(h, w[f"{p}.norm1.weight"], 1e-5)
+        q = P.linear(x, w[f"{p}.mixer.q_proj.weight"]).view(t, 3, 16)
+        k = P.linear(x, w[f"{p}.mixer.k_proj.weight"]).view(t, 1, 16)
+        v = P.linear(x, w[f"{p}.mixer.v_proj.weight"]).view(t, 1, 16)
+        q = torch.cat([P.apply_rope(q[..., :12], cos, sin), q[..., 12:]], -1)
+        k = torch.cat([P.apply_rope(k[..., :12], cos, sin), k[..., 12:]], -1)
+        attn = P.causal_attention(q * (0.25 * 4.0), k, v)
+        h = h + P.linear(attn.reshape(t, 48), w[f"{p}.mixer.o_proj.weight"])
+        x = P.rmsnorm(h, w[f"{p}.norm2.weight"], 1e-5)
+        if layer == 1 and routed:
+            logits = x @ w[f"{p}.ff.router.weight"].T
+            top = logits.topk(2, dim=-1).values
+            margin = min(margin, float((top[:, 0] - top[:, 1]).min()))
+            choice = logits.argmax(-1)
+            gate = torch.softmax(logits, -1)
+            rows = []
+            for i in range(t):
+                e = int(choice[i])
+                mid = torch.relu(x[i] @ w[f"{p}.ff.experts.{e}.up.weight"].T)
+                rows.append(gate[i, e] * (mid @ w[f"{p}.ff.experts.{e}.down.weight"].T))
+            h = h + torch.stack(rows)
+        else:
+            h = h + P.mlp_block(w, f"{p}.ff", x)
+    return P.linear(P.rmsnorm(h, w["final_norm.weight"], 1e-5), w["head.weight"]), margin
+
+
+@pytest.mark.parametrize("routed", [True, False])
+def test_toy_routed_feed_forward_and_toy_position_encoding(tmp_path, routed):
+    """Parts of other kinds than the built-in ones, registered from outside: a routed feed-forward
+    in one layer beside a dense one in the other, and a position encoding of its own behind the
+    attention kernel.  The routed part reads its routing on the host, so the model must not
+    capture decode steps; without it the steps are replayed from a graph, with the toy tables."""
+    from lockstep_amd.config import unregister_architecture
+    from lockstep_amd.engine.model import load_model
+    from lockstep_amd.parts import unregister_part
+    from lockstep_amd.weights import write_random_model
+    from safetensors.torch import load_file
+
+    RoutedToyConfig = _register_routed_toy()
+    try:
+        cfg = RoutedToyConfig(hidden_size=40, vocab_size=75, experts=3, routed=routed)
+        folder = write_random_model(cfg, tmp_path / "routed", seed=8, std=0.25, norm_std=0.1)
+        model = load_model(folder, dtype="float32")
+        w = {k: v.double() for k, v in load_file(str(folder / "model.safetensors")).items()}
+        assert ("layers.1.ff.experts.2.down.weight" in w) == routed and "layers.0.ff.gate_proj.weight" in w
+        tokens = random_tokens(60, 75, seed=4)
+        want, margin = _routed_toy_plain(w, tokens, 40, 3, routed)
+        assert margin > 1e-3, "two experts nearly tie for a token: pick another seed"
+        cache = model.make_cache(num_pages=24, page_size=8, max_requests=3, poison_on_free=True)
+        whole = feed(model, cache, "w", tokens, [])
+        assert rel_err(whole, want) < 5e-5
+        cut = feed(model, cache, "c", tokens, [9, 2, 20] + [1] * 29)     # the tail as decode steps
+        assert rel_err(cut, want) < 5e-5
+        assert (model.graph_replays == 0) == routed, "a part that is not graph safe keeps the steps eager"
+        cache.audit()
+    finally:
+        unregister_part("toy_linear_angles")
+        unregister_part("toy_top1_experts")
+        unregister_architecture(RoutedToyConfig)
