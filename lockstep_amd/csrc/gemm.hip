@@ -623,11 +623,11 @@ __global__ __launch_bounds__(256) void gemm_slices_stream_kernel(const T* __rest
 constexpr int kRowBytes = 128;               // bytes of K per row per stage (two chunks)
 constexpr int kRowStride = kRowBytes + 16;   // padded LDS row
 
-template <typename T, int EPI, int BM, int BN, int PD>
+template <typename T, int EPI, int BM, int BN, int PD, bool AL>
 __global__ __launch_bounds__(256) void gemm_tiled_kernel(const T* __restrict__ X, const T* __restrict__ W,
                                                          void* __restrict__ C, int M, int N, int K, long ldx,
-                                                         long ldc, int kslice, int aligned, int vec_ok,
-                                                         int tiles_m, int tiles_n, int out_cols) {
+                                                         long ldc, int kslice, int vec_ok, int tiles_m, int tiles_n,
+                                                         int out_cols) {
   typedef Atom<T> A;
   typedef typename A::vec_t vec_t;
   constexpr int BK = kRowBytes / sizeof(T);  // elements of K per stage
@@ -676,35 +676,60 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const T* __restrict__ X
       acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
 
-  // PD stages of global loads are in flight in registers (slot = stage % PD)
+  // PD stages of global loads are in flight in registers (slot = stage % PD).
+  // AL (rows and K 16-byte aligned, K a multiple of VEC): the loads are unconditional, from addresses
+  // clamped into the matrix, and nothing reads their registers before the stage is written to LDS, so
+  // the loads of PD stages really are in flight together (a zero selected right behind a load makes the
+  // compiler wait for it there).  Rows beyond M or N then hold copies of the last row: their products
+  // land in outputs that the epilogue does not store.  Only columns from K on must read as zero, and
+  // those are cleared on the way to LDS.
   vec_t wv[PD][WP], xv[PD][XP];
+  const T* w_src[WP];
+  const T* x_src[XP];
+  if (AL) {
+#pragma unroll
+    for (int p = 0; p < WP; ++p) w_src[p] = W + (long)min(n_base + st_row + 32 * p, N - 1) * K;
+#pragma unroll
+    for (int p = 0; p < XP; ++p) x_src[p] = X + (long)min(m_base + st_row + 32 * p, M - 1) * ldx;
+  }
   auto fetch = [&](int slot, int k0) {
+    if (AL) {
+      const int k = min(k0 + st_col, K - A::VEC);
+#pragma unroll
+      for (int p = 0; p < WP; ++p) wv[slot][p] = *reinterpret_cast<const vec_t*>(w_src[p] + k);
+#pragma unroll
+      for (int p = 0; p < XP; ++p) xv[slot][p] = *reinterpret_cast<const vec_t*>(x_src[p] + k);
+      return;
+    }
 #pragma unroll
     for (int p = 0; p < WP; ++p) {
       const int r = st_row + 32 * p;
-      wv[slot][p] = load_vec<T>(W, n_base + r, k0 + st_col, K, K, n_base + r < N, aligned);
+      wv[slot][p] = load_vec<T>(W, n_base + r, k0 + st_col, K, K, n_base + r < N, false);
     }
 #pragma unroll
     for (int p = 0; p < XP; ++p) {
       const int r = st_row + 32 * p;
-      xv[slot][p] = load_vec<T>(X, m_base + r, k0 + st_col, K, ldx, m_base + r < M, aligned);
+      xv[slot][p] = load_vec<T>(X, m_base + r, k0 + st_col, K, ldx, m_base + r < M, false);
     }
   };
-  auto stash = [&](int slot, int buf) {
+  auto stash = [&](int slot, int buf, int k0) {
     unsigned char* w_lds = lds + buf * STAGE_BYTES;
     unsigned char* x_lds = w_lds + BN * kRowStride;
+    const bool past_k = AL && k0 + st_col >= K;  // only in the last stage, where K is no multiple of BK
 #pragma unroll
     for (int p = 0; p < WP; ++p)
-      *reinterpret_cast<vec_t*>(&w_lds[(st_row + 32 * p) * kRowStride + st_col * sizeof(T)]) = wv[slot][p];
+      *reinterpret_cast<vec_t*>(&w_lds[(st_row + 32 * p) * kRowStride + st_col * sizeof(T)]) =
+          past_k ? A::zero() : wv[slot][p];
 #pragma unroll
     for (int p = 0; p < XP; ++p)
-      *reinterpret_cast<vec_t*>(&x_lds[(st_row + 32 * p) * kRowStride + st_col * sizeof(T)]) = xv[slot][p];
+      *reinterpret_cast<vec_t*>(&x_lds[(st_row + 32 * p) * kRowStride + st_col * sizeof(T)]) =
+          past_k ? A::zero() : xv[slot][p];
   };
 
   const int stages = (K + BK - 1) / BK;
   // stage s lives in register slot s % PD until it is written to LDS buffer s % 2
   fetch(0, 0);
-  stash(0, 0);
+  stash(0, 0, 0);
 #pragma unroll
   for (int u = 1; u <= PD; ++u)
     if (u < stages) fetch(u % PD, u * BK);
@@ -726,7 +751,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const T* __restrict__ X
       }
       __syncthreads();  // stage st is in its buffer; the other buffer has been read by every wave
       if (st + 1 < stages) {
-        stash((u + 1) % PD, (st + 1) & 1);
+        stash((u + 1) % PD, (st + 1) & 1, (st + 1) * BK);
         if (st + 1 + PD < stages) fetch((u + 1) % PD, (st + 1 + PD) * BK);
       }
       const unsigned char* w_lds = lds + (st & 1) * STAGE_BYTES;
@@ -867,14 +892,18 @@ int launch_gemm(const void* X, const void* W, void* C, int M, int N, int K, long
     // Large products take 128 x 128 tiles (least LDS traffic per MFMA); smaller ones take
     // 64 x 64 tiles so that every CU has several workgroups, with a deeper register prefetch.
     const long big_tiles = (long)((M + 127) / 128) * ((N + 127) / 128);
-#define LS_TILED(BM_, BN_, PD_)                                                                                 \
+#define LS_TILED(BM_, BN_, PD_, AL_)                                                                           \
   {                                                                                                             \
     const int tiles_m = (M + BM_ - 1) / BM_, tiles_n = (N + BN_ - 1) / BN_;                                       \
-    hipLaunchKernelGGL((gemm_tiled_kernel<T, EPI, BM_, BN_, PD_>), dim3(tiles_m * tiles_n), dim3(256), 0, stream, \
-                       reinterpret_cast<const T*>(X), w, C, M, N, K, ldx, ldc, kslice, aligned, vec_ok, tiles_m,  \
+    hipLaunchKernelGGL((gemm_tiled_kernel<T, EPI, BM_, BN_, PD_, AL_>), dim3(tiles_m * tiles_n), dim3(256), 0,   \
+                       stream, reinterpret_cast<const T*>(X), w, C, M, N, K, ldx, ldc, kslice, vec_ok, tiles_m,   \
                        tiles_n, out_cols);                                                                      \
   }
-    if (big_tiles >= LS_GEMM_BIG) LS_TILED(128, 128, LS_GEMM_PD_BIG) else LS_TILED(64, 64, LS_GEMM_PD_SMALL)
+    // (operands that are not 16-byte aligned take the small tiles, element by element: every tile
+    // shape gives the same bits)
+    if (!aligned) LS_TILED(64, 64, LS_GEMM_PD_SMALL, false)
+    else if (big_tiles >= LS_GEMM_BIG) LS_TILED(128, 128, LS_GEMM_PD_BIG, true)
+    else LS_TILED(64, 64, LS_GEMM_PD_SMALL, true)
 #undef LS_TILED
   }
   return check_launch("gemm");
