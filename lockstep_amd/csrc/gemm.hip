@@ -28,7 +28,7 @@ namespace ls {
 #define LS_GEMM_BIG 512       // from this many 128 x 128 tiles on, use them
 #endif
 #ifndef LS_GEMM_PD_BIG
-#define LS_GEMM_PD_BIG 1      // register prefetch depth (stages) of the 128 x 128 kernel
+#define LS_GEMM_PD_BIG 1      // register prefetch depth (stages) of the 128 x 128 kernel (2: registers run out, a third slower)
 #endif
 #ifndef LS_GEMM_STREAM
 #define LS_GEMM_STREAM 1      // 0: never the streaming kernel
@@ -37,7 +37,7 @@ namespace ls {
 #define LS_GEMM_GROUP_M 4     // row tiles per band of the tile numbering (0: column-major numbering)
 #endif
 #ifndef LS_GEMM_PD_SMALL
-#define LS_GEMM_PD_SMALL 2    // ... and of the 64 x 64 kernel
+#define LS_GEMM_PD_SMALL 4    // ... and of the 64 x 64 kernel (measured 1 to 4: 4 is 2 to 10 % ahead of 2)
 #endif
 
 enum Epilogue : int {
@@ -715,24 +715,33 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const T* __restrict__ X
   auto stash = [&](int slot, int buf, int k0) {
     unsigned char* w_lds = lds + buf * STAGE_BYTES;
     unsigned char* x_lds = w_lds + BN * kRowStride;
-    const bool past_k = AL && k0 + st_col >= K;  // only in the last stage, where K is no multiple of BK
 #pragma unroll
     for (int p = 0; p < WP; ++p)
-      *reinterpret_cast<vec_t*>(&w_lds[(st_row + 32 * p) * kRowStride + st_col * sizeof(T)]) =
-          past_k ? A::zero() : wv[slot][p];
+      *reinterpret_cast<vec_t*>(&w_lds[(st_row + 32 * p) * kRowStride + st_col * sizeof(T)]) = wv[slot][p];
 #pragma unroll
     for (int p = 0; p < XP; ++p)
-      *reinterpret_cast<vec_t*>(&x_lds[(st_row + 32 * p) * kRowStride + st_col * sizeof(T)]) =
-          past_k ? A::zero() : xv[slot][p];
+      *reinterpret_cast<vec_t*>(&x_lds[(st_row + 32 * p) * kRowStride + st_col * sizeof(T)]) = xv[slot][p];
+    if (AL && k0 + BK > K) {  // uniform: the last stage where K is no multiple of BK; its columns from K on are cleared
+      if (k0 + st_col >= K) {
+#pragma unroll
+        for (int p = 0; p < WP; ++p)
+          *reinterpret_cast<vec_t*>(&w_lds[(st_row + 32 * p) * kRowStride + st_col * sizeof(T)]) = A::zero();
+#pragma unroll
+        for (int p = 0; p < XP; ++p)
+          *reinterpret_cast<vec_t*>(&x_lds[(st_row + 32 * p) * kRowStride + st_col * sizeof(T)]) = A::zero();
+      }
+    }
   };
 
   const int stages = (K + BK - 1) / BK;
   // stage s lives in register slot s % PD until it is written to LDS buffer s % 2
   fetch(0, 0);
   stash(0, 0, 0);
+  // (AL: stages past the end are fetched too, from clamped addresses: with no condition around a
+  // fetch the compiler can count which loads are still in flight when a stage goes to LDS)
 #pragma unroll
   for (int u = 1; u <= PD; ++u)
-    if (u < stages) fetch(u % PD, u * BK);
+    if (AL || u < stages) fetch(u % PD, u * BK);
   for (int base = 0; base < stages; base += PD) {
 #pragma unroll
     for (int u = 0; u < PD; ++u) {  // unrolled so that the register slots are static
@@ -750,9 +759,9 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const T* __restrict__ X
           }
       }
       __syncthreads();  // stage st is in its buffer; the other buffer has been read by every wave
-      if (st + 1 < stages) {
+      if (AL || st + 1 < stages) {  // (AL: past the last stage too, into the buffer that nobody reads any more)
         stash((u + 1) % PD, (st + 1) & 1, (st + 1) * BK);
-        if (st + 1 + PD < stages) fetch((u + 1) % PD, (st + 1 + PD) * BK);
+        if (AL || st + 1 + PD < stages) fetch((u + 1) % PD, (st + 1 + PD) * BK);
       }
       const unsigned char* w_lds = lds + (st & 1) * STAGE_BYTES;
       const unsigned char* x_lds = w_lds + BN * kRowStride;
