@@ -1231,7 +1231,7 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
     head16_load_values<T, PASSES>(hx, head_src(vi), D, gl);
     if (vi <= G)
       head16_load_factors<PASSES>(hf, D, vi < G ? fz.q_weight : fz.k_weight, fz.cos_table, fz.sin_table, p_new,
-                                  fz.rot, gl, reinterpret_cast<const float*>(new_row));
+                                  fz.rot, gl);
   };
   if (FUSE) {
     if (owner) page_new = tbl[p_new >> page_shift];

@@ -166,40 +166,38 @@ struct HeadFactors {  // what does not depend on the head's values
   float w[8 * PASSES], c[8 * PASSES], s[8 * PASSES];
 };
 
-// Eight floats from `src` (16-byte aligned) where `ok`, else `fill`.  The loads are unconditional
-// (where not ok they read `safe`, any 32 readable, 16-byte aligned bytes) and the choice comes
-// after them: with a branch around a load the compiler waits for it where the paths meet, and a
-// run of such loads would go to memory one after the other.
 template <int N>
-__device__ __forceinline__ void load_floats8(float* dst, const float* __restrict__ src, bool ok, float fill,
-                                             const float* __restrict__ safe) {
-  const float* from = ok ? src : safe;
-  const f32x4 lo = *reinterpret_cast<const f32x4*>(from);
-  const f32x4 hi = *reinterpret_cast<const f32x4*>(from + 4);
+__device__ __forceinline__ void load_floats8(float* dst, const float* __restrict__ src, bool ok, float fill) {
+  if (ok) {
+    const f32x4 lo = *reinterpret_cast<const f32x4*>(src);
+    const f32x4 hi = *reinterpret_cast<const f32x4*>(src + 4);
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    dst[j] = ok ? lo[j] : fill;
-    dst[4 + j] = ok ? hi[j] : fill;
+    for (int j = 0; j < 4; ++j) {
+      dst[j] = lo[j];
+      dst[4 + j] = hi[j];
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) dst[j] = fill;
   }
 }
 
-// gl: the lane's index in its group of 16.  weight / tables may be nullptr.  safe: see load_floats8.
+// gl: the lane's index in its group of 16.  weight / tables may be nullptr.
 template <int PASSES>
 __device__ __forceinline__ void head16_load_factors(HeadFactors<PASSES>& f, int d, const float* __restrict__ weight,
                                                     const float* __restrict__ cos_table,
-                                                    const float* __restrict__ sin_table, int pos, int rot, int gl,
-                                                    const float* __restrict__ safe) {
+                                                    const float* __restrict__ sin_table, int pos, int rot, int gl) {
   const int half = rot / 2;
 #pragma unroll
   for (int p = 0; p < PASSES; ++p) {
     const int e0 = 128 * p + 8 * gl;
-    load_floats8<8>(f.w + 8 * p, weight + (weight ? e0 : 0), weight != nullptr && e0 < d, 1.f, safe);
+    load_floats8<8>(f.w + 8 * p, weight + (weight ? e0 : 0), weight != nullptr && e0 < d, 1.f);
     if ((half & 7) == 0) {  // uniform: a run of eight lies on one side of the half
       const bool turn = cos_table != nullptr && e0 < rot;
       const int idx = e0 < half ? e0 : e0 - half;
       const long at = turn ? (long)pos * half + idx : 0;
-      load_floats8<8>(f.c + 8 * p, cos_table + at, turn, 1.f, safe);
-      load_floats8<8>(f.s + 8 * p, sin_table + at, turn, 0.f, safe);
+      load_floats8<8>(f.c + 8 * p, cos_table + at, turn, 1.f);
+      load_floats8<8>(f.s + 8 * p, sin_table + at, turn, 0.f);
     } else {
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
@@ -213,21 +211,23 @@ __device__ __forceinline__ void head16_load_factors(HeadFactors<PASSES>& f, int 
   }
 }
 
-// src: the head's first element; 16-byte aligned.  Elements from d on read as zero (their lanes
-// load the head's first elements instead: no branch around the load, see load_floats8).
+// src: the head's first element; 16-byte aligned.
 template <typename T, int PASSES>
 __device__ __forceinline__ void head16_load_values(float (&x)[8 * PASSES], const T* src, int d, int gl) {
 #pragma unroll
   for (int p = 0; p < PASSES; ++p) {
     const int e0 = 128 * p + 8 * gl;
-    const bool in = e0 < d;
-    if (sizeof(T) == 2) {
-      const bf16x8 v = *reinterpret_cast<const bf16x8*>(src + (in ? e0 : 0));
+    if (e0 < d) {
+      if (sizeof(T) == 2) {
+        const bf16x8 v = *reinterpret_cast<const bf16x8*>(src + e0);
 #pragma unroll
-      for (int j = 0; j < 8; ++j) x[8 * p + j] = in ? to_f32(v[j]) : 0.f;
+        for (int j = 0; j < 8; ++j) x[8 * p + j] = to_f32(v[j]);
+      } else {
+        load_floats8<8>(x + 8 * p, reinterpret_cast<const float*>(src) + e0, true, 0.f);
+      }
     } else {
-      load_floats8<8>(x + 8 * p, reinterpret_cast<const float*>(src) + e0, in, 0.f,
-                      reinterpret_cast<const float*>(src));
+#pragma unroll
+      for (int j = 0; j < 8; ++j) x[8 * p + j] = 0.f;
     }
   }
 }

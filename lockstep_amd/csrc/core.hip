@@ -134,18 +134,17 @@ __global__ __launch_bounds__(256) void qk_rope_kv_kernel(
     const int j = threadIdx.x & 15;
     const int t = (vb / col_blocks) * 16 + j;
     if (t >= n_tokens) return;
-    // the values first, then the chain position -> sequence -> block table: they travel together
+    const int pos = tok_pos[t];
+    const SeqMeta sm = seqs[tok_seq[t]];
+    const long page = table[(long)sm.table_row * table_stride + pos / page_size];
+    if (page < 0) return;
+    const int slot = pos % page_size;
     const T* src = qkv + (long)t * ld + (long)(nq + nkv) * d;
+    T* dst = v_pages + page * nkv * d * page_size + slot;
     const int c0 = (vb % col_blocks) * 64 + (threadIdx.x >> 4);
     T v[4];
 #pragma unroll
     for (int u = 0; u < 4; ++u) v[u] = src[min(c0 + 16 * u, width - 1)];
-    const int pos = tok_pos[t];
-    const int table_row = seqs[tok_seq[t]].table_row;
-    const long page = table[(long)table_row * table_stride + pos / page_size];
-    if (page < 0) return;
-    const int slot = pos % page_size;
-    T* dst = v_pages + page * nkv * d * page_size + slot;
 #pragma unroll
     for (int u = 0; u < 4; ++u)
       if (c0 + 16 * u < width) dst[(long)(c0 + 16 * u) * page_size] = v[u];
@@ -160,28 +159,20 @@ __global__ __launch_bounds__(256) void qk_rope_kv_kernel(
   const int head = (int)(gid % heads);
   const bool is_q = head < nq;
   T* src = qkv + (long)t * ld + (long)head * d;
-  // No branch lies between the loads (a query head fetches its token's page too and drops it), so
-  // they go to memory in three rounds: position, sequence, values and weights; rotation factors and
-  // the row of the block table; the page.
   const int pos = tok_pos[t];
-  const int seq = tok_seq[t];
+  T* dst = src;
+  bool held = true;
+  if (!is_q) {
+    const SeqMeta sm = seqs[tok_seq[t]];
+    const long page = table[(long)sm.table_row * table_stride + pos / page_size];
+    held = page >= 0;  // the host never schedules a write to a page it does not hold
+    dst = k_pages + ((max(page, 0L) * nkv + (head - nq)) * page_size + pos % page_size) * d;
+  }
   const float* weight = is_q ? q_weight : k_weight;
   float x[8 * PASSES];
   HeadFactors<PASSES> f;
   head16_load_values<T, PASSES>(x, src, d, gl);
-  head16_load_factors<PASSES>(f, d, weight, cos_table, sin_table, pos, rot, gl,
-                              reinterpret_cast<const float*>(qkv + (long)t * ld));
-  long page = -1;
-  if (write_kv) {  // uniform
-    const int table_row = seqs[seq].table_row;
-    page = table[(long)table_row * table_stride + pos / page_size];
-  }
-  T* dst = src;
-  bool held = true;
-  if (!is_q) {
-    held = page >= 0;  // the host never schedules a write to a page it does not hold
-    dst = k_pages + ((max(page, 0L) * nkv + (head - nq)) * page_size + pos % page_size) * d;
-  }
+  head16_load_factors<PASSES>(f, d, weight, cos_table, sin_table, pos, rot, gl);
   head16_finish<T, PASSES>(x, f, d, weight != nullptr, eps, cos_table != nullptr, rot, gl, [&](int e0, const T (&v)[8]) {
     if (held) store8<T>(dst + e0, v);
   });
