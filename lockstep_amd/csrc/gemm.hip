@@ -25,7 +25,7 @@
 namespace ls {
 
 #ifndef LS_GEMM_BIG
-#define LS_GEMM_BIG 512       // from this many 128 x 128 tiles on, use them
+#define LS_GEMM_BIG 256       // from this many 128 x 128 tiles on (one for every CU), use them; fewer leave CUs idle and 64 x 64 tiles win
 #endif
 #ifndef LS_GEMM_PD_BIG
 #define LS_GEMM_PD_BIG 1      // register prefetch depth (stages) of the 128 x 128 kernel (2: registers run out, a third slower)
