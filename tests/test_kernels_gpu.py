@@ -30,7 +30,10 @@ TOL = {torch.float32: 2e-5, torch.bfloat16: 1.5e-2}
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("m,n,k", [(1, 16, 32), (1, 1000, 96), (5, 48, 200), (16, 100, 64), (17, 33, 72),
                                    (64, 256, 1024), (65, 130, 260), (37, 3072, 1024), (200, 96, 4100),
-                                   (130, 1000, 8), (3, 40, 12)])
+                                   (130, 1000, 8), (3, 40, 12),
+                                   # 128 x 128 tiles with rows, columns and K that end inside a tile (operand
+                                   # loads from clamped addresses), and the same with K not 16-byte aligned
+                                   (2050, 2100, 264), (2050, 2100, 260)])
 def test_gemm_matches_linear(dtype, m, n, k):
     from lockstep_amd.ops import STORE, STORE_F32, ADD_F32
 
