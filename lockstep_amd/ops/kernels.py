@@ -46,24 +46,27 @@ def _ptr(t) -> c_void_p:
 
 
 _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_raw_device = getattr(torch._C, "_cuda_getDevice", None)
 
 
 def _stream() -> c_void_p:
     """The current stream of the current device (asked through the raw call where torch has it:
     a kernel launch asks for it every time, and the Python stream object costs ten times as much)."""
     if _raw_stream is not None:
-        return c_void_p(_raw_stream(torch.cuda.current_device()))
+        return c_void_p(_raw_stream(_raw_device() if _raw_device is not None else torch.cuda.current_device()))
     return c_void_p(torch.cuda.current_stream().cuda_stream)
 
 
-def _need(cond: bool, message: str) -> None:
+def _need(cond: bool, message) -> None:
+    """``message``: the text, or a callable that makes it (so that a message with shapes in it is
+    formatted only when the check fails: these checks run before every launch)."""
     if not cond:
-        raise KernelError(message)
+        raise KernelError(message() if callable(message) else message)
 
 
 def _rows_ok(t: torch.Tensor, name: str) -> None:
-    _need(t.is_cuda, f"{name} must live on the GPU")
-    _need(t.dim() == 2 and t.stride(1) == 1, f"{name} must be 2-D with contiguous rows, got shape "
+    _need(t.is_cuda, lambda: f"{name} must live on the GPU")
+    _need(t.dim() == 2 and t.stride(1) == 1, lambda: f"{name} must be 2-D with contiguous rows, got shape "
           f"{tuple(t.shape)} strides {t.stride()}")
 
 
@@ -91,7 +94,7 @@ class Kernels:
             path = _build.build_attention(head_dim)
             lib = ctypes.CDLL(str(path))
             lib.ls_last_error.restype = ctypes.c_char_p
-            _need(lib.ls_attn_head_dim() == head_dim, f"{path} was built for another head size")
+            _need(lib.ls_attn_head_dim() == head_dim, lambda: f"{path} was built for another head size")
             self._attention[head_dim] = lib
             self.attention_paths[head_dim] = str(path)
         return lib
@@ -143,25 +146,25 @@ class Kernels:
         ``norm_weight`` (float32 ``[K]``): ``x`` is the float32 residual stream and is
         RMS-normalised on the fly with this weight and ``eps`` (at most 16 rows)."""
         _rows_ok(x, "gemm x"); _rows_ok(w, "gemm w"); _rows_ok(out, "gemm out")
-        _need(w.dtype in DTYPE_CODE, f"gemm weights must be float32 or bfloat16, got {w.dtype}")
+        _need(w.dtype in DTYPE_CODE, lambda: f"gemm weights must be float32 or bfloat16, got {w.dtype}")
         if norm_weight is None:
-            _need(x.dtype == w.dtype, f"gemm operands must share a dtype, got {x.dtype} and {w.dtype}")
+            _need(x.dtype == w.dtype, lambda: f"gemm operands must share a dtype, got {x.dtype} and {w.dtype}")
         else:
             _need(x.dtype == torch.float32 and x.shape[0] <= 16, "the fused norm reads at most 16 float32 rows")
             _need(norm_weight.is_cuda and norm_weight.dtype == torch.float32 and norm_weight.is_contiguous()
-                  and norm_weight.shape == (x.shape[1],), f"norm weight must be float32 [{x.shape[1]}]")
+                  and norm_weight.shape == (x.shape[1],), lambda: f"norm weight must be float32 [{x.shape[1]}]")
         m, k = x.shape
         n = w.shape[0]
-        _need(w.shape[1] == k and w.is_contiguous(), f"gemm w must be contiguous [N,{k}], got {tuple(w.shape)}")
+        _need(w.shape[1] == k and w.is_contiguous(), lambda: f"gemm w must be contiguous [N,{k}], got {tuple(w.shape)}")
         if epilogue == SWIGLU:
             cols = out.shape[1]
             _need(n % 32 == 0 and n // 2 - 16 < cols <= n // 2 and out.shape[0] == m,
-                  f"SwiGLU output [{m},{cols}] does not fit {n} interleaved weight rows")
+                  lambda: f"SwiGLU output [{m},{cols}] does not fit {n} interleaved weight rows")
         else:
             cols = n
-            _need(tuple(out.shape) == (m, n), f"gemm out must be [{m},{n}], got {tuple(out.shape)}")
+            _need(tuple(out.shape) == (m, n), lambda: f"gemm out must be [{m},{n}], got {tuple(out.shape)}")
         want = w.dtype if epilogue in (STORE, SWIGLU) else torch.float32
-        _need(out.dtype == want, f"gemm out dtype {out.dtype} does not fit epilogue {epilogue}")
+        _need(out.dtype == want, lambda: f"gemm out dtype {out.dtype} does not fit epilogue {epilogue}")
         if m == 0:
             return
         code = self.core.ls_gemm(c_int(DTYPE_CODE[w.dtype]), c_int(epilogue), _ptr(x), _ptr(w), _ptr(out),
@@ -183,7 +186,7 @@ class Kernels:
               and w.dtype in DTYPE_CODE, "gemm_slices w must be [N, K] contiguous in the dtype of x")
         _need(partials.is_cuda and partials.dtype == torch.float32 and partials.is_contiguous()
               and partials.shape == (self.gemm_slices_count(k), m, n),
-              f"gemm_slices partials must be float32 [{self.gemm_slices_count(k)}, {m}, {n}]")
+              lambda: f"gemm_slices partials must be float32 [{self.gemm_slices_count(k)}, {m}, {n}]")
         code = self.core.ls_gemm_slices(c_int(DTYPE_CODE[w.dtype]), _ptr(x), _ptr(w), _ptr(partials), c_int(m),
                                         c_int(n), c_int(k), c_long(x.stride(0)), _stream())
         self._check(self.core, code)
@@ -221,7 +224,7 @@ class Kernels:
         _rows_ok(table, "embed table"); _rows_ok(out, "embed out")
         _need(table.is_contiguous() and table.dtype in DTYPE_CODE, "embed table must be contiguous float32/bfloat16")
         _need(out.dtype == torch.float32 and out.shape == (tokens.shape[0], table.shape[1]),
-              f"embed out must be float32 [{tokens.shape[0]},{table.shape[1]}]")
+              lambda: f"embed out must be float32 [{tokens.shape[0]},{table.shape[1]}]")
         if tokens.shape[0] == 0:
             return
         code = self.core.ls_embed(c_int(DTYPE_CODE[table.dtype]), _ptr(tokens), _ptr(table), _ptr(out),
@@ -235,12 +238,12 @@ class Kernels:
         _rows_ok(x, "rmsnorm x"); _rows_ok(out, "rmsnorm out")
         _need(x.dtype == torch.float32, "rmsnorm reads the float32 residual stream")
         _need(weight.is_cuda and weight.dtype == torch.float32 and weight.is_contiguous()
-              and weight.shape == (x.shape[1],), f"rmsnorm weight must be float32 [{x.shape[1]}]")
+              and weight.shape == (x.shape[1],), lambda: f"rmsnorm weight must be float32 [{x.shape[1]}]")
         _need(out.dtype in DTYPE_CODE and out.shape[1] == x.shape[1], "rmsnorm out has the wrong width or dtype")
         n = out.shape[0]
         if rows is not None:
             _need(rows.is_cuda and rows.dtype == torch.int32 and rows.is_contiguous() and rows.shape == (n,),
-                  f"rmsnorm rows must be int32 [{n}]")
+                  lambda: f"rmsnorm rows must be int32 [{n}]")
         else:
             _need(x.shape[0] == n, "rmsnorm out must have as many rows as x")
         if n == 0:
@@ -254,7 +257,7 @@ class Kernels:
         _rows_ok(gate_up, "swiglu input"); _rows_ok(out, "swiglu out")
         rows, inter = out.shape
         _need(gate_up.shape == (rows, 2 * inter) and gate_up.dtype == out.dtype and out.dtype in DTYPE_CODE,
-              f"swiglu input must be [{rows},{2 * inter}] of the output's dtype")
+              lambda: f"swiglu input must be [{rows},{2 * inter}] of the output's dtype")
         if rows == 0:
             return
         code = self.core.ls_swiglu(c_int(DTYPE_CODE[out.dtype]), _ptr(gate_up), _ptr(out), c_int(rows), c_int(inter),
@@ -265,7 +268,7 @@ class Kernels:
         _rows_ok(logits, "argmax logits")
         _need(logits.dtype == torch.float32, "argmax reads float32 logits")
         _need(out.is_cuda and out.dtype == torch.int32 and out.is_contiguous() and out.shape == (logits.shape[0],),
-              f"argmax out must be int32 [{logits.shape[0]}]")
+              lambda: f"argmax out must be int32 [{logits.shape[0]}]")
         if logits.shape[0] == 0:
             return
         words = 2 * logits.shape[0] * self.core.ls_argmax_chunks(c_int(logits.shape[1]))
@@ -307,33 +310,33 @@ class Kernels:
         _rows_ok(qkv, "qkv")
         _need(qkv.dtype in DTYPE_CODE and qkv.shape[0] >= n_tokens, "qkv has too few rows or a wrong dtype")
         heads = nq + 2 * nkv if write_kv else nq
-        _need(qkv.shape[1] >= heads * d, f"qkv rows hold {qkv.shape[1]} values, {heads} heads of {d} are needed")
-        _need(d <= MAX_HEAD_DIM, f"head size {d} exceeds the supported maximum {MAX_HEAD_DIM}")
+        _need(qkv.shape[1] >= heads * d, lambda: f"qkv rows hold {qkv.shape[1]} values, {heads} heads of {d} are needed")
+        _need(d <= MAX_HEAD_DIM, lambda: f"head size {d} exceeds the supported maximum {MAX_HEAD_DIM}")
         for name, w in (("q norm weight", q_weight), ("k norm weight", k_weight)):
             if w is not None:
                 _need(w.is_cuda and w.dtype == torch.float32 and w.is_contiguous() and w.shape == (d,),
-                      f"{name} must be float32 [{d}]")
+                      lambda: f"{name} must be float32 [{d}]")
         positions = 0
         if cos is not None:
             _need(sin is not None and cos.shape == sin.shape and cos.dim() == 2 and cos.shape[1] * 2 == rot
                   and cos.dtype == torch.float32 and cos.is_contiguous() and sin.is_contiguous() and cos.is_cuda,
                   "rotation tables must be float32 [positions, rotary_dim/2]")
             positions = cos.shape[0]
-            _need(max_pos < positions, f"position {max_pos} is beyond the rotation tables ({positions})")
+            _need(max_pos < positions, lambda: f"position {max_pos} is beyond the rotation tables ({positions})")
         for name, t in (("tok_seq", tok_seq), ("tok_pos", tok_pos)):
             _need(t.is_cuda and t.dtype == torch.int32 and t.is_contiguous() and t.numel() >= n_tokens,
-                  f"{name} must be int32 with at least {n_tokens} entries")
+                  lambda: f"{name} must be int32 with at least {n_tokens} entries")
         if write_kv:
             _need(table is not None and table.is_cuda and table.dtype == torch.int32 and table.dim() == 2
                   and table.is_contiguous(), "block table must be a contiguous int32 matrix")
             _need(max_pos // page_size < table.shape[1],
-                  f"position {max_pos} needs page {max_pos // page_size}, the block table has {table.shape[1]} columns")
+                  lambda: f"position {max_pos} needs page {max_pos // page_size}, the block table has {table.shape[1]} columns")
             for name, pages in (("key pages", k_pages), ("value pages", v_pages)):
                 _need(pages.is_cuda and pages.dtype == qkv.dtype and pages.is_contiguous() and pages.dim() == 4,
-                      f"{name} must be contiguous 4-D of the compute dtype")
+                      lambda: f"{name} must be contiguous 4-D of the compute dtype")
             _need(k_pages.shape[1:] == (nkv, page_size, d) and v_pages.shape[1:] == (nkv, d, page_size)
                   and k_pages.shape[0] == v_pages.shape[0],
-                  f"cache pages do not have the layout [pages,{nkv},{page_size},{d}] / [pages,{nkv},{d},{page_size}]")
+                  lambda: f"cache pages do not have the layout [pages,{nkv},{page_size},{d}] / [pages,{nkv},{d},{page_size}]")
         if n_tokens == 0:
             return
         code = self.core.ls_qk_rope_kv(
@@ -355,7 +358,7 @@ class Kernels:
         lib = self.attention_lib(d)
         _rows_ok(q, "attention q"); _rows_ok(out, "attention out")
         _need(q.dtype in DTYPE_CODE and out.dtype == q.dtype, "attention q/out dtype")
-        _need(nq % nkv == 0, f"{nq} query heads are not a multiple of {nkv} kv heads")
+        _need(nq % nkv == 0, lambda: f"{nq} query heads are not a multiple of {nkv} kv heads")
         _need(q.shape[1] >= nq * d and out.shape[1] >= nq * d, "attention q/out rows are too short")
         _need(k_pages.dtype == q.dtype and v_pages.dtype == q.dtype and k_pages.is_contiguous()
               and v_pages.is_contiguous() and k_pages.shape[1:] == (nkv, page_size, d)
@@ -381,7 +384,7 @@ class Kernels:
         lib = self.attention_lib(d)
         _rows_ok(qkv, "attention_decode qkv"); _rows_ok(out, "attention_decode out")
         _need(qkv.dtype in DTYPE_CODE and out.dtype == qkv.dtype, "attention_decode qkv/out dtype")
-        _need(nq % nkv == 0, f"{nq} query heads are not a multiple of {nkv} kv heads")
+        _need(nq % nkv == 0, lambda: f"{nq} query heads are not a multiple of {nkv} kv heads")
         heads = nq + 2 * nkv if write_kv else nq
         _need(qkv.shape[1] >= heads * d and out.shape[1] >= nq * d, "attention_decode rows are too short")
         _need(k_pages.dtype == qkv.dtype and v_pages.dtype == qkv.dtype and k_pages.is_contiguous()
