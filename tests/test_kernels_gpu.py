@@ -33,7 +33,9 @@ TOL = {torch.float32: 2e-5, torch.bfloat16: 1.5e-2}
                                    (130, 1000, 8), (3, 40, 12),
                                    # 128 x 128 tiles with rows, columns and K that end inside a tile (operand
                                    # loads from clamped addresses), and the same with K not 16-byte aligned
-                                   (2050, 2100, 264), (2050, 2100, 260)])
+                                   (2050, 2100, 264), (2050, 2100, 260),
+                                   # an odd K: no operand row is 16-byte aligned, in either precision
+                                   (200, 90, 101), (9, 50, 37)])
 def test_gemm_matches_linear(dtype, m, n, k):
     from lockstep_amd.ops import STORE, STORE_F32, ADD_F32
 
