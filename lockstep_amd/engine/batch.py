@@ -58,6 +58,7 @@ class Workspace:
     def __init__(self, device):
         self.device = device
         self._buffers: dict[tuple, torch.Tensor] = {}
+        self._views: dict[tuple, torch.Tensor] = {}     # (name, shape, dtype) -> the view of its buffer
         self.version = 0
         self.plan_templates: dict[tuple, tuple] = {}   # work lists of decode steps by shape
         self._stage = None                             # pinned host buffer of the metadata upload
@@ -78,6 +79,12 @@ class Workspace:
         return self._stage, self._stage_np, self._stage_done
 
     def get(self, name: str, shape, dtype) -> torch.Tensor:
+        # the views handed out are kept: a step asks for some two hundred buffers, mostly with the
+        # shapes of the step before, and making a view costs more than finding one
+        asked = (name, shape if type(shape) is tuple else tuple(shape), dtype)
+        view = self._views.get(asked)
+        if view is not None:
+            return view
         shape = tuple(int(s) for s in shape)
         rows, inner = shape[0], shape[1:]
         key = (name, inner, dtype)
@@ -87,7 +94,12 @@ class Workspace:
             have = torch.empty((grow, *inner), dtype=dtype, device=self.device)
             self._buffers[key] = have
             self.version += 1
-        return have[:rows]
+            self._views = {k: v for k, v in self._views.items() if (k[0], k[1][1:], k[2]) != key}
+        if len(self._views) > 4096:      # many step shapes have gone by: start again
+            self._views.clear()
+        view = have[:rows]
+        self._views[asked] = view
+        return view
 
 
 class StepContext:
