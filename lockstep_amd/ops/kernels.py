@@ -57,17 +57,12 @@ def _stream() -> c_void_p:
     return c_void_p(torch.cuda.current_stream().cuda_stream)
 
 
-def _need(cond: bool, message) -> None:
-    """``message``: the text, or a callable that makes it (so that a message with shapes in it is
-    formatted only when the check fails: these checks run before every launch)."""
-    if not cond:
-        raise KernelError(message() if callable(message) else message)
-
-
+# The checks in front of a launch are plain conditionals whose message is made only when a check
+# fails: a step runs some two thousand of them.
 def _rows_ok(t: torch.Tensor, name: str) -> None:
-    _need(t.is_cuda, lambda: f"{name} must live on the GPU")
-    _need(t.dim() == 2 and t.stride(1) == 1, lambda: f"{name} must be 2-D with contiguous rows, got shape "
-          f"{tuple(t.shape)} strides {t.stride()}")
+    if not (t.is_cuda and t.dim() == 2 and t.stride(1) == 1):
+        raise KernelError(f"{name} must be 2-D with contiguous rows on the GPU, got shape {tuple(t.shape)} "
+                          f"strides {t.stride()} on {t.device}")
 
 
 class Kernels:
@@ -94,7 +89,8 @@ class Kernels:
             path = _build.build_attention(head_dim)
             lib = ctypes.CDLL(str(path))
             lib.ls_last_error.restype = ctypes.c_char_p
-            _need(lib.ls_attn_head_dim() == head_dim, lambda: f"{path} was built for another head size")
+            if not (lib.ls_attn_head_dim() == head_dim):
+                raise KernelError(f"{path} was built for another head size")
             self._attention[head_dim] = lib
             self.attention_paths[head_dim] = str(path)
         return lib
@@ -146,25 +142,32 @@ class Kernels:
         ``norm_weight`` (float32 ``[K]``): ``x`` is the float32 residual stream and is
         RMS-normalised on the fly with this weight and ``eps`` (at most 16 rows)."""
         _rows_ok(x, "gemm x"); _rows_ok(w, "gemm w"); _rows_ok(out, "gemm out")
-        _need(w.dtype in DTYPE_CODE, lambda: f"gemm weights must be float32 or bfloat16, got {w.dtype}")
+        if not (w.dtype in DTYPE_CODE):
+            raise KernelError(f"gemm weights must be float32 or bfloat16, got {w.dtype}")
         if norm_weight is None:
-            _need(x.dtype == w.dtype, lambda: f"gemm operands must share a dtype, got {x.dtype} and {w.dtype}")
+            if not (x.dtype == w.dtype):
+                raise KernelError(f"gemm operands must share a dtype, got {x.dtype} and {w.dtype}")
         else:
-            _need(x.dtype == torch.float32 and x.shape[0] <= 16, "the fused norm reads at most 16 float32 rows")
-            _need(norm_weight.is_cuda and norm_weight.dtype == torch.float32 and norm_weight.is_contiguous()
-                  and norm_weight.shape == (x.shape[1],), lambda: f"norm weight must be float32 [{x.shape[1]}]")
+            if not (x.dtype == torch.float32 and x.shape[0] <= 16):
+                raise KernelError("the fused norm reads at most 16 float32 rows")
+            if not (norm_weight.is_cuda and norm_weight.dtype == torch.float32 and norm_weight.is_contiguous()
+                  and norm_weight.shape == (x.shape[1],)):
+                raise KernelError(f"norm weight must be float32 [{x.shape[1]}]")
         m, k = x.shape
         n = w.shape[0]
-        _need(w.shape[1] == k and w.is_contiguous(), lambda: f"gemm w must be contiguous [N,{k}], got {tuple(w.shape)}")
+        if not (w.shape[1] == k and w.is_contiguous()):
+            raise KernelError(f"gemm w must be contiguous [N,{k}], got {tuple(w.shape)}")
         if epilogue == SWIGLU:
             cols = out.shape[1]
-            _need(n % 32 == 0 and n // 2 - 16 < cols <= n // 2 and out.shape[0] == m,
-                  lambda: f"SwiGLU output [{m},{cols}] does not fit {n} interleaved weight rows")
+            if not (n % 32 == 0 and n // 2 - 16 < cols <= n // 2 and out.shape[0] == m):
+                raise KernelError(f"SwiGLU output [{m},{cols}] does not fit {n} interleaved weight rows")
         else:
             cols = n
-            _need(tuple(out.shape) == (m, n), lambda: f"gemm out must be [{m},{n}], got {tuple(out.shape)}")
+            if not (tuple(out.shape) == (m, n)):
+                raise KernelError(f"gemm out must be [{m},{n}], got {tuple(out.shape)}")
         want = w.dtype if epilogue in (STORE, SWIGLU) else torch.float32
-        _need(out.dtype == want, lambda: f"gemm out dtype {out.dtype} does not fit epilogue {epilogue}")
+        if not (out.dtype == want):
+            raise KernelError(f"gemm out dtype {out.dtype} does not fit epilogue {epilogue}")
         if m == 0:
             return
         code = self.core.ls_gemm(c_int(DTYPE_CODE[w.dtype]), c_int(epilogue), _ptr(x), _ptr(w), _ptr(out),
@@ -182,11 +185,12 @@ class Kernels:
         _rows_ok(x, "gemm_slices x")
         m, k = x.shape
         n = w.shape[0]
-        _need(w.is_cuda and w.dim() == 2 and w.is_contiguous() and w.shape[1] == k and w.dtype == x.dtype
-              and w.dtype in DTYPE_CODE, "gemm_slices w must be [N, K] contiguous in the dtype of x")
-        _need(partials.is_cuda and partials.dtype == torch.float32 and partials.is_contiguous()
-              and partials.shape == (self.gemm_slices_count(k), m, n),
-              lambda: f"gemm_slices partials must be float32 [{self.gemm_slices_count(k)}, {m}, {n}]")
+        if not (w.is_cuda and w.dim() == 2 and w.is_contiguous() and w.shape[1] == k and w.dtype == x.dtype
+              and w.dtype in DTYPE_CODE):
+            raise KernelError("gemm_slices w must be [N, K] contiguous in the dtype of x")
+        if not (partials.is_cuda and partials.dtype == torch.float32 and partials.is_contiguous()
+              and partials.shape == (self.gemm_slices_count(k), m, n)):
+            raise KernelError(f"gemm_slices partials must be float32 [{self.gemm_slices_count(k)}, {m}, {n}]")
         code = self.core.ls_gemm_slices(c_int(DTYPE_CODE[w.dtype]), _ptr(x), _ptr(w), _ptr(partials), c_int(m),
                                         c_int(n), c_int(k), c_long(x.stride(0)), _stream())
         self._check(self.core, code)
@@ -196,19 +200,24 @@ class Kernels:
         """``h[row] += partials[0][row] + partials[1][row] + ...``; then, unless ``out`` is None,
         ``out = rmsnorm(h[row]) * weight`` as ``rmsnorm`` computes it.  ``rows`` selects rows of ``h``."""
         _rows_ok(h, "add_rmsnorm h")
-        _need(h.dtype == torch.float32, "add_rmsnorm works on the float32 residual stream")
-        _need(partials.is_cuda and partials.dtype == torch.float32 and partials.is_contiguous()
-              and partials.dim() == 3 and partials.shape[2] == h.shape[1], "add_rmsnorm partials [slices, rows, width]")
+        if not (h.dtype == torch.float32):
+            raise KernelError("add_rmsnorm works on the float32 residual stream")
+        if not (partials.is_cuda and partials.dtype == torch.float32 and partials.is_contiguous()
+              and partials.dim() == 3 and partials.shape[2] == h.shape[1]):
+            raise KernelError("add_rmsnorm partials [slices, rows, width]")
         n_rows = h.shape[0] if rows is None else rows.shape[0]
         if rows is not None:
-            _need(rows.is_cuda and rows.dtype == torch.int32 and rows.is_contiguous(), "add_rmsnorm rows: int32 on the GPU")
+            if not (rows.is_cuda and rows.dtype == torch.int32 and rows.is_contiguous()):
+                raise KernelError("add_rmsnorm rows: int32 on the GPU")
         dtype = torch.float32
         ld_out = 0
         if out is not None:
             _rows_ok(out, "add_rmsnorm out")
-            _need(out.dtype in DTYPE_CODE and out.shape == (n_rows, h.shape[1]), "add_rmsnorm out shape or dtype")
-            _need(weight is not None and weight.dtype == torch.float32 and weight.is_contiguous()
-                  and weight.numel() == h.shape[1], "add_rmsnorm weight must be float32 [width]")
+            if not (out.dtype in DTYPE_CODE and out.shape == (n_rows, h.shape[1])):
+                raise KernelError("add_rmsnorm out shape or dtype")
+            if not (weight is not None and weight.dtype == torch.float32 and weight.is_contiguous()
+                  and weight.numel() == h.shape[1]):
+                raise KernelError("add_rmsnorm weight must be float32 [width]")
             dtype, ld_out = out.dtype, out.stride(0)
         if n_rows == 0:
             return
@@ -219,12 +228,13 @@ class Kernels:
 
     # -- rows -------------------------------------------------------------------
     def embed(self, tokens: torch.Tensor, table: torch.Tensor, out: torch.Tensor) -> None:
-        _need(tokens.is_cuda and tokens.dtype == torch.int32 and tokens.dim() == 1 and tokens.is_contiguous(),
-              "embed tokens must be a contiguous int32 vector on the GPU")
+        if not (tokens.is_cuda and tokens.dtype == torch.int32 and tokens.dim() == 1 and tokens.is_contiguous()):
+            raise KernelError("embed tokens must be a contiguous int32 vector on the GPU")
         _rows_ok(table, "embed table"); _rows_ok(out, "embed out")
-        _need(table.is_contiguous() and table.dtype in DTYPE_CODE, "embed table must be contiguous float32/bfloat16")
-        _need(out.dtype == torch.float32 and out.shape == (tokens.shape[0], table.shape[1]),
-              lambda: f"embed out must be float32 [{tokens.shape[0]},{table.shape[1]}]")
+        if not (table.is_contiguous() and table.dtype in DTYPE_CODE):
+            raise KernelError("embed table must be contiguous float32/bfloat16")
+        if not (out.dtype == torch.float32 and out.shape == (tokens.shape[0], table.shape[1])):
+            raise KernelError(f"embed out must be float32 [{tokens.shape[0]},{table.shape[1]}]")
         if tokens.shape[0] == 0:
             return
         code = self.core.ls_embed(c_int(DTYPE_CODE[table.dtype]), _ptr(tokens), _ptr(table), _ptr(out),
@@ -236,16 +246,20 @@ class Kernels:
                 rows: torch.Tensor | None = None) -> None:
         """Rows of float ``x`` (all, or those listed in ``rows``) normalised into ``out``."""
         _rows_ok(x, "rmsnorm x"); _rows_ok(out, "rmsnorm out")
-        _need(x.dtype == torch.float32, "rmsnorm reads the float32 residual stream")
-        _need(weight.is_cuda and weight.dtype == torch.float32 and weight.is_contiguous()
-              and weight.shape == (x.shape[1],), lambda: f"rmsnorm weight must be float32 [{x.shape[1]}]")
-        _need(out.dtype in DTYPE_CODE and out.shape[1] == x.shape[1], "rmsnorm out has the wrong width or dtype")
+        if not (x.dtype == torch.float32):
+            raise KernelError("rmsnorm reads the float32 residual stream")
+        if not (weight.is_cuda and weight.dtype == torch.float32 and weight.is_contiguous()
+              and weight.shape == (x.shape[1],)):
+            raise KernelError(f"rmsnorm weight must be float32 [{x.shape[1]}]")
+        if not (out.dtype in DTYPE_CODE and out.shape[1] == x.shape[1]):
+            raise KernelError("rmsnorm out has the wrong width or dtype")
         n = out.shape[0]
         if rows is not None:
-            _need(rows.is_cuda and rows.dtype == torch.int32 and rows.is_contiguous() and rows.shape == (n,),
-                  lambda: f"rmsnorm rows must be int32 [{n}]")
+            if not (rows.is_cuda and rows.dtype == torch.int32 and rows.is_contiguous() and rows.shape == (n,)):
+                raise KernelError(f"rmsnorm rows must be int32 [{n}]")
         else:
-            _need(x.shape[0] == n, "rmsnorm out must have as many rows as x")
+            if not (x.shape[0] == n):
+                raise KernelError("rmsnorm out must have as many rows as x")
         if n == 0:
             return
         code = self.core.ls_rmsnorm(c_int(DTYPE_CODE[out.dtype]), _ptr(x), _ptr(weight), _ptr(out), _ptr(rows),
@@ -256,8 +270,8 @@ class Kernels:
     def swiglu(self, gate_up: torch.Tensor, out: torch.Tensor) -> None:
         _rows_ok(gate_up, "swiglu input"); _rows_ok(out, "swiglu out")
         rows, inter = out.shape
-        _need(gate_up.shape == (rows, 2 * inter) and gate_up.dtype == out.dtype and out.dtype in DTYPE_CODE,
-              lambda: f"swiglu input must be [{rows},{2 * inter}] of the output's dtype")
+        if not (gate_up.shape == (rows, 2 * inter) and gate_up.dtype == out.dtype and out.dtype in DTYPE_CODE):
+            raise KernelError(f"swiglu input must be [{rows},{2 * inter}] of the output's dtype")
         if rows == 0:
             return
         code = self.core.ls_swiglu(c_int(DTYPE_CODE[out.dtype]), _ptr(gate_up), _ptr(out), c_int(rows), c_int(inter),
@@ -266,9 +280,10 @@ class Kernels:
 
     def argmax(self, logits: torch.Tensor, out: torch.Tensor) -> None:
         _rows_ok(logits, "argmax logits")
-        _need(logits.dtype == torch.float32, "argmax reads float32 logits")
-        _need(out.is_cuda and out.dtype == torch.int32 and out.is_contiguous() and out.shape == (logits.shape[0],),
-              lambda: f"argmax out must be int32 [{logits.shape[0]}]")
+        if not (logits.dtype == torch.float32):
+            raise KernelError("argmax reads float32 logits")
+        if not (out.is_cuda and out.dtype == torch.int32 and out.is_contiguous() and out.shape == (logits.shape[0],)):
+            raise KernelError(f"argmax out must be int32 [{logits.shape[0]}]")
         if logits.shape[0] == 0:
             return
         words = 2 * logits.shape[0] * self.core.ls_argmax_chunks(c_int(logits.shape[1]))
@@ -287,12 +302,15 @@ class Kernels:
         tokens are appended to ``ring[counter]``.  ``lists``: (offset, count) of the attention
         work-item lists inside ``meta`` (16 ints an item)."""
         for t in (meta, picked, ring, counter):
-            _need(t.is_cuda and t.dtype == torch.int32 and t.is_contiguous(), "advance_decode works on int32 GPU tensors")
-        _need(picked.numel() >= n_seqs and len(lists) <= 4, "advance_decode: picked too short or more than four lists")
+            if not (t.is_cuda and t.dtype == torch.int32 and t.is_contiguous()):
+                raise KernelError("advance_decode works on int32 GPU tensors")
+        if not (picked.numel() >= n_seqs and len(lists) <= 4):
+            raise KernelError("advance_decode: picked too short or more than four lists")
         offsets = (ctypes.c_int * 4)(*([o for o, _ in lists] + [0] * (4 - len(lists))))
         counts = (ctypes.c_int * 4)(*([c for _, c in lists] + [0] * (4 - len(lists))))
         for o, c in lists:
-            _need(0 <= o and o + 16 * c <= meta.numel(), "advance_decode: an item list lies outside the metadata")
+            if not (0 <= o and o + 16 * c <= meta.numel()):
+                raise KernelError("advance_decode: an item list lies outside the metadata")
         code = self.core.ls_advance_decode(_ptr(meta), c_int(n_seqs), c_int(off_tokens), c_int(off_positions),
                                            c_int(off_seqs), _ptr(picked), _ptr(ring), _ptr(counter), offsets, counts,
                                            c_int(len(lists)), _stream())
@@ -308,35 +326,40 @@ class Kernels:
         tables); ``table`` is the group's block table ``[rows, stride]``.
         """
         _rows_ok(qkv, "qkv")
-        _need(qkv.dtype in DTYPE_CODE and qkv.shape[0] >= n_tokens, "qkv has too few rows or a wrong dtype")
+        if not (qkv.dtype in DTYPE_CODE and qkv.shape[0] >= n_tokens):
+            raise KernelError("qkv has too few rows or a wrong dtype")
         heads = nq + 2 * nkv if write_kv else nq
-        _need(qkv.shape[1] >= heads * d, lambda: f"qkv rows hold {qkv.shape[1]} values, {heads} heads of {d} are needed")
-        _need(d <= MAX_HEAD_DIM, lambda: f"head size {d} exceeds the supported maximum {MAX_HEAD_DIM}")
+        if not (qkv.shape[1] >= heads * d):
+            raise KernelError(f"qkv rows hold {qkv.shape[1]} values, {heads} heads of {d} are needed")
+        if not (d <= MAX_HEAD_DIM):
+            raise KernelError(f"head size {d} exceeds the supported maximum {MAX_HEAD_DIM}")
         for name, w in (("q norm weight", q_weight), ("k norm weight", k_weight)):
             if w is not None:
-                _need(w.is_cuda and w.dtype == torch.float32 and w.is_contiguous() and w.shape == (d,),
-                      lambda: f"{name} must be float32 [{d}]")
+                if not (w.is_cuda and w.dtype == torch.float32 and w.is_contiguous() and w.shape == (d,)):
+                    raise KernelError(f"{name} must be float32 [{d}]")
         positions = 0
         if cos is not None:
-            _need(sin is not None and cos.shape == sin.shape and cos.dim() == 2 and cos.shape[1] * 2 == rot
-                  and cos.dtype == torch.float32 and cos.is_contiguous() and sin.is_contiguous() and cos.is_cuda,
-                  "rotation tables must be float32 [positions, rotary_dim/2]")
+            if not (sin is not None and cos.shape == sin.shape and cos.dim() == 2 and cos.shape[1] * 2 == rot
+                  and cos.dtype == torch.float32 and cos.is_contiguous() and sin.is_contiguous() and cos.is_cuda):
+                raise KernelError("rotation tables must be float32 [positions, rotary_dim/2]")
             positions = cos.shape[0]
-            _need(max_pos < positions, lambda: f"position {max_pos} is beyond the rotation tables ({positions})")
+            if not (max_pos < positions):
+                raise KernelError(f"position {max_pos} is beyond the rotation tables ({positions})")
         for name, t in (("tok_seq", tok_seq), ("tok_pos", tok_pos)):
-            _need(t.is_cuda and t.dtype == torch.int32 and t.is_contiguous() and t.numel() >= n_tokens,
-                  lambda: f"{name} must be int32 with at least {n_tokens} entries")
+            if not (t.is_cuda and t.dtype == torch.int32 and t.is_contiguous() and t.numel() >= n_tokens):
+                raise KernelError(f"{name} must be int32 with at least {n_tokens} entries")
         if write_kv:
-            _need(table is not None and table.is_cuda and table.dtype == torch.int32 and table.dim() == 2
-                  and table.is_contiguous(), "block table must be a contiguous int32 matrix")
-            _need(max_pos // page_size < table.shape[1],
-                  lambda: f"position {max_pos} needs page {max_pos // page_size}, the block table has {table.shape[1]} columns")
+            if not (table is not None and table.is_cuda and table.dtype == torch.int32 and table.dim() == 2
+                  and table.is_contiguous()):
+                raise KernelError("block table must be a contiguous int32 matrix")
+            if not (max_pos // page_size < table.shape[1]):
+                raise KernelError(f"position {max_pos} needs page {max_pos // page_size}, the block table has {table.shape[1]} columns")
             for name, pages in (("key pages", k_pages), ("value pages", v_pages)):
-                _need(pages.is_cuda and pages.dtype == qkv.dtype and pages.is_contiguous() and pages.dim() == 4,
-                      lambda: f"{name} must be contiguous 4-D of the compute dtype")
-            _need(k_pages.shape[1:] == (nkv, page_size, d) and v_pages.shape[1:] == (nkv, d, page_size)
-                  and k_pages.shape[0] == v_pages.shape[0],
-                  lambda: f"cache pages do not have the layout [pages,{nkv},{page_size},{d}] / [pages,{nkv},{d},{page_size}]")
+                if not (pages.is_cuda and pages.dtype == qkv.dtype and pages.is_contiguous() and pages.dim() == 4):
+                    raise KernelError(f"{name} must be contiguous 4-D of the compute dtype")
+            if not (k_pages.shape[1:] == (nkv, page_size, d) and v_pages.shape[1:] == (nkv, d, page_size)
+                  and k_pages.shape[0] == v_pages.shape[0]):
+                raise KernelError(f"cache pages do not have the layout [pages,{nkv},{page_size},{d}] / [pages,{nkv},{d},{page_size}]")
         if n_tokens == 0:
             return
         code = self.core.ls_qk_rope_kv(
@@ -357,15 +380,20 @@ class Kernels:
         with half the rows a block (for steps with few rows)."""
         lib = self.attention_lib(d)
         _rows_ok(q, "attention q"); _rows_ok(out, "attention out")
-        _need(q.dtype in DTYPE_CODE and out.dtype == q.dtype, "attention q/out dtype")
-        _need(nq % nkv == 0, lambda: f"{nq} query heads are not a multiple of {nkv} kv heads")
-        _need(q.shape[1] >= nq * d and out.shape[1] >= nq * d, "attention q/out rows are too short")
-        _need(k_pages.dtype == q.dtype and v_pages.dtype == q.dtype and k_pages.is_contiguous()
+        if not (q.dtype in DTYPE_CODE and out.dtype == q.dtype):
+            raise KernelError("attention q/out dtype")
+        if not (nq % nkv == 0):
+            raise KernelError(f"{nq} query heads are not a multiple of {nkv} kv heads")
+        if not (q.shape[1] >= nq * d and out.shape[1] >= nq * d):
+            raise KernelError("attention q/out rows are too short")
+        if not (k_pages.dtype == q.dtype and v_pages.dtype == q.dtype and k_pages.is_contiguous()
               and v_pages.is_contiguous() and k_pages.shape[1:] == (nkv, page_size, d)
-              and v_pages.shape[1:] == (nkv, d, page_size), "attention cache pages have the wrong layout or dtype")
-        _need(table.dtype == torch.int32 and table.dim() == 2 and table.is_contiguous(), "attention block table")
-        _need(items.dtype == torch.int32 and items.is_contiguous() and items.numel() >= ATTENTION_ITEM_INTS * n_items,
-              "attention items must hold 16 int32 each (see pack_attention_items)")
+              and v_pages.shape[1:] == (nkv, d, page_size)):
+            raise KernelError("attention cache pages have the wrong layout or dtype")
+        if not (table.dtype == torch.int32 and table.dim() == 2 and table.is_contiguous()):
+            raise KernelError("attention block table")
+        if not (items.dtype == torch.int32 and items.is_contiguous() and items.numel() >= ATTENTION_ITEM_INTS * n_items):
+            raise KernelError("attention items must hold 16 int32 each (see pack_attention_items)")
         if n_items == 0:
             return
         code = lib.ls_attention(
@@ -383,24 +411,30 @@ class Kernels:
         in one launch.  ``qkv`` is the raw fused projection; every request brings exactly one token."""
         lib = self.attention_lib(d)
         _rows_ok(qkv, "attention_decode qkv"); _rows_ok(out, "attention_decode out")
-        _need(qkv.dtype in DTYPE_CODE and out.dtype == qkv.dtype, "attention_decode qkv/out dtype")
-        _need(nq % nkv == 0, lambda: f"{nq} query heads are not a multiple of {nkv} kv heads")
+        if not (qkv.dtype in DTYPE_CODE and out.dtype == qkv.dtype):
+            raise KernelError("attention_decode qkv/out dtype")
+        if not (nq % nkv == 0):
+            raise KernelError(f"{nq} query heads are not a multiple of {nkv} kv heads")
         heads = nq + 2 * nkv if write_kv else nq
-        _need(qkv.shape[1] >= heads * d and out.shape[1] >= nq * d, "attention_decode rows are too short")
-        _need(k_pages.dtype == qkv.dtype and v_pages.dtype == qkv.dtype and k_pages.is_contiguous()
+        if not (qkv.shape[1] >= heads * d and out.shape[1] >= nq * d):
+            raise KernelError("attention_decode rows are too short")
+        if not (k_pages.dtype == qkv.dtype and v_pages.dtype == qkv.dtype and k_pages.is_contiguous()
               and v_pages.is_contiguous() and k_pages.shape[1:] == (nkv, page_size, d)
-              and v_pages.shape[1:] == (nkv, d, page_size), "attention cache pages have the wrong layout or dtype")
-        _need(table.dtype == torch.int32 and table.dim() == 2 and table.is_contiguous(), "attention block table")
-        _need(items.dtype == torch.int32 and items.is_contiguous() and items.numel() >= ATTENTION_ITEM_INTS * n_items,
-              "attention items must hold 16 int32 each (see pack_attention_items)")
+              and v_pages.shape[1:] == (nkv, d, page_size)):
+            raise KernelError("attention cache pages have the wrong layout or dtype")
+        if not (table.dtype == torch.int32 and table.dim() == 2 and table.is_contiguous()):
+            raise KernelError("attention block table")
+        if not (items.dtype == torch.int32 and items.is_contiguous() and items.numel() >= ATTENTION_ITEM_INTS * n_items):
+            raise KernelError("attention items must hold 16 int32 each (see pack_attention_items)")
         for w in (q_weight, k_weight):
-            _need(w is None or (w.dtype == torch.float32 and w.is_contiguous() and w.numel() == d),
-                  "per-head norm weights must be float32 [head_dim]")
+            if not (w is None or (w.dtype == torch.float32 and w.is_contiguous() and w.numel() == d)):
+                raise KernelError("per-head norm weights must be float32 [head_dim]")
         positions = 0
         if cos is not None:
-            _need(sin is not None and cos.dtype == torch.float32 and sin.dtype == torch.float32
+            if not (sin is not None and cos.dtype == torch.float32 and sin.dtype == torch.float32
                   and cos.is_contiguous() and sin.is_contiguous() and cos.shape == sin.shape
-                  and cos.shape[1] == rot // 2, "rotation tables must be float32 [positions, rot/2]")
+                  and cos.shape[1] == rot // 2):
+                raise KernelError("rotation tables must be float32 [positions, rot/2]")
             positions = cos.shape[0]
         if n_items == 0:
             return
@@ -416,9 +450,10 @@ class Kernels:
                           out: torch.Tensor) -> None:
         lib = self.attention_lib(d)
         _rows_ok(out, "combine out")
-        _need(out.dtype in DTYPE_CODE and out.shape[1] >= nq * d, "combine out rows are too short")
-        _need(items.dtype == torch.int32 and items.is_contiguous() and items.numel() >= COMBINE_ITEM_INTS * n_items,
-              "combine items must hold 8 int32 each (see pack_combine_items)")
+        if not (out.dtype in DTYPE_CODE and out.shape[1] >= nq * d):
+            raise KernelError("combine out rows are too short")
+        if not (items.dtype == torch.int32 and items.is_contiguous() and items.numel() >= COMBINE_ITEM_INTS * n_items):
+            raise KernelError("combine items must hold 8 int32 each (see pack_combine_items)")
         if n_items == 0:
             return
         code = lib.ls_attention_combine(c_int(DTYPE_CODE[out.dtype]), _ptr(seqs), _ptr(items), c_int(n_items),
