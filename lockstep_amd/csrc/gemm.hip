@@ -959,12 +959,21 @@ extern "C" int ls_gemm_slices_count(int K) {
   return (K + kslice - 1) / kslice;
 }
 
-// Slice sums of X [M,K] @ W [N,K]^T for M <= 64: P [slices][M][N] float, P[s] = the sum over K slice s.
-// The product is P[0] + P[1] + ... added in this order, starting from +0.
+// Rows that ls_gemm_slices takes for a product over K: 64 always; 256 where the kernel that keeps
+// its rows of X in registers has an instance for the slice length (more rows are further groups of
+// workgroups that walk the same weights).
+extern "C" int ls_gemm_slices_max_rows(int dtype, int K) {
+  const int xc = ls::kslice_for(K) / (dtype == ls::kF32 ? 16 : 32);
+  return (LS_GEMM_STREAM && (xc == 8 || xc == 16)) ? 256 : 64;
+}
+
+// Slice sums of X [M,K] @ W [N,K]^T for M <= ls_gemm_slices_max_rows: P [slices][M][N] float, P[s] = the
+// sum over K slice s.  The product is P[0] + P[1] + ... added in this order, starting from +0.
 extern "C" int ls_gemm_slices(int dtype, const void* X, const void* W, float* P, int M, int N, int K, long ldx,
                               void* stream) {
   using namespace ls;
-  LS_REQUIRE(M > 0 && M <= 64 && N > 0 && K > 0, "gemm_slices: takes 1 to 64 rows, got M=%d N=%d K=%d", M, N, K);
+  LS_REQUIRE(M > 0 && M <= ls_gemm_slices_max_rows(dtype, K) && N > 0 && K > 0,
+             "gemm_slices: takes 1 to %d rows with K=%d, got M=%d N=%d", ls_gemm_slices_max_rows(dtype, K), K, M, N);
   LS_REQUIRE(ldx >= K && X && W && P, "gemm_slices: bad operands");
   LS_REQUIRE(reinterpret_cast<uintptr_t>(P) % 16 == 0, "gemm_slices: the partial sums must be 16-byte aligned");
   const int kslice = kslice_for(K);
@@ -990,9 +999,10 @@ extern "C" int ls_gemm_slices(int dtype, const void* X, const void* W, float* P,
   // (24 chunks a slice with two tiles need 268 registers: one wave a SIMD, measured slower than the plain kernel)
   const int group_tiles = xc <= 8 ? std::min(mt, 4) : (xc <= 16 ? std::min(mt, 2) : 0);
   const int row_groups = group_tiles > 0 ? (mt + group_tiles - 1) / group_tiles : 0;
-  const int rounds =
+  int rounds =
       (int)std::min<long>(4, (long)col_blocks * groups * std::max(row_groups, 1) / (2L * compute_units()));
-  if (rounds >= 2 && mt >= 2 && group_tiles > 0 && xc % 4 == 0 && LS_GEMM_STREAM) {
+  if (mt > 4 && rounds < 1) rounds = 1;  // more than 64 rows: this kernel only, if with one column block a workgroup
+  if ((rounds >= 2 || mt > 4) && mt >= 2 && group_tiles > 0 && xc % 4 == 0 && LS_GEMM_STREAM) {
     int walkers = (col_blocks + rounds - 1) / rounds;
     if (row_groups > 1) walkers = (walkers + 7) / 8 * 8;  // the groups' workgroups of a walk sit on the same XCD
     dim3 walk_grid(walkers, groups, row_groups);
@@ -1011,6 +1021,7 @@ extern "C" int ls_gemm_slices(int dtype, const void* X, const void* W, float* P,
 #undef LS_WALK
     if (launched) return check_launch("gemm_slices");
   }
+  LS_REQUIRE(mt <= 4, "gemm_slices: no kernel for %d rows with K=%d", M, K);
 #define LS_SLICES(T_, MT_)                                                                                       \
   hipLaunchKernelGGL((gemm_slices_kernel<T_, MT_>), grid, dim3(64 * per_group), 0, s, (const T_*)X, (const T_*)W, P, M, \
                      N, K, ldx, kslice, aligned, per_group)

@@ -179,9 +179,16 @@ class Kernels:
         """K slices of a product over ``k`` (first dimension of ``gemm_slices``'s output)."""
         return self._memo(("slices", k), lambda: int(self.core.ls_gemm_slices_count(c_int(k))))
 
+    def gemm_slices_max_rows(self, k: int, dtype: torch.dtype) -> int:
+        """Most rows ``gemm_slices`` takes for a product over ``k``: 64, or 256 where the kernel that walks
+        the column blocks with its rows in registers has an instance for the slice length."""
+        return self._memo(("slices_rows", k, dtype),
+                          lambda: int(self.core.ls_gemm_slices_max_rows(c_int(DTYPE_CODE[dtype]), c_int(k))))
+
     def gemm_slices(self, x: torch.Tensor, w: torch.Tensor, partials: torch.Tensor) -> None:
-        """Slice sums of ``x @ w.T`` for at most 64 rows: ``partials [slices, M, N]`` float32, to be added
-        in ascending order by the consumer (``add_rmsnorm``).  The work is cut over K as well as over N."""
+        """Slice sums of ``x @ w.T`` for at most ``gemm_slices_max_rows`` rows: ``partials [slices, M, N]``
+        float32, to be added in ascending order by the consumer (``add_rmsnorm``).  The work is cut over K
+        as well as over N."""
         _rows_ok(x, "gemm_slices x")
         m, k = x.shape
         n = w.shape[0]

@@ -19,7 +19,7 @@ import torch
 
 from ..config.base import PartSpec
 from ..ops import ADD_F32, STORE_F32
-from .base import DEFER_ADD_ROWS, Mixer, PagedKVSpec, PendingAdd, WeightSpec, build_part, register_part
+from .base import Mixer, PagedKVSpec, PendingAdd, WeightSpec, build_part, deferred_rows, register_part
 
 import os
 
@@ -165,7 +165,7 @@ class Attention(Mixer):
 
     def _project_out(self, ctx, attn, out, accumulate: bool, defer: bool):
         k = ctx.rt.kernels
-        if defer and accumulate and 0 < ctx.n_tokens <= DEFER_ADD_ROWS:
+        if defer and accumulate and 0 < ctx.n_tokens <= deferred_rows(ctx, self.nq * self.d, out.shape[1]):
             slices = k.gemm_slices_count(self.nq * self.d)
             partials = ctx.buf("attention.out_slices", (slices * ctx.n_tokens, out.shape[1]), torch.float32)
             partials = partials.view(slices, ctx.n_tokens, out.shape[1])

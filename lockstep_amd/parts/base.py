@@ -221,8 +221,24 @@ class PendingAdd:
 
 
 #: steps of at most this many tokens leave the residual additions of the output products to the
-#: following norm (their work is then cut over K as well, which fills the GPU); 0 switches it off
-DEFER_ADD_ROWS = int(__import__("os").environ.get("LOCKSTEP_DEFER_ADD_ROWS", "64"))
+#: following norm (their work is then cut over K as well, which fills the GPU); 0 switches it off.
+#: Up to 64 rows every product is left so; beyond, up to this bound, a product whose slice length
+#: has a many-row kernel and whose slice sums stay small (``deferred_rows``).
+DEFER_ADD_ROWS = int(__import__("os").environ.get("LOCKSTEP_DEFER_ADD_ROWS", "256"))
+
+#: slices x output width up to which more than 64 rows are left as slice sums: the sums are that
+#: many floats a row, written and read once, which beyond this outweighs what cutting K gains
+#: (measured: 8 to 12 slices of 1,024 columns gain, 16 slices of 4,096 columns lose)
+DEFER_MANY_ROWS_SUMS = 16384
+
+
+def deferred_rows(ctx, k: int, n: int) -> int:
+    """The most tokens of a step for which a product over ``k`` with ``n`` outputs is left as
+    K-slice sums."""
+    kernels = ctx.rt.kernels
+    if kernels.gemm_slices_count(k) * n > DEFER_MANY_ROWS_SUMS:
+        return min(DEFER_ADD_ROWS, 64)
+    return min(DEFER_ADD_ROWS, kernels.gemm_slices_max_rows(k, ctx.rt.dtype))
 
 
 def graph_safe_tree(part: Part) -> bool:

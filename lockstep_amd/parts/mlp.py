@@ -11,7 +11,7 @@ import torch
 
 from ..config.base import PartSpec
 from ..ops import ADD_F32, STORE_F32, SWIGLU, interleave_gate_up
-from .base import DEFER_ADD_ROWS, FeedForward, PendingAdd, WeightSpec, register_part
+from .base import FeedForward, PendingAdd, WeightSpec, deferred_rows, register_part
 
 
 @register_part("gated_mlp")
@@ -53,7 +53,7 @@ class GatedMLP(FeedForward):
             rt.kernels.gemm(x, self.w_gate_up, act, SWIGLU)
         else:
             rt.kernels.gemm(x, self.w_gate_up, act, SWIGLU, norm_weight=norm.weight, eps=norm.eps)
-        if defer and accumulate and 0 < ctx.n_tokens <= DEFER_ADD_ROWS:
+        if defer and accumulate and 0 < ctx.n_tokens <= deferred_rows(ctx, self.inter, out.shape[1]):
             slices = rt.kernels.gemm_slices_count(self.inter)
             partials = ctx.buf("mlp.down_slices", (slices * ctx.n_tokens, out.shape[1]), torch.float32)
             partials = partials.view(slices, ctx.n_tokens, out.shape[1])

@@ -657,16 +657,25 @@ def test_gemm_with_fused_norm_equals_norm_then_gemm(dtype, m, n, k):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("m", [1, 8, 16, 17, 40, 64])
+@pytest.mark.parametrize("m", [1, 8, 16, 17, 40, 64, 65, 100, 200, 256])
 @pytest.mark.parametrize("n,k", [(1024, 3072), (96, 520), (1024, 2048), (40, 64), (4096, 1024), (5120, 96),
                                  (1028, 4096), (16384, 64), (16388, 64),
                                  # enough column blocks and slices that workgroups walk several blocks
                                  (4104, 4096), (4104, 12288), (4200, 8192), (8200, 2048)])
 def test_slice_sums_and_fused_add_norm_equal_the_separate_kernels(dtype, m, n, k):
     """gemm_slices + add_rmsnorm give the bits of gemm(ADD_F32) + rmsnorm: the residual row and the
-    normalised row; also for a list of rows and for the plain addition."""
+    normalised row; also for a list of rows and for the plain addition.  More than 64 rows (several
+    groups of rows walking the same weights) where the slice length has such a kernel; elsewhere the
+    product says so."""
     from lockstep_amd.ops import ADD_F32
 
+    most = K().gemm_slices_max_rows(k, dtype)
+    assert most in (64, 256) and (most == 256) == (k <= (8192 if dtype is torch.bfloat16 else 4096))
+    if m > most:
+        with pytest.raises(RuntimeError, match="gemm_slices"):
+            K().gemm_slices(torch.zeros(m, k, dtype=dtype, device="cuda"), torch.zeros(n, k, dtype=dtype, device="cuda"),
+                            torch.zeros(K().gemm_slices_count(k), m, n, device="cuda"))
+        return
     g = torch.Generator().manual_seed(n + k + m)
     x = torch.randn(m, k, generator=g).to(dtype).cuda()
     w = (torch.randn(n, k, generator=g) * 0.1).to(dtype).cuda()
