@@ -161,3 +161,20 @@ def test_sharded_checkpoints_are_read_through_their_index(tmp_path):
     (tmp_path / "model.safetensors.index.json").write_text(json.dumps(index))
     store = load_weights(tmp_path, collect_weight_specs(spec), collect_ties(spec))
     assert torch.equal(store.get(names[-1]), tensors[names[-1]])
+
+
+def test_graph_safety_is_asked_of_every_part_of_a_layer():
+    """A layer may run inside a captured graph only if the arrangement, its mixer (and the mixer's
+    position encoding), its feed-forward and its norms all say so."""
+    from lockstep_amd.config.presets import preset
+    from lockstep_amd.parts import part_class
+    from lockstep_amd.parts.base import graph_safe_tree
+
+    spec = preset("tiny-a").model_spec()
+    layer = part_class(spec.layers[0].arrangement.kind)(spec.layers[0])
+    assert graph_safe_tree(layer)
+    for part in (layer.feed_forward, layer.mixer.position, layer.mixer_norm):
+        part.graph_safe = False          # on the instance: the class keeps its value
+        assert not graph_safe_tree(layer)
+        del part.graph_safe
+    assert graph_safe_tree(layer)
