@@ -5,7 +5,10 @@
 // a matrix product is in the compute dtype T (float or bfloat16).  All
 // reductions are per row with an order fixed by the row's width alone.
 
+#include <mutex>
+
 #include "common.h"
+#include "core_api.h"
 
 namespace ls {
 
@@ -590,6 +593,59 @@ extern "C" int ls_argmax(const float* x, int* out, int rows, int width, long ld,
                      chunks);
   if (chunks > 1) hipLaunchKernelGGL(argmax_final_kernel, dim3(rows), dim3(256), 0, s, part_v, part_i, out, chunks);
   return check_launch("argmax");
+}
+
+// ---------------------------------------------------------------------------
+// Arg-max for callers that cannot allocate (see core_api.h).  The chunks'
+// winners go to `argmax_scratch`, an array in the library's device image:
+// values in the first LS_ARGMAX_STATIC_PAIRS words, indices in the second.
+// In host code the array's name is only a stand-in for the symbol; the
+// address of each GPU's own copy is asked from the runtime once per device
+// (g_argmax_scratch_ptr) and only that pointer is handed to kernels.
+// ---------------------------------------------------------------------------
+static __device__ __align__(256) unsigned int argmax_scratch[2 * LS_ARGMAX_STATIC_PAIRS];
+
+namespace ls {
+constexpr int kMaxDevices = 64;
+static void* g_argmax_scratch_ptr[kMaxDevices] = {nullptr};
+static std::mutex g_argmax_scratch_mutex;
+
+// The current device's copy of argmax_scratch; looked up at the first call on that device.
+static int argmax_scratch_of_current_device(void** out) {
+  int device = -1;
+  hipError_t e = hipGetDevice(&device);
+  if (e != hipSuccess) return fail("argmax_static: hipGetDevice: %s", hipGetErrorString(e));
+  if (device < 0 || device >= kMaxDevices) return fail("argmax_static: device %d is outside [0, %d)", device, kMaxDevices);
+  std::lock_guard<std::mutex> lock(g_argmax_scratch_mutex);
+  if (g_argmax_scratch_ptr[device] == nullptr) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(argmax_scratch));
+    if (e != hipSuccess || ptr == nullptr)
+      return fail("argmax_static: hipGetSymbolAddress on device %d: %s", device, hipGetErrorString(e));
+    g_argmax_scratch_ptr[device] = ptr;
+  }
+  *out = g_argmax_scratch_ptr[device];
+  return 0;
+}
+}  // namespace ls
+
+extern "C" int ls_argmax_static(const float* x, int* out, int rows, int width, long ld, void* stream) {
+  LS_REQUIRE(x && out && rows > 0 && width > 0 && ld >= width, "argmax_static: bad operands or sizes");
+  const int chunks = ls_argmax_chunks(width);
+  LS_REQUIRE((long)rows * chunks <= (long)LS_ARGMAX_STATIC_PAIRS,
+             "argmax_static: %d rows of %d chunks need %ld scratch entries, the static array holds %d "
+             "(use ls_argmax with a scratch buffer of your own)",
+             rows, chunks, (long)rows * chunks, LS_ARGMAX_STATIC_PAIRS);
+  void* ptr = nullptr;
+  if (int code = argmax_scratch_of_current_device(&ptr)) return code;
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  // both halves sized for the capacity, so the layout does not depend on the call
+  float* part_v = reinterpret_cast<float*>(ptr);
+  int* part_i = reinterpret_cast<int*>(ptr) + LS_ARGMAX_STATIC_PAIRS;
+  hipLaunchKernelGGL(argmax_chunk_kernel, dim3(chunks, rows), dim3(256), 0, s, x, out, part_v, part_i, width, ld,
+                     chunks);
+  if (chunks > 1) hipLaunchKernelGGL(argmax_final_kernel, dim3(rows), dim3(256), 0, s, part_v, part_i, out, chunks);
+  return check_launch("argmax_static");
 }
 
 // meta: the step's uploaded metadata; picked [n_seqs]: the tokens chosen for the requests; ring

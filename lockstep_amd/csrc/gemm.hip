@@ -21,6 +21,7 @@
 #include <type_traits>
 
 #include "common.h"
+#include "core_api.h"
 
 namespace ls {
 

@@ -38,16 +38,31 @@ FLAGS = [
 ]
 CORE_SOURCES = ("core.hip", "gemm.hip")
 ATTENTION_SOURCES = ("attention.hip",)
-HEADERS = ("common.h",)
 
 
 class BuildError(RuntimeError):
     pass
 
 
+def _headers(sources) -> tuple:
+    """The headers of this folder that ``sources`` include, directly or through one another."""
+    found: list[str] = []
+    queue = list(sources)
+    while queue:
+        text = (CSRC / queue.pop(0)).read_text()
+        for line in text.splitlines():
+            line = line.strip()
+            if line.startswith('#include "'):
+                name = line.split('"')[1]
+                if name not in found and (CSRC / name).is_file():
+                    found.append(name)
+                    queue.append(name)
+    return tuple(sorted(found))
+
+
 def _hash(sources, defines) -> str:
     digest = hashlib.sha256()
-    for name in tuple(sources) + HEADERS:
+    for name in tuple(sources) + _headers(sources):
         digest.update(name.encode())
         digest.update((CSRC / name).read_bytes())
     digest.update(" ".join(FLAGS + list(defines)).encode())
