@@ -11,8 +11,21 @@ in the next step.  By default the pick is fed back on the device
 reads the tokens once at the end); ``--host-sampling`` brings every step's
 logits to the ``Sampler`` on the host instead.  Requests start from 512-token random prompts (prefilled
 outside the timed region); K timed steps follow W untimed ones, bracketed by
-device synchronisation.  One JSON line is printed.  The reference publishes no
-tokens-a-second figure (it states ratios only), so ``vs_baseline`` is null.
+device synchronisation; the run is repeated (``--repeats``, default 5) from freshly
+prefilled requests and the median run is reported with the fastest and slowest beside it
+(reference bench/lockstep_runner.py:30-42 and README.md:184-222: an untimed warm-up pass, then
+the median of at least five runs with their spread).  One JSON line is printed.  The reference
+publishes no tokens-a-second figure (it states ratios only), so ``vs_baseline`` is null.
+
+    python bench.py --workload serve --model qwen3-8b
+
+runs a whole workload through the scheduler instead, as the reference's own benchmark does
+(bench/lockstep_runner.py:35-51: every request submitted at once, ``Scheduler.run()``, one
+untimed pass first): 64 requests with prompt lengths uniform in [128, 4096] and 256 new tokens
+each in prompt portions of 2,048 tokens (``qwen3-0.6b``, ``qwen3-8b``), or 16 requests of 8,192
+tokens with 128 new tokens each (``qwen3-32b``).  ``--workload reference-trace`` runs the shape
+of the reference's committed trace (eight prompts of 64 to 700 tokens, 32 new tokens each,
+bench/throughput.py:35-45).  The value is all tokens (prompt and new) a second.
 """
 
 from __future__ import annotations
@@ -83,8 +96,9 @@ def random_prompts(n: int, length: int, vocab: int, seed: int):
 
 
 def measure_decode(model, cfg, batch: int, prompt_len: int, steps: int, warmup: int, page_size: int,
-                   device_loop: bool = True):
-    """(seconds of the timed steps, mean context length during them)."""
+                   device_loop: bool = True, repeats: int = 1):
+    """(seconds of the timed steps of every repeat, mean context length during them).  Every
+    repeat starts from freshly prefilled requests and times exactly ``steps`` decode steps."""
     import torch
 
     from lockstep_amd.engine.batch import StepEntry
@@ -121,21 +135,30 @@ def measure_decode(model, cfg, batch: int, prompt_len: int, steps: int, warmup: 
             tokens = sampler.sample(logits, requests)
         return tokens
 
+    def close_all():
+        for r in requests:
+            cache.close(r.uid)
+
     tokens = prefill()
     decode(tokens, warmup)
-    for r in requests:
-        cache.close(r.uid)
-    tokens = prefill()
-    decode(tokens, 1)          # the first step of a shape records its graph; keep that out of the timing
-    torch.cuda.synchronize()
-    started = time.perf_counter()
-    decode(tokens, steps)
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - started
-    for r in requests:
-        cache.close(r.uid)
+    close_all()
+    times = []
+    for _ in range(max(1, repeats)):
+        tokens = prefill()
+        decode(tokens, 1)          # the first step of a shape records its graph; keep that out of the timing
+        torch.cuda.synchronize()
+        started = time.perf_counter()
+        decode(tokens, steps)
+        torch.cuda.synchronize()
+        times.append(time.perf_counter() - started)
+        close_all()
     del cache
-    return elapsed, prompt_len + 1 + steps / 2.0
+    return times, prompt_len + 1 + steps / 2.0
+
+
+def spread(times, steps: int) -> dict:
+    return {"runs": len(times), "min_ms_per_step": round(1e3 * min(times) / steps, 4),
+            "max_ms_per_step": round(1e3 * max(times) / steps, 4)}
 
 
 def measure_prefill(model, cfg, length: int, page_size: int, repeats: int = 5):
@@ -159,6 +182,118 @@ def measure_prefill(model, cfg, length: int, page_size: int, repeats: int = 5):
     return statistics.median(times)
 
 
+def kernel_digest(model) -> str:
+    """Names of the loaded kernel libraries; each carries a hash of its sources and flags, which
+    fixes every tile and split constant (reference engine/kernels/registry.py:163-166)."""
+    kernels = model.rt.kernels
+    names = [Path(kernels.core_path).stem] + [Path(p).stem for _, p in sorted(kernels.attention_paths.items())]
+    return ",".join(n.replace("liblockstep_", "") for n in names)
+
+
+def serve_trace(kind: str, model_name: str, vocab: int, n_requests: int = 0):
+    """(prompts, new tokens each, prompt portion) of a serving workload, seeded."""
+    import random
+
+    import torch
+
+    g = torch.Generator().manual_seed(20260805)
+    rng = random.Random(64)
+    if kind == "reference-trace":
+        lengths, new, chunk = [64, 544, 96, 600, 80, 520, 112, 700], 32, None
+    elif model_name == "qwen3-32b":
+        lengths, new, chunk = [8192] * 16, 128, 2048
+    else:
+        lengths, new, chunk = [rng.randint(128, 4096) for _ in range(64)], 256, 2048
+    if n_requests:
+        lengths = lengths[:n_requests]
+    return [torch.randint(0, vocab, (n,), generator=g).tolist() for n in lengths], new, chunk
+
+
+def measure_serve(model, prompts, new_tokens: int, chunk, page_size: int, max_batched_tokens, repeats: int):
+    """Run the workload ``repeats`` + 1 times through the scheduler (the first pass untimed).
+    Returns per timed pass (seconds, seconds until no prompt token was left, scheduler steps,
+    steps of the decode-only phase)."""
+    import torch
+
+    from lockstep_amd.engine.policy import DefaultPolicy, FixedChunkPolicy
+    from lockstep_amd.engine.scheduler import Request, Scheduler
+
+    n = len(prompts)
+    longest = max(len(p) for p in prompts) + new_tokens
+    pages = sum(-(-(len(p) + new_tokens) // page_size) for p in prompts) + 8
+    cache = model.make_cache(num_pages=pages, page_size=page_size, max_requests=n, max_tokens_per_request=longest)
+    passes = []
+    for i in range(repeats + 1):
+        policy = FixedChunkPolicy(chunk, max_running=n) if chunk else DefaultPolicy(max_running=n)
+        scheduler = Scheduler(model, num_blocks=pages, policy=policy, audit=False, block_size=page_size,
+                              max_batched_tokens=max_batched_tokens, cache=cache, decode_burst=32)
+        for j, prompt in enumerate(prompts):
+            scheduler.submit(Request(uid=f"r{j:02d}", prompt=prompt, seed=j, max_new_tokens=new_tokens))
+        torch.cuda.synchronize()
+        started = time.perf_counter()
+        prompts_done_at, steps_at = None, 0
+        while scheduler.advance():
+            if prompts_done_at is None and not scheduler.waiting and all(
+                    r.kv_len >= len(r.prompt) for r in scheduler.running):
+                torch.cuda.synchronize()
+                prompts_done_at, steps_at = time.perf_counter() - started, scheduler.step_index
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - started
+        done = {r.uid: len(r.generated) for r in scheduler.done}
+        if len(done) != n or any(v != new_tokens for v in done.values()):
+            raise RuntimeError(f"the workload did not finish: {len(done)} of {n} requests done")
+        if i:
+            passes.append((elapsed, prompts_done_at if prompts_done_at is not None else elapsed,
+                           scheduler.step_index, scheduler.step_index - steps_at))
+    del cache
+    return passes
+
+
+def serve_record(args, model, cfg, full_layers) -> dict:
+    prompts, new_tokens, chunk = serve_trace(args.workload, args.model, cfg.vocab_size, args.requests)
+    if args.prefill_chunk is not None:
+        chunk = args.prefill_chunk or None
+    passes = measure_serve(model, prompts, new_tokens, chunk, args.page_size, args.max_batched_tokens,
+                           args.repeats)
+    order = sorted(passes, key=lambda t: t[0])
+    elapsed, prompts_done, steps, decode_steps = order[len(order) // 2]
+    prompt_tokens = sum(len(p) for p in prompts)
+    total_new = new_tokens * len(prompts)
+    decode_seconds = elapsed - prompts_done
+    return {
+        "metric": (f"serve tok/s, prompt and new tokens ({args.model} layer sizes, {len(prompts)} requests through the "
+                   f"scheduler, {args.workload})"),
+        "value": round((prompt_tokens + total_new) / elapsed, 1),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": steps,
+        "warmup": 1,
+        "ms_per_step": round(1e3 * elapsed / steps, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": args.dtype,
+        "data": "synthetic: uniform random token ids, random weights N(0, 0.02)",
+        "config": {
+            "model": args.model, "layers": cfg.num_hidden_layers, "layers_of_model": full_layers,
+            "hidden_size": cfg.hidden_size, "intermediate_size": cfg.intermediate_size,
+            "num_attention_heads": cfg.num_attention_heads, "num_key_value_heads": cfg.num_key_value_heads,
+            "head_dim": cfg.head_dim, "vocab_size": cfg.vocab_size, "tie_word_embeddings": cfg.tie_word_embeddings,
+            "requests": len(prompts), "prompt_tokens": prompt_tokens, "longest_prompt": max(len(p) for p in prompts),
+            "new_tokens": new_tokens, "prefill_chunk": chunk or 0, "max_batched_tokens": args.max_batched_tokens or 0,
+            "page_size": args.page_size, "parallelism": "single GPU", "decode_loop": "hip graphs, device token feedback",
+            "kernels": kernel_digest(model),
+        },
+        "serve": {
+            "seconds": round(elapsed, 4), "runs": len(passes), "min_s": round(order[0][0], 4),
+            "max_s": round(order[-1][0], 4), "new_tokens_per_s": round(total_new / elapsed, 1),
+            "until_prompts_done_s": round(prompts_done, 4), "decode_only_s": round(decode_seconds, 4),
+            "decode_only_steps": decode_steps,
+            "decode_only_step_ms": round(1e3 * decode_seconds / decode_steps, 4) if decode_steps else None,
+        },
+    }
+
+
 def main(argv=None) -> int:
     p = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     p.add_argument("--gpus", type=int, default=1)
@@ -174,6 +309,12 @@ def main(argv=None) -> int:
     p.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points and the prefill")
     p.add_argument("--host-sampling", action="store_true",
                    help="pick every step's tokens on the host (Model.step + Sampler) instead of the device-side loop")
+    p.add_argument("--workload", default="decode", choices=["decode", "serve", "reference-trace"],
+                   help="decode: fixed batches (the headline); serve / reference-trace: a workload through the scheduler")
+    p.add_argument("--repeats", type=int, default=5, help="timed runs; the median is reported with the spread")
+    p.add_argument("--requests", type=int, default=0, help="serve: only the first N requests of the workload")
+    p.add_argument("--prefill-chunk", type=int, default=None, help="serve: prompt portion (0: whole prompts)")
+    p.add_argument("--max-batched-tokens", type=int, default=8192, help="serve: token budget of a step (0: none)")
     p.add_argument("--only-prefill", action="store_true",
                    help="run the prefill measurement alone and print its record (for profiling)")
     args = p.parse_args(argv)
@@ -187,14 +328,19 @@ def main(argv=None) -> int:
     model, cfg, full_layers = build_model(args)
     element = 2 if args.dtype == "bf16" else 4
 
+    if args.workload != "decode":
+        print(json.dumps(serve_record(args, model, cfg, full_layers)))
+        return 0
+
     if args.only_prefill:
         seconds = measure_prefill(model, cfg, args.prefill_len, args.page_size)
         print(json.dumps({"prefill": {"value": round(args.prefill_len / seconds, 1), "tokens": args.prefill_len,
                                       "ms": round(1e3 * seconds, 3)}}))
         return 0
 
-    elapsed, context = measure_decode(model, cfg, args.batch, args.prompt_len, args.steps, args.warmup,
-                                      args.page_size, not args.host_sampling)
+    times, context = measure_decode(model, cfg, args.batch, args.prompt_len, args.steps, args.warmup,
+                                    args.page_size, not args.host_sampling, args.repeats)
+    elapsed = statistics.median(times)
     ms_per_step = 1e3 * elapsed / args.steps
     value = args.batch * args.steps / elapsed
     bytes_step = decode_bytes(cfg, args.batch, context, element)
@@ -220,9 +366,12 @@ def main(argv=None) -> int:
             "head_dim": cfg.head_dim, "vocab_size": cfg.vocab_size, "tie_word_embeddings": cfg.tie_word_embeddings,
             "global_batch": args.batch, "prompt_len": args.prompt_len, "new_tokens": args.steps,
             "seq_len": args.prompt_len + args.steps, "max_context": 4096, "page_size": args.page_size,
-            "prefill_len": args.prefill_len, "parallelism": "single GPU", "hip_graphs": bool(model.use_graphs),
-            "token_feedback": "host" if args.host_sampling else "device",
+            "prefill_len": args.prefill_len, "parallelism": "single GPU",
+            "decode_loop": ("hip graphs" if model.use_graphs else "eager") +
+                           (", host sampling" if args.host_sampling else ", device token feedback"),
+            "kernels": kernel_digest(model),
         },
+        "spread": spread(times, args.steps),
         "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": PEAK_HBM / 1e9,
                      "unit": "GB/s", "frac": round(achieved / PEAK_HBM, 4)},
     }
@@ -233,12 +382,14 @@ def main(argv=None) -> int:
         record["prefill"] = {"value": round(args.prefill_len / seconds, 1), "tokens": args.prefill_len,
                              "ms": round(1e3 * seconds, 3),
                              "frac": round(flops / seconds / PEAK_FLOPS[args.dtype], 4)}
-        points = {}
+        points, point_spread = {}, {}
         for batch, steps in ((1, args.steps), (64, args.steps)):
             t, _ = measure_decode(model, cfg, batch, args.prompt_len, steps, min(args.warmup, 4), args.page_size,
-                                  not args.host_sampling)
-            points[f"decode_b{batch}"] = round(batch * steps / t, 1)
+                                  not args.host_sampling, args.repeats)
+            points[f"decode_b{batch}"] = round(batch * steps / statistics.median(t), 1)
+            point_spread[f"decode_b{batch}"] = spread(t, steps)
         record["points"] = points
+        record["points_spread"] = point_spread
     torch.cuda.synchronize()
     print(json.dumps(record))
     return 0

@@ -133,6 +133,20 @@ class CacheGroup:
         return 2 * len(self.units) * self.spec.num_kv_heads * self.spec.head_dim * element_size
 
 
+class GraphStore(dict):
+    """Captured step graphs that point into one cache manager's storage, by step shape.  They
+    belong to the model that captured them, live here because they are valid for this storage
+    only, and die with the manager.  The least recently captured ones make room for new ones."""
+
+    def __init__(self, capacity: int = 32):
+        super().__init__()
+        self.capacity = capacity
+
+    def make_room(self) -> None:
+        while len(self) >= self.capacity:
+            del self[next(iter(self))]
+
+
 class CacheManager:
     def __init__(self, unit_specs: Sequence[object], page_size: int, num_pages, max_requests: int,
                  max_tokens_per_request: int, torch_dtype=None, device=None, poison_on_free: bool = False):
@@ -177,6 +191,7 @@ class CacheManager:
                 self.state[unit] = torch.zeros((max_requests, *spec.shape), dtype=torch.float32, device=device)
 
         self.ever_shared = False     # set once a page got a second holder (prefix sharing)
+        self.step_graphs = GraphStore()
         self._free_slots = list(range(max_requests))
         heapq.heapify(self._free_slots)
         self.requests: dict[Hashable, _Request] = {}

@@ -65,6 +65,8 @@ class Model:
                 raise ValueError(f"the schedule names layer {run.layer}, the model has {len(self.layers)}")
         self.workspace = Workspace(rt.device)
         self.use_graphs = os.environ.get("LOCKSTEP_NO_GRAPHS", "") in ("", "0")
+        # debugging aid: every replayed decode step is also run eagerly and the logits compared bit for bit
+        self.verify_graphs = os.environ.get("LOCKSTEP_VERIFY_GRAPHS", "") not in ("", "0")
         self._graph_safe = all(graph_safe_tree(part)
                                for part in (self.embedding, *self.layers, self.final_norm, self.head))
         # which arrangements, and the final norm, take over an addition the previous layer left open
@@ -186,19 +188,24 @@ class Model:
         replays.  The first step of a shape runs eagerly (that also sizes the
         workspace), then the same launches are recorded for the steps to come.
         Graphs are kept on the cache manager they point into and die with it."""
-        graphs = cache.__dict__.setdefault("_step_graphs", {})
+        graphs = cache.step_graphs
         key = self._graph_key(ctx)
         held = graphs.get(key)
         if held is not None:
             graph, logits = held
             graph.replay()
             self.graph_replays += 1
+            if self.verify_graphs:
+                replayed = logits.clone()
+                eager = self._forward(ctx)
+                if not torch.equal(replayed, eager):
+                    raise RuntimeError("a replayed step graph and the same step run eagerly disagree: a device "
+                                       "buffer the graph points at was replaced without the graph key changing")
             return logits.clone()
         logits = torch.empty((ctx.n_want, self.spec.vocab_size), dtype=torch.float32, device=self.rt.device)
         self._forward(ctx, logits)
         key = self._graph_key(ctx)                 # the eager run may have grown the workspace
-        if len(graphs) >= 32:
-            graphs.clear()
+        graphs.make_room()
         result = logits.clone()
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()
@@ -280,7 +287,7 @@ class Model:
             kernels.advance_decode(layout["meta"], n, layout["tokens"], layout["positions"], layout["seqs"], picked,
                                    ring, counter, layout["item_lists"])
 
-        graphs = cache.__dict__.setdefault("_step_graphs", {})
+        graphs = cache.step_graphs
         key = ("loop",) + self._graph_key(ctx)
         held = graphs.get(key)
         done = 0
@@ -289,8 +296,7 @@ class Model:
             one_step(logits)                              # sizes the workspace; it is the loop's first step
             done = 1
             key = ("loop",) + self._graph_key(ctx)
-            if len(graphs) >= 32:
-                graphs.clear()
+            graphs.make_room()
             torch.cuda.synchronize()
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):

@@ -372,8 +372,13 @@ class Scheduler:
         self._retire_finished()
         return True
 
+    def advance(self, max_steps: int = 1 << 20) -> bool:
+        """One iteration of the serving loop (a run of decode steps on the device, or one step);
+        False when nothing waits and nothing runs, or ``max_steps`` steps have been taken."""
+        return bool(self._burst(max_steps) or self.step()) and self.step_index < max_steps
+
     def run(self, max_steps: int = 1 << 20) -> dict:
-        while (self._burst(max_steps) or self.step()) and self.step_index < max_steps:
+        while self.advance(max_steps):
             pass
         if self.audit_enabled:
             self.cache.audit()

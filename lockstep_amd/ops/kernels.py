@@ -285,7 +285,15 @@ class Kernels:
                                    c_long(gate_up.stride(0)), c_long(out.stride(0)), _stream())
         self._check(self.core, code)
 
+    #: (row, chunk) pairs the library's static arg-max scratch holds (LS_ARGMAX_STATIC_PAIRS)
+    ARGMAX_STATIC_PAIRS = 16384
+
     def argmax(self, logits: torch.Tensor, out: torch.Tensor) -> None:
+        """Lowest index among the maxima of every float32 row.  Calls that fit the library's static
+        scratch array go through the entry point that allocates nothing: that array never moves, so
+        a captured graph that contains the launch stays valid whatever runs in between.  Larger
+        calls bring a scratch buffer; a buffer that was outgrown is kept until the process ends,
+        because a captured graph may still write into it."""
         _rows_ok(logits, "argmax logits")
         if not (logits.dtype == torch.float32):
             raise KernelError("argmax reads float32 logits")
@@ -293,11 +301,17 @@ class Kernels:
             raise KernelError(f"argmax out must be int32 [{logits.shape[0]}]")
         if logits.shape[0] == 0:
             return
-        words = 2 * logits.shape[0] * self.core.ls_argmax_chunks(c_int(logits.shape[1]))
-        scratch = self._argmax_scratch.get(logits.device)
-        if scratch is None or scratch.numel() < words:
-            scratch = torch.empty(max(words, 4096), dtype=torch.int32, device=logits.device)
-            self._argmax_scratch[logits.device] = scratch
+        pairs = logits.shape[0] * self.core.ls_argmax_chunks(c_int(logits.shape[1]))
+        if pairs <= self.ARGMAX_STATIC_PAIRS:
+            code = self.core.ls_argmax_static(_ptr(logits), _ptr(out), c_int(logits.shape[0]), c_int(logits.shape[1]),
+                                              c_long(logits.stride(0)), _stream())
+            self._check(self.core, code)
+            return
+        held = self._argmax_scratch.setdefault(logits.device, [])
+        if not held or held[-1].numel() < 2 * pairs:
+            held.append(torch.empty(max(2 * pairs, 2 * held[-1].numel() if held else 0), dtype=torch.int32,
+                                    device=logits.device))
+        scratch = held[-1]
         code = self.core.ls_argmax(_ptr(logits), _ptr(out), c_int(logits.shape[0]), c_int(logits.shape[1]),
                                    c_long(logits.stride(0)), _ptr(scratch), c_long(scratch.numel()), _stream())
         self._check(self.core, code)

@@ -198,6 +198,25 @@ def test_argmax_takes_the_lowest_index_among_maxima():
     want = [int(torch.nonzero(r == r.max())[0]) for r in x]
     assert out.cpu().tolist() == want
     assert want[1] == 77 and want[2] == 0 and want[3] == 151935
+
+
+def test_argmax_with_more_rows_than_the_static_scratch_holds():
+    """Beyond 16,384 (row, chunk) pairs the wrapper brings a scratch buffer, and a larger call
+    after a smaller one grows it; the results are those of the static path."""
+    k = K()
+    g = torch.Generator().manual_seed(5)
+    for rows in (2100, 2900):                       # 3 chunks a row: 6,300 and 8,700 pairs, the static array
+        x = torch.randn(rows, 9000, generator=g)
+        x[:, 8999] = x.max(dim=1).values            # a tie with the last column: the lower index wins
+        out = torch.empty(rows, dtype=torch.int32, device="cuda")
+        k.argmax(x.cuda(), out)
+        assert torch.equal(out.long().cpu(), (x == x.max(1, keepdim=True).values).int().argmax(1))
+    for rows in (5600, 7000):                       # 16,800 and 21,000 pairs: beyond the static array, growing
+        assert rows * 3 > k.ARGMAX_STATIC_PAIRS
+        x = torch.randn(rows, 9000, generator=g)
+        out = torch.empty(rows, dtype=torch.int32, device="cuda")
+        k.argmax(x.cuda(), out)
+        assert torch.equal(out.long().cpu(), x.argmax(dim=1))
     small = torch.tensor([[1.0, 5.0, 5.0, 5.0, 2.0]]).cuda()
     one = torch.empty(1, dtype=torch.int32, device="cuda")
     K().argmax(small, one)

@@ -165,6 +165,41 @@ def test_the_device_side_loop_at_real_layer_sizes(models):
     assert picked["loop"] == picked["steps"]
 
 
+def test_a_captured_decode_loop_survives_a_large_argmax_in_between(models):
+    """The arg-max inside the captured loop writes its partial results (this vocabulary has two
+    chunks a row) to memory that must still be the loop's when the graph is replayed after an
+    arg-max over many more rows."""
+    from lockstep_amd.engine.batch import StepEntry
+
+    folder, config = models["0.6b-like"]
+    model = load(folder, "bfloat16")
+    kernels = model.rt.kernels
+    prompts = {f"r{i}": random_tokens(30 + 11 * i, config.vocab_size, seed=90 + i) for i in range(8)}
+
+    def run(disturb: bool):
+        cache = model.make_cache(num_pages=64, page_size=16, max_requests=8)
+        first = []
+        for rid, toks in prompts.items():
+            cache.open(rid)
+            logits = model.step(cache, [StepEntry(rid, toks, [len(toks) - 1])])
+            first.append(int(logits[0].argmax()))
+        a = model.decode_greedy(cache, list(prompts), first, 6)
+        if disturb:
+            for rows in (64, 9000):                 # 9,000 rows of two chunks: beyond the static scratch array
+                big = torch.randn(rows, config.vocab_size, device="cuda")
+                kernels.argmax(big, torch.empty(rows, dtype=torch.int32, device="cuda"))
+                del big
+            torch.cuda.synchronize()
+            torch.cuda.empty_cache()
+            filler = torch.full((1 << 22,), -1, dtype=torch.int32, device="cuda")    # takes freed blocks, if any
+        replays = model.graph_replays
+        b = model.decode_greedy(cache, list(prompts), a[-1].tolist(), 6)
+        assert model.graph_replays > replays
+        return a.tolist() + b.tolist()
+
+    assert run(disturb=True) == run(disturb=False)
+
+
 @pytest.mark.parametrize("name", list(SIZES))
 def test_random_mixes_at_real_layer_sizes(models, name):
     """Random mixes of one to five requests (lengths on both sides of the tile, split and row-block
