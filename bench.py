@@ -234,12 +234,12 @@ def measure_serve(model, prompts, new_tokens: int, chunk, page_size: int, max_ba
         prompts_done_at, steps_at = None, 0
         while scheduler.advance():
             if prompts_done_at is None and not scheduler.waiting and all(
-                    r.kv_len >= len(r.prompt) for r in scheduler.running):
+                    r.cached >= r.n_prompt for r in scheduler.running):
                 torch.cuda.synchronize()
                 prompts_done_at, steps_at = time.perf_counter() - started, scheduler.step_index
         torch.cuda.synchronize()
         elapsed = time.perf_counter() - started
-        done = {r.uid: len(r.generated) for r in scheduler.done}
+        done = {r.uid: r.n_generated for r in scheduler.done}
         if len(done) != n or any(v != new_tokens for v in done.values()):
             raise RuntimeError(f"the workload did not finish: {len(done)} of {n} requests done")
         if i:

@@ -20,6 +20,7 @@ _LAZY = {
     "Request": ("lockstep_amd.engine.scheduler", "Request"),
     "OversizedRequest": ("lockstep_amd.engine.scheduler", "OversizedRequest"),
     "LLM": ("lockstep_amd.engine.llm", "LLM"),
+    "EngineConfig": ("lockstep_amd.engine.config", "EngineConfig"),
     "generate_greedy": ("lockstep_amd.engine.llm", "generate_greedy"),
     "DefaultPolicy": ("lockstep_amd.engine.policy", "DefaultPolicy"),
     "FixedChunkPolicy": ("lockstep_amd.engine.policy", "FixedChunkPolicy"),

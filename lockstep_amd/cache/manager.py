@@ -15,7 +15,8 @@ page and pins of the prefix index (reference engine/kv/paged.py:116-139).
 
 Every request also owns a *slot*: its row in the block tables on the device
 and its index into the state tensors of the units that keep a ``StateSpec``.
-State is zeroed when the slot is taken.
+State is zeroed when the slot is taken and, like freed pages, poisoned when
+the slot is given back (``poison_on_free``); the audit and the digest cover it.
 
 The manager does its accounting on the host; with ``device=None`` it holds no
 storage at all, which is how the tests without a GPU drive it.
@@ -187,13 +188,17 @@ class CacheManager:
         if device is not None and self.state_units:
             import torch
 
+            kinds = {"float32": torch.float32, "bfloat16": torch.bfloat16, "int32": torch.int32}
             for unit, spec in self.state_units.items():
-                self.state[unit] = torch.zeros((max_requests, *spec.shape), dtype=torch.float32, device=device)
+                if spec.dtype not in kinds:
+                    raise TypeError(f"cache unit {unit} asks for state of dtype {spec.dtype!r}; known: {sorted(kinds)}")
+                self.state[unit] = torch.zeros((max_requests, *spec.shape), dtype=kinds[spec.dtype], device=device)
 
         self.ever_shared = False     # set once a page got a second holder (prefix sharing)
         self.step_graphs = GraphStore()
         self._free_slots = list(range(max_requests))
         heapq.heapify(self._free_slots)
+        self._ever_used: set[int] = set()
         self.requests: dict[Hashable, _Request] = {}
 
     # -- requests ---------------------------------------------------------------
@@ -204,6 +209,7 @@ class CacheManager:
         if not self._free_slots:
             raise OutOfPages(f"all {self.max_requests} request slots are taken")
         slot = heapq.heappop(self._free_slots)
+        self._ever_used.add(slot)
         self.requests[request_id] = _Request(slot=slot, groups=[_RequestPages() for _ in self.groups])
         for tensor in self.state.values():
             tensor[slot].zero_()
@@ -301,7 +307,14 @@ class CacheManager:
                 group.table_host[request.slot, : len(mine.pages)] = -1
                 group.dirty_rows.add(request.slot)
             mine.pages.clear()
+        if self.poison_on_free:
+            for tensor in self.state.values():      # a later reader of the slot's old state must notice
+                tensor[request.slot].fill_(self._poison_value(tensor))
         heapq.heappush(self._free_slots, request.slot)
+
+    @staticmethod
+    def _poison_value(tensor):
+        return float("nan") if tensor.dtype.is_floating_point else -(1 << 30)
 
     def _release_page(self, group: CacheGroup, page: int) -> None:
         if group.pool.release(page) and self.poison_on_free:
@@ -404,6 +417,7 @@ class CacheManager:
             raise CacheAuditError("two requests share a slot")
         if sorted(slots + self._free_slots) != list(range(self.max_requests)):
             raise CacheAuditError("request slots are lost or duplicated")
+        self._audit_state()
         for gi, group in enumerate(self.groups):
             expected = [0] * group.pool.num_pages
             for page, count in group.pinned.items():
@@ -434,9 +448,43 @@ class CacheManager:
                     raise CacheAuditError(f"group {gi} page {page} has {group.pool.holders[page]} holders but is "
                                           f"{'in' if page in free else 'not in'} the free list")
 
-    def state_digest(self) -> tuple:
-        """Allocator state as a comparable value (reference engine/kv/paged.py:225-237)."""
-        return tuple(
+    def _audit_state(self) -> None:
+        """State units: every unit has a row per slot; with poisoning on, the rows of free slots
+        hold the poison and the rows of live requests hold none of it."""
+        for unit, spec in self.state_units.items():
+            tensor = self.state.get(unit)
+            if self.device is None:
+                continue
+            if tensor is None or tuple(tensor.shape) != (self.max_requests, *spec.shape):
+                raise CacheAuditError(f"state unit {unit} does not hold {self.max_requests} rows of {spec.shape}")
+            if not self.poison_on_free:
+                continue
+            rows = tensor.reshape(self.max_requests, -1)
+            bad = rows.isnan().any(dim=1) if tensor.dtype.is_floating_point else (rows == -(1 << 30)).any(dim=1)
+            bad = bad.cpu().tolist()
+            live = {r.slot: rid for rid, r in self.requests.items()}
+            for slot, poisoned in enumerate(bad):
+                if slot in live and poisoned:
+                    raise CacheAuditError(f"state unit {unit}: request {live[slot]!r} (slot {slot}) holds poisoned state")
+                if slot not in live and slot in self._ever_used and not poisoned:
+                    raise CacheAuditError(f"state unit {unit}: free slot {slot} was not poisoned when it was given back")
+
+    def state_digest(self, content: bool = False) -> tuple:
+        """Allocator state as a comparable value (reference engine/kv/paged.py:225-237); the
+        state units' declarations are part of it, and with ``content`` a hash of the state rows
+        of the live requests (read back from the device)."""
+        states = tuple((unit, tuple(spec.shape), spec.dtype) for unit, spec in sorted(self.state_units.items()))
+        if content and self.state:
+            import hashlib
+
+            slots = sorted(r.slot for r in self.requests.values())
+            rows = hashlib.sha256()
+            for unit in sorted(self.state):
+                if slots:
+                    picked = self.state[unit][slots].contiguous().view(-1)
+                    rows.update(picked.view(dtype=__import__("torch").uint8).cpu().numpy().tobytes())
+            states += (rows.hexdigest(),)
+        return states + tuple(
             (tuple(g.pool.holders), tuple(g.pool.free_set()), tuple(sorted(g.pinned.items())),
              tuple((repr(rid), r.slot, r.length, tuple(r.groups[gi].pages))
                    for rid, r in sorted(self.requests.items(), key=lambda kv: repr(kv[0]))))

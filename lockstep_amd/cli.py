@@ -61,6 +61,7 @@ def cmd_run(argv) -> int:
 
     import tempfile
 
+    from .engine.config import EngineConfig
     from .engine.llm import LLM
     from .engine.scheduler import Request
 
@@ -88,11 +89,11 @@ def cmd_run(argv) -> int:
             from .weights import write_random_model
 
             folder = write_random_model(preset(args.random), scratch, args.seed)
-        llm = LLM(folder, dtype=args.dtype, num_pages=args.num_blocks, page_size=args.block_size,
-                  max_batched_tokens=args.max_batched_tokens, prefill_chunk=args.prefill_chunk,
-                  max_running=args.max_running, enable_prefix_cache=args.enable_prefix_cache,
-                  eos_token_ids=args.eos, reserve=args.reserve, decode_burst=args.decode_burst)
-        outputs = llm.generate(requests)
+        engine = EngineConfig(dtype=args.dtype, num_pages=args.num_blocks, page_size=args.block_size,
+                              max_batched_tokens=args.max_batched_tokens, prefill_chunk=args.prefill_chunk,
+                              max_running=args.max_running, enable_prefix_cache=args.enable_prefix_cache,
+                              eos_token_ids=tuple(args.eos), reserve=args.reserve, decode_burst=args.decode_burst)
+        outputs = LLM(folder, engine).generate(requests)
     for uid in sorted(outputs):
         print(json.dumps({"uid": uid, "tokens": outputs[uid]}))
     return 0

@@ -79,6 +79,8 @@ class ModelSpec:
     schedule: tuple[ScheduleEntry, ...]
     final_norm: PartSpec
     head: PartSpec
+    #: positions a request may use (its tokens are at positions 0 .. max_positions - 1); None: no bound
+    max_positions: int | None = None
 
     def cache_units(self) -> int:
         return 1 + max((e.cache for e in self.schedule), default=-1)

@@ -2,7 +2,8 @@
 
 The eleven keys are the ones the reference reads, all without defaults
 (reference engine/model/qwen3.py:49-80); any other key is ignored there and
-here.  ``model_spec`` states the architecture once, as data: token embedding,
+here.  ``max_position_embeddings``, which the reference stores and never uses,
+bounds a request here: no token may sit at a position beyond it.  ``model_spec`` states the architecture once, as data: token embedding,
 ``num_hidden_layers`` pre-norm residual layers of grouped-query attention
 (per-head q/k RMSNorm, half-rotation RoPE over the whole head, full causal
 mask) and a SwiGLU MLP, a final RMSNorm and an untied or tied head
@@ -100,4 +101,5 @@ class Qwen3Config(ModelConfig):
                 "name": "lm_head.weight", "tied_to": "model.embed_tokens.weight"
                 if self.tie_word_embeddings else None,
                 "vocab_size": self.vocab_size, "hidden_size": self.hidden_size}),
+            max_positions=self.max_position_embeddings,
         )

@@ -1,17 +1,22 @@
-"""Counters of the paths a run took, and a running digest of what it did.
+"""Evidence of what a run did: counters of the paths it took, and a ledger of
+its steps that two runs can be compared by.
 
-A test that claims "preemption leaves tokens unchanged" must be able to show
-that a preemption happened; the counters are that evidence (reference
-engine/audit/counters.py:8-99).  The trajectory hash absorbs every step's
-work list, emitted tokens, sampled logit rows and the cache manager's state,
-so two runs can be compared step by step (reference
-engine/audit/trajectory.py:15-59).
+A test that claims "preemption leaves the tokens unchanged" has to show that
+a preemption happened; ``Counters.require_fired`` is that check (the idea of
+the reference's engine/audit/counters.py:86-99).  The ledger answers the other
+question, "where did two runs part and in what": every step leaves one record
+of four digests (the batch that ran, the tokens it emitted, the logit rows
+they were sampled from, the state of cache manager and prefix index), and the
+records are chained, so equal chains mean equal runs (the reference keeps one
+rolling hash, engine/audit/trajectory.py:15-59; here the parts stay apart so
+that a difference names what differs).
 """
 
 from __future__ import annotations
 
 import hashlib
 from collections import Counter
+from dataclasses import dataclass
 
 PATHS = {
     "admit": "a waiting request was admitted",
@@ -34,6 +39,7 @@ PATHS = {
     "finish_eos": "a request finished on an end-of-sequence token",
     "finish_limit": "a request finished at max_new_tokens",
     "out_of_pages": "nothing could run and nothing could be admitted",
+    "position_limit": "a request was refused because it would pass the model's last position",
 }
 
 
@@ -59,31 +65,64 @@ class Counters:
             raise VacuousRun(f"the run never took: {', '.join(missing)}")
 
 
-class TrajectoryHash:
+def _digest(*chunks: bytes) -> bytes:
+    h = hashlib.sha256()
+    for chunk in chunks:
+        h.update(len(chunk).to_bytes(8, "little"))
+        h.update(chunk)
+    return h.digest()
+
+
+@dataclass(frozen=True)
+class StepRecord:
+    """One step of a run, as digests of its four aspects, and the chain value after it."""
+
+    step: int
+    batch: bytes
+    tokens: bytes
+    logits: bytes
+    state: bytes
+    chain: bytes
+
+    ASPECTS = ("batch", "tokens", "logits", "state")
+
+
+class StepLedger:
+    """The chained records of a run's steps."""
+
     def __init__(self):
-        self._digest = hashlib.sha256()
-        self.per_step: list[str] = []
+        self.records: list[StepRecord] = []
 
-    def _absorb(self, label: str, payload: bytes) -> None:
-        self._digest.update(label.encode())
-        self._digest.update(len(payload).to_bytes(8, "big"))
-        self._digest.update(payload)
+    def observe_step(self, step: int, batch, emitted, logits_bytes: bytes, state) -> StepRecord:
+        """``batch``: what ran (uid, tokens, start) per request; ``emitted``: (uid, token) pairs;
+        ``logits_bytes``: the raw float32 rows the tokens were picked from; ``state``: any value
+        with a stable ``repr`` that describes the cache manager and the prefix index."""
+        previous = self.records[-1].chain if self.records else b"\0" * 32
+        parts = (_digest(repr(batch).encode()), _digest(repr(emitted).encode()), _digest(logits_bytes),
+                 _digest(repr(state).encode()))
+        record = StepRecord(step, *parts, chain=_digest(previous, str(step).encode(), *parts))
+        self.records.append(record)
+        return record
 
-    def observe_step(self, step: int, work, emitted, logits_bytes: bytes, cache_state) -> None:
-        self._absorb("step", str(step).encode())
-        self._absorb("work", repr(work).encode())
-        self._absorb("emitted", repr(emitted).encode())
-        self._absorb("logits", logits_bytes)
-        self._absorb("cache", repr(cache_state).encode())
-        self.per_step.append(self._digest.hexdigest())
+    @property
+    def per_step(self) -> list[str]:
+        return [r.chain.hex() for r in self.records]
 
     def hexdigest(self) -> str:
-        return self._digest.hexdigest()
+        return self.records[-1].chain.hex() if self.records else _digest().hex()
 
-    def first_divergence(self, other: "TrajectoryHash"):
-        for i, (a, b) in enumerate(zip(self.per_step, other.per_step)):
-            if a != b:
-                return i
-        if len(self.per_step) != len(other.per_step):
-            return min(len(self.per_step), len(other.per_step))
+    def first_divergence(self, other: "StepLedger"):
+        """Index of the first step at which the two runs differ, or None."""
+        found = self.first_difference(other)
+        return None if found is None else found[0]
+
+    def first_difference(self, other: "StepLedger"):
+        """(index, aspects) of the first step that differs: the names of the digests that are not
+        equal there ("length" when one run simply has more steps), or None for equal runs."""
+        for i, (mine, theirs) in enumerate(zip(self.records, other.records)):
+            if mine.chain != theirs.chain:
+                aspects = tuple(a for a in StepRecord.ASPECTS if getattr(mine, a) != getattr(theirs, a))
+                return i, aspects or ("step",)
+        if len(self.records) != len(other.records):
+            return min(len(self.records), len(other.records)), ("length",)
         return None

@@ -15,9 +15,11 @@ from __future__ import annotations
 from typing import Iterable, Sequence
 
 from .batch import StepEntry
+from .config import EngineConfig
 from .model import Model, load_model
-from .policy import DefaultPolicy, FixedChunkPolicy, Policy
+from .policy import Policy
 from .scheduler import Request, Scheduler
+from .scheduler import Sequence as SchedulerSequence
 
 
 def generate_greedy(model: Model, prompt_ids: Sequence[int], max_new_tokens: int, eos_token_ids=None,
@@ -32,44 +34,34 @@ def generate_greedy(model: Model, prompt_ids: Sequence[int], max_new_tokens: int
     cache.open("seq")
     sampler = Sampler(model.rt.kernels)
     eos = set(eos_token_ids or ())
-    request = Request(uid="seq", prompt=list(prompt_ids), max_new_tokens=max_new_tokens)
-    tokens = list(prompt_ids)
-    generated, step_logits = [], []
+    seq = SchedulerSequence(Request(uid="seq", prompt=list(prompt_ids), max_new_tokens=max_new_tokens))
+    feed = list(seq.tokens)
+    step_logits = []
     for _ in range(max_new_tokens):
-        logits = model.step(cache, [StepEntry("seq", tokens, [len(tokens) - 1])])
+        logits = model.step(cache, [StepEntry("seq", feed, [len(feed) - 1])])
         step_logits.append(logits[0].clone())
-        token = sampler.sample(logits, [request])[0]
-        generated.append(token)
-        request.generated.append(token)
+        token = sampler.sample(logits, [seq])[0]
+        seq.tokens.append(token)
         if token in eos:
             break
-        tokens = [token]
+        feed = [token]
     cache.close("seq")
-    return generated, step_logits
+    return seq.generated, step_logits
 
 
 class LLM:
-    """A loaded model plus what a workload needs to run on it."""
+    """A loaded model plus what a workload needs to run on it.  Options are an ``EngineConfig``
+    or its fields as keywords."""
 
-    def __init__(self, model_dir, dtype: str = "bfloat16", device: str = "cuda:0", num_pages: int = 512,
-                 page_size: int = 16, max_batched_tokens: int | None = None, prefill_chunk: int | None = None,
-                 max_running: int = 64, enable_prefix_cache: bool = False, eos_token_ids=None,
-                 reserve: str = "full", audit: bool = False, max_tokens_per_request: int | None = None,
-                 decode_burst: int = 32):
-        self.model = load_model(model_dir, dtype=dtype, device=device)
-        self.options = dict(num_blocks=num_pages, block_size=page_size, max_batched_tokens=max_batched_tokens,
-                            enable_prefix_cache=enable_prefix_cache, eos_token_ids=eos_token_ids, reserve=reserve,
-                            audit=audit, max_tokens_per_request=max_tokens_per_request, decode_burst=decode_burst)
-        self.prefill_chunk = prefill_chunk
-        self.max_running = max_running
+    def __init__(self, model_dir, config: EngineConfig | None = None, device: str = "cuda:0", **options):
+        self.config = (config or EngineConfig()).with_(**options) if options else (config or EngineConfig())
+        self.model = load_model(model_dir, dtype=self.config.dtype, device=device)
 
     def policy(self) -> Policy:
-        if self.prefill_chunk:
-            return FixedChunkPolicy(self.prefill_chunk, max_running=self.max_running)
-        return DefaultPolicy(max_running=self.max_running)
+        return self.config.policy()
 
     def scheduler(self, policy: Policy | None = None) -> Scheduler:
-        return Scheduler(self.model, policy=policy or self.policy(), **self.options)
+        return Scheduler.from_config(self.model, self.config, policy)
 
     def generate(self, requests: Iterable[Request], policy: Policy | None = None) -> dict:
         """Run the requests to completion; ``{uid: generated token ids}``."""

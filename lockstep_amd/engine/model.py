@@ -91,6 +91,12 @@ class Model:
         self.head.load(weights, self.rt)
         return self
 
+    def weight_cast_report(self) -> dict:
+        """What casting the checkpoint's tensors to the dtypes they are used in cost: elements
+        cast, how many changed value, largest absolute and relative change (all zero for a
+        bfloat16 checkpoint on either path)."""
+        return dict(self.rt.cast_report)
+
     # -- cache ------------------------------------------------------------------
     def cache_unit_specs(self) -> list:
         units = [None] * self.spec.cache_units()
@@ -129,8 +135,12 @@ class Model:
             for w in e.want:
                 if not 0 <= w < len(e.tokens):
                     raise ValueError(f"request {e.request!r} wants logits at {w}, it brings {len(e.tokens)} tokens")
+        limit = self.spec.max_positions
         for e in entries:
             start = cache.length(e.request)
+            if limit is not None and start + len(e.tokens) > limit:
+                raise ValueError(f"request {e.request!r} would reach {start + len(e.tokens)} tokens; the model's "
+                                 f"positions end at {limit}")
             cache.reserve(e.request, start + len(e.tokens))
             if cache.ever_shared:
                 for gi in range(len(cache.groups)):
@@ -260,7 +270,11 @@ class Model:
     def _decode_loop(self, cache, requests, tokens, n_steps):
         n = len(requests)
         starts = [cache.length(r) for r in requests]
+        limit = self.spec.max_positions
         for r, start in zip(requests, starts):
+            if limit is not None and start + n_steps > limit:
+                raise ValueError(f"request {r!r} would reach {start + n_steps} tokens; the model's positions end "
+                                 f"at {limit}")
             cache.reserve(r, start + n_steps)          # every page the loop will write, now
             if cache.ever_shared:
                 for gi in range(len(cache.groups)):

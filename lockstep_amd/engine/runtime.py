@@ -5,6 +5,7 @@ from __future__ import annotations
 import torch
 
 from ..ops import kernels as load_kernels
+from ..weights.cast import CastLedger
 
 DTYPES = {
     "bfloat16": torch.bfloat16, "bf16": torch.bfloat16,
@@ -42,20 +43,28 @@ class Runtime:
         self.dtype = parse_dtype(dtype)
         self.kernels = load_kernels()
         self._shared: dict[str, torch.Tensor] = {}
+        self.casts = CastLedger(self.dtype)     # what casting stored tensors to their working dtypes cost
 
     def matrix(self, tensor: torch.Tensor, share_key: str | None = None) -> torch.Tensor:
         """An operand of a matrix product: compute dtype, contiguous, on the device.
         Tensors loaded under the same ``share_key`` share one buffer (tied weights)."""
         if share_key is not None and share_key in self._shared:
             return self._shared[share_key]
-        out = tensor.to(device=self.device, dtype=self.dtype).contiguous()
+        out = self._cast(tensor, self.dtype).to(device=self.device).contiguous()
         if share_key is not None:
             self._shared[share_key] = out
         return out
 
     def vector(self, tensor: torch.Tensor) -> torch.Tensor:
         """A tensor used in 32-bit arithmetic (norm weights): float32 on the device."""
-        return tensor.to(device=self.device, dtype=torch.float32).contiguous()
+        return self._cast(tensor, torch.float32).to(device=self.device).contiguous()
+
+    def _cast(self, tensor: torch.Tensor, target: torch.dtype) -> torch.Tensor:
+        return self.casts.cast(tensor, target)
+
+    @property
+    def cast_report(self) -> dict:
+        return self.casts.report
 
     def element_size(self) -> int:
         return 2 if self.dtype is torch.bfloat16 else 4

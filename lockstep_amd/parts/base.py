@@ -69,9 +69,11 @@ class PagedKVSpec:
 
 @dataclass(frozen=True)
 class StateSpec:
-    """A state of fixed size per request (``shape`` elements of float32)."""
+    """A state of fixed size per request: ``shape`` elements of ``dtype`` ("float32",
+    "bfloat16" or "int32"), all zero when a request starts."""
 
     shape: tuple[int, ...]
+    dtype: str = "float32"
 
 
 class Part:
@@ -234,8 +236,10 @@ DEFER_MANY_ROWS_SUMS = 16384
 
 def deferred_rows(ctx, k: int, n: int) -> int:
     """The most tokens of a step for which a product over ``k`` with ``n`` outputs is left as
-    K-slice sums."""
+    K-slice sums (0: never; the kernel that adds the sums moves four columns at a time)."""
     kernels = ctx.rt.kernels
+    if n % 4:
+        return 0
     if kernels.gemm_slices_count(k) * n > DEFER_MANY_ROWS_SUMS:
         return min(DEFER_ADD_ROWS, 64)
     return min(DEFER_ADD_ROWS, kernels.gemm_slices_max_rows(k, ctx.rt.dtype))

@@ -5,9 +5,11 @@ with the ``WeightSpec`` list of the model and raises one ``WeightError`` that
 lists every missing, unexpected and mis-shaped tensor.  Tensors stay on the
 CPU here (memory-mapped); parts move what they use to the device.
 
-Dtypes are normalised, not chosen: 16-bit floating tensors are kept as
-bfloat16, integer tables become int32, and a tensor stored in 32-bit (or
-64-bit) floating point stays float32.
+Dtypes are normalised, not chosen: bfloat16 and float16 tensors are kept as
+stored, integer tables become int32, and a tensor stored in 32-bit (or
+64-bit) floating point stays float32.  The cast to the compute dtype happens
+where a part puts a tensor on the device (``Runtime.matrix`` / ``vector``),
+which also keeps the record of what a lossy cast cost.
 
 A tied head follows the reference (engine/model/qwen3.py:159-174,201-202):
 when the configuration ties the head to the embedding and the checkpoint
@@ -36,10 +38,8 @@ class WeightError(ValueError):
 
 
 def normalise_dtype(tensor: torch.Tensor) -> torch.Tensor:
-    if tensor.dtype in (torch.bfloat16, torch.float32):
+    if tensor.dtype in (torch.bfloat16, torch.float32, torch.float16):
         return tensor
-    if tensor.dtype is torch.float16:
-        return tensor.to(torch.bfloat16)
     if tensor.dtype is torch.float64:
         return tensor.to(torch.float32)
     if tensor.dtype in (torch.int64, torch.int32, torch.int16, torch.int8, torch.uint8, torch.bool):

@@ -43,7 +43,14 @@ TINY_B_INIT = dict(seed=2, std=0.05, norm_std=0.1, page_size=8)
 TINY = {"A": (TINY_A, TINY_A_INIT), "B": (TINY_B, TINY_B_INIT)}
 
 
-def make_model_dir(tmp_path_factory, name: str, sharpen: float = 1.0, std: float | None = None) -> Path:
+# The configurations' own position bounds (256 and 512) hold the workloads they are defined with; the
+# tests of tile, split and page edges run longer sequences, so their folders carry wider bounds
+# (still different from each other).  ``max_position=None`` keeps the configuration's own.
+LONG_POSITIONS = {"A": 1024, "B": 2048}
+
+
+def make_model_dir(tmp_path_factory, name: str, sharpen: float = 1.0, std: float | None = None,
+                   max_position: int | None = -1) -> Path:
     """Write tiny configuration ``name`` with random weights.  ``sharpen``
     multiplies the per-head q/k norm weights so that attention is peaked and a
     wrong key or a wrong position changes the logits visibly (the float32 path
@@ -57,6 +64,10 @@ def make_model_dir(tmp_path_factory, name: str, sharpen: float = 1.0, std: float
     import json
 
     raw, init = TINY[name]
+    if max_position == -1:
+        max_position = LONG_POSITIONS[name]
+    if max_position is not None:
+        raw = dict(raw, max_position_embeddings=max_position)
     config = Qwen3Config.from_dict(raw)
     out = tmp_path_factory.mktemp(f"tiny{name}")
     tensors = random_tensors(config, init["seed"], std or init["std"], init["norm_std"], torch.bfloat16)

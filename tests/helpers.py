@@ -6,8 +6,19 @@ from __future__ import annotations
 import numpy as np
 import torch
 
-FP32_TOL = 5e-5    # max |engine - plain| / max |plain| over a request, 32-bit path
-BF16_TOL = 4e-2    # same, bfloat16 path
+# Bounds on max |engine - plain| / max |plain| over a request.  Each is about three times the
+# largest error measured on the MI355X for the weights it is used with, so a fault that moves
+# the logits by a few times the rounding noise fails.
+FP32_TOL = 2e-5        # 32-bit path on the sharpened weights (measured up to 7e-6: peaked attention
+                       # multiplies the rounding of the scores; 1e-6 on weights as drawn)
+FP32_TOL_SOFT = 5e-6   # 32-bit path on weights as drawn and on the generation weights (measured up to 2e-6)
+BF16_TOL = 2e-2        # bfloat16 path against exact arithmetic, weights as drawn (measured up to 6e-3)
+# bfloat16 path against the plain forward that stores in bfloat16 where the engine does
+# (``store=bf16``): until the first value lands on the other side of a rounding boundary the two agree
+# to 1e-7; afterwards the difference is that of a few flipped roundings (measured up to 2.2e-2 on the
+# sharpened weights of configuration B at 700 tokens, 4e-3 on A)
+BF16_STORED_TOL = 5e-2
+BF16_EXACT_PREFIX_TOL = 1e-6   # ... and the bound while no rounding has flipped yet (the first positions)
 
 
 def rel_err(got, want) -> float:

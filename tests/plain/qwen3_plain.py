@@ -10,6 +10,18 @@ from (paths are relative to the reference checkout).
 The default precision is float64; ``dtype=torch.float32`` gives the 32-bit
 variant.  Weights are used at the values the checkpoint holds (bfloat16
 values upcast exactly), as in bench/fp64_reference.py:76-80.
+
+``store`` (optional, on the functions that take it) is applied wherever the
+engine under test keeps a value in its 16-bit compute dtype between kernels:
+the normalised rows that enter a projection, the projected q, k and v, q and
+k after norm and rotation, the probabilities that multiply the values (the
+row sum is formed from the unrounded ones, engine/kernels/attention.py:111-112),
+the attention output, the activated feed-forward rows and the final
+normalised rows.  The residual stream and the logits stay unrounded, which is
+the engine's own contract (the reference rounds its residual stream too,
+engine/model/qwen3.py:360,370).  With ``store=bf16`` the plain forward is the
+exact-arithmetic model of the bfloat16 path: what is left between the two is
+the order of sums and values that sit on a rounding boundary.
 """
 
 from __future__ import annotations
@@ -102,6 +114,15 @@ def apply_rope(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.T
     return torch.cat([lo * c - hi * s, hi * c + lo * s], dim=-1)
 
 
+def bf16(x: torch.Tensor) -> torch.Tensor:
+    """Round to the nearest bfloat16 (ties to even), kept in the input's dtype."""
+    return x.to(torch.float32).to(torch.bfloat16).to(x.dtype)
+
+
+def _keep(x: torch.Tensor) -> torch.Tensor:
+    return x
+
+
 def stable_softmax(scores: torch.Tensor) -> torch.Tensor:
     """Explicit max-subtract softmax over the last dimension
     (bench/fp64_reference.py:41-50)."""
@@ -116,6 +137,8 @@ def causal_attention(
     v: torch.Tensor,
     q_positions: torch.Tensor | None = None,
     window: int | None = None,
+    store=None,
+    also_hidden: torch.Tensor | None = None,
 ) -> torch.Tensor:
     """Grouped-query causal attention of whole sequences.
 
@@ -127,6 +150,8 @@ def causal_attention(
     ``Tk - Tq + arange(Tq)``: the queries are the tail of the keys
     (engine/kernels/attention.py:224-227).  ``window`` is not in the
     reference: when given, a key is also dropped once ``p - n >= window``.
+    ``also_hidden`` (bool ``[Tq, Tk]``, not in the reference either) hides further
+    keys: tests use it to state what a fault (a dropped key, a lost page) would give.
     """
     tq, nq, d = q.shape
     tk, nkv, _ = k.shape
@@ -140,8 +165,14 @@ def causal_attention(
     hidden = key_positions[None, :] > q_positions[:, None]
     if window is not None:
         hidden = hidden | (q_positions[:, None] - key_positions[None, :] >= window)
+    if also_hidden is not None:
+        hidden = hidden | also_hidden
     scores = scores.masked_fill(hidden[None], float("-inf"))
-    return torch.einsum("hqk,khd->qhd", stable_softmax(scores), v)
+    if store is None:
+        return torch.einsum("hqk,khd->qhd", stable_softmax(scores), v)
+    # the stored probabilities multiply the values, the unrounded ones form the row sum
+    e = (scores - scores.max(dim=-1, keepdim=True).values).exp()
+    return torch.einsum("hqk,khd->qhd", store(e), v) / e.sum(dim=-1).transpose(0, 1)[..., None]
 
 
 def swiglu(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
@@ -150,34 +181,37 @@ def swiglu(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
     return gate * torch.sigmoid(gate) * up
 
 
-def attention_block(cfg: dict, w: dict, prefix: str, x: torch.Tensor, positions: torch.Tensor):
+def attention_block(cfg: dict, w: dict, prefix: str, x: torch.Tensor, positions: torch.Tensor, store=None,
+                    window: int | None = None, also_hidden: torch.Tensor | None = None):
     """Projections, per-head q/k norm, rotation, attention, output projection
     (engine/model/qwen3.py:327-363; bench/fp64_reference.py:122-148).  The
     per-head norm uses one ``[d]`` weight for all heads, is applied to q and k
     only, and comes before the rotation."""
+    keep = store or _keep
     t = x.shape[0]
     nq, nkv, d = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
-    q = linear(x, w[f"{prefix}.q_proj.weight"]).view(t, nq, d)
-    k = linear(x, w[f"{prefix}.k_proj.weight"]).view(t, nkv, d)
-    v = linear(x, w[f"{prefix}.v_proj.weight"]).view(t, nkv, d)
+    q = keep(linear(x, w[f"{prefix}.q_proj.weight"])).view(t, nq, d)
+    k = keep(linear(x, w[f"{prefix}.k_proj.weight"])).view(t, nkv, d)
+    v = keep(linear(x, w[f"{prefix}.v_proj.weight"])).view(t, nkv, d)
     q = rmsnorm(q, w[f"{prefix}.q_norm.weight"], cfg["rms_norm_eps"])
     k = rmsnorm(k, w[f"{prefix}.k_norm.weight"], cfg["rms_norm_eps"])
     cos, sin = rope_tables(d, cfg["rope_theta"], positions)
-    q = apply_rope(q, cos, sin)
-    k = apply_rope(k, cos, sin)
-    attn = causal_attention(q, k, v, q_positions=positions - positions[0])
+    q = keep(apply_rope(q, cos, sin))
+    k = keep(apply_rope(k, cos, sin))
+    attn = keep(causal_attention(q, k, v, q_positions=positions - positions[0], window=window, store=store,
+                                 also_hidden=also_hidden))
     return linear(attn.reshape(t, nq * d), w[f"{prefix}.o_proj.weight"])
 
 
-def mlp_block(w: dict, prefix: str, x: torch.Tensor) -> torch.Tensor:
+def mlp_block(w: dict, prefix: str, x: torch.Tensor, store=None) -> torch.Tensor:
     """``down(swiglu(gate(x), up(x)))`` (engine/model/qwen3.py:368-370;
     bench/fp64_reference.py:150-153)."""
     gate = linear(x, w[f"{prefix}.gate_proj.weight"])
     up = linear(x, w[f"{prefix}.up_proj.weight"])
-    return linear(swiglu(gate, up), w[f"{prefix}.down_proj.weight"])
+    return linear((store or _keep)(swiglu(gate, up)), w[f"{prefix}.down_proj.weight"])
 
 
-def hidden_states(cfg: dict, w: dict, token_ids, dtype=torch.float64) -> torch.Tensor:
+def hidden_states(cfg: dict, w: dict, token_ids, dtype=torch.float64, store=None, also_hidden=None) -> torch.Tensor:
     """Final normalised hidden states ``[T, H]`` of one whole sequence from
     position 0: embedding, then per layer ``h += attn(norm(h))`` and
     ``h += mlp(norm(h))``, then the final norm
@@ -186,20 +220,22 @@ def hidden_states(cfg: dict, w: dict, token_ids, dtype=torch.float64) -> torch.T
     positions = torch.arange(ids.shape[0])
     h = w["model.embed_tokens.weight"][ids].to(dtype)
     eps = cfg["rms_norm_eps"]
+    keep = store or _keep
     for layer in range(cfg["num_hidden_layers"]):
         p = f"model.layers.{layer}"
-        normed = rmsnorm(h, w[f"{p}.input_layernorm.weight"], eps)
-        h = h + attention_block(cfg, w, f"{p}.self_attn", normed, positions)
-        normed = rmsnorm(h, w[f"{p}.post_attention_layernorm.weight"], eps)
-        h = h + mlp_block(w, f"{p}.mlp", normed)
-    return rmsnorm(h, w["model.norm.weight"], eps)
+        normed = keep(rmsnorm(h, w[f"{p}.input_layernorm.weight"], eps))
+        h = h + attention_block(cfg, w, f"{p}.self_attn", normed, positions, store,
+                                also_hidden=(also_hidden or {}).get(layer))
+        normed = keep(rmsnorm(h, w[f"{p}.post_attention_layernorm.weight"], eps))
+        h = h + mlp_block(w, f"{p}.mlp", normed, store)
+    return keep(rmsnorm(h, w["model.norm.weight"], eps))
 
 
-def logits(cfg: dict, w: dict, token_ids, dtype=torch.float64) -> torch.Tensor:
+def logits(cfg: dict, w: dict, token_ids, dtype=torch.float64, store=None, also_hidden=None) -> torch.Tensor:
     """Logits ``[T, V]`` at every position: ``norm(h) @ lm_head^T``, no bias
     and no scaling (engine/model/qwen3.py:372-373;
     bench/fp64_reference.py:157-164)."""
-    return linear(hidden_states(cfg, w, token_ids, dtype), w["lm_head.weight"])
+    return linear(hidden_states(cfg, w, token_ids, dtype, store, also_hidden), w["lm_head.weight"])
 
 
 class PlainModel:
@@ -210,8 +246,9 @@ class PlainModel:
         self.dtype = dtype
         self.w = read_weights(model_dir, self.cfg, dtype)
 
-    def logits(self, token_ids) -> torch.Tensor:
-        return logits(self.cfg, self.w, token_ids, self.dtype)
+    def logits(self, token_ids, store=None, also_hidden=None) -> torch.Tensor:
+        """``also_hidden``: {layer: bool [T, T]} of keys to hide from queries in that layer."""
+        return logits(self.cfg, self.w, token_ids, self.dtype, store, also_hidden)
 
     def generate_greedy(self, prompt, max_new_tokens: int, eos=()) -> list[int]:
         """Whole-sequence recomputation at every step, lowest-id tie-break

@@ -97,6 +97,44 @@ def test_state_slots_are_handed_out_lowest_first():
     c.audit()
 
 
+def test_state_is_zeroed_when_taken_poisoned_when_given_back_and_in_the_ledger():
+    import torch
+
+    def build(**kw):
+        return CacheManager([FULL, StateSpec((3,)), StateSpec((2, 2), dtype="int32")], 16, 4, max_requests=2,
+                            max_tokens_per_request=64, torch_dtype=torch.float32, device=torch.device("cpu"), **kw)
+
+    c = build(poison_on_free=True)
+    assert c.unit_state(1).dtype is torch.float32 and c.unit_state(2).dtype is torch.int32
+    c.open("a"); c.open("b")
+    c.unit_state(1)[c.slot("a")] = torch.tensor([1.0, 2.0, 3.0])
+    c.unit_state(2)[c.slot("b")] += 5
+    c.audit()
+    with_content = c.state_digest(content=True)
+    c.unit_state(1)[c.slot("a"), 0] = 9.0
+    assert c.state_digest(content=True) != with_content            # the rows of live requests are in the digest
+    assert c.state_digest() == c.state_digest()                     # ... and only when asked for
+    assert c.state_digest()[:2] == ((1, (3,), "float32"), (2, (2, 2), "int32"))
+    c.close("a")
+    assert bool(c.unit_state(1)[0].isnan().all()) and bool((c.unit_state(2)[0] == -(1 << 30)).all())
+    c.audit()
+    c.unit_state(1)[0] = 0.0                                        # someone wrote into a slot nobody owns
+    with pytest.raises(CacheAuditError, match="not poisoned"):
+        c.audit()
+    assert c.open("c") == 0 and bool((c.unit_state(1)[0] == 0).all()) and bool((c.unit_state(2)[0] == 0).all())
+    c.audit()
+    c.unit_state(1)[c.slot("b"), 1] = float("nan")                  # a live request that read poison
+    with pytest.raises(CacheAuditError, match="poisoned state"):
+        c.audit()
+    with pytest.raises(TypeError):
+        CacheManager([StateSpec((3,), dtype="float64")], 16, 4, 2, 64, torch_dtype=torch.float32,
+                     device=torch.device("cpu"))
+    quiet = build()
+    quiet.open("a"); quiet.unit_state(1)[0] = 4.0; quiet.close("a")
+    assert bool((quiet.unit_state(1)[0] == 4.0).all())              # without poisoning the row is left as it was
+    quiet.audit()
+
+
 def test_audit_catches_a_lost_a_doubled_and_a_twice_freed_page():
     # reference tests/test_paged_kv.py:67-85
     c = manager()
@@ -154,27 +192,43 @@ def test_random_orders_of_requests_keep_the_ledger_balanced(seed):
     assert c.free_pages == [24, 10] and c.free_slots == 5 and len(digests) > 50
 
 
-def test_prefix_index_shares_whole_pages_and_evicts_only_unused_ones():
+def test_prefix_index_shares_whole_pages_and_drops_only_unused_leaves():
     c = manager(num_pages=8, page_size=8, specs=(FULL,), max_tokens=64)
     index = PrefixIndex(8)
     tokens = list(range(22))
     c.open("a"); c.reserve("a", 22); c.commit("a", 22)
-    assert index.insert(tokens, c.request_pages("a"), c) == 2       # two whole pages
+    assert index.remember(tokens, c.request_pages("a"), c) == 2       # two whole pages
+    assert index.remember(tokens, c.request_pages("a"), c) == 0       # nothing new the second time
     c.close("a")
     assert c.free_pages == [6]                                        # the index still holds two
-    hit, pages = index.lookup(tokens[:16] + [99, 98])
-    assert hit == 16 and pages == [0, 1]
-    assert index.lookup([0, 1, 2, 9] + tokens[4:16])[0] == 0          # a changed first page breaks the chain
+    pages = index.match(tokens[:16] + [99, 98])
+    assert pages == [0, 1]
+    assert index.match([0, 1, 2, 9] + tokens[4:16]) == []             # a changed first page: nothing after it counts
+    assert index.match(tokens[:15]) == [0]                            # whole pages only
     c.open("b"); c.adopt("b", pages); c.commit("b", 16); c.reserve("b", 18)
     assert c.request_pages("b") == [0, 1, 2]
     c.audit()
-    assert index.evictable(c) == []                                   # b maps them
+    assert index.droppable(c) == [] and index.reclaimable(c) == 0     # b maps them
     with pytest.raises(CacheAuditError):
         c.assert_exclusive("b", 0, 0)                                 # a write into a shared page is refused
     c.assert_exclusive("b", 0, 2)
+    # b finishes with a longer context: its third page joins the chain below the shared two
+    c.commit("b", 24)
+    assert index.remember(tokens[:16] + list(range(100, 108)), c.request_pages("b"), c) == 1
     c.close("b")
-    assert index.evictable(c) == [0, 1]
-    assert index.evict(0, c) and c.free_pages == [7]
+    assert index.reclaimable(c) == 3 and index.droppable(c) == [2]    # only the leaf may go
+    assert not index.drop(0, c) and not index.drop(1, c)              # a page inside a chain stays
+    assert index.drop(2, c) and index.droppable(c) == [1]
+    assert index.drop(1, c) and index.drop(0, c) and c.free_pages == [8] and len(index) == 0
+    c.audit()
+    # two requests that computed the same first page on pages of their own share one node
+    c.open("x"); c.reserve("x", 16); c.commit("x", 16)
+    c.open("y"); c.reserve("y", 16); c.commit("y", 16)
+    assert index.remember(tokens[:16], c.request_pages("x"), c) == 2
+    assert index.remember(tokens[:8] + list(range(50, 58)), c.request_pages("y"), c) == 1
+    assert sorted(index.by_page) == [0, 1, 3] and len(index.digest()) == 3
+    c.close("x"); c.close("y")
+    assert index.droppable(c) == [1, 3]                               # both leaves; their common parent stays
     c.audit()
     windowed = manager(specs=(FULL, PagedKVSpec(2, 16, 8)))
     assert not windowed.shareable()

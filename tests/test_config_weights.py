@@ -109,8 +109,49 @@ def test_dtypes_are_normalised_not_chosen(tmp_path):
     spec = cfg.model_spec()
     store = load_weights(tmp_path, collect_weight_specs(spec), collect_ties(spec))
     assert store.get("model.norm.weight").dtype is torch.float32
-    assert store.get("model.layers.0.mlp.up_proj.weight").dtype is torch.bfloat16
+    assert store.get("model.layers.0.mlp.up_proj.weight").dtype is torch.float16  # kept as stored until it is used
     assert store.get("model.embed_tokens.weight").dtype is torch.bfloat16
+
+
+def test_a_lossy_cast_of_the_checkpoint_is_measured():
+    # reference engine/model/qwen3.py:176-216: element count, inexact count, largest errors
+    from lockstep_amd.weights.cast import CastLedger
+
+    ledger = CastLedger(torch.bfloat16)
+    stored = torch.tensor([1.0, 1.0 + 2.0 ** -10, -3.0, 0.3330078125], dtype=torch.float16)
+    used = ledger.cast(stored, torch.bfloat16)
+    assert used.dtype is torch.bfloat16
+    assert ledger.report["elements"] == 4 and ledger.report["lossy_tensors"] == 1
+    assert ledger.report["inexact_elements"] == 2                 # 1 + 2^-10 and 0.333 need more than 8 bits
+    assert ledger.report["max_abs_error"] == pytest.approx(2.0 ** -10, rel=0.5)
+    assert 0 < ledger.report["max_rel_error"] < 2.0 ** -8
+    before = dict(ledger.report)
+    assert ledger.cast(torch.ones(5, dtype=torch.bfloat16), torch.bfloat16).dtype is torch.bfloat16
+    assert ledger.report == before                                # same dtype: not a cast
+    wide = CastLedger(torch.float32)
+    assert torch.equal(wide.cast(stored, torch.float32), stored.float())
+    assert wide.report["elements"] == 4 and wide.report["lossy_tensors"] == 0 and wide.report["inexact_elements"] == 0
+    assert wide.cast(torch.tensor([3], dtype=torch.int32), torch.float32).dtype is torch.int32   # tables are left alone
+
+
+def test_the_position_bound_comes_from_the_configuration():
+    spec = Qwen3Config.from_dict(TINY_A).model_spec()
+    assert spec.max_positions == TINY_A["max_position_embeddings"] == 256
+    assert Qwen3Config.from_dict(TINY_B).model_spec().max_positions == 512
+
+
+def test_engine_config_is_typed_and_checked():
+    from lockstep_amd.engine.config import EngineConfig
+    from lockstep_amd.engine.policy import DefaultPolicy, FixedChunkPolicy
+
+    cfg = EngineConfig(page_size=8, num_pages=40, prefill_chunk=12, eos_token_ids=[3, 7])
+    assert cfg.eos_token_ids == (3, 7) and isinstance(cfg.policy(), FixedChunkPolicy) and cfg.policy().chunk == 12
+    assert isinstance(EngineConfig().policy(), DefaultPolicy) and EngineConfig().policy().max_running == 64
+    assert cfg.with_(num_pages=9).num_pages == 9 and cfg.to_dict()["page_size"] == 8
+    for bad in (dict(page_size=48), dict(dtype="float16"), dict(reserve="eager"), dict(num_pages=0),
+                dict(prefill_chunk=0), dict(decode_burst=0)):
+        with pytest.raises(ValueError):
+            EngineConfig(**bad)
 
 
 def test_one_error_lists_missing_unexpected_and_misshapen(tmp_path):

@@ -6,19 +6,23 @@ from __future__ import annotations
 import pytest
 import torch
 
-from helpers import BF16_TOL, FP32_TOL, feed, random_tokens, rel_err
+from helpers import (BF16_EXACT_PREFIX_TOL, BF16_STORED_TOL, BF16_TOL, FP32_TOL, FP32_TOL_SOFT, feed, random_tokens,
+                     rel_err)
 
 pytestmark = pytest.mark.gpu
 
 DTYPES = ["float32", "bfloat16"]
-TOL = {"float32": FP32_TOL, "bfloat16": BF16_TOL}
+# what each path is held to on the sharpened weights: the 32-bit path against exact arithmetic, the
+# bfloat16 path against the plain forward that stores in bfloat16 where the engine does
+TOL = {"float32": FP32_TOL, "bfloat16": BF16_STORED_TOL}
 
 
 @pytest.fixture(scope="module")
 def plain_logits(tiny_dirs):
-    """Plain float64 logits of the test sequences, computed once.  Keys are
-    ``name`` (the sharpened weights) and ``(name, "soft")`` (weights as drawn)."""
-    from plain.qwen3_plain import PlainModel
+    """Plain float64 logits of the test sequences, computed once.  ``[name]``: (folder, {n:
+    (tokens, exact logits, logits with bfloat16 storage)}) on the sharpened weights; ``[(name,
+    "soft")]``: (folder, {n: (tokens, exact logits)}) on the weights as drawn."""
+    from plain.qwen3_plain import PlainModel, bf16
 
     out = {}
     for name in ("A", "B"):
@@ -27,15 +31,25 @@ def plain_logits(tiny_dirs):
             plain = PlainModel(folder)
             vocab = plain.cfg["vocab_size"]
             seqs = {n: random_tokens(n, vocab, seed=100 + n) for n in (1, 7, 40, 333)}
-            out[(name, variant)] = (folder, {n: (t, plain.logits(t)) for n, t in seqs.items()})
-        out[name] = out[(name, "sharp")]
+            if variant == "sharp":
+                out[name] = (folder, {n: (t, plain.logits(t), plain.logits(t, store=bf16)) for n, t in seqs.items()})
+            else:
+                out[(name, variant)] = (folder, {n: (t, plain.logits(t)) for n, t in seqs.items()})
     out["gen"] = {name: tiny_dirs[(name, "gen")] for name in ("A", "B")}
     return out
 
 
-def for_plain(plain_logits, name, dtype):
-    """The weights on which ``dtype`` is compared with the plain implementation."""
-    return plain_logits[(name, "sharp" if dtype == "float32" else "soft")]
+def want_for(entry, dtype):
+    """The plain logits a path is compared with on the sharpened weights."""
+    return entry[1] if dtype == "float32" else entry[2]
+
+
+def plain_of(folder, dtype):
+    """tokens -> plain logits as ``dtype`` is compared with them."""
+    from plain.qwen3_plain import PlainModel, bf16
+
+    plain = PlainModel(folder)
+    return plain, (lambda tokens: plain.logits(tokens, store=None if dtype == "float32" else bf16))
 
 
 def load(folder, dtype):
@@ -47,16 +61,62 @@ def load(folder, dtype):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name,page_size", [("A", 16), ("B", 8)])
 def test_whole_prompts_match_plain(plain_logits, dtype, name, page_size):
-    folder, seqs = for_plain(plain_logits, name, dtype)
+    folder, seqs = plain_logits[name]
     model = load(folder, dtype)
     cache = model.make_cache(num_pages=64, page_size=page_size, poison_on_free=True)
-    for n, (tokens, want) in seqs.items():
-        got = feed(model, cache, f"r{n}", tokens, [])
-        err = rel_err(got, want)
+    for n, entry in seqs.items():
+        got = feed(model, cache, f"r{n}", entry[0], [])
+        err = rel_err(got, want_for(entry, dtype))
         print(f"{name} {dtype} whole n={n}: rel err {err:.3e}")
         assert err < TOL[dtype], f"n={n}"
+        if dtype == "bfloat16" and n == 1:         # nothing can have flipped yet: the stored forward is exact
+            assert err < BF16_EXACT_PREFIX_TOL
         cache.close(f"r{n}")
     cache.audit()
+    # the weights as drawn: the 32-bit path at its tightest, the bfloat16 path against exact arithmetic
+    folder, seqs = plain_logits[(name, "soft")]
+    model = load(folder, dtype)
+    cache = model.make_cache(num_pages=64, page_size=page_size)
+    for n, (tokens, want) in seqs.items():
+        err = rel_err(feed(model, cache, f"s{n}", tokens, []), want)
+        print(f"{name} {dtype} whole n={n}, weights as drawn: rel err {err:.3e}")
+        assert err < (FP32_TOL_SOFT if dtype == "float32" else BF16_TOL), f"n={n}"
+        cache.close(f"s{n}")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name,page_size", [("A", 16), ("B", 8)])
+def test_a_lost_far_page_or_key_would_show(plain_logits, dtype, name, page_size):
+    """700 tokens (three splits of the keys) on the sharpened weights.  The plain forward states what
+    a fault would give -- a far page hidden from the last 64 queries in every layer, the same in the
+    first layer only, a single far key hidden -- and the engine has to lie far closer to the
+    faultless logits than any of them does, in 32-bit and, against the forward that stores in
+    bfloat16, in bfloat16."""
+    folder, _ = plain_logits[name]
+    plain, reference = plain_of(folder, dtype)
+    store = None if dtype == "float32" else __import__("plain.qwen3_plain", fromlist=["bf16"]).bf16
+    n, tail = 700, 64
+    tokens = random_tokens(n, plain.cfg["vocab_size"], seed=100 + n)
+    good = reference(tokens)
+    layers = plain.cfg["num_hidden_layers"]
+    page = {"A": 2, "B": 16}[name]                      # far behind the last queries, inside the first split
+
+    def faulty(keys, where):
+        hide = torch.zeros(n, n, dtype=torch.bool)
+        hide[-tail:, keys] = True
+        return rel_err(plain.logits(tokens, store=store, also_hidden={l: hide for l in where})[-tail:], good[-tail:])
+
+    lost_page = faulty(slice(page * page_size, (page + 1) * page_size), range(layers))
+    lost_page_one_layer = faulty(slice(page * page_size, (page + 1) * page_size), [0])
+    lost_key = faulty(slice(page * page_size + 3, page * page_size + 4), range(layers))
+    model = load(folder, dtype)
+    cache = model.make_cache(num_pages=-(-n // page_size) + 2, page_size=page_size, poison_on_free=True)
+    got = feed(model, cache, "far", tokens, [n - tail] + [1] * tail)     # the last queries as decoded tokens
+    err = rel_err(got[-tail:], good[-tail:])
+    print(f"{name} {dtype}: engine {err:.2e}; a lost page {lost_page:.2e}, in one layer {lost_page_one_layer:.2e}, "
+          f"a lost key {lost_key:.2e}")
+    assert err < TOL[dtype]
+    assert lost_page > 3 * TOL[dtype] and lost_page_one_layer > 3 * err and lost_key > 3 * err
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -67,11 +127,10 @@ def test_cuttings_give_the_same_bits(plain_logits, dtype, name, page_size):
     folder, seqs = plain_logits[name]
     model = load(folder, dtype)
     cache = model.make_cache(num_pages=64, page_size=page_size, poison_on_free=True)
-    tokens, want = seqs[333]
+    tokens = seqs[333][0]
     whole = feed(model, cache, "whole", tokens, [])
     cache.close("whole")
-    if dtype == "float32":
-        assert rel_err(whole, want) < TOL[dtype]
+    assert rel_err(whole, want_for(seqs[333], dtype)) < TOL[dtype]
     cuttings = {
         "last32": [len(tokens) - 32] + [1] * 32,
         "ragged": [7, 17, 37, 2, 64, 3, 129, 2],
@@ -97,10 +156,9 @@ def test_mixed_batches_with_reused_pages(plain_logits, dtype, name, page_size):
     between): every request's logits equal its whole run bit for bit and the
     plain implementation within tolerance."""
     from helpers import make_mixed_trace, max_live_tokens, replay_in_process
-    from plain.qwen3_plain import PlainModel
 
-    folder, _ = for_plain(plain_logits, name, dtype)
-    plain = PlainModel(folder)
+    folder, _ = plain_logits[name]
+    plain, reference = plain_of(folder, dtype)
     vocab = plain.cfg["vocab_size"]
     lengths = [70, 45, 33, 90, 21, 64, 130, 17]
     requests = {f"q{i}": random_tokens(n, vocab, seed=500 + i) for i, n in enumerate(lengths)}
@@ -119,21 +177,19 @@ def test_mixed_batches_with_reused_pages(plain_logits, dtype, name, page_size):
         whole = feed(model, roomy, rid, tokens, [])
         roomy.close(rid)
         assert torch.equal(got[rid], whole), f"{rid}: mixed run differs from the whole run"
-        assert rel_err(got[rid], plain.logits(tokens)) < TOL[dtype], rid
+        assert rel_err(got[rid], reference(tokens)) < TOL[dtype], rid
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_long_decoding_matches_plain(plain_logits, dtype):
     """Forty tokens at once, then three hundred one by one (past two splits of the keys)."""
-    from plain.qwen3_plain import PlainModel
-
-    folder, _ = for_plain(plain_logits, "B", dtype)
-    plain = PlainModel(folder)
+    folder, _ = plain_logits["B"]
+    plain, reference = plain_of(folder, dtype)
     tokens = random_tokens(340, plain.cfg["vocab_size"], seed=77)
     model = load(folder, dtype)
     cache = model.make_cache(num_pages=48, page_size=8, poison_on_free=True)
     got = feed(model, cache, "long", tokens, [40] + [1] * 300)
-    err = rel_err(got, plain.logits(tokens))
+    err = rel_err(got, reference(tokens))
     print(f"long decode {dtype}: rel err {err:.3e}")
     assert err < TOL[dtype]
 
@@ -166,7 +222,7 @@ def test_greedy_generation_through_the_entry_points(plain_logits, name, page_siz
     half = LLM(folder, dtype="bfloat16", num_pages=64, page_size=page_size, audit=True)
     base = half.generate(requests())
     assert half.generate(requests(), policy=FixedChunkPolicy(12)) == base
-    half.options["max_batched_tokens"] = 20
+    half.config = half.config.with_(max_batched_tokens=20)
     assert half.generate(requests(), policy=FixedChunkPolicy(5)) == base
     assert half.generate(requests()[1:2]) == {"r1": base["r1"]}
     # decode steps in bursts on the GPU (no audit, default policy): the same tokens, float32 and bfloat16
@@ -209,7 +265,7 @@ def test_decode_steps_from_a_captured_graph_equal_eager_steps(plain_logits, dtyp
     from lockstep_amd.engine.batch import StepEntry
 
     folder, seqs = plain_logits["B"]
-    tokens, _ = seqs[333]
+    tokens = seqs[333][0]
     other = random_tokens(50, 1000, seed=4)
     eager = load(folder, dtype)
     eager.use_graphs = False
@@ -280,8 +336,8 @@ def test_the_first_tokens_of_a_sequence(plain_logits, dtype, name, page_size):
     """A sequence decoded one by one from its very first token (position 0 has one key, the first
     page and the first tile are being filled): right against the plain implementation, and the
     same bits as the whole prompt in one step."""
-    folder, seqs = for_plain(plain_logits, name, dtype)
-    tokens, want = seqs[40]
+    folder, seqs = plain_logits[name]
+    tokens, want = seqs[40][0], want_for(seqs[40], dtype)
     model = load(folder, dtype)
     cache = model.make_cache(num_pages=16, page_size=page_size, poison_on_free=True)
     whole = feed(model, cache, "whole", tokens, [])
@@ -292,8 +348,7 @@ def test_the_first_tokens_of_a_sequence(plain_logits, dtype, name, page_size):
     assert rel_err(stepwise[:3], want[:3]) < TOL[dtype]
     assert rel_err(stepwise, want) < TOL[dtype]
     assert torch.equal(stepwise, whole) and torch.equal(pair, whole)
-    one_folder, one_seqs = for_plain(plain_logits, name, dtype)
-    single, single_want = one_seqs[1]
+    single, single_want = seqs[1][0], want_for(seqs[1], dtype)
     cache.close("pair")
     assert rel_err(feed(model, cache, "one", single, []), single_want) < TOL[dtype]
 

@@ -11,7 +11,7 @@ from __future__ import annotations
 import pytest
 import torch
 
-from helpers import BF16_TOL, FP32_TOL, feed, random_tokens, rel_err
+from helpers import BF16_TOL, FP32_TOL_SOFT, feed, random_tokens, rel_err
 
 pytestmark = pytest.mark.gpu
 
@@ -127,7 +127,7 @@ def test_the_32_bit_path_matches_plain_at_real_layer_sizes(models):
     folder, config = models["0.6b-like"]
     tokens = random_tokens(300, config.vocab_size, seed=9)
     want = PlainModel(folder).logits(tokens)
-    for dtype, tol in (("float32", FP32_TOL), ("bfloat16", BF16_TOL)):
+    for dtype, tol in (("float32", FP32_TOL_SOFT), ("bfloat16", BF16_TOL)):
         model = load(folder, dtype)
         cache = model.make_cache(num_pages=40, page_size=16)
         got = feed(model, cache, "a", tokens, [270] + [1] * 30)

@@ -208,3 +208,44 @@ def test_tied_head_refuses_a_differing_tensor(tmp_path):
     save_file(w, str(folder / "model.safetensors"))
     with pytest.raises(ValueError):
         P.PlainModel(folder)
+
+
+def test_bf16_rounds_to_nearest_even_and_stays_in_the_dtype():
+    x = torch.tensor([1.0, 1.0 + 2.0 ** -8, 1.0 + 3 * 2.0 ** -8, 1.0 + 2.0 ** -7, -0.1, 3e38], dtype=torch.float64)
+    y = P.bf16(x)
+    assert y.dtype is torch.float64
+    # 1 + 2^-8 lies halfway between 1 and 1 + 2^-7: the even neighbour (1) wins; 1 + 3*2^-8 goes up to 1 + 2^-6
+    assert y[:4].tolist() == [1.0, 1.0, 1.0 + 2.0 ** -6, 1.0 + 2.0 ** -7]
+    assert y[4] == torch.tensor(-0.1).to(torch.bfloat16).double() and torch.isfinite(y[5])
+
+
+def test_stored_probabilities_multiply_the_values_and_unrounded_ones_form_the_sum():
+    # reference engine/kernels/attention.py:111-112: l sums p, the product uses p in the value dtype
+    q = torch.randn(6, 2, 8, dtype=torch.float64)
+    k = torch.randn(6, 1, 8, dtype=torch.float64)
+    v = torch.randn(6, 1, 8, dtype=torch.float64)
+    exact = P.causal_attention(q, k, v)
+    assert torch.equal(P.causal_attention(q, k, v, store=lambda t: t), exact) or \
+        torch.allclose(P.causal_attention(q, k, v, store=lambda t: t), exact, atol=1e-15)
+    stored = P.causal_attention(q, k, v, store=P.bf16)
+    assert 0 < float((stored - exact).abs().max()) < 2.0 ** -7
+    assert torch.equal(stored[0], v[0].expand(2, 8))              # one visible key: p = 1 is stored exactly
+    # the rows of the stored probabilities do not sum to one; dividing by the stored sum instead would show
+    scores = torch.einsum("qhd,khd->hqk", q, k.repeat_interleave(2, 1)) / math.sqrt(8)
+    scores = scores.masked_fill(torch.triu(torch.ones(6, 6, dtype=torch.bool), 1)[None], float("-inf"))
+    e = (scores - scores.max(-1, keepdim=True).values).exp()
+    wrong = torch.einsum("hqk,khd->qhd", P.bf16(e) / P.bf16(e).sum(-1, keepdim=True), v.repeat_interleave(2, 1))
+    assert float((wrong - stored).abs().max()) > 1e-5
+
+
+def test_hidden_keys_state_what_a_dropped_key_would_give():
+    q = torch.randn(5, 2, 8, dtype=torch.float64)
+    k = torch.randn(5, 2, 8, dtype=torch.float64)
+    v = torch.randn(5, 2, 8, dtype=torch.float64)
+    hide = torch.zeros(5, 5, dtype=torch.bool)
+    hide[3:, 1] = True                                              # queries 3 and 4 do not see key 1
+    out = P.causal_attention(q, k, v, also_hidden=hide)
+    assert torch.equal(out[:3], P.causal_attention(q, k, v)[:3])
+    keep = [0, 2, 3, 4]
+    want = P.causal_attention(q[3:], k[keep], v[keep], q_positions=torch.tensor([2, 3]))
+    assert torch.allclose(out[3:], want, atol=1e-14)

@@ -164,7 +164,7 @@ def test_lazy_reservation_preempts_the_newest_and_recomputes():
     out, s, model = run(reqs(ps, n=12), num_blocks=8, block_size=8, reserve="lazy", policy=Eager())
     assert out == want
     assert s.counters["preempt_for_pages"] > 0 and s.counters["resume"] > 0
-    assert any(r.preempt_count for r in s.done)
+    assert any(r.preemptions for r in s.done)
     s.cache.audit()
     assert s.cache.free_pages == [8]
 
@@ -187,7 +187,7 @@ def test_scripted_preemption_leaves_tokens_unchanged():
         out, s, _ = run(reqs(ps, n=8), policy=PreemptAtStepsPolicy("r0", steps, chunk=7))
         assert out == want
         assert s.counters["preempt_fired"] == len(steps) and s.counters["resume"] == len(steps)
-        assert [r.preempt_count for r in s.done if r.uid == "r0"] == [len(steps)]
+        assert [r.preemptions for r in s.done if r.uid == "r0"] == [len(steps)]
         assert Event.PREEMPT in s.lifecycle["r0"] and Event.RESUME in s.lifecycle["r0"]
 
 
@@ -206,7 +206,7 @@ def test_prefix_index_hits_trims_a_whole_prompt_hit_and_evicts_under_pressure():
         model.prompts[r.uid] = list(r.prompt); s.submit(r)
     s.run()
     done = {r.uid: r for r in s.done}
-    assert done["b"].cache_hit_tokens == 32 and done["c"].cache_hit_tokens == 24
+    assert done["b"].reused == 32 and done["c"].reused == 24
     assert s.counters["cache_hit"] == 2 and s.counters["cache_full_prompt_trimmed"] == 1
     assert done["b"].generated == expected_greedy(b.prompt, 4)
     assert done["c"].generated == expected_greedy(c.prompt, 4)
@@ -303,3 +303,54 @@ def test_decode_bursts_change_neither_tokens_nor_counts():
     many = [Request(uid=f"w{i}", prompt=ps[0], max_new_tokens=8) for i in range(3)]
     out, s3, m3 = run(many, audit=False, decode_burst=16, policy=None, num_blocks=2)   # pages for two at a time
     assert out == {f"w{i}": expected_greedy(ps[0], 8) for i in range(3)}
+
+
+def test_a_request_beyond_the_models_last_position_is_refused():
+    class Bounded(StandInModel):
+        class spec:                      # what the scheduler reads of a model
+            max_positions = 40
+
+    s = Scheduler(Bounded(), num_blocks=64)
+    s.submit(Request(uid="fits", prompt=[1] * 30, max_new_tokens=10))
+    with pytest.raises(OversizedRequest, match="positions end at 40"):
+        s.submit(Request(uid="long", prompt=[1] * 30, max_new_tokens=11))
+    assert s.counters["position_limit"] == 1 and [q.uid for q in s.waiting] == ["fits"]
+
+
+def test_policies_are_put_together_from_rules():
+    from lockstep_amd.engine.policy import AtSteps, EveryTokens, Listed, Policy
+
+    ps = prompts(9, 23)
+    want = {f"r{i}": expected_greedy(p, 8) for i, p in enumerate(ps)}
+    rule = AtSteps([("r0", 3), ("r0", 7), ("r1", 1)])     # r1 has produced nothing at step 1: it is not asked about
+    out, s, model = run(reqs(ps, n=8), policy=Policy(portion=EveryTokens(5), preemption=rule))
+    assert out == want and rule.fired == [("r0", 3), ("r0", 7)] and s.counters["preempt_fired"] == 2
+    assert all(n <= 5 for b in model.batches for _, _, n in b)
+    assert not Policy(preemption=rule).same_answers_every_step()
+    assert not Policy(portion=Listed([3])).same_answers_every_step()
+    assert Policy(portion=EveryTokens(5)).same_answers_every_step() and FixedChunkPolicy(7).same_answers_every_step()
+
+    class Own(DefaultPolicy):
+        def chunk_boundary(self, view, uid, remaining):
+            return 1
+
+    assert not Own().same_answers_every_step()
+    with pytest.raises(ValueError, match="between 1 and"):
+        run(reqs(ps), policy=Policy(portion=lambda view, uid, remaining: remaining + 1))
+
+
+def test_the_ledger_names_what_differs_between_two_runs():
+    from lockstep_amd.engine.audit import StepLedger
+
+    def ledger(logits=b"abc", state=(1, 2), steps=3):
+        out = StepLedger()
+        for i in range(steps):
+            out.observe_step(i, [("r", [i], i)], [("r", i)], logits if i == 1 else b"same", state)
+        return out
+
+    a = ledger()
+    assert a.first_difference(ledger()) is None and a.hexdigest() == ledger().hexdigest()
+    assert a.first_difference(ledger(logits=b"abd")) == (1, ("logits",))
+    assert a.first_difference(ledger(state=(1, 3))) == (0, ("state",))
+    assert a.first_difference(ledger(steps=2)) == (2, ("length",)) and a.first_divergence(ledger(steps=2)) == 2
+    assert len(set(a.per_step)) == 3

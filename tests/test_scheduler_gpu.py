@@ -1,0 +1,184 @@
+"""The schedules that only a real model can check: pages adopted from the prefix index and
+read by the attention kernels, preemption with recomputation, lazy reservation with preemption
+for pages -- each with freed pages poisoned, a pool small enough that pages are used again, and
+the logits every token was picked from compared bit for bit with the request run alone
+(reference harness/mr/state.py:174-216 and harness/mr/relations.py: outputs do not depend on
+cache hits, preemption depth or cohabitants, and every relation shows that its mechanism fired)."""
+
+from __future__ import annotations
+
+import pytest
+import torch
+
+from helpers import FP32_TOL_SOFT, random_tokens, rel_err
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = ["float32", "bfloat16"]
+CASES = [("A", 16), ("B", 8)]
+
+
+def load(folder, dtype):
+    from lockstep_amd.engine.model import load_model
+
+    return load_model(folder, dtype=dtype)
+
+
+def alone(model, request, page_size):
+    """Tokens and the logit rows they were picked from, for the request on its own."""
+    from lockstep_amd import Request, Scheduler
+
+    s = Scheduler(model, num_blocks=-(-(len(request.prompt) + request.max_new_tokens) // page_size) + 1,
+                  block_size=page_size, keep_logits=True, audit=False)
+    s.submit(Request(**vars(request)))
+    return s.run()[request.uid], torch.stack(s.emitted_logits[request.uid])
+
+
+def serve(model, requests, page_size, num_pages, **options):
+    from lockstep_amd import Scheduler
+
+    cache = model.make_cache(num_pages=num_pages, page_size=page_size, max_requests=8, poison_on_free=True)
+    s = Scheduler(model, num_blocks=num_pages, block_size=page_size, cache=cache, keep_logits=True, audit=True,
+                  **options)
+    out = {}
+    for wave in requests:
+        for r in wave:
+            s.submit(r)
+        out.update(s.run())
+    return out, s
+
+
+def check(model, waves, out, s, page_size, plain=None):
+    for wave in waves:
+        for r in wave:
+            tokens, rows = alone(model, r, page_size)
+            assert out[r.uid] == tokens, r.uid
+            assert torch.equal(torch.stack(s.emitted_logits[r.uid]), rows), r.uid
+            if plain is not None:                      # float32: the plain implementation's logits at the same places
+                want = plain.logits(list(r.prompt) + tokens)[len(r.prompt) - 1: -1]
+                assert rel_err(rows.cpu(), want) < FP32_TOL_SOFT, r.uid
+    s.cache.audit()
+    assert s.cache.free_slots == s.cache.max_requests
+
+
+def plain_for(folder, dtype):
+    if dtype != "float32":
+        return None
+    from plain.qwen3_plain import PlainModel
+
+    return PlainModel(folder)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name,page_size", CASES)
+def test_prefix_hits_read_adopted_pages_and_evict_under_pressure(tiny_dirs, dtype, name, page_size):
+    """A second wave shares two to five whole pages with finished requests (one prompt is indexed
+    whole and gives its last page back); a third wave needs the indexed pages' room."""
+    from lockstep_amd import Request
+
+    folder = tiny_dirs[(name, "gen")]
+    model = load(folder, dtype)
+    vocab = model.spec.vocab_size
+    base = random_tokens(5 * page_size, vocab, seed=31)
+    first = [Request(uid="a0", prompt=base + random_tokens(3, vocab, seed=32), max_new_tokens=6),
+             Request(uid="a1", prompt=random_tokens(2 * page_size + 5, vocab, seed=33), max_new_tokens=5)]
+    second = [Request(uid="b0", prompt=base[: 2 * page_size] + random_tokens(7, vocab, seed=34), max_new_tokens=6),
+              Request(uid="b1", prompt=base + random_tokens(page_size + 1, vocab, seed=35), max_new_tokens=4),
+              Request(uid="b2", prompt=list(base[: 3 * page_size]), max_new_tokens=5),       # indexed whole
+              Request(uid="b3", prompt=base[: 4 * page_size] + [1, 2], max_new_tokens=3, temperature=0.7, seed=5)]
+    third = [Request(uid="c0", prompt=random_tokens(18 * page_size, vocab, seed=36), max_new_tokens=4)]
+    waves = [first, second, third]
+    out, s = serve(model, waves, page_size, num_pages=26, enable_prefix_cache=True)
+    s.counters.require_fired("cache_hit", "cache_insert", "cache_full_prompt_trimmed", "eviction_taken")
+    reused = {q.uid: q.reused for q in s.done}
+    assert reused["b0"] == 2 * page_size and reused["b1"] == 5 * page_size
+    assert reused["b2"] == 2 * page_size and reused["b3"] == 4 * page_size and reused["c0"] == 0
+    assert s.cache.groups[0].pool.taken_total > 26                 # pages were used again
+    check(model, waves, out, s, page_size, plain_for(folder, dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name,page_size", CASES)
+def test_preempted_requests_recompute_to_the_same_bits(tiny_dirs, dtype, name, page_size):
+    """One request is preempted one to three times while others run beside it; it comes back to
+    the head of the queue, its context (prompt and what it has generated) runs again in portions,
+    and every later token comes from the same logits."""
+    from lockstep_amd import Request
+    from lockstep_amd.engine.policy import PreemptAtStepsPolicy
+
+    folder = tiny_dirs[(name, "gen")]
+    model = load(folder, dtype)
+    vocab = model.spec.vocab_size
+    wave = [Request(uid="p0", prompt=random_tokens(2 * page_size + 3, vocab, seed=41), max_new_tokens=14),
+            Request(uid="p1", prompt=random_tokens(37, vocab, seed=42), max_new_tokens=9),
+            Request(uid="p2", prompt=random_tokens(5, vocab, seed=43), max_new_tokens=12, temperature=0.9, seed=7)]
+    plain = plain_for(folder, dtype)
+    for steps in ((5,), (5, 9), (5, 8, 12)):
+        fresh = [[Request(**vars(r)) for r in wave]]
+        policy = PreemptAtStepsPolicy("p0", steps, chunk=page_size + 3)
+        out, s = serve(model, fresh, page_size, num_pages=24, policy=policy, max_batched_tokens=40)
+        s.counters.require_fired("preempt_fired", "resume", "prefill_chunk", "decode_step")
+        assert s.counters["preempt_fired"] == len(steps) and policy.fired_at == list(steps)
+        assert {q.uid: q.preemptions for q in s.done}["p0"] == len(steps)
+        check(model, fresh, out, s, page_size, plain if len(steps) == 3 else None)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name,page_size", CASES)
+def test_lazy_reservation_preempts_for_pages_and_gives_the_same_bits(tiny_dirs, dtype, name, page_size):
+    """Pages are taken step by step from a pool that cannot hold every request to its end: the
+    request that started last is preempted when another cannot grow, and recomputed later."""
+    from lockstep_amd import Request
+    from lockstep_amd.engine.policy import Policy
+
+    folder = tiny_dirs[(name, "gen")]
+    model = load(folder, dtype)
+    vocab = model.spec.vocab_size
+    wave = [[Request(uid=f"z{i}", prompt=random_tokens(n, vocab, seed=50 + i), max_new_tokens=3 * page_size)
+             for i, n in enumerate((2 * page_size - 1, page_size + 2, 3 * page_size))]]
+    # admit on what the prompt needs now; growth is found out later
+    eager = Policy(admission=lambda view, uid, pages: len(view.running) < 3 and view.free_pages >= 3)
+    out, s = serve(model, wave, page_size, num_pages=11, reserve="lazy", policy=eager)
+    s.counters.require_fired("preempt_for_pages", "resume")
+    assert any(q.preemptions for q in s.done) and s.cache.free_pages == [11]
+    assert s.cache.groups[0].pool.taken_total > 11
+    check(model, wave, out, s, page_size, plain_for(folder, dtype))
+
+
+def test_replayed_decode_steps_are_checked_against_eager_ones(tiny_dirs, monkeypatch):
+    """With LOCKSTEP_VERIFY_GRAPHS every replayed step graph is followed by the same step run
+    eagerly and the two sets of logits must be equal bit for bit; a serving run passes it."""
+    from lockstep_amd import Request
+
+    monkeypatch.setenv("LOCKSTEP_VERIFY_GRAPHS", "1")
+    model = load(tiny_dirs[("B", "gen")], "bfloat16")
+    assert model.verify_graphs
+    wave = [[Request(uid=f"v{i}", prompt=random_tokens(n, 1000, seed=60 + i), max_new_tokens=20)
+             for i, n in enumerate((3, 40, 9, 120))]]
+    out, s = serve(model, wave, 8, num_pages=40)
+    assert model.graph_replays > 10 and all(len(t) == 20 for t in out.values())
+
+
+def test_the_position_bound_is_enforced_by_the_step_and_by_submit(tmp_path_factory):
+    """Tiny configuration A with its own bound of 256 positions."""
+    from conftest import make_model_dir
+    from lockstep_amd import OversizedRequest, Request, Scheduler, StepEntry
+
+    model = load(make_model_dir(tmp_path_factory, "A", max_position=None), "float32")
+    assert model.spec.max_positions == 256
+    cache = model.make_cache(num_pages=40, page_size=16, max_requests=2)
+    cache.open("r")
+    assert model.step(cache, [StepEntry("r", random_tokens(255, 512, seed=1), [254])]).shape == (1, 512)
+    assert model.step(cache, [StepEntry("r", [5], [0])]).shape == (1, 512)           # position 255: the last one
+    with pytest.raises(ValueError, match="positions end at 256"):
+        model.step(cache, [StepEntry("r", [6], [0])])
+    assert cache.length("r") == 256
+    cache.open("q")
+    model.step(cache, [StepEntry("q", random_tokens(250, 512, seed=2), [249])])
+    with pytest.raises(ValueError, match="positions end at 256"):
+        model.decode_greedy(cache, ["q"], [3], 7)
+    s = Scheduler(model, num_blocks=32)
+    with pytest.raises(OversizedRequest, match="positions end at 256"):
+        s.submit(Request(uid="x", prompt=[1] * 250, max_new_tokens=7))
+    s.submit(Request(uid="y", prompt=[1] * 250, max_new_tokens=6))
+    assert len(s.run()["y"]) == 6
