@@ -42,6 +42,10 @@
 #error "compile with -DLS_HEAD_DIM=<head size, a multiple of 16>"
 #endif
 
+#ifdef LS_MUTANTS
+__device__ int ls_mutants_dev = 0;  // external linkage: the compiler must not assume it stays zero
+#endif
+
 namespace ls {
 
 constexpr int D = LS_HEAD_DIM;
@@ -1568,6 +1572,18 @@ __global__ __launch_bounds__(256) void combine_kernel(const SeqMeta* __restrict_
   // The partial results of several splits are requested together (a request far away has many splits and
   // the fold of each waits for its loads); they are folded in ascending order all the same.
   constexpr int BATCH = DB <= 8 ? 4 : 2;
+  if (LS_MUTANT_DEVICE(kMutantReversedFold)) {
+    for (int s = item.n_splits - 1; s >= 0; --s) {
+      f32x4 acc[DB];
+      const long pr = pr0 + s;
+#pragma unroll
+      for (int blk = 0; blk < DB; ++blk)
+        acc[blk] = *reinterpret_cast<const f32x4*>(part_acc + pr * D + blk * 16 + 4 * g);
+      fold_split<T>(run, acc, part_ml[pr * 2], part_ml[pr * 2 + 1]);
+    }
+    store_output<T>(run, out + (long)(item.q_off + qi) * ldo + (long)head * D, g);
+    return;
+  }
   for (int s0 = 0; s0 < item.n_splits; s0 += BATCH) {
     f32x4 acc[BATCH][DB];
     float m[BATCH], l[BATCH];
@@ -1590,6 +1606,7 @@ __global__ __launch_bounds__(256) void combine_kernel(const SeqMeta* __restrict_
 }  // namespace ls
 
 LS_DEFINE_ERROR_API
+LS_DEFINE_MUTANT_API
 
 using namespace ls;
 

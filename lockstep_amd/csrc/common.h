@@ -339,6 +339,38 @@ inline int check_launch(const char* what) {
 #define LS_DEFINE_ERROR_API \
   extern "C" const char* ls_last_error() { return ls::g_error; }
 
+// Positive controls.  A library built with -DLS_MUTANTS (the tests build one beside the product
+// library, under a name of its own) carries deliberately wrong variants of a few reductions, each
+// switched on by a bit of a mask that ls_set_mutants() sets: variants whose summation order
+// depends on how many rows or work items a launch has.  They exist so that the tests of batch
+// independence can be shown to fail when the property is broken.  Without the define the
+// conditions below are constant false and nothing of this is in the product library.
+namespace ls {
+// bits of the mask, core library
+constexpr int kMutantKsliceByRows = 1;  // the skinny product cuts K into other slices above 16 rows
+constexpr int kMutantNormByRows = 2;    // RMSNorm adds its wave sums in another order in launches of more than four rows
+// bits of the mask, attention libraries
+constexpr int kMutantReversedFold = 1;  // the combine kernel folds the splits from the last to the first
+}  // namespace ls
+#ifdef LS_MUTANTS
+namespace ls {
+inline int g_mutants = 0;  // host-side copy of the mask
+}
+#define LS_MUTANT_HOST(bit) ((ls::g_mutants & (bit)) != 0)
+#define LS_MUTANT_DEVICE(bit) ((ls_mutants_dev & (bit)) != 0)
+#define LS_DEFINE_MUTANT_API                                                                       \
+  extern "C" int ls_set_mutants(int mask) {                                                        \
+    ls::g_mutants = mask;                                                                          \
+    hipError_t e = hipMemcpyToSymbol(HIP_SYMBOL(ls_mutants_dev), &mask, sizeof(int));              \
+    if (e != hipSuccess) return ls::fail("set_mutants: %s", hipGetErrorString(e));                 \
+    return 0;                                                                                      \
+  }
+#else
+#define LS_MUTANT_HOST(bit) false
+#define LS_MUTANT_DEVICE(bit) false
+#define LS_DEFINE_MUTANT_API
+#endif
+
 #define LS_REQUIRE(cond, ...)                   \
   do {                                          \
     if (!(cond)) return ls::fail(__VA_ARGS__);  \

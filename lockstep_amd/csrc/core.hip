@@ -10,6 +10,10 @@
 #include "common.h"
 #include "core_api.h"
 
+#ifdef LS_MUTANTS
+__device__ int ls_mutants_dev = 0;  // external linkage: the compiler must not assume it stays zero
+#endif
+
 namespace ls {
 
 // ---------------------------------------------------------------------------
@@ -70,7 +74,9 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ 
     part = wave_sum(part);
     if ((threadIdx.x & 63) == 0) wave_part[threadIdx.x >> 6] = part;
     __syncthreads();
-    const float total = ((wave_part[0] + wave_part[1]) + wave_part[2]) + wave_part[3];
+    float total = ((wave_part[0] + wave_part[1]) + wave_part[2]) + wave_part[3];
+    if (LS_MUTANT_DEVICE(kMutantNormByRows) && gridDim.x > 4)
+      total = ((wave_part[3] + wave_part[2]) + wave_part[1]) + wave_part[0];
     const float scale = 1.0f / sqrtf(total / (float)width + eps);
 #pragma unroll
     for (int c = 0; c < KEEP; ++c) {
@@ -92,7 +98,9 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ 
   float part = wave_sum(row_sumsq_part(src, width, threadIdx.x, vec_ok));
   if ((threadIdx.x & 63) == 0) wave_part[threadIdx.x >> 6] = part;
   __syncthreads();
-  const float total = ((wave_part[0] + wave_part[1]) + wave_part[2]) + wave_part[3];
+  float total = ((wave_part[0] + wave_part[1]) + wave_part[2]) + wave_part[3];
+  if (LS_MUTANT_DEVICE(kMutantNormByRows) && gridDim.x > 4)
+    total = ((wave_part[3] + wave_part[2]) + wave_part[1]) + wave_part[0];
   const float scale = 1.0f / sqrtf(total / (float)width + eps);
   for (int e = threadIdx.x; e < width; e += 256) dst[e] = from_f32<T>((src[e] * scale) * weight[e]);
 }
@@ -450,6 +458,7 @@ __global__ __launch_bounds__(256) void advance_decode_kernel(int* __restrict__ m
 }  // namespace ls
 
 LS_DEFINE_ERROR_API
+LS_DEFINE_MUTANT_API
 
 using namespace ls;
 

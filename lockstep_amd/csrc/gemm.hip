@@ -829,7 +829,8 @@ inline int compute_units() {
 template <typename T, int EPI>
 int launch_gemm(const void* X, const void* W, void* C, int M, int N, int K, long ldx, long ldc, const float* norm_w,
                 float eps, int out_cols, hipStream_t stream) {
-  const int kslice = kslice_for(K);
+  int kslice = kslice_for(K);
+  if (LS_MUTANT_HOST(kMutantKsliceByRows) && M > 16 && M <= 64) kslice *= 2;  // the mutant: K blocking that depends on the rows of the launch
   const int nslices = (K + kslice - 1) / kslice;
   constexpr int VEC = Atom<T>::VEC;
   constexpr int NT = (EPI == kSwiGLU) ? 2 : 1;

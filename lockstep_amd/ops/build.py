@@ -162,13 +162,30 @@ def build_attention(head_dim: int, force: bool = False) -> Path:
     return build(f"attention{head_dim}", ATTENTION_SOURCES, (f"-DLS_HEAD_DIM={head_dim}",), force)
 
 
+MUTANT_DEFINE = "-DLS_MUTANTS"
+
+
+def build_core_mutants(force: bool = False) -> Path:
+    """The core library with its switchable wrong variants compiled in (positive controls of the
+    tests); a file of its own, never loaded by the engine."""
+    return build("core.mutants", CORE_SOURCES, (MUTANT_DEFINE,), force)
+
+
+def build_attention_mutants(head_dim: int, force: bool = False) -> Path:
+    return build(f"attention{head_dim}.mutants", ATTENTION_SOURCES, (f"-DLS_HEAD_DIM={head_dim}", MUTANT_DEFINE), force)
+
+
 DEFAULT_HEAD_DIMS = (16, 32, 48, 64, 80, 128, 256)
+MUTANT_HEAD_DIMS = (16, 32, 128)     # the head sizes of the tests that use the controls
 
 
-def build_all(head_dims=DEFAULT_HEAD_DIMS, force: bool = True) -> list[Path]:
+def build_all(head_dims=DEFAULT_HEAD_DIMS, force: bool = True, mutants: bool = True) -> list[Path]:
     """Compile the core library and the attention library of each head size,
-    a few at a time."""
+    a few at a time; with ``mutants`` also the control libraries of the tests."""
     jobs = [lambda: build_core(force)] + [lambda d=d: build_attention(d, force) for d in head_dims]
+    if mutants:
+        jobs += [lambda: build_core_mutants(force)] + [lambda d=d: build_attention_mutants(d, force)
+                                                       for d in MUTANT_HEAD_DIMS]
     results: list = [None] * len(jobs)
     errors: list = []
 

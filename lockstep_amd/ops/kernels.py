@@ -68,8 +68,12 @@ def _rows_ok(t: torch.Tensor, name: str) -> None:
 class Kernels:
     """The loaded libraries.  One instance per process (see ``kernels()``)."""
 
-    def __init__(self):
-        self.core_path = _build.build_core()
+    def __init__(self, mutants: bool = False):
+        """``mutants``: load the control libraries instead (built with their deliberately wrong
+        variants compiled in, all switched off until ``set_mutants``); the tests' positive
+        controls use them, the engine never does."""
+        self.mutants = mutants
+        self.core_path = _build.build_core_mutants() if mutants else _build.build_core()
         self.core = ctypes.CDLL(str(self.core_path))
         self.core.ls_last_error.restype = ctypes.c_char_p
         self._attention: dict[int, ctypes.CDLL] = {}
@@ -86,14 +90,29 @@ class Kernels:
     def attention_lib(self, head_dim: int):
         lib = self._attention.get(head_dim)
         if lib is None:
-            path = _build.build_attention(head_dim)
+            path = _build.build_attention_mutants(head_dim) if self.mutants else _build.build_attention(head_dim)
             lib = ctypes.CDLL(str(path))
             lib.ls_last_error.restype = ctypes.c_char_p
             if not (lib.ls_attn_head_dim() == head_dim):
                 raise KernelError(f"{path} was built for another head size")
+            if self.mutants and getattr(self, "_attention_mask", 0):
+                self._check(lib, lib.ls_set_mutants(c_int(self._attention_mask)))
             self._attention[head_dim] = lib
             self.attention_paths[head_dim] = str(path)
         return lib
+
+    #: bits of ``set_mutants`` (csrc/common.h)
+    MUTANT_KSLICE_BY_ROWS, MUTANT_NORM_BY_ROWS = 1, 2      # core library
+    MUTANT_REVERSED_FOLD = 1                               # attention libraries
+
+    def set_mutants(self, core: int = 0, attention: int = 0) -> None:
+        """Switch wrong variants of the control libraries on (bit masks) or off (0)."""
+        if not self.mutants:
+            raise KernelError("these are the product libraries: they hold no mutants")
+        self._check(self.core, self.core.ls_set_mutants(c_int(core)))
+        for lib in self._attention.values():
+            self._check(lib, lib.ls_set_mutants(c_int(attention)))
+        self._attention_mask = attention
 
     def _memo(self, key, compute):
         """Capability queries do not change while the process runs: ask the library once."""

@@ -393,3 +393,32 @@ def test_the_device_side_decode_loop_picks_the_tokens_of_stepwise_greedy_decodin
     probe = [StepEntry(r, [int(t)], [0]) for r, t in zip(ids, want[-1])]
     assert torch.equal(model.step(loop_cache, probe), model.step(stepwise_cache, probe))
     loop_cache.audit(); stepwise_cache.audit()
+
+
+def test_a_width_that_is_no_multiple_of_four(tmp_path):
+    """hidden_size 66: rows of the residual stream are not 16-byte aligned, so the products add to
+    it in their own epilogue instead of leaving slice sums to the next norm.  Whole, cut and decoded
+    one by one: the plain implementation's logits (float32), the same bits (both precisions)."""
+    from lockstep_amd.config import Qwen3Config
+    from lockstep_amd.weights import write_random_model
+    from plain.qwen3_plain import PlainModel
+
+    config = Qwen3Config(hidden_size=66, intermediate_size=100, num_hidden_layers=2, num_attention_heads=3,
+                         num_key_value_heads=1, head_dim=16, vocab_size=301, rms_norm_eps=1e-6, rope_theta=10000.0,
+                         max_position_embeddings=128, tie_word_embeddings=False)
+    folder = write_random_model(config, tmp_path / "odd", seed=8, std=0.1, norm_std=0.1)
+    tokens = random_tokens(90, 301, seed=4)
+    want = PlainModel(folder).logits(tokens)
+    for dtype in DTYPES:
+        model = load(folder, dtype)
+        cache = model.make_cache(num_pages=24, page_size=8, poison_on_free=True)
+        whole = feed(model, cache, "w", tokens, [])
+        if dtype == "float32":
+            assert rel_err(whole, want) < FP32_TOL_SOFT
+        else:
+            assert rel_err(whole, want) < BF16_TOL
+        cache.close("w")
+        assert torch.equal(feed(model, cache, "c", tokens, [7, 2, 30, 1, 1, 17]), whole)
+        cache.close("c")
+        assert torch.equal(feed(model, cache, "d", tokens, [60] + [1] * 30), whole)
+        cache.audit()

@@ -354,3 +354,54 @@ def test_the_ledger_names_what_differs_between_two_runs():
     assert a.first_difference(ledger(state=(1, 3))) == (0, ("state",))
     assert a.first_difference(ledger(steps=2)) == (2, ("length",)) and a.first_divergence(ledger(steps=2)) == 2
     assert len(set(a.per_step)) == 3
+
+
+# -- positive controls on the host (the GPU ones are in test_controls_gpu.py) ------------------------
+
+def test_a_draw_keyed_on_the_step_instead_of_the_position_is_caught(monkeypatch):
+    """Sampled tokens must not depend on who else is served (reference harness/fuzz/faults.py:
+    rng_keyed_on_global_step).  With the draw keyed on a running count of draws they do."""
+    from lockstep_amd.sampling import philox
+
+    ps = prompts(5, 9, 14)
+
+    def sampled(subset):
+        rs = [Request(uid=f"r{i}", prompt=ps[i], seed=10 + i, max_new_tokens=10, temperature=0.8, top_p=0.95)
+              for i in subset]
+        return run(rs)[0]
+
+    def survivors_keep_their_tokens():
+        everyone = sampled([0, 1, 2])
+        return sampled([1]) == {"r1": everyone["r1"]} and sampled([0, 2]) == {k: everyone[k] for k in ("r0", "r2")}
+
+    assert survivors_keep_their_tokens()
+    original, count = philox.uniform, [0]
+
+    def keyed_on_the_count(seed, uid, position, index=0):
+        count[0] += 1
+        return original(seed, uid, count[0], index)
+
+    monkeypatch.setattr(philox, "uniform", keyed_on_the_count)
+    assert not survivors_keep_their_tokens()
+    monkeypatch.setattr(philox, "uniform", original)
+    assert survivors_keep_their_tokens()
+
+
+def test_a_page_given_back_without_its_count_going_down_is_caught(monkeypatch):
+    """reference harness/fuzz/faults.py: refcount_decrement_missing_on_free -- the audit of every step sees it."""
+    from lockstep_amd.cache import CacheAuditError
+    from lockstep_amd.cache.manager import PagePool
+
+    ps = prompts(20, 20)
+    run(reqs(ps, n=4), num_blocks=8, block_size=8)                    # the unbroken run passes its audits
+    original = PagePool.release
+
+    def forgets_page_two(self, page):
+        if page == 2:
+            return False
+        return original(self, page)
+
+    monkeypatch.setattr(PagePool, "release", forgets_page_two)
+    with pytest.raises(CacheAuditError):
+        run(reqs(ps, n=4) + [Request(uid="late", prompt=ps[0], max_new_tokens=4)], num_blocks=8, block_size=8,
+            policy=DefaultPolicy(max_running=1))

@@ -52,6 +52,17 @@ def run_trace(model_dir, dtype, steps, out_dir, vocab, max_tokens):
     return {rid: np.stack(rows) for rid, rows in logits.items()}
 
 
+def read_digests(out_dir) -> dict:
+    """(request, position) -> sha256 of the logit row, from the ``<step>.sha256`` files."""
+    digests = {}
+    for path in Path(out_dir).glob("*.sha256"):
+        for line in path.read_text().splitlines():
+            rid, position, digest = line.split()
+            assert (rid, int(position)) not in digests, f"position {position} of {rid} was written twice"
+            digests[(rid, int(position))] = digest
+    return digests
+
+
 def whole(requests):
     return [{"step": i, "entries": [{"id": rid, "tokens": t, "want": list(range(len(t)))}], "end": [rid]}
             for i, (rid, t) in enumerate(requests.items())]
@@ -116,6 +127,14 @@ def test_replay_under_four_cuttings(tiny_dirs, tmp_path, dtype, name):
     for label in ("tail", "portions", "mixed"):
         for rid in requests:
             assert np.array_equal(results[label][rid], results["whole"][rid]), f"{label} {rid} differs from whole"
+    # the digests written beside the logits name every (request, position) once and agree between the cuttings
+    import hashlib
+
+    reference = read_digests(tmp_path / "whole")
+    assert set(reference) == {(rid, i) for rid, t in requests.items() for i in range(len(t))}
+    assert reference[("t2", 1)] == hashlib.sha256(results["whole"]["t2"][1].astype("<f4").tobytes()).hexdigest()
+    for label in ("tail", "portions", "mixed"):
+        assert read_digests(tmp_path / label) == reference, label
 
 
 def test_steps_without_wanted_logits_write_no_file(tiny_a_dir, tmp_path):
