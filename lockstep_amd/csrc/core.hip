@@ -418,21 +418,17 @@ __global__ __launch_bounds__(256) void argmax_final_kernel(const float* __restri
 // ---------------------------------------------------------------------------
 // Between two decode steps that run without the host: every request takes the
 // token that was picked for it as its next input, at the next position.  The
-// step's metadata (see the engine's upload) is advanced in place: token ids,
-// token positions, the requests' rows (q_start, kv_len) and the copies of those
-// rows inside the attention work items.  The picked tokens are also appended
-// to a ring the host reads later: ring[step][request], step = *counter, which
-// is incremented.
+// step's metadata (see the engine's upload) is advanced in place: the token
+// ids are replaced, and every value named by the table of runs (first, stride,
+// count) inside the metadata moves on by one -- token positions, the requests'
+// first position and length, and whatever copies of them the parts keep in
+// blocks of their own (the host checks that no value is named twice).  The
+// picked tokens are also appended to a ring the host reads later:
+// ring[step][request], step = *counter, which is incremented.
 // ---------------------------------------------------------------------------
-struct AdvanceLists {
-  int offset[4];  // first int of a list of 16-int attention items inside meta
-  int count[4];   // items in it
-};
-
 __global__ __launch_bounds__(256) void advance_decode_kernel(int* __restrict__ meta, int n_seqs, int off_tokens,
-                                                             int off_positions, int off_seqs,
                                                              const int* __restrict__ picked, int* __restrict__ ring,
-                                                             int* __restrict__ counter, AdvanceLists lists) {
+                                                             int* __restrict__ counter, int off_runs, int n_runs) {
   // one workgroup, so that the counter can be read by all of it before one thread moves it on
   const int tid = threadIdx.x;
   const int stride = blockDim.x;
@@ -440,17 +436,12 @@ __global__ __launch_bounds__(256) void advance_decode_kernel(int* __restrict__ m
   for (int i = tid; i < n_seqs; i += stride) {
     const int token = picked[i];
     meta[off_tokens + i] = token;
-    meta[off_positions + i] += 1;
-    meta[off_seqs + 8 * i + 2] += 1;  // q_start
-    meta[off_seqs + 8 * i + 3] += 1;  // kv_len
     ring[(long)step * n_seqs + i] = token;
   }
-#pragma unroll
-  for (int l = 0; l < 4; ++l)
-    for (int i = tid; i < lists.count[l]; i += stride) {
-      meta[lists.offset[l] + 16 * i + 10] += 1;  // AttnItem.sm.q_start
-      meta[lists.offset[l] + 16 * i + 11] += 1;  // AttnItem.sm.kv_len
-    }
+  for (int r = 0; r < n_runs; ++r) {
+    const int first = meta[off_runs + 3 * r], step_ints = meta[off_runs + 3 * r + 1], count = meta[off_runs + 3 * r + 2];
+    for (int i = tid; i < count; i += stride) meta[first + step_ints * i] += 1;
+  }
   __syncthreads();
   if (tid == 0) *counter = step + 1;
 }
@@ -657,21 +648,17 @@ extern "C" int ls_argmax_static(const float* x, int* out, int rows, int width, l
   return check_launch("argmax_static");
 }
 
-// meta: the step's uploaded metadata; picked [n_seqs]: the tokens chosen for the requests; ring
-// [steps][n_seqs] and counter: where the loop's output goes.  lists: up to four (offset, count) pairs of
-// attention work-item lists inside meta (offset in ints; unused pairs have count 0).
-extern "C" int ls_advance_decode(int* meta, int n_seqs, int off_tokens, int off_positions, int off_seqs,
-                                 const int* picked, int* ring, int* counter, const int* list_offsets,
-                                 const int* list_counts, int n_lists, void* stream) {
+// meta [meta_ints]: the step's uploaded metadata; picked [n_seqs]: the tokens chosen for the requests; ring
+// [steps][n_seqs] and counter: where the loop's output goes.  The table of n_runs runs (first, stride, count)
+// lies at meta[off_runs]; the caller has checked that every run stays inside meta and outside the table.
+extern "C" int ls_advance_decode(int* meta, long meta_ints, int n_seqs, int off_tokens, const int* picked, int* ring,
+                                 int* counter, int off_runs, int n_runs, void* stream) {
   LS_REQUIRE(meta && picked && ring && counter && n_seqs > 0, "advance_decode: bad operands");
-  LS_REQUIRE(n_lists >= 0 && n_lists <= 4, "advance_decode: at most four item lists, got %d", n_lists);
-  AdvanceLists lists;
-  for (int l = 0; l < 4; ++l) {
-    lists.offset[l] = l < n_lists ? list_offsets[l] : 0;
-    lists.count[l] = l < n_lists ? list_counts[l] : 0;
-  }
+  LS_REQUIRE(off_tokens >= 0 && off_tokens + (long)n_seqs <= meta_ints, "advance_decode: the token ids lie outside the metadata");
+  LS_REQUIRE(n_runs >= 0 && off_runs >= 0 && off_runs + 3L * n_runs <= meta_ints,
+             "advance_decode: the table of %d runs at %d lies outside the %ld ints of metadata", n_runs, off_runs, meta_ints);
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-  hipLaunchKernelGGL(advance_decode_kernel, dim3(1), dim3(256), 0, s, meta, n_seqs, off_tokens, off_positions,
-                     off_seqs, picked, ring, counter, lists);
+  hipLaunchKernelGGL(advance_decode_kernel, dim3(1), dim3(256), 0, s, meta, n_seqs, off_tokens, picked, ring, counter,
+                     off_runs, n_runs);
   return check_launch("advance_decode");
 }

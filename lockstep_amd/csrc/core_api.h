@@ -49,9 +49,8 @@ int ls_argmax(const float* x, int* out, int rows, int width, long ld, void* scra
 #define LS_ARGMAX_STATIC_PAIRS 16384
 int ls_argmax_static(const float* x, int* out, int rows, int width, long ld, void* stream);
 
-int ls_advance_decode(int* meta, int n_seqs, int off_tokens, int off_positions, int off_seqs, const int* picked,
-                      int* ring, int* counter, const int* list_offsets, const int* list_counts, int n_lists,
-                      void* stream);
+int ls_advance_decode(int* meta, long meta_ints, int n_seqs, int off_tokens, const int* picked, int* ring,
+                      int* counter, int off_runs, int n_runs, void* stream);
 
 // Matrix products C = X W^T with a fixed summation order (see gemm.hip).
 int ls_gemm(int dtype, int epilogue, const void* X, const void* W, void* C, int M, int N, int K, long ldx, long ldc,

@@ -287,8 +287,6 @@ class Model:
             mixer.prepare(ctx)
         ctx.upload()
         layout = ctx.meta_layout()
-        if len(layout["item_lists"]) > 4:
-            return None                                   # more work lists than the advance kernel takes
         kernels = self.rt.kernels
         ring = self.workspace.get("loop.ring", (self.LOOP_CAPACITY * max(n, 64),), torch.int32)
         counter = self.workspace.get("loop.counter", (1,), torch.int32)
@@ -298,8 +296,7 @@ class Model:
         def one_step(logits):
             self._forward(ctx, logits)
             kernels.argmax(logits, picked[:n])
-            kernels.advance_decode(layout["meta"], n, layout["tokens"], layout["positions"], layout["seqs"], picked,
-                                   ring, counter, layout["item_lists"])
+            kernels.advance_decode(layout["meta"], n, layout["tokens"], picked, ring, counter, *layout["runs"])
 
         graphs = cache.step_graphs
         key = ("loop",) + self._graph_key(ctx)

@@ -335,25 +335,20 @@ class Kernels:
                                    c_long(logits.stride(0)), _ptr(scratch), c_long(scratch.numel()), _stream())
         self._check(self.core, code)
 
-    def advance_decode(self, meta: torch.Tensor, n_seqs: int, off_tokens: int, off_positions: int, off_seqs: int,
-                       picked: torch.Tensor, ring: torch.Tensor, counter: torch.Tensor, lists) -> None:
+    def advance_decode(self, meta: torch.Tensor, n_seqs: int, off_tokens: int, picked: torch.Tensor,
+                       ring: torch.Tensor, counter: torch.Tensor, off_runs: int, n_runs: int) -> None:
         """Between two decode steps that run without the host: the picked tokens become the next
-        inputs, positions and lengths inside the uploaded metadata ``meta`` move on by one, and the
-        tokens are appended to ``ring[counter]``.  ``lists``: (offset, count) of the attention
-        work-item lists inside ``meta`` (16 ints an item)."""
+        inputs inside the uploaded metadata ``meta``, every value named by the ``n_runs`` runs
+        (first, stride, count) of the table at ``meta[off_runs]`` moves on by one, and the tokens
+        are appended to ``ring[counter]``.  The step's upload builds the table and checks it."""
         for t in (meta, picked, ring, counter):
             if not (t.is_cuda and t.dtype == torch.int32 and t.is_contiguous()):
                 raise KernelError("advance_decode works on int32 GPU tensors")
-        if not (picked.numel() >= n_seqs and len(lists) <= 4):
-            raise KernelError("advance_decode: picked too short or more than four lists")
-        offsets = (ctypes.c_int * 4)(*([o for o, _ in lists] + [0] * (4 - len(lists))))
-        counts = (ctypes.c_int * 4)(*([c for _, c in lists] + [0] * (4 - len(lists))))
-        for o, c in lists:
-            if not (0 <= o and o + 16 * c <= meta.numel()):
-                raise KernelError("advance_decode: an item list lies outside the metadata")
-        code = self.core.ls_advance_decode(_ptr(meta), c_int(n_seqs), c_int(off_tokens), c_int(off_positions),
-                                           c_int(off_seqs), _ptr(picked), _ptr(ring), _ptr(counter), offsets, counts,
-                                           c_int(len(lists)), _stream())
+        if not (picked.numel() >= n_seqs):
+            raise KernelError("advance_decode: picked is too short")
+        code = self.core.ls_advance_decode(_ptr(meta), c_long(meta.numel()), c_int(n_seqs), c_int(off_tokens),
+                                           _ptr(picked), _ptr(ring), _ptr(counter), c_int(off_runs), c_int(n_runs),
+                                           _stream())
         self._check(self.core, code)
 
     # -- attention ----------------------------------------------------------------

@@ -15,13 +15,15 @@ one kernel; attention is one launch for all requests of the step.
 
 from __future__ import annotations
 
+import os
+from dataclasses import dataclass
+
+import numpy as np
 import torch
 
 from ..config.base import PartSpec
-from ..ops import ADD_F32, STORE_F32
+from ..ops import ADD_F32, STORE_F32, pack_attention_items, pack_combine_items
 from .base import Mixer, PagedKVSpec, PendingAdd, WeightSpec, build_part, deferred_rows, register_part
-
-import os
 
 # Steps of single decoded tokens run norm, rotation and cache write inside the
 # attention kernel (one launch less per layer); "0" keeps the separate kernel.
@@ -29,6 +31,139 @@ FUSE_DECODE = os.environ.get("LOCKSTEP_FUSE_DECODE", "1") not in ("", "0")
 # From this many attention workgroups on (two a CU: the kernel is then bound by the cache it streams) the
 # prologue of the fused kernel costs more than the separate norm/rotation launch; measured +2 % at batch 64.
 FUSE_DECODE_BELOW = int(os.environ.get("LOCKSTEP_FUSE_DECODE_BELOW", "512"))
+
+
+# ---------------------------------------------------------------------------
+# The step's attention work, laid out on the host.  The lists go into the step's
+# upload as one declared block per set of attention constants (layers with the
+# same constants share it); the kernels read them from there.
+# ---------------------------------------------------------------------------
+
+@dataclass
+class AttentionPlan:
+    """Where the lists of one set of attention constants lie inside their block, and what the
+    launches need to know about them."""
+
+    n_items: int              # staged / direct items (16 ints each), first in the block
+    n_combine: int            # combine items (8 ints each)
+    n_coop: int               # cooperative items (decoded tokens)
+    coop_max_rows: int
+    n_wide: int               # wide items (long prompt portions)
+    part_rows: int            # rows of partial results the split items leave
+    decode_fused: bool        # every request brings one token and the fused decode kernel can take the step
+    wide_variant: int = 4     # 4: row blocks of 128 rows, 5: of 64
+
+    ITEM, COMBINE = 16, 8
+
+    def offsets(self):
+        items = 0
+        combine = items + self.ITEM * self.n_items
+        coop = combine + self.COMBINE * self.n_combine
+        wide = coop + self.ITEM * self.n_coop
+        return items, combine, coop, wide, wide + self.ITEM * self.n_wide
+
+    def signature(self):
+        return (self.n_items, self.n_combine, self.n_coop, self.n_wide, self.part_rows, self.decode_fused,
+                self.wide_variant)
+
+
+def plan_attention(ctx, group_size: int, nkv: int, head_dim: int, window: int):
+    """Work items of one set of attention constants for this step: (plan, ints of the block).
+
+    Requests are cut at the kernels' own, position-anchored splits; which kernel takes a request
+    and whether a workgroup walks all splits or leaves one partial result per split is chosen
+    here freely, because every choice gives the same bits.  With ``ctx.fixed_shape`` the size of
+    the lists depends only on the number of requests and on a bucket of the longest context:
+    every request gets one item per split up to the bucket (items past a request's own length
+    leave empty partial results, which the fold skips), so a captured graph of the step stays
+    valid from one decode step to the next."""
+    kernels, dtype, page_size = ctx.rt.kernels, ctx.rt.dtype, ctx.cache.page_size
+    tile, split = kernels.attention_geometry(head_dim)
+    coop_ok = kernels.coop_supported(head_dim, dtype, page_size)
+    # with a workgroup per CU anyway, one workgroup walks all splits of a request itself
+    whole_requests = ctx.n_seqs * nkv >= 256
+    wide_ok = kernels.wide_supported(head_dim, dtype, page_size)
+    wide_variant, wide_rows = 4, kernels.attention_block_rows(head_dim, 4)
+    if wide_ok:
+        # so few rows that the large row blocks would leave half of the CUs without a workgroup: smaller blocks
+        blocks = sum(-(-(int(q) * group_size) // wide_rows) for q in ctx.q_len if int(q) * group_size > 64)
+        if 0 < blocks * nkv <= kernels.compute_units() // 2:
+            wide_variant, wide_rows = 5, kernels.attention_block_rows(head_dim, 5)
+    items, coop, wide, combine = [], [], [], []
+    coop_max_rows = part_rows = bucket = 0
+    if ctx.fixed_shape:
+        longest = (int(ctx.kv_len.max()) + ctx.horizon - 1) // split + 1
+        bucket = 1
+        while bucket < longest:
+            bucket = bucket * 2 if bucket < 8 else bucket + 8
+        if coop_ok and group_size <= 16 and ctx.single_tokens:
+            # a decode step: the lists depend on its shape only, the requests' rows are appended
+            shape = ("attention.template", ctx.n_seqs, group_size, nkv, bucket, whole_requests)
+            made = ctx.memo.get(shape)
+            if made is None:
+                for i in range(ctx.n_seqs):
+                    if whole_requests:
+                        coop.append((i, 0, 0, bucket, -1, 0, 0, 0))
+                    else:
+                        base = part_rows
+                        part_rows += nkv * group_size * bucket
+                        coop += [(i, 0, s, s + 1, base, bucket, 0, 0) for s in range(bucket)]
+                        combine.append((i, 0, base, bucket))
+                made = (np.asarray(coop, dtype=np.int64).reshape(-1, 8),
+                        np.asarray(combine, dtype=np.int64).reshape(-1, 4), part_rows)
+                ctx.memo[shape] = made
+            coop_t, combine_t, part_rows = made
+            plan = AttentionPlan(0, len(combine_t), len(coop_t), group_size, 0, part_rows,
+                                 kernels.decode_fused_supported(head_dim, dtype, page_size))
+            return plan, np.concatenate([pack_combine_items(combine_t, ctx.seq_rows),
+                                         pack_attention_items(coop_t, ctx.seq_rows)])
+    for i in range(ctx.n_seqs):
+        q_len, q_start, kv_len = int(ctx.q_len[i]), int(ctx.q_start[i]), int(ctx.kv_len[i])
+        rows = q_len * group_size
+        lo_valid = max(0, q_start - window + 1) if window > 0 else 0
+        split_lo = lo_valid // split
+        n_splits = (kv_len - 1) // split + 1 - split_lo
+        if ctx.fixed_shape:
+            split_lo, n_splits = 0, bucket
+        # items of at most 16 rows (decoded tokens) go to the cooperative kernel
+        target = coop if (coop_ok and rows <= 16) else items
+        if target is coop:
+            coop_max_rows = max(coop_max_rows, rows)
+        if rows <= 64 and (n_splits > 1 or ctx.fixed_shape) and not (target is coop and whole_requests):
+            base = part_rows
+            part_rows += nkv * rows * n_splits
+            for s in range(split_lo, split_lo + n_splits):
+                target.append((i, 0, s, s + 1, base, n_splits, split_lo, 0))
+            combine.append((i, 0, base, n_splits))
+        else:
+            # long portions go to the wide kernel, in larger row blocks
+            if wide_ok and rows > 64:
+                target, block_rows = wide, wide_rows
+            else:
+                block_rows = 64
+            for block in range(-(-rows // block_rows)):
+                first_pos = q_start + (block * block_rows) // group_size
+                last_pos = q_start + min((block + 1) * block_rows - 1, rows - 1) // group_size
+                begin = (max(0, first_pos - window + 1) // split) if window > 0 else 0
+                target.append((i, block, begin, last_pos // split + 1, -1, 0, 0, 0))
+    decode_fused = (coop_ok and not items and not wide and bool((ctx.q_len == 1).all())
+                    and kernels.decode_fused_supported(head_dim, dtype, page_size))
+    # the longest row blocks first: they decide when the launch ends
+    wide.sort(key=lambda it: it[2] - it[3])
+    plan = AttentionPlan(len(items), len(combine), len(coop), coop_max_rows, len(wide), part_rows, decode_fused,
+                         wide_variant)
+    return plan, np.concatenate([pack_attention_items(items, ctx.seq_rows), pack_combine_items(combine, ctx.seq_rows),
+                                 pack_attention_items(coop, ctx.seq_rows), pack_attention_items(wide, ctx.seq_rows)])
+
+
+def advancing_fields(plan: AttentionPlan):
+    """The copies of a request's first position and length inside the attention items: they move
+    on with every token decoded without the host."""
+    items, _, coop, wide, _ = plan.offsets()
+    runs = []
+    for first, count in ((items, plan.n_items), (coop, plan.n_coop), (wide, plan.n_wide)):
+        runs += [(first + 10, 16, count), (first + 11, 16, count)]
+    return [r for r in runs if r[2]]
 
 
 @register_part("attention")
@@ -110,9 +245,18 @@ class Attention(Mixer):
             return None
         return ("attention", self.nq, self.nkv, self.d, self.window, share())
 
+    def _block_key(self):
+        window = int(self.window) if self.window is not None else 0
+        return ("attention", self.nq // self.nkv, self.nkv, self.d, window)
+
     def prepare(self, ctx) -> None:
         self.position.ensure(ctx.max_position + 1, ctx.rt)
-        ctx.plan_attention(self.nq // self.nkv, self.nkv, self.d, int(self.window) if self.window is not None else 0)
+        key = self._block_key()
+        if ctx.declared(key):
+            return
+        plan, ints = plan_attention(ctx, *key[1:])
+        ctx.declare(key, ints, advance=advancing_fields(plan), signature=plan.signature())
+        ctx.notes[key] = plan                         # for forward, which runs after the upload
 
     def forward(self, ctx, run, x, out, accumulate: bool, norm=None, defer: bool = False):
         """``norm``: when given, ``x`` is the float32 residual stream and ``norm``
@@ -133,34 +277,41 @@ class Attention(Mixer):
             k.gemm(x, self.w_q, qkv[:, : nq * d], **fused)
         attn = ctx.buf("attention.out", (t, nq * d), rt.dtype)
         window = int(self.window) if self.window is not None else 0
-        plan = ctx.attention_plan(nq // nkv, nkv, d, window)
+        key = self._block_key()
+        plan = ctx.notes[key]
+        block = ctx.block(key)
+        at_items, at_combine, at_coop, at_wide, end = plan.offsets()
+        items, combine_items = block[at_items:at_combine], block[at_combine:at_coop]
+        coop_items, wide_items = block[at_coop:at_wide], block[at_wide:end]
+        part_acc = part_ml = None
+        if plan.part_rows:
+            part_acc = ctx.buf(f"attention.part_acc.{d}", (plan.part_rows, d), torch.float32)
+            part_ml = ctx.buf("attention.part_ml", (plan.part_rows, 2), torch.float32)
         if plan.decode_fused and FUSE_DECODE and plan.n_coop * nkv < FUSE_DECODE_BELOW:
             # single decoded tokens: norm, rotation and cache write happen inside the attention kernel
             k.attention_decode(qkv, nq, nkv, d, key_pages, value_pages, group.page_size, group.table, ctx.seqs,
-                               plan.coop_items, plan.n_coop, attn, plan.part_acc, plan.part_ml, self.scale, window,
+                               coop_items, plan.n_coop, attn, part_acc, part_ml, self.scale, window,
                                self.q_norm, self.k_norm, self.norm_eps, self.position.cos, self.position.sin,
                                self.position.rotary_dim, ctx.max_position, run.writes_cache)
             if plan.n_combine:
-                k.attention_combine(d, ctx.seqs, plan.combine_items, plan.n_combine, nq, nkv, plan.part_acc,
-                                    plan.part_ml, attn)
+                k.attention_combine(d, ctx.seqs, combine_items, plan.n_combine, nq, nkv, part_acc, part_ml, attn)
             return self._project_out(ctx, attn, out, accumulate, defer)
         k.qk_rope_kv(qkv, t, nq, nkv, d, self.q_norm, self.k_norm, self.norm_eps, self.position.cos,
                      self.position.sin, self.position.rotary_dim, ctx.tok_seq, ctx.tok_pos, ctx.seqs,
                      ctx.max_position, group.table, key_pages, value_pages, group.page_size, run.writes_cache)
         if plan.n_items:
             k.attention(qkv, nq, nkv, d, key_pages, value_pages, group.page_size, group.table, ctx.seqs,
-                        plan.items, plan.n_items, attn, plan.part_acc, plan.part_ml, self.scale, window)
+                        items, plan.n_items, attn, part_acc, part_ml, self.scale, window)
         if plan.n_coop:
             k.attention(qkv, nq, nkv, d, key_pages, value_pages, group.page_size, group.table, ctx.seqs,
-                        plan.coop_items, plan.n_coop, attn, plan.part_acc, plan.part_ml, self.scale, window,
+                        coop_items, plan.n_coop, attn, part_acc, part_ml, self.scale, window,
                         variant=3, max_rows=plan.coop_max_rows)
         if plan.n_wide:
             k.attention(qkv, nq, nkv, d, key_pages, value_pages, group.page_size, group.table, ctx.seqs,
-                        plan.wide_items, plan.n_wide, attn, plan.part_acc, plan.part_ml, self.scale, window,
+                        wide_items, plan.n_wide, attn, part_acc, part_ml, self.scale, window,
                         variant=plan.wide_variant)
         if plan.n_combine:
-            k.attention_combine(d, ctx.seqs, plan.combine_items, plan.n_combine, nq, nkv, plan.part_acc,
-                                plan.part_ml, attn)
+            k.attention_combine(d, ctx.seqs, combine_items, plan.n_combine, nq, nkv, part_acc, part_ml, attn)
         return self._project_out(ctx, attn, out, accumulate, defer)
 
     def _project_out(self, ctx, attn, out, accumulate: bool, defer: bool):

@@ -206,7 +206,14 @@ def _register_toy():
 
     @register_part("toy_decay")
     class DecayMixer(Mixer):
-        """s_t = decay * s_{t-1} + x_t (one state vector per request); out_t = s_t @ W^T."""
+        """s_t = decay * s_{t-1} + x_t / (1 + position_t % 5) (one state vector per request);
+        out_t = s_t @ W^T.  The mixer owns device-side metadata of the step: a block of two ints
+        a request (its state slot, the position of its token) whose positions move on by one with
+        every token decoded without the host.  Steps of single decoded tokens read nothing on the
+        host (torch operations indexed by that block, the engine's own matrix product), so the
+        part is graph safe; prompt portions walk their rows on the host."""
+
+        graph_safe = True
 
         def __init__(self, spec, prefix=""):
             super().__init__(spec, prefix)
@@ -222,14 +229,29 @@ def _register_toy():
         def load(self, weights, rt):
             self.w = rt.vector(weights.get(f"{self.prefix}.mix.weight"))
 
+        def prepare(self, ctx):
+            if ctx.single_tokens and not ctx.declared("toy_decay"):
+                ints = [v for slot, pos in zip(ctx.slots, ctx.q_start) for v in (int(slot), int(pos))]
+                ctx.declare("toy_decay", ints, advance=[(1, 2, ctx.n_seqs)])
+
         def forward(self, ctx, run, x, out, accumulate):
+            from lockstep_amd.ops import ADD_F32, STORE_F32
+
             state = ctx.cache.unit_state(run.cache)
+            if ctx.single_tokens:                       # device side only: may be captured and replayed
+                block = ctx.block("toy_decay").view(ctx.n_seqs, 2)
+                slots, positions = block[:, 0].long(), block[:, 1]
+                gain = 1.0 / (1 + positions % 5).to(torch.float32)
+                fresh = self.decay * state.index_select(0, slots) + x.float() * gain[:, None]
+                state.index_copy_(0, slots, fresh)
+                ctx.rt.kernels.gemm(fresh.contiguous(), self.w, out, ADD_F32 if accumulate else STORE_F32)
+                return
             for i in range(ctx.n_seqs):
-                lo, n, slot = int(ctx.q_off[i]), int(ctx.q_len[i]), int(ctx.slots[i])
+                lo, n, slot, start = int(ctx.q_off[i]), int(ctx.q_len[i]), int(ctx.slots[i]), int(ctx.q_start[i])
                 s = state[slot]
                 rows = []
                 for t in range(n):
-                    s = self.decay * s + x[lo + t].float()
+                    s = self.decay * s + x[lo + t].float() / (1 + (start + t) % 5)
                     rows.append(s)
                 state[slot] = s
                 y = torch.stack(rows) @ self.w.T
@@ -284,7 +306,7 @@ def _toy_plain(cfg, w, tokens, schedule):
             s = torch.zeros(cfg["hidden_size"], dtype=torch.float64)
             rows = []
             for i in range(t):
-                s = cfg["decay"] * s + x[i]
+                s = cfg["decay"] * s + x[i] / (1 + i % 5)
                 rows.append(s)
             h = h + torch.stack(rows) @ w[f"{p}.mixer.mix.weight"].T
         else:
@@ -338,6 +360,42 @@ def test_toy_architecture_registers_builds_and_steps(tmp_path, schedule):
         cache.close("w"); cache.close("o")
         again = feed(model, cache, "w2", tokens, [25])                          # a reused slot starts from zero state
         assert rel_err(again, want) < 5e-5
+        cache.audit()
+        cache.close("c"); cache.close("w2")
+        # The mixer declared itself graph safe: steps of single decoded tokens are replayed from a captured
+        # graph, with its block of slots and positions uploaded beside the attention layers' work lists ...
+        replays = model.graph_replays
+        tail = feed(model, cache, "t", tokens, [20] + [1] * 30)
+        assert model.graph_replays - replays >= 25 and rel_err(tail, want) < 5e-5
+        beside = random_tokens(50, 90, seed=3)                                  # ... two requests in a step
+        want_beside = _toy_plain({"hidden_size": 48, "decay": 0.9}, w, beside, schedule)
+        cache.close("t")
+        feed(model, cache, "p", tokens[:30], [], want_all=False); feed(model, cache, "q", beside[:11], [], want_all=False)
+        from lockstep_amd.engine.batch import StepEntry
+        rows_p, rows_q = [], []
+        for i in range(20):
+            logits = model.step(cache, [StepEntry("p", [tokens[30 + i]], [0]), StepEntry("q", [beside[11 + i]], [0])])
+            rows_p.append(logits[0].cpu()); rows_q.append(logits[1].cpu())
+        assert rel_err(torch.stack(rows_p), want[30:50]) < 5e-5
+        assert rel_err(torch.stack(rows_q), want_beside[11:31]) < 5e-5
+        # ... and the device-side loop advances the mixer's positions itself: greedy tokens equal stepwise decoding
+        picked = {}
+        for way in ("loop", "steps"):
+            cache.close("p"); cache.close("q")
+            feed(model, cache, "p", tokens[:30], [], want_all=False); feed(model, cache, "q", beside[:11], [], want_all=False)
+            cur = [tokens[30], beside[11]]
+            if way == "loop":
+                before = model.graph_replays
+                picked[way] = model.decode_greedy(cache, ["p", "q"], cur, 12).tolist()
+                assert model.graph_replays - before >= 10
+            else:
+                got = []
+                for _ in range(12):
+                    logits = model.step(cache, [StepEntry("p", cur[:1], [0]), StepEntry("q", cur[1:], [0])])
+                    cur = [int(row.argmax()) for row in logits]
+                    got.append(cur)
+                picked[way] = got
+        assert picked["loop"] == picked["steps"]
         cache.audit()
     finally:
         unregister_part("toy_decay")
