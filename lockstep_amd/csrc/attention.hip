@@ -71,6 +71,8 @@ constexpr int DB = D / 16;          // 16-column blocks of the head
 struct SeqMeta {
   int q_off, q_len, q_start, kv_len, table_row, reserved[3];
 };
+// An item of all zeros stands for no work (lists of graph-replayed steps are rounded up with them): a request
+// of no rows has no row to load for and none to write, and the kernels need no test of their own for it.
 struct AttnItem {  // one workgroup column of the attention launch (16 ints)
   int seq;         // index into SeqMeta
   int row_block;   // row block of the sequence's rows
@@ -1055,7 +1057,7 @@ struct DecodeFuse {
   T* v_out;
 };
 
-template <typename T, int NBUF, bool FUSE>
+template <typename T, int NBUF, bool FUSE, bool SPANS>
 __global__ __launch_bounds__(256) void attention_coop_kernel(
     const T* __restrict__ q, long ldq, const T* __restrict__ k_pages, const T* __restrict__ v_pages, int nkv,
     int page_size, int page_shift, const int* __restrict__ table, int table_stride,
@@ -1211,6 +1213,22 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
     cur_acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
     run_acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
+
+  // The sums of one split to their place among the partial results (an item may hold several splits).
+  auto write_partial = [&](int split, const f32x4 (&acc)[MYDB], float m, float l) {
+    if (!row_ok) return;
+    const long pr = item.part_base + ((long)kvh * rows_total + r) * item.n_splits + (split - item.split_lo);
+    float* pa = part_acc + pr * D;
+#pragma unroll
+    for (int j = 0; j < MYDB; ++j) {
+      const int blk = wave + 4 * j;
+      if (blk < DB) *reinterpret_cast<f32x4*>(pa + blk * 16 + 4 * g) = acc[j];
+    }
+    if (wave == 0 && g == 0) {
+      part_ml[pr * 2] = m;
+      part_ml[pr * 2 + 1] = l;
+    }
+  };
 
   // FUSE: one new token per request at position q_start; its tile is patched by the workgroup that walks it.
   // The heads to process are numbered vi: the G query heads, then the new key, then the new value;
@@ -1476,6 +1494,15 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
       }
     }
     PROBE(11)
+    if (SPANS) {
+      if (!direct && (ti + 1) % TILES_PER_SPLIT == 0 && ti + 1 < ti_hi) {  // an item of several splits: this one's
+        write_partial(ti / TILES_PER_SPLIT, cur_acc, cur_m, cur_l);        // sums go to their place
+#pragma unroll
+        for (int j = 0; j < MYDB; ++j) cur_acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+        cur_m = kNegSentinel;
+        cur_l = 0.f;
+      }
+    }
     if (direct && ((ti + 1) % TILES_PER_SPLIT == 0 || ti + 1 == ti_hi)) {
       if (cur_l > 0.f) {  // the fold of fold_split, on this wave's blocks
         const float m_fold = fmaxf(run_m, cur_m);
@@ -1528,18 +1555,31 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
       }
     }
   } else {
-    const int split = item.split_begin;
-    const long pr = item.part_base + ((long)kvh * rows_total + r) * item.n_splits + (split - item.split_lo);
-    float* pa = part_acc + pr * D;
+    // the item's splits that hold no tile for these rows (past the request's end, or behind the window)
+    // leave empty sums: the fold reads every split's place and skips those
+    if (!SPANS) {  // one split an item (checked on the host): its sums, empty if it holds no tile for these rows
+      const int split = item.split_begin;
+      const long pr = item.part_base + ((long)kvh * rows_total + r) * item.n_splits + (split - item.split_lo);
+      float* pa = part_acc + pr * D;
 #pragma unroll
-    for (int j = 0; j < MYDB; ++j) {
-      const int blk = wave + 4 * j;
-      if (blk < DB) *reinterpret_cast<f32x4*>(pa + blk * 16 + 4 * g) = cur_acc[j];
+      for (int j = 0; j < MYDB; ++j) {
+        const int blk = wave + 4 * j;
+        if (blk < DB) *reinterpret_cast<f32x4*>(pa + blk * 16 + 4 * g) = cur_acc[j];
+      }
+      if (wave == 0 && g == 0) {
+        part_ml[pr * 2] = cur_m;
+        part_ml[pr * 2 + 1] = cur_l;
+      }
+      return;
     }
-    if (wave == 0 && g == 0) {
-      part_ml[pr * 2] = cur_m;
-      part_ml[pr * 2 + 1] = cur_l;
+    const int first_done = ti_lo / TILES_PER_SPLIT, last_done = (ti_hi - 1) / TILES_PER_SPLIT;
+    if (ti_lo < ti_hi) {  // the sums of the last split walked
+      write_partial(last_done, cur_acc, cur_m, cur_l);
+#pragma unroll
+      for (int j = 0; j < MYDB; ++j) cur_acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
+    for (int split = item.split_begin; split < item.split_end; ++split)
+      if (ti_lo >= ti_hi || split < first_done || split > last_done) write_partial(split, cur_acc, kNegSentinel, 0.f);
   }
 }
 
@@ -1647,14 +1687,14 @@ constexpr size_t coop_kernel_lds() { return NBUF * (2 * (size_t)kTileKeys * D * 
 
 // Whether this instantiation can be launched (its LDS fits; above 64 KB the
 // function attribute is raised once).
-template <typename T, int NBUF, bool FUSE>
+template <typename T, int NBUF, bool FUSE, bool SPANS = false>
 static bool coop_kernel_ready() {
   constexpr size_t bytes = coop_kernel_lds<T, NBUF>();
   if (bytes > kLdsLimit) return false;
   if (bytes <= 64 * 1024) return true;
   static int state = 0;  // 0 unknown, 1 granted, -1 refused
   if (state == 0) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_coop_kernel<T, NBUF, FUSE>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_coop_kernel<T, NBUF, FUSE, SPANS>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
     if (e != hipSuccess) (void)hipGetLastError();
     state = e == hipSuccess ? 1 : -1;
@@ -1666,27 +1706,41 @@ static bool coop_kernel_ready() {
 // where they fit; when the grid brings at least two workgroups per CU, with
 // one buffer instead, so that two workgroups share a CU and overlap each
 // other's loads.
-template <typename T, bool FUSE>
-static int launch_coop(dim3 grid, hipStream_t s, const void* q, long ldq, const void* k_pages, const void* v_pages,
-                       int nkv, int page_size, int page_shift, const int* table, int table_stride, const void* seqs,
-                       const void* items, void* out, long ldo, float* part_acc, float* part_ml, int G, float scale,
-                       int window, DecodeFuse<T> fz) {
+template <typename T, bool FUSE, bool SPANS>
+static int launch_coop_as(dim3 grid, hipStream_t s, const void* q, long ldq, const void* k_pages, const void* v_pages,
+                          int nkv, int page_size, int page_shift, const int* table, int table_stride, const void* seqs,
+                          const void* items, void* out, long ldo, float* part_acc, float* part_ml, int G, float scale,
+                          int window, DecodeFuse<T> fz) {
   constexpr int BUFS = coop_bufs(sizeof(T));
   const bool crowded = (long)grid.x * grid.y >= 512;
 #define LS_COOP(NBUF_)                                                                                              \
-  hipLaunchKernelGGL((attention_coop_kernel<T, NBUF_, FUSE>), grid, dim3(256), (coop_kernel_lds<T, NBUF_>()), s,       \
+  hipLaunchKernelGGL((attention_coop_kernel<T, NBUF_, FUSE, SPANS>), grid, dim3(256), (coop_kernel_lds<T, NBUF_>()), s, \
                      (const T*)q, ldq, (const T*)k_pages, (const T*)v_pages, nkv, page_size, page_shift, table,        \
                      table_stride, (const SeqMeta*)seqs, (const AttnItem*)items, (T*)out, ldo, part_acc, part_ml, G,   \
                      scale, window, fz)
-  if (BUFS == 2 && !(crowded && coop_kernel_ready<T, 1, FUSE>())) {
-    if (!coop_kernel_ready<T, 2, FUSE>()) return fail("attention: the cooperative kernel does not fit into LDS");
+  if (BUFS == 2 && !(crowded && coop_kernel_ready<T, 1, FUSE, SPANS>())) {
+    if (!coop_kernel_ready<T, 2, FUSE, SPANS>()) return fail("attention: the cooperative kernel does not fit into LDS");
     LS_COOP(2);
   } else {
-    if (!coop_kernel_ready<T, 1, FUSE>()) return fail("attention: the cooperative kernel does not fit into LDS");
+    if (!coop_kernel_ready<T, 1, FUSE, SPANS>()) return fail("attention: the cooperative kernel does not fit into LDS");
     LS_COOP(1);
   }
 #undef LS_COOP
   return 0;
+}
+
+// ``spans``: items may hold several splits and leave a partial result for each (an instance of its own, so
+// that the usual one-split items keep their code).
+template <typename T, bool FUSE>
+static int launch_coop(bool spans, dim3 grid, hipStream_t s, const void* q, long ldq, const void* k_pages,
+                       const void* v_pages, int nkv, int page_size, int page_shift, const int* table, int table_stride,
+                       const void* seqs, const void* items, void* out, long ldo, float* part_acc, float* part_ml, int G,
+                       float scale, int window, DecodeFuse<T> fz) {
+  if (spans)
+    return launch_coop_as<T, FUSE, true>(grid, s, q, ldq, k_pages, v_pages, nkv, page_size, page_shift, table,
+                                         table_stride, seqs, items, out, ldo, part_acc, part_ml, G, scale, window, fz);
+  return launch_coop_as<T, FUSE, false>(grid, s, q, ldq, k_pages, v_pages, nkv, page_size, page_shift, table,
+                                        table_stride, seqs, items, out, ldo, part_acc, part_ml, G, scale, window, fz);
 }
 
 static bool coop_supported(int dtype) {
@@ -1718,7 +1772,7 @@ extern "C" int ls_attention_decode(int dtype, const void* qkv, long ld, void* k_
                                    const void* items, int n_items, void* out, long ldo, float* part_acc,
                                    float* part_ml, float scale, int window, const float* q_weight,
                                    const float* k_weight, float eps, const float* cos_table, const float* sin_table,
-                                   int rot, int table_positions, int max_pos, int write_kv, void* stream) {
+                                   int rot, int table_positions, int max_pos, int write_kv, int spans, void* stream) {
   LS_REQUIRE(n_items > 0 && nkv > 0 && nq > 0 && nq % nkv == 0, "decode attention: bad sizes");
   const int G = nq / nkv;
   LS_REQUIRE(G <= 16, "decode attention: %d query heads per kv head, at most 16 fit a work item", G);
@@ -1747,12 +1801,12 @@ extern "C" int ls_attention_decode(int dtype, const void* qkv, long ld, void* k_
   int rc = 0;
   if (dtype == kF32) {
     DecodeFuse<float> fz{q_weight, k_weight, eps, cos_table, sin_table, rot, nq, write_kv, (float*)k_pages, (float*)v_pages};
-    rc = launch_coop<float, true>(grid, s, qkv, ld, k_pages, v_pages, nkv, page_size, page_shift, table, table_stride,
+    rc = launch_coop<float, true>(spans != 0, grid, s, qkv, ld, k_pages, v_pages, nkv, page_size, page_shift, table, table_stride,
                                   seqs, items, out, ldo, part_acc, part_ml, G, scale, window, fz);
   } else if (dtype == kBF16) {
     DecodeFuse<bf16_t> fz{q_weight, k_weight, eps, cos_table, sin_table, rot, nq, write_kv, (bf16_t*)k_pages,
                           (bf16_t*)v_pages};
-    rc = launch_coop<bf16_t, true>(grid, s, qkv, ld, k_pages, v_pages, nkv, page_size, page_shift, table, table_stride,
+    rc = launch_coop<bf16_t, true>(spans != 0, grid, s, qkv, ld, k_pages, v_pages, nkv, page_size, page_shift, table, table_stride,
                                    seqs, items, out, ldo, part_acc, part_ml, G, scale, window, fz);
   } else {
     return fail("decode attention: unknown dtype %d", dtype);
@@ -1801,7 +1855,7 @@ extern "C" int ls_attn_block_rows(int variant) {
 extern "C" int ls_attention(int dtype, const void* q, long ldq, const void* k_pages, const void* v_pages, int nkv,
                             int page_size, const int* table, int table_stride, const void* seqs, const void* items,
                             int n_items, void* out, long ldo, float* part_acc, float* part_ml, int G, float scale,
-                            int window, int variant, int max_rows, void* stream) {
+                            int window, int variant, int max_rows, int spans, void* stream) {
   LS_REQUIRE(n_items > 0 && nkv > 0 && G > 0, "attention: bad sizes (items %d, kv heads %d, group %d)", n_items, nkv, G);
   LS_REQUIRE(page_size >= 4 && page_size % 4 == 0 && kTileKeys % page_size == 0,
              "attention: page size %d must be a multiple of 4 that divides the key tile %d", page_size, kTileKeys);
@@ -1824,10 +1878,10 @@ extern "C" int ls_attention(int dtype, const void* q, long ldq, const void* k_pa
     LS_REQUIRE(page_size >= 8, "attention: the cooperative variant needs pages of at least 8 keys, got %d", page_size);
     int rc = 0;
     if (dtype == kF32)
-      rc = launch_coop<float, false>(grid, s, q, ldq, k_pages, v_pages, nkv, page_size, page_shift, table, table_stride,
+      rc = launch_coop<float, false>(spans != 0, grid, s, q, ldq, k_pages, v_pages, nkv, page_size, page_shift, table, table_stride,
                                      seqs, items, out, ldo, part_acc, part_ml, G, scale, window, DecodeFuse<float>{});
     else if (dtype == kBF16)
-      rc = launch_coop<bf16_t, false>(grid, s, q, ldq, k_pages, v_pages, nkv, page_size, page_shift, table,
+      rc = launch_coop<bf16_t, false>(spans != 0, grid, s, q, ldq, k_pages, v_pages, nkv, page_size, page_shift, table,
                                       table_stride, seqs, items, out, ldo, part_acc, part_ml, G, scale, window,
                                       DecodeFuse<bf16_t>{});
     else

@@ -282,7 +282,8 @@ class Model:
                         cache.assert_exclusive(r, gi, logical)
         cache.sync_tables()
         entries = [StepEntry(r, [t], [0]) for r, t in zip(requests, tokens)]
-        ctx = StepContext(self.rt, cache, self.workspace, entries, fixed_shape=True, horizon=n_steps - 1)
+        # (a loop of one step is laid out like longer ones, so that they share a graph)
+        ctx = StepContext(self.rt, cache, self.workspace, entries, fixed_shape=True, horizon=max(n_steps - 1, 1))
         for mixer in self._preparers:
             mixer.prepare(ctx)
         ctx.upload()

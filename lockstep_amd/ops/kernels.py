@@ -407,12 +407,13 @@ class Kernels:
 
     def attention(self, q: torch.Tensor, nq: int, nkv: int, d: int, k_pages, v_pages, page_size: int, table,
                   seqs, items, n_items: int, out: torch.Tensor, part_acc, part_ml, scale: float,
-                  window: int, variant: int = 0, max_rows: int = 0) -> None:
+                  window: int, variant: int = 0, max_rows: int = 0, spans: bool = False) -> None:
         """Launch the attention kernel over ``n_items`` work items (see attention.hip).
         ``variant``: 0 staged through LDS where it fits, 1 direct from global memory, 2 staged or
         error, 3 cooperative (every item has at most 16 rows; ``max_rows`` states the largest),
         4 wide (prompt portions; items count row blocks of ``attention_block_rows``), 5 the same
-        with half the rows a block (for steps with few rows)."""
+        with half the rows a block (for steps with few rows).  ``spans`` (cooperative only): items
+        that leave partial results may hold several splits each."""
         lib = self.attention_lib(d)
         _rows_ok(q, "attention q"); _rows_ok(out, "attention out")
         if not (q.dtype in DTYPE_CODE and out.dtype == q.dtype):
@@ -435,13 +436,13 @@ class Kernels:
             c_int(DTYPE_CODE[q.dtype]), _ptr(q), c_long(q.stride(0)), _ptr(k_pages), _ptr(v_pages), c_int(nkv),
             c_int(page_size), _ptr(table), c_int(table.shape[1]), _ptr(seqs), _ptr(items), c_int(n_items),
             _ptr(out), c_long(out.stride(0)), _ptr(part_acc), _ptr(part_ml), c_int(nq // nkv), c_float(scale),
-            c_int(window), c_int(variant), c_int(max_rows), _stream())
+            c_int(window), c_int(variant), c_int(max_rows), c_int(1 if spans else 0), _stream())
         self._check(lib, code)
 
     def attention_decode(self, qkv: torch.Tensor, nq: int, nkv: int, d: int, k_pages, v_pages, page_size: int,
                          table, seqs, items, n_items: int, out: torch.Tensor, part_acc, part_ml, scale: float,
                          window: int, q_weight, k_weight, eps: float, cos, sin, rot: int, max_pos: int,
-                         write_kv: bool) -> None:
+                         write_kv: bool, spans: bool = False) -> None:
         """A step of single decoded tokens: what ``qk_rope_kv`` and ``attention`` (cooperative items) do,
         in one launch.  ``qkv`` is the raw fused projection; every request brings exactly one token."""
         lib = self.attention_lib(d)
@@ -478,7 +479,7 @@ class Kernels:
             c_int(nkv), c_int(page_size), _ptr(table), c_int(table.shape[1]), _ptr(seqs), _ptr(items),
             c_int(n_items), _ptr(out), c_long(out.stride(0)), _ptr(part_acc), _ptr(part_ml), c_float(scale),
             c_int(window), _ptr(q_weight), _ptr(k_weight), c_float(eps), _ptr(cos), _ptr(sin), c_int(rot),
-            c_int(positions), c_int(max_pos), c_int(1 if write_kv else 0), _stream())
+            c_int(positions), c_int(max_pos), c_int(1 if write_kv else 0), c_int(1 if spans else 0), _stream())
         self._check(lib, code)
 
     def attention_combine(self, d: int, seqs, items, n_items: int, nq: int, nkv: int, part_acc, part_ml,
@@ -504,7 +505,7 @@ COMBINE_ITEM_INTS = 8
 def pack_attention_items(items, seqs) -> "np.ndarray":
     """Work items of the attention kernels as the device wants them.  ``items``:
     rows of (seq, row_block, split_begin, split_end, part_base, n_splits,
-    split_lo, 0); ``seqs``: the step's rows of (q_off, q_len, q_start, kv_len,
+    split_lo, 0), seq -1 for an item that stands for no work; ``seqs``: the step's rows of (q_off, q_len, q_start, kv_len,
     table_row, 0, 0, 0).  Each item gets a copy of its request's row appended, so
     that a workgroup learns its work from one load."""
     import numpy as np
@@ -513,7 +514,11 @@ def pack_attention_items(items, seqs) -> "np.ndarray":
     seqs = np.asarray(seqs, dtype=np.int64).reshape(-1, 8)
     if not len(items):
         return np.zeros(0, dtype=np.int64)
-    return np.concatenate([items, seqs[items[:, 0]]], axis=1).reshape(-1)
+    null = items[:, 0] < 0
+    rows = seqs[np.maximum(items[:, 0], 0)]
+    rows[null] = 0                               # a null item is all zeros: a request of no rows, no splits
+    items = np.where(null[:, None], 0, items)
+    return np.concatenate([items, rows], axis=1).reshape(-1)
 
 
 def pack_combine_items(items, seqs) -> "np.ndarray":
@@ -525,7 +530,11 @@ def pack_combine_items(items, seqs) -> "np.ndarray":
     if not len(items):
         return np.zeros(0, dtype=np.int64)
     pad = np.zeros((len(items), 2), dtype=np.int64)
-    return np.concatenate([items, seqs[items[:, 0], :2], pad], axis=1).reshape(-1)
+    null = items[:, 0] < 0
+    rows = seqs[np.maximum(items[:, 0], 0), :2]
+    rows[null] = 0
+    items = np.where(null[:, None], 0, items)
+    return np.concatenate([items, rows, pad], axis=1).reshape(-1)
 
 
 _INSTANCE: Kernels | None = None

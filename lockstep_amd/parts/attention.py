@@ -31,6 +31,9 @@ FUSE_DECODE = os.environ.get("LOCKSTEP_FUSE_DECODE", "1") not in ("", "0")
 # From this many attention workgroups on (two a CU: the kernel is then bound by the cache it streams) the
 # prologue of the fused kernel costs more than the separate norm/rotation launch; measured +2 % at batch 64.
 FUSE_DECODE_BELOW = int(os.environ.get("LOCKSTEP_FUSE_DECODE_BELOW", "512"))
+# The most splits (of 256 keys) one cooperative workgroup walks when a request is cut over several.
+MAX_SPAN = int(os.environ.get("LOCKSTEP_ATTENTION_MAX_SPAN", "4"))
+PART_ROWS_STEP = 4096      # rows of partial results are taken in steps of this many (sizes of replayed steps)
 
 
 # ---------------------------------------------------------------------------
@@ -52,6 +55,7 @@ class AttentionPlan:
     part_rows: int            # rows of partial results the split items leave
     decode_fused: bool        # every request brings one token and the fused decode kernel can take the step
     wide_variant: int = 4     # 4: row blocks of 128 rows, 5: of 64
+    spans: bool = False       # cooperative items that leave partial results hold several splits each
 
     ITEM, COMBINE = 16, 8
 
@@ -64,24 +68,36 @@ class AttentionPlan:
 
     def signature(self):
         return (self.n_items, self.n_combine, self.n_coop, self.n_wide, self.part_rows, self.decode_fused,
-                self.wide_variant)
+                self.wide_variant, self.spans)
+
+
+def _round_up(n: int, buckets=(1, 2, 4, 8, 16, 32, 64), step: int = 64) -> int:
+    """``n`` rounded up to one of a few sizes (then to a multiple of ``step``): list sizes of
+    graph-replayed steps, so that one graph serves many steps."""
+    for b in buckets:
+        if n <= b:
+            return b
+    return -(-n // step) * step
 
 
 def plan_attention(ctx, group_size: int, nkv: int, head_dim: int, window: int):
     """Work items of one set of attention constants for this step: (plan, ints of the block).
 
     Requests are cut at the kernels' own, position-anchored splits; which kernel takes a request
-    and whether a workgroup walks all splits or leaves one partial result per split is chosen
-    here freely, because every choice gives the same bits.  With ``ctx.fixed_shape`` the size of
-    the lists depends only on the number of requests and on a bucket of the longest context:
-    every request gets one item per split up to the bucket (items past a request's own length
-    leave empty partial results, which the fold skips), so a captured graph of the step stays
-    valid from one decode step to the next."""
+    and whether a workgroup walks a request's splits itself or leaves a partial result per split
+    to the fold is chosen here freely, because every choice gives the same bits.
+
+    Decoded tokens (at most 16 rows a kv head) go to the cooperative kernel.  While the step's
+    splits would not fill the GPU twice over, every split is a work item of its own.  Beyond
+    that a workgroup walks a whole request and writes the output -- unless the requests are of
+    very different lengths: a workgroup takes a few microseconds a tile whatever else runs, so
+    the longest request would decide when the launch ends; requests are then cut into items of
+    MAX_SPAN splits.  With ``ctx.fixed_shape`` (a step whose launches are captured and replayed)
+    the lists are laid out for the lengths the requests will have ``ctx.horizon`` tokens on,
+    and their sizes are rounded up with null items, so that one graph serves the steps to come."""
     kernels, dtype, page_size = ctx.rt.kernels, ctx.rt.dtype, ctx.cache.page_size
     tile, split = kernels.attention_geometry(head_dim)
     coop_ok = kernels.coop_supported(head_dim, dtype, page_size)
-    # with a workgroup per CU anyway, one workgroup walks all splits of a request itself
-    whole_requests = ctx.n_seqs * nkv >= 256
     wide_ok = kernels.wide_supported(head_dim, dtype, page_size)
     wide_variant, wide_rows = 4, kernels.attention_block_rows(head_dim, 4)
     if wide_ok:
@@ -89,69 +105,64 @@ def plan_attention(ctx, group_size: int, nkv: int, head_dim: int, window: int):
         blocks = sum(-(-(int(q) * group_size) // wide_rows) for q in ctx.q_len if int(q) * group_size > 64)
         if 0 < blocks * nkv <= kernels.compute_units() // 2:
             wide_variant, wide_rows = 5, kernels.attention_block_rows(head_dim, 5)
+
+    # splits every request has (when the step's last token of the horizon is in): first, count
+    first_query = ctx.q_start
+    lo = (np.maximum(0, first_query - window + 1) // split) if window > 0 else np.zeros(ctx.n_seqs, dtype=np.int64)
+    counts = (ctx.kv_len + ctx.horizon - 1) // split + 1 - lo
+    rows_of = ctx.q_len * group_size
+    to_coop = (rows_of <= 16) & coop_ok
+    span = 1
+    if to_coop.any():
+        mine = counts[to_coop]
+        if int(mine.sum()) * nkv >= 2 * kernels.compute_units():
+            ragged = int(mine.max()) > 2 * float(mine.mean())
+            span = MAX_SPAN if ragged else int(mine.max())      # the latter: every request is walked whole
+
     items, coop, wide, combine = [], [], [], []
-    coop_max_rows = part_rows = bucket = 0
-    if ctx.fixed_shape:
-        longest = (int(ctx.kv_len.max()) + ctx.horizon - 1) // split + 1
-        bucket = 1
-        while bucket < longest:
-            bucket = bucket * 2 if bucket < 8 else bucket + 8
-        if coop_ok and group_size <= 16 and ctx.single_tokens:
-            # a decode step: the lists depend on its shape only, the requests' rows are appended
-            shape = ("attention.template", ctx.n_seqs, group_size, nkv, bucket, whole_requests)
-            made = ctx.memo.get(shape)
-            if made is None:
-                for i in range(ctx.n_seqs):
-                    if whole_requests:
-                        coop.append((i, 0, 0, bucket, -1, 0, 0, 0))
-                    else:
-                        base = part_rows
-                        part_rows += nkv * group_size * bucket
-                        coop += [(i, 0, s, s + 1, base, bucket, 0, 0) for s in range(bucket)]
-                        combine.append((i, 0, base, bucket))
-                made = (np.asarray(coop, dtype=np.int64).reshape(-1, 8),
-                        np.asarray(combine, dtype=np.int64).reshape(-1, 4), part_rows)
-                ctx.memo[shape] = made
-            coop_t, combine_t, part_rows = made
-            plan = AttentionPlan(0, len(combine_t), len(coop_t), group_size, 0, part_rows,
-                                 kernels.decode_fused_supported(head_dim, dtype, page_size))
-            return plan, np.concatenate([pack_combine_items(combine_t, ctx.seq_rows),
-                                         pack_attention_items(coop_t, ctx.seq_rows)])
+    coop_max_rows = part_rows = 0
     for i in range(ctx.n_seqs):
-        q_len, q_start, kv_len = int(ctx.q_len[i]), int(ctx.q_start[i]), int(ctx.kv_len[i])
-        rows = q_len * group_size
-        lo_valid = max(0, q_start - window + 1) if window > 0 else 0
-        split_lo = lo_valid // split
-        n_splits = (kv_len - 1) // split + 1 - split_lo
-        if ctx.fixed_shape:
-            split_lo, n_splits = 0, bucket
-        # items of at most 16 rows (decoded tokens) go to the cooperative kernel
-        target = coop if (coop_ok and rows <= 16) else items
-        if target is coop:
+        q_len, q_start = int(ctx.q_len[i]), int(ctx.q_start[i])
+        rows = int(rows_of[i])
+        split_lo, n_splits = int(lo[i]), int(counts[i])
+        if to_coop[i]:
             coop_max_rows = max(coop_max_rows, rows)
-        if rows <= 64 and (n_splits > 1 or ctx.fixed_shape) and not (target is coop and whole_requests):
+            if n_splits <= span:
+                coop.append((i, 0, split_lo, split_lo + n_splits, -1, 0, 0, 0))       # writes the output itself
+            else:
+                base = part_rows
+                part_rows += nkv * rows * n_splits
+                for first in range(split_lo, split_lo + n_splits, span):
+                    coop.append((i, 0, first, min(first + span, split_lo + n_splits), base, n_splits, split_lo, 0))
+                combine.append((i, 0, base, n_splits))
+        elif rows <= 64 and (n_splits > 1 or ctx.fixed_shape):
             base = part_rows
             part_rows += nkv * rows * n_splits
-            for s in range(split_lo, split_lo + n_splits):
-                target.append((i, 0, s, s + 1, base, n_splits, split_lo, 0))
+            for first in range(split_lo, split_lo + n_splits):
+                items.append((i, 0, first, first + 1, base, n_splits, split_lo, 0))
             combine.append((i, 0, base, n_splits))
         else:
             # long portions go to the wide kernel, in larger row blocks
-            if wide_ok and rows > 64:
-                target, block_rows = wide, wide_rows
-            else:
-                block_rows = 64
+            target, block_rows = (wide, wide_rows) if (wide_ok and rows > 64) else (items, 64)
             for block in range(-(-rows // block_rows)):
                 first_pos = q_start + (block * block_rows) // group_size
                 last_pos = q_start + min((block + 1) * block_rows - 1, rows - 1) // group_size
                 begin = (max(0, first_pos - window + 1) // split) if window > 0 else 0
                 target.append((i, block, begin, last_pos // split + 1, -1, 0, 0, 0))
+    if ctx.fixed_shape:
+        # null work (request -1 here, an item of zeros on the device) up to a size that many steps share
+        null_item, null_fold = (-1, 0, 0, 0, -1, 0, 0, 0), (-1, 0, 0, 0)
+        for work, null in ((items, null_item), (coop, null_item), (combine, null_fold)):
+            if work:
+                work += [null] * (_round_up(len(work)) - len(work))
+        part_rows = _round_up(part_rows, buckets=(), step=PART_ROWS_STEP) if part_rows else 0
     decode_fused = (coop_ok and not items and not wide and bool((ctx.q_len == 1).all())
                     and kernels.decode_fused_supported(head_dim, dtype, page_size))
     # the longest row blocks first: they decide when the launch ends
     wide.sort(key=lambda it: it[2] - it[3])
+    spans = any(it[4] >= 0 and it[3] - it[2] > 1 for it in coop)
     plan = AttentionPlan(len(items), len(combine), len(coop), coop_max_rows, len(wide), part_rows, decode_fused,
-                         wide_variant)
+                         wide_variant, spans)
     return plan, np.concatenate([pack_attention_items(items, ctx.seq_rows), pack_combine_items(combine, ctx.seq_rows),
                                  pack_attention_items(coop, ctx.seq_rows), pack_attention_items(wide, ctx.seq_rows)])
 
@@ -292,7 +303,7 @@ class Attention(Mixer):
             k.attention_decode(qkv, nq, nkv, d, key_pages, value_pages, group.page_size, group.table, ctx.seqs,
                                coop_items, plan.n_coop, attn, part_acc, part_ml, self.scale, window,
                                self.q_norm, self.k_norm, self.norm_eps, self.position.cos, self.position.sin,
-                               self.position.rotary_dim, ctx.max_position, run.writes_cache)
+                               self.position.rotary_dim, ctx.max_position, run.writes_cache, plan.spans)
             if plan.n_combine:
                 k.attention_combine(d, ctx.seqs, combine_items, plan.n_combine, nq, nkv, part_acc, part_ml, attn)
             return self._project_out(ctx, attn, out, accumulate, defer)
@@ -305,7 +316,7 @@ class Attention(Mixer):
         if plan.n_coop:
             k.attention(qkv, nq, nkv, d, key_pages, value_pages, group.page_size, group.table, ctx.seqs,
                         coop_items, plan.n_coop, attn, part_acc, part_ml, self.scale, window,
-                        variant=3, max_rows=plan.coop_max_rows)
+                        variant=3, max_rows=plan.coop_max_rows, spans=plan.spans)
         if plan.n_wide:
             k.attention(qkv, nq, nkv, d, key_pages, value_pages, group.page_size, group.table, ctx.seqs,
                         wide_items, plan.n_wide, attn, part_acc, part_ml, self.scale, window,

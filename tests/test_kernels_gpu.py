@@ -288,7 +288,10 @@ class PagedCase:
         K().qk_rope_kv(qkv, t, self.nq, self.nkv, self.d, q_norm, k_norm, eps, cos, sin, rot, tok_seq, tok_pos,
                        self.seqs(q_start, t), q_start + t - 1, self.table, self.k_pages, self.v_pages, self.ps, True)
 
-    def attend(self, qkv, q_start, scale, window=0, force_split=None, variant=0, repeat=1):
+    def attend(self, qkv, q_start, scale, window=0, force_split=None, variant=0, repeat=1, span=1, pad_splits=0):
+        """``span``: splits one work item walks when the request is cut (the cooperative kernel takes more
+        than one and leaves a partial result for each); ``pad_splits``: lay the items out for that many
+        more splits than the request has (as the fixed-shape lists of graph-replayed steps do)."""
         from lockstep_amd.ops import kernels
 
         t = qkv.shape[0]
@@ -303,10 +306,11 @@ class PagedCase:
         items, combine, part_rows = [], [], 0
         br = kernels().attention_block_rows(self.d, variant)       # rows of a work item's row block
         if use_split:
+            n_splits += pad_splits
             part_rows = self.nkv * rows * n_splits
             for b in range(-(-rows // br)):
-                for s in range(split_lo, split_lo + n_splits):
-                    items += [0, b, s, s + 1, 0, n_splits, split_lo, 0]
+                for s in range(split_lo, split_lo + n_splits, span):
+                    items += [0, b, s, min(s + span, split_lo + n_splits), 0, n_splits, split_lo, 0]
             for b in range(-(-rows // 64)):
                 combine += [0, b, 0, n_splits]
         else:
@@ -326,7 +330,7 @@ class PagedCase:
         part_ml = torch.full((max(part_rows, 1), 2), float("nan"), dtype=torch.float32, device="cuda")
         K().attention(qkv, self.nq, self.nkv, self.d, self.k_pages, self.v_pages, self.ps, self.table,
                       self.seqs(q_start, t), items_t, n_items, out, part_acc, part_ml, scale, window,
-                      variant, rows)
+                      variant, rows, spans=span > 1)
         if combine:
             comb = torch.from_numpy(pack_combine_items(combine, seq_row)).to(torch.int32).cuda()
             K().attention_combine(self.d, self.seqs(q_start, t), comb, len(combine) // 4, self.nq, self.nkv,
@@ -550,6 +554,28 @@ def test_decode_attention_is_the_same_in_every_kernel(dtype, nq, nkv, d, ps):
         for variant, split in variants:
             got = case.attend(dev[start:start + n], start, d ** -0.5, variant=variant, force_split=split)
             assert torch.equal(got, ref), f"start={start} n={n} variant={variant} split={split}"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nq,nkv,d,ps", [(16, 8, 128, 16), (4, 4, 16, 8), (6, 2, 48, 16), (3, 3, 32, 8)])
+def test_cooperative_items_of_several_splits_leave_the_same_partial_results(dtype, nq, nkv, d, ps):
+    """A long request cut into work items of one, two, three or four splits each (a partial result a
+    split, folded by the combine kernel), laid out for more splits than it has, with and without
+    a window: the bits of one workgroup walking the whole request."""
+    if not K().coop_supported(d, dtype, ps):
+        pytest.skip("the cooperative kernel's tiles do not fit")
+    kv_len = 1400                                     # six splits, the last one partly filled
+    qkv = rand_qkv(kv_len, nq, nkv, d, dtype, seed=3 * d + nq, sharp=(9,))
+    case = PagedCase(dtype, nq, nkv, d, ps, kv_len, shuffle_seed=5)
+    dev = qkv.cuda()
+    case.write(dev, 0)
+    for window in (0, 700):
+        for start in (1399, 1279, 1024, 511):
+            ref = case.attend(dev[start:start + 1], start, d ** -0.5, window=window, variant=3, force_split=False)
+            for span, pad in ((1, 0), (2, 0), (3, 1), (4, 0), (4, 3), (8, 0)):
+                got = case.attend(dev[start:start + 1], start, d ** -0.5, window=window, variant=3, force_split=True,
+                                  span=span, pad_splits=pad)
+                assert torch.equal(got, ref), f"start={start} window={window} span={span} pad={pad}"
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

@@ -119,6 +119,48 @@ def test_many_requests_decode_with_the_bits_of_one(models, name):
         assert torch.equal(torch.stack([t[i] for t in together]), want), f"request {i} (context {lengths[i]})"
 
 
+def test_requests_of_very_different_lengths_decode_with_the_bits_of_one(models):
+    """Forty requests between 20 and 1,500 tokens in one decode step: there are so many splits that
+    the long requests are cut into work items of several splits each (partial results and a fold),
+    the short ones are walked whole, and the graph-replayed steps lay every request out for the
+    longest; each request has the bits it has alone, eagerly and from the replayed graph."""
+    from lockstep_amd.engine.batch import StepEntry
+
+    folder, config = models["0.6b-like"]
+    model = load(folder, "bfloat16")
+    vocab = config.vocab_size
+    n_req, n_decode = 40, 3
+    lengths = [20 + (37 * i * i) % 1480 for i in range(n_req)]
+    assert max(lengths) > 1300 and min(lengths) < 100
+    prompts = [random_tokens(m + n_decode, vocab, seed=150 + i) for i, m in enumerate(lengths)]
+    cache = model.make_cache(num_pages=sum(-(-(m + n_decode) // 16) for m in lengths) + 4, page_size=16,
+                             max_requests=n_req)
+    for i in range(n_req):
+        cache.open(f"r{i}")
+        model.step(cache, [StepEntry(f"r{i}", prompts[i][:lengths[i]], [])])
+    replays = model.graph_replays
+    together = [model.step(cache, [StepEntry(f"r{i}", [prompts[i][lengths[i] + k]], [0]) for i in range(n_req)]).cpu()
+                for k in range(n_decode)]
+    assert model.graph_replays > replays
+    # the same step through the lists of a step that is not replayed (a portion of two tokens beside it)
+    extra = random_tokens(300, vocab, seed=3)
+    cache2 = model.make_cache(num_pages=sum(-(-(m + n_decode) // 16) for m in lengths) + 40, page_size=16,
+                              max_requests=n_req + 1)
+    for i in range(n_req):
+        cache2.open(f"r{i}")
+        model.step(cache2, [StepEntry(f"r{i}", prompts[i][:lengths[i]], [])])
+    cache2.open("x")
+    model.step(cache2, [StepEntry("x", extra[:298], [])])
+    mixed = model.step(cache2, [StepEntry(f"r{i}", [prompts[i][lengths[i]]], [0]) for i in range(n_req)]
+                       + [StepEntry("x", extra[298:], [1])]).cpu()
+    assert torch.equal(mixed[:n_req], together[0])
+    longest, shortest = lengths.index(max(lengths)), lengths.index(min(lengths))
+    for i in (0, longest, shortest, n_req - 1):
+        alone = model.make_cache(num_pages=100, page_size=16)
+        want = feed(model, alone, "x", prompts[i], [lengths[i]] + [1] * n_decode)[lengths[i]:]
+        assert torch.equal(torch.stack([t[i] for t in together]), want), f"request {i} (context {lengths[i]})"
+
+
 def test_the_32_bit_path_matches_plain_at_real_layer_sizes(models):
     """float32 against the plain float64 implementation, and bfloat16 within its tolerance, on the
     two-layer configuration (whole prompt and decoded tail)."""
