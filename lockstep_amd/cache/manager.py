@@ -400,6 +400,15 @@ class CacheManager:
         """State tensor ``[slots, *shape]`` of a unit with a ``StateSpec``."""
         return self.state[unit]
 
+    def unit_tensors(self, unit: int) -> tuple:
+        """The device tensors that are this unit's own: (key pages, value pages), (state,) or ()."""
+        if unit in self.unit_place:
+            gi, position = self.unit_place[unit]
+            return (self.groups[gi].keys[position], self.groups[gi].values[position])
+        if unit in self.state:
+            return (self.state[unit],)
+        return ()
+
     # -- accounting -----------------------------------------------------------------
     @property
     def free_pages(self) -> list[int]:

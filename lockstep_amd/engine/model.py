@@ -12,6 +12,7 @@ from __future__ import annotations
 
 import itertools
 import os
+import weakref
 from typing import Sequence
 
 import numpy as np
@@ -24,6 +25,7 @@ from ..parts.base import device_epoch, graph_safe_tree, takes
 from ..weights.store import load_weights, weights_from_dict
 from .batch import StepContext, StepEntry, Workspace
 from .runtime import Runtime
+from .tape import LayerTape, RunKinds
 
 
 def collect_weight_specs(spec: ModelSpec) -> list[WeightSpec]:
@@ -81,6 +83,17 @@ class Model:
                 if group is not None:
                     seen.add(group)
         self.graph_replays = 0
+        # layers alike repeat the launches of the second of them (engine/tape.py)
+        self.use_tapes = os.environ.get("LOCKSTEP_NO_TAPES", "") in ("", "0")
+        self.verify_tapes = os.environ.get("LOCKSTEP_VERIFY_TAPE", "") not in ("", "0")
+        self._run_kinds = weakref.WeakKeyDictionary()      # cache manager -> (device epoch, RunKinds)
+        self.layers_repeated = 0
+
+    def _kinds_for(self, cache) -> RunKinds:
+        held = self._run_kinds.get(cache)
+        if held is None or held[0] != device_epoch():
+            held = self._run_kinds[cache] = (device_epoch(), RunKinds(self, cache))
+        return held[1]
 
     # -- weights --------------------------------------------------------------
     def load(self, weights) -> "Model":
@@ -166,15 +179,48 @@ class Model:
         h = ctx.buf("residual", (ctx.n_tokens, self.spec.hidden_size), torch.float32)
         self.embedding.forward(ctx, ctx.token_ids, h)
         pending = None          # an addition to h that a layer left to the next reader of h
-        for run in self.schedule:
-            layer = self.layers[run.layer]
-            if self._layer_takes_pending[run.layer]:
-                pending = layer.forward(ctx, run, h, pending=pending)
-            else:
-                if pending is not None:
-                    pending.flush(ctx, h)
-                pending = None
-                layer.forward(ctx, run, h)
+        kernels = self.rt.kernels
+        kinds = self._kinds_for(ctx.cache) if self.use_tapes else None
+        met: dict = {}          # kind of run -> None after its first run, then (tape, situation, what it left)
+        for index, run in enumerate(self.schedule):
+            kind = kinds.kind[index] if kinds is not None else None
+            situation = None
+            if kind is not None:
+                situation = (self.workspace.version,
+                             None if pending is None else (pending.partials.data_ptr(), tuple(pending.partials.shape)))
+                held = met.get(kind)
+                if held is not None and held[1] == situation and not self.verify_tapes:
+                    held[0].repeat(kinds.addresses[index])
+                    pending = held[2]
+                    self.layers_repeated += 1
+                    continue
+            noting = kind is not None and kind in met
+            if noting:
+                outer, kernels.tape = kernels.tape, []
+            try:
+                layer = self.layers[run.layer]
+                if self._layer_takes_pending[run.layer]:
+                    pending = layer.forward(ctx, run, h, pending=pending)
+                else:
+                    if pending is not None:
+                        pending.flush(ctx, h)
+                    pending = None
+                    layer.forward(ctx, run, h)
+            finally:
+                if noting:
+                    launches, kernels.tape = kernels.tape, outer
+                    if outer is not None:
+                        outer.extend(launches)
+            if kind is None:
+                continue
+            if not noting:
+                met[kind] = None
+                continue
+            held = met[kind]
+            if held is not None and held[1] == situation:          # only with verify_tapes
+                held[0].compare(launches, kinds.addresses[index], f"layer run {index}")
+            if situation[0] == self.workspace.version:             # the run did not move the workspace
+                met[kind] = (LayerTape(launches, kinds.addresses[index]), situation, pending)
         if ctx.n_want:
             x = ctx.buf("final.normed", (ctx.n_want, self.spec.hidden_size), self.rt.dtype)
             if pending is not None and self._final_takes_pending:

@@ -1,0 +1,145 @@
+"""Repeating one layer's launches for the layers that are like it.
+
+A step that is not replayed from a captured graph launches some eight kernels a layer, and the
+Python that leads up to each launch (the part's ``forward``, the checks of the kernel wrapper,
+building the arguments) costs twice what the launch itself costs.  Layers of one model mostly
+differ in nothing but the addresses of their weights and of their unit of the cache.  So within a
+step the engine runs a layer's ``forward`` in Python only for the first two layers of a kind: the
+second run is noted launch by launch (``Kernels.tape``), and for every further layer of that kind
+the noted launches are made again with this layer's addresses in the place of that layer's.
+
+What makes two schedule entries *alike* (``RunKinds``): parts that all say ``repeatable``, equal
+layer specifications apart from the tensor-name prefix, the same answer to ``writes_cache``, and
+cache units in the same group of the cache.  The first run of a kind is never noted, because parts
+may do once a step what later layers find done.  A noted run stands for later ones only while they
+arrive in the same situation: the same pending addition (or none) and an unchanged workspace.
+
+``LOCKSTEP_VERIFY_TAPE=1`` runs every layer in Python all the same and compares its launches,
+argument by argument, with what the tape would have launched.
+"""
+
+from __future__ import annotations
+
+import dataclasses
+from ctypes import c_void_p
+
+import torch
+
+from ..ops.kernels import KernelError
+from ..parts.base import Part
+
+
+def device_constants(part: Part) -> dict:
+    """Device tensors that ``part`` and the parts below it hold, by a name that is the same for
+    every layer of the same build: attribute names along the path through ``parts()``."""
+    found: dict = {}
+
+    def collect(value, name):
+        if isinstance(value, torch.Tensor):
+            if value.is_cuda and value.numel():
+                found[name] = value
+        elif isinstance(value, (list, tuple)):
+            for i, v in enumerate(value):
+                if isinstance(v, torch.Tensor):
+                    collect(v, f"{name}[{i}]")
+        elif isinstance(value, dict):
+            for k, v in value.items():
+                if isinstance(v, torch.Tensor):
+                    collect(v, f"{name}[{k!r}]")
+
+    def walk(p, path):
+        for name, value in vars(p).items():
+            if not isinstance(value, Part):
+                collect(value, f"{path}{name}")
+        for i, child in enumerate(p.parts()):
+            walk(child, f"{path}{i}/")
+
+    walk(part, "")
+    return found
+
+
+def repeatable_tree(part: Part) -> bool:
+    return bool(getattr(part, "repeatable", False)) and all(repeatable_tree(p) for p in part.parts())
+
+
+def _spec_without_prefix(layer_spec):
+    if dataclasses.is_dataclass(layer_spec):
+        fields = {f.name: getattr(layer_spec, f.name) for f in dataclasses.fields(layer_spec)}
+        fields.pop("prefix", None)
+        return fields
+    return layer_spec
+
+
+class RunKinds:
+    """For one model and one cache: which schedule entries are alike, and every entry's addresses."""
+
+    def __init__(self, model, cache):
+        self.kind: list = []            # per schedule entry: a small int, or None (always run in Python)
+        self.addresses: list = []       # per schedule entry: name -> (address, bytes)
+        seen: list = []
+        for run in model.schedule:
+            layer = model.layers[run.layer]
+            tensors = dict(device_constants(layer))
+            for i, t in enumerate(cache.unit_tensors(run.cache)):
+                tensors[f"cache[{i}]"] = t
+            group = cache.unit_place.get(run.cache, (None,))[0]
+            self.addresses.append({name: (t.data_ptr(), t.numel() * t.element_size()) for name, t in tensors.items()})
+            if not repeatable_tree(layer):
+                self.kind.append(None)
+                continue
+            key = (_spec_without_prefix(model.spec.layers[run.layer]), bool(run.writes_cache), group,
+                   tuple((name, tuple(t.shape), t.dtype) for name, t in tensors.items()))
+            for i, known in enumerate(seen):
+                if known == key:
+                    self.kind.append(i)
+                    break
+            else:
+                seen.append(key)
+                self.kind.append(len(seen) - 1)
+
+
+def _value(arg):
+    return getattr(arg, "value", arg)
+
+
+class LayerTape:
+    """The launches of one layer run, with the places marked where an address of that layer stands."""
+
+    def __init__(self, launches, addresses: dict):
+        ranges = sorted((base, base + size, name) for name, (base, size) in addresses.items())
+        self.calls = []
+        for lib, entry, args in launches:
+            marks = []
+            for i, a in enumerate(args):
+                if isinstance(a, c_void_p) and a.value:
+                    for lo, hi, name in ranges:
+                        if lo <= a.value < hi:
+                            marks.append((i, name, a.value - lo))
+                            break
+            self.calls.append((lib, entry, args, tuple(marks)))
+
+    def arguments(self, addresses: dict):
+        """(library, entry point, arguments) of every launch, for the layer with these addresses."""
+        for lib, entry, args, marks in self.calls:
+            if marks:
+                args = list(args)
+                for i, name, offset in marks:
+                    args[i] = c_void_p(addresses[name][0] + offset)
+            yield lib, entry, args
+
+    def repeat(self, addresses: dict) -> None:
+        for lib, entry, args in self.arguments(addresses):
+            if entry(*args) != 0:
+                raise KernelError(lib.ls_last_error().decode())
+
+    def compare(self, launches, addresses: dict, what: str) -> None:
+        """Raise unless ``launches`` (of a layer run in Python) are what ``repeat`` would launch."""
+        mine = list(self.arguments(addresses))
+        if len(mine) != len(launches):
+            raise RuntimeError(f"{what}: the layer launched {len(launches)} kernels, the tape holds {len(mine)}")
+        for n, ((_, entry, args), (_, entry2, args2)) in enumerate(zip(mine, launches)):
+            same = entry == entry2 and len(args) == len(args2) and all(
+                _value(a) == _value(b) for a, b in zip(args, args2))
+            if not same:
+                raise RuntimeError(f"{what}: launch {n} ({getattr(entry2, '__name__', entry2)}) differs from the "
+                                   f"tape's: {[_value(a) for a in args2]} against {[_value(a) for a in args]}")

@@ -80,12 +80,21 @@ class Kernels:
         self.attention_paths: dict[int, str] = {}
         self._argmax_scratch: dict = {}
         self._capabilities: dict = {}
+        #: while this is a list, every launch is noted on it as (library, entry point, arguments):
+        #: the engine repeats the launches of one layer for the next layers that are alike
+        self.tape: list | None = None
 
     # -- helpers ------------------------------------------------------------
     @staticmethod
     def _check(lib, code: int) -> None:
         if code != 0:
             raise KernelError(lib.ls_last_error().decode())
+
+    def _launch(self, lib, entry, args: tuple) -> None:
+        if entry(*args) != 0:
+            raise KernelError(lib.ls_last_error().decode())
+        if self.tape is not None:
+            self.tape.append((lib, entry, args))
 
     def attention_lib(self, head_dim: int):
         lib = self._attention.get(head_dim)
@@ -189,10 +198,9 @@ class Kernels:
             raise KernelError(f"gemm out dtype {out.dtype} does not fit epilogue {epilogue}")
         if m == 0:
             return
-        code = self.core.ls_gemm(c_int(DTYPE_CODE[w.dtype]), c_int(epilogue), _ptr(x), _ptr(w), _ptr(out),
-                                 c_int(m), c_int(n), c_int(k), c_long(x.stride(0)), c_long(out.stride(0)),
-                                 _ptr(norm_weight), c_float(eps), c_int(cols), _stream())
-        self._check(self.core, code)
+        self._launch(self.core, self.core.ls_gemm, (
+            c_int(DTYPE_CODE[w.dtype]), c_int(epilogue), _ptr(x), _ptr(w), _ptr(out), c_int(m), c_int(n), c_int(k),
+            c_long(x.stride(0)), c_long(out.stride(0)), _ptr(norm_weight), c_float(eps), c_int(cols), _stream()))
 
     def gemm_slices_count(self, k: int) -> int:
         """K slices of a product over ``k`` (first dimension of ``gemm_slices``'s output)."""
@@ -217,9 +225,9 @@ class Kernels:
         if not (partials.is_cuda and partials.dtype == torch.float32 and partials.is_contiguous()
               and partials.shape == (self.gemm_slices_count(k), m, n)):
             raise KernelError(f"gemm_slices partials must be float32 [{self.gemm_slices_count(k)}, {m}, {n}]")
-        code = self.core.ls_gemm_slices(c_int(DTYPE_CODE[w.dtype]), _ptr(x), _ptr(w), _ptr(partials), c_int(m),
-                                        c_int(n), c_int(k), c_long(x.stride(0)), _stream())
-        self._check(self.core, code)
+        self._launch(self.core, self.core.ls_gemm_slices, (
+            c_int(DTYPE_CODE[w.dtype]), _ptr(x), _ptr(w), _ptr(partials), c_int(m), c_int(n), c_int(k),
+            c_long(x.stride(0)), _stream()))
 
     def add_rmsnorm(self, h: torch.Tensor, partials: torch.Tensor, weight, out, eps: float = 0.0,
                     rows: torch.Tensor | None = None) -> None:
@@ -247,10 +255,10 @@ class Kernels:
             dtype, ld_out = out.dtype, out.stride(0)
         if n_rows == 0:
             return
-        code = self.core.ls_add_rmsnorm(c_int(DTYPE_CODE[dtype]), _ptr(h), _ptr(partials), c_int(partials.shape[0]),
-                                        c_int(partials.shape[1]), _ptr(weight), _ptr(out), _ptr(rows), c_int(n_rows),
-                                        c_int(h.shape[1]), c_long(h.stride(0)), c_long(ld_out), c_float(eps), _stream())
-        self._check(self.core, code)
+        self._launch(self.core, self.core.ls_add_rmsnorm, (
+            c_int(DTYPE_CODE[dtype]), _ptr(h), _ptr(partials), c_int(partials.shape[0]), c_int(partials.shape[1]),
+            _ptr(weight), _ptr(out), _ptr(rows), c_int(n_rows), c_int(h.shape[1]), c_long(h.stride(0)),
+            c_long(ld_out), c_float(eps), _stream()))
 
     # -- rows -------------------------------------------------------------------
     def embed(self, tokens: torch.Tensor, table: torch.Tensor, out: torch.Tensor) -> None:
@@ -263,10 +271,9 @@ class Kernels:
             raise KernelError(f"embed out must be float32 [{tokens.shape[0]},{table.shape[1]}]")
         if tokens.shape[0] == 0:
             return
-        code = self.core.ls_embed(c_int(DTYPE_CODE[table.dtype]), _ptr(tokens), _ptr(table), _ptr(out),
-                                  c_int(tokens.shape[0]), c_int(table.shape[0]), c_int(table.shape[1]),
-                                  c_long(out.stride(0)), _stream())
-        self._check(self.core, code)
+        self._launch(self.core, self.core.ls_embed, (
+            c_int(DTYPE_CODE[table.dtype]), _ptr(tokens), _ptr(table), _ptr(out), c_int(tokens.shape[0]),
+            c_int(table.shape[0]), c_int(table.shape[1]), c_long(out.stride(0)), _stream()))
 
     def rmsnorm(self, x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, eps: float,
                 rows: torch.Tensor | None = None) -> None:
@@ -288,10 +295,9 @@ class Kernels:
                 raise KernelError("rmsnorm out must have as many rows as x")
         if n == 0:
             return
-        code = self.core.ls_rmsnorm(c_int(DTYPE_CODE[out.dtype]), _ptr(x), _ptr(weight), _ptr(out), _ptr(rows),
-                                    c_int(n), c_int(x.shape[1]), c_long(x.stride(0)), c_long(out.stride(0)),
-                                    c_float(eps), _stream())
-        self._check(self.core, code)
+        self._launch(self.core, self.core.ls_rmsnorm, (
+            c_int(DTYPE_CODE[out.dtype]), _ptr(x), _ptr(weight), _ptr(out), _ptr(rows), c_int(n), c_int(x.shape[1]),
+            c_long(x.stride(0)), c_long(out.stride(0)), c_float(eps), _stream()))
 
     def swiglu(self, gate_up: torch.Tensor, out: torch.Tensor) -> None:
         _rows_ok(gate_up, "swiglu input"); _rows_ok(out, "swiglu out")
@@ -300,9 +306,9 @@ class Kernels:
             raise KernelError(f"swiglu input must be [{rows},{2 * inter}] of the output's dtype")
         if rows == 0:
             return
-        code = self.core.ls_swiglu(c_int(DTYPE_CODE[out.dtype]), _ptr(gate_up), _ptr(out), c_int(rows), c_int(inter),
-                                   c_long(gate_up.stride(0)), c_long(out.stride(0)), _stream())
-        self._check(self.core, code)
+        self._launch(self.core, self.core.ls_swiglu, (
+            c_int(DTYPE_CODE[out.dtype]), _ptr(gate_up), _ptr(out), c_int(rows), c_int(inter),
+            c_long(gate_up.stride(0)), c_long(out.stride(0)), _stream()))
 
     #: (row, chunk) pairs the library's static arg-max scratch holds (LS_ARGMAX_STATIC_PAIRS)
     ARGMAX_STATIC_PAIRS = 16384
@@ -322,18 +328,18 @@ class Kernels:
             return
         pairs = logits.shape[0] * self.core.ls_argmax_chunks(c_int(logits.shape[1]))
         if pairs <= self.ARGMAX_STATIC_PAIRS:
-            code = self.core.ls_argmax_static(_ptr(logits), _ptr(out), c_int(logits.shape[0]), c_int(logits.shape[1]),
-                                              c_long(logits.stride(0)), _stream())
-            self._check(self.core, code)
+            self._launch(self.core, self.core.ls_argmax_static, (
+                _ptr(logits), _ptr(out), c_int(logits.shape[0]), c_int(logits.shape[1]), c_long(logits.stride(0)),
+                _stream()))
             return
         held = self._argmax_scratch.setdefault(logits.device, [])
         if not held or held[-1].numel() < 2 * pairs:
             held.append(torch.empty(max(2 * pairs, 2 * held[-1].numel() if held else 0), dtype=torch.int32,
                                     device=logits.device))
         scratch = held[-1]
-        code = self.core.ls_argmax(_ptr(logits), _ptr(out), c_int(logits.shape[0]), c_int(logits.shape[1]),
-                                   c_long(logits.stride(0)), _ptr(scratch), c_long(scratch.numel()), _stream())
-        self._check(self.core, code)
+        self._launch(self.core, self.core.ls_argmax, (
+            _ptr(logits), _ptr(out), c_int(logits.shape[0]), c_int(logits.shape[1]), c_long(logits.stride(0)),
+            _ptr(scratch), c_long(scratch.numel()), _stream()))
 
     def advance_decode(self, meta: torch.Tensor, n_seqs: int, off_tokens: int, picked: torch.Tensor,
                        ring: torch.Tensor, counter: torch.Tensor, off_runs: int, n_runs: int) -> None:
@@ -346,10 +352,9 @@ class Kernels:
                 raise KernelError("advance_decode works on int32 GPU tensors")
         if not (picked.numel() >= n_seqs):
             raise KernelError("advance_decode: picked is too short")
-        code = self.core.ls_advance_decode(_ptr(meta), c_long(meta.numel()), c_int(n_seqs), c_int(off_tokens),
-                                           _ptr(picked), _ptr(ring), _ptr(counter), c_int(off_runs), c_int(n_runs),
-                                           _stream())
-        self._check(self.core, code)
+        self._launch(self.core, self.core.ls_advance_decode, (
+            _ptr(meta), c_long(meta.numel()), c_int(n_seqs), c_int(off_tokens), _ptr(picked), _ptr(ring),
+            _ptr(counter), c_int(off_runs), c_int(n_runs), _stream()))
 
     # -- attention ----------------------------------------------------------------
     def qk_rope_kv(self, qkv: torch.Tensor, n_tokens: int, nq: int, nkv: int, d: int, q_weight, k_weight,
@@ -397,13 +402,12 @@ class Kernels:
                 raise KernelError(f"cache pages do not have the layout [pages,{nkv},{page_size},{d}] / [pages,{nkv},{d},{page_size}]")
         if n_tokens == 0:
             return
-        code = self.core.ls_qk_rope_kv(
+        self._launch(self.core, self.core.ls_qk_rope_kv, (
             c_int(DTYPE_CODE[qkv.dtype]), _ptr(qkv), c_long(qkv.stride(0)), c_int(n_tokens), c_int(nq), c_int(nkv),
             c_int(d), _ptr(q_weight), _ptr(k_weight), c_float(eps), _ptr(cos), _ptr(sin), c_int(rot),
-            c_int(positions), _ptr(tok_seq), _ptr(tok_pos), _ptr(seqs), _ptr(table),
-            c_int(table.shape[1] if table is not None else 0), _ptr(k_pages), _ptr(v_pages), c_int(page_size),
-            c_int(1 if write_kv else 0), _stream())
-        self._check(self.core, code)
+            c_int(positions), _ptr(tok_seq), _ptr(tok_pos), _ptr(seqs), _ptr(table), c_int(table.shape[1] if table
+            is not None else 0), _ptr(k_pages), _ptr(v_pages), c_int(page_size), c_int(1 if write_kv else 0),
+            _stream()))
 
     def attention(self, q: torch.Tensor, nq: int, nkv: int, d: int, k_pages, v_pages, page_size: int, table,
                   seqs, items, n_items: int, out: torch.Tensor, part_acc, part_ml, scale: float,
@@ -432,12 +436,11 @@ class Kernels:
             raise KernelError("attention items must hold 16 int32 each (see pack_attention_items)")
         if n_items == 0:
             return
-        code = lib.ls_attention(
+        self._launch(lib, lib.ls_attention, (
             c_int(DTYPE_CODE[q.dtype]), _ptr(q), c_long(q.stride(0)), _ptr(k_pages), _ptr(v_pages), c_int(nkv),
             c_int(page_size), _ptr(table), c_int(table.shape[1]), _ptr(seqs), _ptr(items), c_int(n_items),
             _ptr(out), c_long(out.stride(0)), _ptr(part_acc), _ptr(part_ml), c_int(nq // nkv), c_float(scale),
-            c_int(window), c_int(variant), c_int(max_rows), c_int(1 if spans else 0), _stream())
-        self._check(lib, code)
+            c_int(window), c_int(variant), c_int(max_rows), c_int(1 if spans else 0), _stream()))
 
     def attention_decode(self, qkv: torch.Tensor, nq: int, nkv: int, d: int, k_pages, v_pages, page_size: int,
                          table, seqs, items, n_items: int, out: torch.Tensor, part_acc, part_ml, scale: float,
@@ -474,13 +477,12 @@ class Kernels:
             positions = cos.shape[0]
         if n_items == 0:
             return
-        code = lib.ls_attention_decode(
+        self._launch(lib, lib.ls_attention_decode, (
             c_int(DTYPE_CODE[qkv.dtype]), _ptr(qkv), c_long(qkv.stride(0)), _ptr(k_pages), _ptr(v_pages), c_int(nq),
             c_int(nkv), c_int(page_size), _ptr(table), c_int(table.shape[1]), _ptr(seqs), _ptr(items),
             c_int(n_items), _ptr(out), c_long(out.stride(0)), _ptr(part_acc), _ptr(part_ml), c_float(scale),
             c_int(window), _ptr(q_weight), _ptr(k_weight), c_float(eps), _ptr(cos), _ptr(sin), c_int(rot),
-            c_int(positions), c_int(max_pos), c_int(1 if write_kv else 0), c_int(1 if spans else 0), _stream())
-        self._check(lib, code)
+            c_int(positions), c_int(max_pos), c_int(1 if write_kv else 0), c_int(1 if spans else 0), _stream()))
 
     def attention_combine(self, d: int, seqs, items, n_items: int, nq: int, nkv: int, part_acc, part_ml,
                           out: torch.Tensor) -> None:
@@ -492,10 +494,9 @@ class Kernels:
             raise KernelError("combine items must hold 8 int32 each (see pack_combine_items)")
         if n_items == 0:
             return
-        code = lib.ls_attention_combine(c_int(DTYPE_CODE[out.dtype]), _ptr(seqs), _ptr(items), c_int(n_items),
-                                        c_int(nkv), _ptr(part_acc), _ptr(part_ml), _ptr(out),
-                                        c_long(out.stride(0)), c_int(nq // nkv), _stream())
-        self._check(lib, code)
+        self._launch(lib, lib.ls_attention_combine, (
+            c_int(DTYPE_CODE[out.dtype]), _ptr(seqs), _ptr(items), c_int(n_items), c_int(nkv), _ptr(part_acc),
+            _ptr(part_ml), _ptr(out), c_long(out.stride(0)), c_int(nq // nkv), _stream()))
 
 
 ATTENTION_ITEM_INTS = 16

@@ -32,7 +32,8 @@ FUSE_DECODE = os.environ.get("LOCKSTEP_FUSE_DECODE", "1") not in ("", "0")
 # prologue of the fused kernel costs more than the separate norm/rotation launch; measured +2 % at batch 64.
 FUSE_DECODE_BELOW = int(os.environ.get("LOCKSTEP_FUSE_DECODE_BELOW", "512"))
 # The most splits (of 256 keys) one cooperative workgroup walks when a request is cut over several.
-MAX_SPAN = int(os.environ.get("LOCKSTEP_ATTENTION_MAX_SPAN", "4"))
+MAX_SPAN = 4               # splits of a work item where requests of a ragged batch are cut
+RAGGED_RATIO = 2.0         # a batch is ragged when its longest request has more than this many times the mean splits
 PART_ROWS_STEP = 4096      # rows of partial results are taken in steps of this many (sizes of replayed steps)
 
 
@@ -116,7 +117,7 @@ def plan_attention(ctx, group_size: int, nkv: int, head_dim: int, window: int):
     if to_coop.any():
         mine = counts[to_coop]
         if int(mine.sum()) * nkv >= 2 * kernels.compute_units():
-            ragged = int(mine.max()) > 2 * float(mine.mean())
+            ragged = int(mine.max()) > RAGGED_RATIO * float(mine.mean())
             span = MAX_SPAN if ragged else int(mine.max())      # the latter: every request is walked whole
 
     items, coop, wide, combine = [], [], [], []
@@ -185,6 +186,7 @@ class Attention(Mixer):
     None for all), ``bias`` (must be False), ``scale`` (score multiplier)."""
 
     graph_safe = True
+    repeatable = True
 
     def parts(self):
         return (self.position,)

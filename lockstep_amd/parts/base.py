@@ -88,6 +88,15 @@ class Part:
     #: such part anywhere in the model switches the graphs off for the model.
     graph_safe = False
 
+    #: True if all that ``forward`` does is launch kernels through ``ctx.rt.kernels``, with arguments
+    #: that depend on the layer only through the addresses of device tensors the part holds in its
+    #: attributes (weights) and of its unit of the cache.  The engine then runs ``forward`` for the
+    #: first two layers of a kind in a step and repeats the second one's launches, with each layer's
+    #: own addresses, for the others.  A part that launches in another way (torch operations), keeps
+    #: per-layer state on the host or passes per-layer numbers to a kernel leaves this False, and
+    #: every layer that contains it runs its ``forward`` every time.
+    repeatable = False
+
     def __init__(self, spec: PartSpec, prefix: str = ""):
         self.spec = spec
         self.prefix = prefix

@@ -16,6 +16,7 @@ class PreNormResidual(Arrangement):
     """
 
     graph_safe = True
+    repeatable = True
 
     def __init__(self, layer_spec, prefix: str = ""):
         super().__init__(layer_spec, build_part)

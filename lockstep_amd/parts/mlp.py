@@ -19,6 +19,7 @@ class GatedMLP(FeedForward):
     """Parameters: ``hidden_size``, ``intermediate_size``, ``activation``."""
 
     graph_safe = True
+    repeatable = True
 
     def __init__(self, spec: PartSpec, prefix: str = ""):
         super().__init__(spec, prefix)

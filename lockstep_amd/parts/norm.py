@@ -12,6 +12,7 @@ class RMSNorm(Norm):
     """Parameters: ``size``, ``eps``; ``name`` overrides the tensor name."""
 
     graph_safe = True
+    repeatable = True
 
     def __init__(self, spec: PartSpec, prefix: str = ""):
         super().__init__(spec, prefix)

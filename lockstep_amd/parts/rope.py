@@ -20,6 +20,7 @@ class RotaryHalf(PositionEncoding):
     """Parameters: ``rotary_dim`` (even, at most the head size), ``theta``."""
 
     graph_safe = True
+    repeatable = True
 
     def __init__(self, spec: PartSpec, prefix: str = ""):
         super().__init__(spec, prefix)
@@ -69,6 +70,7 @@ class NoPosition(PositionEncoding):
     """Leaves queries and keys as they are."""
 
     graph_safe = True
+    repeatable = True
 
     rotary_dim = 0
     cos = None

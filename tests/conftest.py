@@ -50,7 +50,7 @@ LONG_POSITIONS = {"A": 1024, "B": 2048}
 
 
 def make_model_dir(tmp_path_factory, name: str, sharpen: float = 1.0, std: float | None = None,
-                   max_position: int | None = -1) -> Path:
+                   max_position: int | None = -1, overrides: dict | None = None) -> Path:
     """Write tiny configuration ``name`` with random weights.  ``sharpen``
     multiplies the per-head q/k norm weights so that attention is peaked and a
     wrong key or a wrong position changes the logits visibly (the float32 path
@@ -58,7 +58,8 @@ def make_model_dir(tmp_path_factory, name: str, sharpen: float = 1.0, std: float
     is amplified by the same factor squared, so the bfloat16 comparison with
     the plain implementation uses the unsharpened weights and the sharpened
     ones serve its bit-for-bit comparisons).  ``std`` overrides the spread of
-    the matrices (larger values separate the logits, for token comparisons)."""
+    the matrices (larger values separate the logits, for token comparisons).
+    ``overrides`` replaces keys of the configuration (more layers, for instance)."""
     from lockstep_amd.config import Qwen3Config
     from lockstep_amd.weights import random_tensors, save_file
     import json
@@ -68,6 +69,8 @@ def make_model_dir(tmp_path_factory, name: str, sharpen: float = 1.0, std: float
         max_position = LONG_POSITIONS[name]
     if max_position is not None:
         raw = dict(raw, max_position_embeddings=max_position)
+    if overrides:
+        raw = dict(raw, **overrides)
     config = Qwen3Config.from_dict(raw)
     out = tmp_path_factory.mktemp(f"tiny{name}")
     tensors = random_tensors(config, init["seed"], std or init["std"], init["norm_std"], torch.bfloat16)
