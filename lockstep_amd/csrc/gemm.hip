@@ -31,6 +31,15 @@ namespace ls {
 #ifndef LS_GEMM_PD_BIG
 #define LS_GEMM_PD_BIG 1      // register prefetch depth (stages) of the 128 x 128 kernel (2: registers run out, a third slower)
 #endif
+#ifndef LS_GEMM_SLICES_WIDE
+#define LS_GEMM_SLICES_WIDE 1       // 0: never the wide slice kernel
+#endif
+#ifndef LS_GEMM_SLICES_WIDE_WGS
+#define LS_GEMM_SLICES_WIDE_WGS 192  // its workgroups (64 columns, up to four slices) must be at least this many
+#endif
+#ifndef LS_GEMM_SLICES_WIDE_UNR
+#define LS_GEMM_SLICES_WIDE_UNR 2   // chunks it loads at a time
+#endif
 #ifndef LS_GEMM_STREAM
 #define LS_GEMM_STREAM 1      // 0: never the streaming kernel
 #endif
@@ -515,6 +524,77 @@ __global__ __launch_bounds__(256) void gemm_slices_kernel(const T* __restrict__ 
   }
 }
 
+// The slice kernel for many rows and many columns: a wave takes one K slice of NTL column tiles (16 * NTL
+// columns) and all the rows, so a chunk of X that it has loaded meets NTL chunks of weights and a chunk of
+// weights MT chunks of X: at 64 rows and 64 columns the rows of X are read once for every byte of weights,
+// where the kernel above reads them four times over.  The chain of a slice is the same (ascending chunks,
+// from zero), so are the bits.  UNR chunks are loaded at a time, then multiplied; the CU's other waves
+// cover the wait.
+template <typename T, int MT, int NTL, int UNR>
+__global__ __launch_bounds__(256) void gemm_slices_wide_kernel(const T* __restrict__ X, const T* __restrict__ W,
+                                                               float* __restrict__ P, int M, int N, int K, long ldx,
+                                                               int kslice, int aligned, int slices_per_group) {
+  typedef Atom<T> A;
+  typedef typename A::vec_t vec_t;
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int n0 = blockIdx.x * 16 * NTL;
+  const int row16 = lane & 15;
+  const int g = lane >> 4;
+  const int nslices = (K + kslice - 1) / kslice;
+  const int s = blockIdx.y * slices_per_group + wave;
+  if (wave >= slices_per_group || s >= nslices) return;
+
+  f32x4 acc[NTL][MT];
+#pragma unroll
+  for (int i = 0; i < NTL; ++i)
+#pragma unroll
+    for (int j = 0; j < MT; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const int k_begin = s * kslice;
+  const int k_end = min(K, k_begin + kslice);
+  for (int k0 = k_begin; k0 < k_end; k0 += UNR * A::KCHUNK) {
+    vec_t w[UNR][NTL], x[UNR][MT];
+#pragma unroll
+    for (int u = 0; u < UNR; ++u) {
+      const int k = k0 + u * A::KCHUNK + g * A::VEC;
+      const bool in = k0 + u * A::KCHUNK < k_end;
+#pragma unroll
+      for (int i = 0; i < NTL; ++i) {
+        const int n = n0 + i * 16 + row16;
+        w[u][i] = load_vec<T>(W, n, k, K, K, n < N && in, aligned);
+      }
+#pragma unroll
+      for (int j = 0; j < MT; ++j)
+        x[u][j] = load_vec<T>(X, j * 16 + row16, k, K, ldx, j * 16 + row16 < M && in, aligned);
+    }
+#pragma unroll
+    for (int u = 0; u < UNR; ++u) {
+      if (k0 + u * A::KCHUNK >= k_end) break;  // uniform: a chunk is visited iff it starts inside the slice
+#pragma unroll
+      for (int i = 0; i < NTL; ++i)
+#pragma unroll
+        for (int j = 0; j < MT; ++j) A::mma(acc[i][j], w[u][i], x[u][j]);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < NTL; ++i) {
+    const int n = n0 + i * 16 + g * 4;
+#pragma unroll
+    for (int j = 0; j < MT; ++j) {
+      const int m = j * 16 + row16;
+      if (m >= M || n >= N) continue;
+      float* dst = P + ((long)s * M + m) * N + n;
+      if (n + 3 < N && (N & 3) == 0) {
+        *reinterpret_cast<f32x4*>(dst) = acc[i][j];
+      } else {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          if (n + r < N) dst[r] = acc[i][j][r];
+      }
+    }
+  }
+}
+
 // The slice kernel as a walk (products with many K slices and enough column
 // blocks that workgroups can take several): wave = slice, its rows of X stay
 // in registers, the weights of the next units are in flight across column
@@ -844,6 +924,13 @@ int launch_gemm(const void* X, const void* W, void* C, int M, int N, int K, long
   // head) its workgroups re-read all rows of X for 16 columns each, and the tiled kernel reads less.
   const int mt_rows = (M + 15) / 16;
   const int col_blocks = (N + 16 * NT - 1) / (16 * NT);
+  // With more than 16 rows the tiled kernel does better wherever it has a workgroup for every CU (its
+  // workgroups read the rows of X once for 64 columns, through LDS, and 64 columns of weights a workgroup
+  // keep enough loads in flight): from 33 rows on always (Qwen3-8B sizes, gate and up at 64 rows: 85 -> 50
+  // us), from 17 rows on for SwiGLU, where the streaming kernel has two weight tiles a column block and
+  // holds less in flight (58 -> 46 us at 32 rows; the logits head at 24 rows: streaming 257, tiled 307 us).
+  const bool tiled_fills = !norm_w && M <= 64 && (N + 63) / 64 >= compute_units() &&
+                           (M > 32 || (M > 16 && EPI == kSwiGLU));
   const int xc = kslice / Atom<T>::KCHUNK;  // chunks per slice
   // The streaming kernel where a workgroup would get more than one column block: a CU holds 16 waves
   // of it (one per K slice), so 16 / nslices workgroups.
@@ -855,7 +942,7 @@ int launch_gemm(const void* X, const void* W, void* C, int M, int N, int K, long
   // (two groups read the weights twice, the second time rarely from L2 in practice: with very many
   // columns, where the tiled kernel does well, they are not worth it)
   // (with fewer than eight slices the skinny kernel's small workgroups, several a CU, do as well or better)
-  if (!norm_w && mt_rows <= 4 && xc % 4 == 0 && xc * group_tiles <= 16 && nslices >= 8 && nslices <= 16 &&
+  if (!norm_w && mt_rows <= 4 && !tiled_fills && xc % 4 == 0 && xc * group_tiles <= 16 && nslices >= 8 && nslices <= 16 &&
       col_blocks * row_groups > stream_wgs && stream_lds <= 128 * 1024 && !(row_groups > 1 && N >= 32768) &&
       LS_GEMM_STREAM) {
     int walkers = stream_wgs / row_groups;
@@ -878,7 +965,7 @@ int launch_gemm(const void* X, const void* W, void* C, int M, int N, int K, long
 #undef LS_STREAM
     if (launched) return check_launch("gemm");
   }
-  if (M <= 64 && !(M > 16 && N >= 32768)) {
+  if (M <= 64 && !tiled_fills && !(M > 16 && N >= 32768)) {
     const int mt = (M + 15) / 16;
     // 16 waves leave 128 registers a lane: only for one or two row tiles
     const int nw = (nslices > 8 && mt * NT <= 2) ? 16 : (nslices > 4 ? 8 : 4);
@@ -1004,6 +1091,25 @@ extern "C" int ls_gemm_slices(int dtype, const void* X, const void* W, float* P,
   int rounds =
       (int)std::min<long>(4, (long)col_blocks * groups * std::max(row_groups, 1) / (2L * compute_units()));
   if (mt > 4 && rounds < 1) rounds = 1;  // more than 64 rows: this kernel only, if with one column block a workgroup
+  // More than 16 rows and enough columns that workgroups of 64 columns fill the GPU: the wide kernel.
+  {
+    const int wide_blocks = (N + 63) / 64;
+    const int wide_per_group = std::min(4, nslices);
+    const int wide_groups = (nslices + wide_per_group - 1) / wide_per_group;
+    if (mt >= 2 && mt <= 4 && (long)wide_blocks * wide_groups >= LS_GEMM_SLICES_WIDE_WGS && xc % LS_GEMM_SLICES_WIDE_UNR == 0 &&
+        LS_GEMM_SLICES_WIDE) {
+      dim3 wide_grid(wide_blocks, wide_groups);
+#define LS_WIDE(T_, MT_)                                                                                          \
+  hipLaunchKernelGGL((gemm_slices_wide_kernel<T_, MT_, 4, LS_GEMM_SLICES_WIDE_UNR>), wide_grid, dim3(64 * wide_per_group), 0, s, \
+                     (const T_*)X, (const T_*)W, P, M, N, K, ldx, kslice, aligned, wide_per_group)
+#define LS_WIDE_MT(T_)                                       \
+  if (mt == 2) LS_WIDE(T_, 2); else if (mt == 3) LS_WIDE(T_, 3); else LS_WIDE(T_, 4)
+      if (dtype == kF32) { LS_WIDE_MT(float); } else if (dtype == kBF16) { LS_WIDE_MT(bf16_t); } else return fail("gemm_slices: unknown dtype %d", dtype);
+#undef LS_WIDE_MT
+#undef LS_WIDE
+      return check_launch("gemm_slices");
+    }
+  }
   if ((rounds >= 2 || mt > 4) && mt >= 2 && group_tiles > 0 && xc % 4 == 0 && LS_GEMM_STREAM) {
     int walkers = (col_blocks + rounds - 1) / rounds;
     if (row_groups > 1) walkers = (walkers + 7) / 8 * 8;  // the groups' workgroups of a walk sit on the same XCD
