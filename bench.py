@@ -26,6 +26,11 @@ each in prompt portions of 2,048 tokens (``qwen3-0.6b``, ``qwen3-8b``), or 16 re
 tokens with 128 new tokens each (``qwen3-32b``).  ``--workload reference-trace`` runs the shape
 of the reference's committed trace (eight prompts of 64 to 700 tokens, 32 new tokens each,
 bench/throughput.py:35-45).  The value is all tokens (prompt and new) a second.
+
+    python bench.py --workload contexts --model qwen3-8b --steps 32
+
+measures a prompt in portions of 2,048 tokens and decode steps at batch 1, 8 and 64 at the
+context lengths of ``--contexts`` (default 4,096, 8,192 and 16,384 tokens).
 """
 
 from __future__ import annotations
@@ -182,6 +187,70 @@ def measure_prefill(model, cfg, length: int, page_size: int, repeats: int = 5):
     return statistics.median(times)
 
 
+def measure_prefill_portions(model, cfg, length: int, portion: int, page_size: int, repeats: int = 3):
+    """Median seconds of a ``length``-token prompt run in portions of ``portion`` tokens (one request)."""
+    import torch
+
+    from lockstep_amd.engine.batch import StepEntry
+
+    cache = model.make_cache(num_pages=-(-length // page_size) + 1, page_size=page_size, max_requests=1,
+                             max_tokens_per_request=length)
+    prompt = random_prompts(1, length, cfg.vocab_size, seed=length)[0]
+    times = []
+    for i in range(repeats + 1):
+        cache.open("p")
+        torch.cuda.synchronize()
+        started = time.perf_counter()
+        for lo in range(0, length, portion):
+            part = prompt[lo:lo + portion]
+            model.step(cache, [StepEntry("p", part, [len(part) - 1] if lo + portion >= length else [])])
+        torch.cuda.synchronize()
+        if i:
+            times.append(time.perf_counter() - started)
+        cache.close("p")
+    del cache
+    return statistics.median(times)
+
+
+def contexts_record(args, model, cfg, full_layers: int) -> dict:
+    """Prefill and decode at longer contexts: for every context length a prompt of that length in
+    portions of ``--prefill-chunk`` tokens, and ``--steps`` decode steps of batches of 1, 8 and 64
+    requests that hold that many tokens each (batches whose cache would not fit are left out)."""
+    import torch
+
+    element = 2 if args.dtype == "bf16" else 4
+    portion = args.prefill_chunk or 2048
+    rows = {}
+    for context in [int(c) for c in args.contexts.split(",")]:
+        seconds = measure_prefill_portions(model, cfg, context, portion, args.page_size)
+        flops = sum(step_flops(cfg, min(portion, context - lo), lo, 0) for lo in range(0, context, portion))
+        row = {"prefill_tok_s": round(context / seconds, 1), "prefill_ms": round(1e3 * seconds, 2),
+               "prefill_frac": round(flops / seconds / PEAK_FLOPS[args.dtype], 4)}
+        for batch in (1, 8, 64):
+            cache_bytes = (batch * (context + args.steps + 64) * cfg.num_hidden_layers * 2
+                           * cfg.num_key_value_heads * cfg.head_dim * element)
+            free, _ = torch.cuda.mem_get_info()
+            if cache_bytes > free - (12 << 30):
+                continue
+            t, mean_context = measure_decode(model, cfg, batch, context, args.steps, 2, args.page_size,
+                                             not args.host_sampling, 1)
+            step_s = t[0] / args.steps
+            row[f"decode_b{batch}_tok_s"] = round(batch / step_s, 1)
+            row[f"decode_b{batch}_ms"] = round(1e3 * step_s, 3)
+            row[f"decode_b{batch}_hbm_frac"] = round(decode_bytes(cfg, batch, mean_context, element) / step_s
+                                                     / PEAK_HBM, 4)
+            torch.cuda.empty_cache()
+        rows[str(context)] = row
+    return {
+        "metric": f"prefill and decode tok/s by context length ({args.model} layer sizes)",
+        "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "dtype": args.dtype,
+        "data": "synthetic: uniform random token ids, random weights N(0, 0.02)",
+        "config": {"model": args.model, "layers": cfg.num_hidden_layers, "layers_of_model": full_layers,
+                   "prefill_portion": portion, "page_size": args.page_size, "kernels": kernel_digest(model)},
+        "contexts": rows,
+    }
+
+
 def kernel_digest(model) -> str:
     """Names of the loaded kernel libraries; each carries a hash of its sources and flags, which
     fixes every tile and split constant (reference engine/kernels/registry.py:163-166)."""
@@ -309,8 +378,10 @@ def main(argv=None) -> int:
     p.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points and the prefill")
     p.add_argument("--host-sampling", action="store_true",
                    help="pick every step's tokens on the host (Model.step + Sampler) instead of the device-side loop")
-    p.add_argument("--workload", default="decode", choices=["decode", "serve", "reference-trace"],
-                   help="decode: fixed batches (the headline); serve / reference-trace: a workload through the scheduler")
+    p.add_argument("--workload", default="decode", choices=["decode", "serve", "reference-trace", "contexts"],
+                   help="decode: fixed batches (the headline); serve / reference-trace: a workload through the "
+                        "scheduler; contexts: prefill and decode at the context lengths of --contexts")
+    p.add_argument("--contexts", default="4096,8192,16384", help="contexts: the context lengths, comma separated")
     p.add_argument("--repeats", type=int, default=5, help="timed runs; the median is reported with the spread")
     p.add_argument("--requests", type=int, default=0, help="serve: only the first N requests of the workload")
     p.add_argument("--prefill-chunk", type=int, default=None, help="serve: prompt portion (0: whole prompts)")
@@ -328,6 +399,9 @@ def main(argv=None) -> int:
     model, cfg, full_layers = build_model(args)
     element = 2 if args.dtype == "bf16" else 4
 
+    if args.workload == "contexts":
+        print(json.dumps(contexts_record(args, model, cfg, full_layers)))
+        return 0
     if args.workload != "decode":
         print(json.dumps(serve_record(args, model, cfg, full_layers)))
         return 0

@@ -1643,6 +1643,93 @@ __global__ __launch_bounds__(256) void combine_kernel(const SeqMeta* __restrict_
   store_output<T>(run, out + (long)(item.q_off + qi) * ldo + (long)head * D, g);
 }
 
+// The fold for requests of at most 16 rows a kv head (decoded tokens), where a request far away has dozens
+// of splits: the fold of one split has to wait for the one before, so what takes time is the loads.  Here
+// the four waves share the columns (wave w has the column blocks w, w + 4, ..., as in the cooperative
+// kernel), so a lane holds a quarter of a row's sums and can ask for sixteen splits at a time.  Every
+// element goes through the operations of fold_split in the same order: the same bits.
+template <typename T>
+__global__ __launch_bounds__(256) void combine_few_rows_kernel(const SeqMeta* __restrict__ seqs,
+                                                               const CombineItem* __restrict__ items,
+                                                               const float* __restrict__ part_acc,
+                                                               const float* __restrict__ part_ml,
+                                                               T* __restrict__ out, long ldo, int G) {
+  constexpr int MYDB = (DB + 3) / 4;
+  constexpr int BATCH = MYDB <= 2 ? 16 : 8;
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const CombineItem item = items[blockIdx.x];
+  const int kvh = blockIdx.y;
+  const int rows_total = item.q_len * G;  // <= 16, checked on the host
+  const int r = lane & 15;
+  if (r >= rows_total) return;
+  const int g = lane >> 4;
+  const int qi = r / G;
+  const int head = kvh * G + r % G;
+
+  f32x4 run_acc[MYDB];
+  float run_m = kNegSentinel, run_l = 0.f;
+#pragma unroll
+  for (int j = 0; j < MYDB; ++j) run_acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const long pr0 = item.part_base + ((long)kvh * rows_total + r) * item.n_splits;
+  auto fold = [&](const f32x4 (&acc)[MYDB], float m, float l) {  // fold_split on this wave's blocks
+    if (!(l > 0.f)) return;
+    const float m_new = fmaxf(run_m, m);
+    const float a = softmax_exp<T>(run_m - m_new);
+    const float b = softmax_exp<T>(m - m_new);
+#pragma unroll
+    for (int j = 0; j < MYDB; ++j)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) run_acc[j][e] = run_acc[j][e] * a + acc[j][e] * b;
+    run_l = run_l * a + l * b;
+    run_m = m_new;
+  };
+  auto load = [&](f32x4 (&acc)[MYDB], float& m, float& l, long pr) {
+#pragma unroll
+    for (int j = 0; j < MYDB; ++j) {
+      const int blk = min(wave + 4 * j, DB - 1);
+      acc[j] = *reinterpret_cast<const f32x4*>(part_acc + pr * D + blk * 16 + 4 * g);
+    }
+    m = part_ml[pr * 2];
+    l = part_ml[pr * 2 + 1];
+  };
+  if (LS_MUTANT_DEVICE(kMutantReversedFold)) {
+    for (int s = item.n_splits - 1; s >= 0; --s) {
+      f32x4 acc[MYDB];
+      float m, l;
+      load(acc, m, l, pr0 + s);
+      fold(acc, m, l);
+    }
+  } else {
+    for (int s0 = 0; s0 < item.n_splits; s0 += BATCH) {
+      f32x4 acc[BATCH][MYDB];
+      float m[BATCH], l[BATCH];
+#pragma unroll
+      for (int u = 0; u < BATCH; ++u) load(acc[u], m[u], l[u], pr0 + min(s0 + u, item.n_splits - 1));  // clamped: loaded, not used
+#pragma unroll
+      for (int u = 0; u < BATCH; ++u)
+        if (s0 + u < item.n_splits) fold(acc[u], m[u], l[u]);
+    }
+  }
+  T* dst = out + (long)(item.q_off + qi) * ldo + (long)head * D;
+#pragma unroll
+  for (int j = 0; j < MYDB; ++j) {
+    const int blk = wave + 4 * j;
+    if (blk >= DB) continue;
+    float o[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) o[e] = run_l > 0.f ? run_acc[j][e] / run_l : 0.f;
+    T* p = dst + blk * 16 + 4 * g;
+    if (sizeof(T) == 2) {
+      bf16x4 v;
+      v[0] = (bf16_t)o[0]; v[1] = (bf16_t)o[1]; v[2] = (bf16_t)o[2]; v[3] = (bf16_t)o[3];
+      *reinterpret_cast<bf16x4*>(p) = v;
+    } else {
+      *reinterpret_cast<f32x4*>(p) = f32x4{o[0], o[1], o[2], o[3]};
+    }
+  }
+}
+
 }  // namespace ls
 
 LS_DEFINE_ERROR_API
@@ -1939,18 +2026,24 @@ extern "C" int ls_attention(int dtype, const void* q, long ldq, const void* k_pa
 
 extern "C" int ls_attention_combine(int dtype, const void* seqs, const void* items, int n_items, int nkv,
                                     const float* part_acc, const float* part_ml, void* out, long ldo, int G,
-                                    void* stream) {
-  LS_REQUIRE(n_items > 0 && nkv > 0 && G > 0, "combine: bad sizes");
+                                    int max_rows, void* stream) {
+  // max_rows: the most rows (tokens times query heads a kv head) any item's request brings, or 0 if unknown;
+  // up to 16 rows the kernel that shares a row's columns among the waves is taken.
+  LS_REQUIRE(n_items > 0 && nkv > 0 && G > 0 && max_rows >= 0, "combine: bad sizes");
   LS_REQUIRE(ldo % 4 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0, "combine: output not vector aligned");
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   dim3 grid(n_items, nkv);
-  if (dtype == kF32)
-    hipLaunchKernelGGL(combine_kernel<float>, grid, dim3(256), 0, s, (const SeqMeta*)seqs, (const CombineItem*)items,
-                       part_acc, part_ml, (float*)out, ldo, G);
-  else if (dtype == kBF16)
-    hipLaunchKernelGGL(combine_kernel<bf16_t>, grid, dim3(256), 0, s, (const SeqMeta*)seqs,
-                       (const CombineItem*)items, part_acc, part_ml, (bf16_t*)out, ldo, G);
-  else
+  const bool few = max_rows > 0 && max_rows <= 16;
+#define LS_COMBINE(KERNEL_, T_)                                                                              \
+  hipLaunchKernelGGL(KERNEL_<T_>, grid, dim3(256), 0, s, (const SeqMeta*)seqs, (const CombineItem*)items, \
+                     part_acc, part_ml, (T_*)out, ldo, G)
+  if (dtype == kF32) {
+    if (few) LS_COMBINE(combine_few_rows_kernel, float); else LS_COMBINE(combine_kernel, float);
+  } else if (dtype == kBF16) {
+    if (few) LS_COMBINE(combine_few_rows_kernel, bf16_t); else LS_COMBINE(combine_kernel, bf16_t);
+  } else {
     return fail("combine: unknown dtype %d", dtype);
+  }
+#undef LS_COMBINE
   return check_launch("combine");
 }

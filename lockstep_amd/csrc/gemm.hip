@@ -539,11 +539,10 @@ __global__ __launch_bounds__(256) void gemm_slices_wide_kernel(const T* __restri
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int n0 = blockIdx.x * 16 * NTL;
+  const int s = blockIdx.y * slices_per_group + wave;
+  if (wave >= slices_per_group || s >= (K + kslice - 1) / kslice) return;
   const int row16 = lane & 15;
   const int g = lane >> 4;
-  const int nslices = (K + kslice - 1) / kslice;
-  const int s = blockIdx.y * slices_per_group + wave;
-  if (wave >= slices_per_group || s >= nslices) return;
 
   f32x4 acc[NTL][MT];
 #pragma unroll
@@ -1100,8 +1099,9 @@ extern "C" int ls_gemm_slices(int dtype, const void* X, const void* W, float* P,
         LS_GEMM_SLICES_WIDE) {
       dim3 wide_grid(wide_blocks, wide_groups);
 #define LS_WIDE(T_, MT_)                                                                                          \
-  hipLaunchKernelGGL((gemm_slices_wide_kernel<T_, MT_, 4, LS_GEMM_SLICES_WIDE_UNR>), wide_grid, dim3(64 * wide_per_group), 0, s, \
-                     (const T_*)X, (const T_*)W, P, M, N, K, ldx, kslice, aligned, wide_per_group)
+  hipLaunchKernelGGL((gemm_slices_wide_kernel<T_, MT_, 4, LS_GEMM_SLICES_WIDE_UNR>), wide_grid,                 \
+                     dim3(64 * wide_per_group), 0, s, (const T_*)X, (const T_*)W, P, M, N, K, ldx, kslice, aligned, \
+                     wide_per_group)
 #define LS_WIDE_MT(T_)                                       \
   if (mt == 2) LS_WIDE(T_, 2); else if (mt == 3) LS_WIDE(T_, 3); else LS_WIDE(T_, 4)
       if (dtype == kF32) { LS_WIDE_MT(float); } else if (dtype == kBF16) { LS_WIDE_MT(bf16_t); } else return fail("gemm_slices: unknown dtype %d", dtype);

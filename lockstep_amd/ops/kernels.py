@@ -485,7 +485,10 @@ class Kernels:
             c_int(positions), c_int(max_pos), c_int(1 if write_kv else 0), c_int(1 if spans else 0), _stream()))
 
     def attention_combine(self, d: int, seqs, items, n_items: int, nq: int, nkv: int, part_acc, part_ml,
-                          out: torch.Tensor) -> None:
+                          out: torch.Tensor, max_rows: int = 0) -> None:
+        """Fold the splits' partial results of the requests in ``items`` into ``out``.  ``max_rows``: the
+        most rows (tokens times query heads a kv head) a request of an item brings, 0 if unknown; with
+        at most 16 the fold that asks for many splits at a time is taken (same bits)."""
         lib = self.attention_lib(d)
         _rows_ok(out, "combine out")
         if not (out.dtype in DTYPE_CODE and out.shape[1] >= nq * d):
@@ -496,7 +499,7 @@ class Kernels:
             return
         self._launch(lib, lib.ls_attention_combine, (
             c_int(DTYPE_CODE[out.dtype]), _ptr(seqs), _ptr(items), c_int(n_items), c_int(nkv), _ptr(part_acc),
-            _ptr(part_ml), _ptr(out), c_long(out.stride(0)), c_int(nq // nkv), _stream()))
+            _ptr(part_ml), _ptr(out), c_long(out.stride(0)), c_int(nq // nkv), c_int(max_rows), _stream()))
 
 
 ATTENTION_ITEM_INTS = 16

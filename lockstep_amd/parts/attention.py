@@ -33,6 +33,7 @@ FUSE_DECODE = os.environ.get("LOCKSTEP_FUSE_DECODE", "1") not in ("", "0")
 FUSE_DECODE_BELOW = int(os.environ.get("LOCKSTEP_FUSE_DECODE_BELOW", "512"))
 # The most splits (of 256 keys) one cooperative workgroup walks when a request is cut over several.
 MAX_SPAN = 4               # splits of a work item where requests of a ragged batch are cut
+WORKGROUPS_A_CU = 2         # work items (times kv heads) a CU that a decode step is cut for
 RAGGED_RATIO = 2.0         # a batch is ragged when its longest request has more than this many times the mean splits
 PART_ROWS_STEP = 4096      # rows of partial results are taken in steps of this many (sizes of replayed steps)
 
@@ -90,9 +91,12 @@ def plan_attention(ctx, group_size: int, nkv: int, head_dim: int, window: int):
 
     Decoded tokens (at most 16 rows a kv head) go to the cooperative kernel.  While the step's
     splits would not fill the GPU twice over, every split is a work item of its own.  Beyond
-    that a workgroup walks a whole request and writes the output -- unless the requests are of
-    very different lengths: a workgroup takes a few microseconds a tile whatever else runs, so
-    the longest request would decide when the launch ends; requests are then cut into items of
+    that a workgroup walks a whole request and writes the output -- unless there are too few
+    requests for that to give every CU two workgroups (a CU alone streams slowly: eight
+    requests of 4,096 tokens walked whole keep a quarter of the GPU busy), then requests are cut
+    into the longest items that still do; and unless the requests are of very different
+    lengths: a workgroup takes a few microseconds a tile whatever else runs, so the longest
+    request would decide when the launch ends; requests are then cut into items of at most
     MAX_SPAN splits.  With ``ctx.fixed_shape`` (a step whose launches are captured and replayed)
     the lists are laid out for the lengths the requests will have ``ctx.horizon`` tokens on,
     and their sizes are rounded up with null items, so that one graph serves the steps to come."""
@@ -116,9 +120,20 @@ def plan_attention(ctx, group_size: int, nkv: int, head_dim: int, window: int):
     span = 1
     if to_coop.any():
         mine = counts[to_coop]
-        if int(mine.sum()) * nkv >= 2 * kernels.compute_units():
-            ragged = int(mine.max()) > RAGGED_RATIO * float(mine.mean())
-            span = MAX_SPAN if ragged else int(mine.max())      # the latter: every request is walked whole
+        enough = WORKGROUPS_A_CU * kernels.compute_units()
+        if int(mine.sum()) * nkv >= enough:
+            span = int(mine.max())                              # every request is walked whole ...
+            if len(mine) * nkv < kernels.compute_units():       # ... unless that leaves CUs without work: the
+                low, high = 1, span                             # longest items that still give every CU two
+                while low < high:
+                    middle = (low + high + 1) // 2
+                    if int((-(-mine // middle)).sum()) * nkv >= enough:
+                        low = middle
+                    else:
+                        high = middle - 1
+                span = low
+            if int(mine.max()) > RAGGED_RATIO * float(mine.mean()):
+                span = min(span, MAX_SPAN)
 
     items, coop, wide, combine = [], [], [], []
     coop_max_rows = part_rows = 0
@@ -133,8 +148,10 @@ def plan_attention(ctx, group_size: int, nkv: int, head_dim: int, window: int):
             else:
                 base = part_rows
                 part_rows += nkv * rows * n_splits
-                for first in range(split_lo, split_lo + n_splits, span):
-                    coop.append((i, 0, first, min(first + span, split_lo + n_splits), base, n_splits, split_lo, 0))
+                pieces = -(-n_splits // span)
+                even = -(-n_splits // pieces)               # items of even length: the longest decides
+                for first in range(split_lo, split_lo + n_splits, even):
+                    coop.append((i, 0, first, min(first + even, split_lo + n_splits), base, n_splits, split_lo, 0))
                 combine.append((i, 0, base, n_splits))
         elif rows <= 64 and (n_splits > 1 or ctx.fixed_shape):
             base = part_rows
@@ -307,7 +324,8 @@ class Attention(Mixer):
                                self.q_norm, self.k_norm, self.norm_eps, self.position.cos, self.position.sin,
                                self.position.rotary_dim, ctx.max_position, run.writes_cache, plan.spans)
             if plan.n_combine:
-                k.attention_combine(d, ctx.seqs, combine_items, plan.n_combine, nq, nkv, part_acc, part_ml, attn)
+                k.attention_combine(d, ctx.seqs, combine_items, plan.n_combine, nq, nkv, part_acc, part_ml, attn,
+                                    max_rows=plan.coop_max_rows if not plan.n_items else 0)
             return self._project_out(ctx, attn, out, accumulate, defer)
         k.qk_rope_kv(qkv, t, nq, nkv, d, self.q_norm, self.k_norm, self.norm_eps, self.position.cos,
                      self.position.sin, self.position.rotary_dim, ctx.tok_seq, ctx.tok_pos, ctx.seqs,
@@ -324,7 +342,8 @@ class Attention(Mixer):
                         wide_items, plan.n_wide, attn, part_acc, part_ml, self.scale, window,
                         variant=plan.wide_variant)
         if plan.n_combine:
-            k.attention_combine(d, ctx.seqs, combine_items, plan.n_combine, nq, nkv, part_acc, part_ml, attn)
+            k.attention_combine(d, ctx.seqs, combine_items, plan.n_combine, nq, nkv, part_acc, part_ml, attn,
+                                    max_rows=plan.coop_max_rows if not plan.n_items else 0)
         return self._project_out(ctx, attn, out, accumulate, defer)
 
     def _project_out(self, ctx, attn, out, accumulate: bool, defer: bool):

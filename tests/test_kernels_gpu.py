@@ -288,8 +288,10 @@ class PagedCase:
         K().qk_rope_kv(qkv, t, self.nq, self.nkv, self.d, q_norm, k_norm, eps, cos, sin, rot, tok_seq, tok_pos,
                        self.seqs(q_start, t), q_start + t - 1, self.table, self.k_pages, self.v_pages, self.ps, True)
 
-    def attend(self, qkv, q_start, scale, window=0, force_split=None, variant=0, repeat=1, span=1, pad_splits=0):
-        """``span``: splits one work item walks when the request is cut (the cooperative kernel takes more
+    def attend(self, qkv, q_start, scale, window=0, force_split=None, variant=0, repeat=1, span=1, pad_splits=0,
+               few_rows=False):
+        """``few_rows``: tell the fold that no request has more than 16 rows (it then takes the kernel that
+        asks for many splits at a time).  ``span``: splits one work item walks when the request is cut (the cooperative kernel takes more
         than one and leaves a partial result for each); ``pad_splits``: lay the items out for that many
         more splits than the request has (as the fixed-shape lists of graph-replayed steps do)."""
         from lockstep_amd.ops import kernels
@@ -334,7 +336,7 @@ class PagedCase:
         if combine:
             comb = torch.from_numpy(pack_combine_items(combine, seq_row)).to(torch.int32).cuda()
             K().attention_combine(self.d, self.seqs(q_start, t), comb, len(combine) // 4, self.nq, self.nkv,
-                                  part_acc, part_ml, out)
+                                  part_acc, part_ml, out, max_rows=rows if few_rows else 0)
         return out.view(t, self.nq, self.d)
 
 
@@ -573,9 +575,32 @@ def test_cooperative_items_of_several_splits_leave_the_same_partial_results(dtyp
         for start in (1399, 1279, 1024, 511):
             ref = case.attend(dev[start:start + 1], start, d ** -0.5, window=window, variant=3, force_split=False)
             for span, pad in ((1, 0), (2, 0), (3, 1), (4, 0), (4, 3), (8, 0)):
-                got = case.attend(dev[start:start + 1], start, d ** -0.5, window=window, variant=3, force_split=True,
-                                  span=span, pad_splits=pad)
-                assert torch.equal(got, ref), f"start={start} window={window} span={span} pad={pad}"
+                for few in (False, True):
+                    got = case.attend(dev[start:start + 1], start, d ** -0.5, window=window, variant=3,
+                                      force_split=True, span=span, pad_splits=pad, few_rows=few)
+                    assert torch.equal(got, ref), f"start={start} window={window} span={span} pad={pad} few={few}"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nq,nkv,d,ps", [(16, 8, 128, 16), (4, 4, 16, 8), (6, 2, 48, 16), (2, 1, 256, 16)])
+def test_the_fold_for_few_rows_has_the_bits_of_the_general_fold_over_many_splits(dtype, nq, nkv, d, ps):
+    """Forty-one splits (more than two of the fold's rounds of sixteen), one and three tokens."""
+    if not K().coop_supported(d, dtype, ps):
+        pytest.skip("the cooperative kernel's tiles do not fit")
+    kv_len = 256 * 40 + 77
+    qkv = rand_qkv(kv_len, nq, nkv, d, dtype, seed=5 * d + nq, sharp=(300,))
+    case = PagedCase(dtype, nq, nkv, d, ps, kv_len, shuffle_seed=6)
+    dev = qkv.cuda()
+    case.write(dev, 0)
+    for tokens in (1, 3):
+        if tokens * (nq // nkv) > 16:
+            continue
+        start = kv_len - tokens
+        ref = case.attend(dev[start:], start, d ** -0.5, variant=3, force_split=False)
+        for span in (1, 5):
+            general = case.attend(dev[start:], start, d ** -0.5, variant=3, force_split=True, span=span)
+            few = case.attend(dev[start:], start, d ** -0.5, variant=3, force_split=True, span=span, few_rows=True)
+            assert torch.equal(general, ref) and torch.equal(few, ref), f"tokens={tokens} span={span}"
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

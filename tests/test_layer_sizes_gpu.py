@@ -161,6 +161,64 @@ def test_requests_of_very_different_lengths_decode_with_the_bits_of_one(models):
         assert torch.equal(torch.stack([t[i] for t in together]), want), f"request {i} (context {lengths[i]})"
 
 
+def test_few_long_requests_are_cut_so_that_every_cu_has_work(tmp_path):
+    """Three requests of some 12,300 tokens in one decode step: walked whole they would be 24 workgroups;
+    the planner cuts them into the longest items that still give every CU two (here two splits an
+    item), the decode loop lays the same out for the lengths to come, and each request has the bits
+    it has alone."""
+    import lockstep_amd.parts.attention as attention_module
+    from lockstep_amd.config import Qwen3Config
+    from lockstep_amd.engine.batch import StepEntry
+    from lockstep_amd.weights import write_random_model
+
+    config = Qwen3Config.from_dict(dict(SIZES["0.6b-like"], num_hidden_layers=1, max_position_embeddings=16384))
+    write_random_model(config, tmp_path, seed=12, std=0.02, norm_std=0.1)
+    model = load(tmp_path, "bfloat16")
+    vocab = config.vocab_size
+    lengths, n_decode = [12300, 12290, 12310], 3
+    prompts = [random_tokens(m + n_decode + 8, vocab, seed=170 + i) for i, m in enumerate(lengths)]
+    cache = model.make_cache(num_pages=4 * 780, page_size=16, max_requests=4)
+
+    def prefill(rid, tokens):
+        cache.open(rid)
+        for lo in range(0, len(tokens), 4096):
+            part = tokens[lo:lo + 4096]
+            logits = model.step(cache, [StepEntry(rid, part, [len(part) - 1])])
+        return logits[0]
+
+    for i, m in enumerate(lengths):
+        prefill(f"r{i}", prompts[i][:m])
+    seen = []
+    original = attention_module.plan_attention
+
+    def watching(ctx, *args):
+        plan, ints = original(ctx, *args)
+        seen.append(plan)
+        return plan, ints
+
+    attention_module.plan_attention = watching
+    try:
+        together = [model.step(cache, [StepEntry(f"r{i}", [prompts[i][lengths[i] + k]], [0]) for i in range(3)]).cpu()
+                    for k in range(n_decode)]
+    finally:
+        attention_module.plan_attention = original
+    assert seen and all(p.spans and p.n_combine >= 3 and 8 * p.n_coop >= 512 for p in seen), seen
+    prefill("alone", prompts[1][:lengths[1]])
+    for k in range(n_decode):
+        want = model.step(cache, [StepEntry("alone", [prompts[1][lengths[1] + k]], [0])]).cpu()
+        assert torch.equal(together[k][1], want[0]), k
+    # and through the device-side loop: the greedy continuation of one of three equals its own alone
+    for rid in ("r0", "r1", "r2", "alone"):
+        cache.close(rid)
+    firsts = [int(prefill(f"q{i}", prompts[i][:m]).argmax()) for i, m in enumerate(lengths)]
+    picked = model.decode_greedy(cache, ["q0", "q1", "q2"], firsts, 6)
+    token = int(prefill("alone", prompts[1][:lengths[1]]).argmax())
+    assert token == firsts[1]
+    for k in range(6):
+        token = int(model.step(cache, [StepEntry("alone", [token], [0])])[0].argmax())
+        assert token == int(picked[k][1]), k
+
+
 def test_the_32_bit_path_matches_plain_at_real_layer_sizes(models):
     """float32 against the plain float64 implementation, and bfloat16 within its tolerance, on the
     two-layer configuration (whole prompt and decoded tail)."""
