@@ -66,31 +66,58 @@ def build_model(args):
     return model, config, full_layers
 
 
-def matrix_params_per_layer(cfg) -> int:
-    qkv = (cfg.num_attention_heads + 2 * cfg.num_key_value_heads) * cfg.head_dim * cfg.hidden_size
-    out = cfg.hidden_size * cfg.num_attention_heads * cfg.head_dim
-    mlp = 3 * cfg.intermediate_size * cfg.hidden_size
-    return qkv + out + mlp
+class Workload:
+    """What a step costs, read from the model's own description (its parts' tensors and cache
+    units) rather than from one architecture's formulas: per run of a layer the elements of its
+    matrices and vectors, and for an attention mixer its heads; the head's matrix."""
+
+    def __init__(self, model):
+        from lockstep_amd.parts import part_class
+
+        spec = model.spec
+        per_layer = []
+        for layer in spec.layers:
+            tensors = part_class(layer.arrangement.kind).weight_specs(layer)
+            matrices = sum(_numel(w.shape) for w in tensors if w.kind == "matrix")
+            vectors = sum(_numel(w.shape) for w in tensors if w.kind != "matrix")
+            mixer = layer.mixer.params if layer.mixer.kind == "attention" else None
+            per_layer.append((matrices, vectors, mixer))
+        self.runs = [per_layer[run.layer] for run in spec.schedule]
+        self.writers = [per_layer[run.layer][2] for run in spec.schedule if run.writes_cache]
+        self.head = spec.vocab_size * spec.hidden_size
+        self.hidden = spec.hidden_size
+
+    def step_flops(self, tokens: int, start: int, wanted: int) -> float:
+        """Multiply-adds times two of a step of ``tokens`` new tokens at positions ``start``.. of
+        one request with ``wanted`` logit rows."""
+        total = 2.0 * wanted * self.head
+        for matrices, _, mixer in self.runs:
+            total += 2.0 * tokens * matrices
+            if mixer is not None:
+                window = mixer.get("window")
+                pairs = sum(min(start + i + 1, window or start + i + 1) for i in range(tokens))   # visible (query, key) pairs
+                total += 4.0 * mixer["head_dim"] * mixer["num_heads"] * pairs
+        return total
+
+    def decode_bytes(self, batch: int, context: float, element: int) -> float:
+        """Bytes a decode step has to read: every weight it uses once, and the cache of the
+        live requests."""
+        weights = sum(matrices * element + vectors * 4 for matrices, vectors, _ in self.runs)
+        weights += self.head * element + self.hidden * 4                     # head and final norm
+        weights += batch * self.hidden * element                             # embedding rows
+        kv = 0.0
+        for mixer in self.writers:
+            if mixer is not None:
+                held = min(context, mixer.get("window") or context)
+                kv += batch * held * 2 * mixer["num_kv_heads"] * mixer["head_dim"] * element
+        return weights + kv
 
 
-def step_flops(cfg, tokens: int, start: int, wanted: int) -> float:
-    """Multiply-adds times two of a step of ``tokens`` new tokens at positions
-    ``start``.. of one request with ``wanted`` logit rows."""
-    dense = 2.0 * tokens * matrix_params_per_layer(cfg)
-    pairs = sum(start + i + 1 for i in range(tokens))               # visible (query, key) pairs
-    attention = 4.0 * cfg.head_dim * cfg.num_attention_heads * pairs
-    return cfg.num_hidden_layers * (dense + attention) + 2.0 * wanted * cfg.vocab_size * cfg.hidden_size
-
-
-def decode_bytes(cfg, batch: int, context: float, element: int) -> float:
-    """Bytes a decode step has to read: every weight it uses once, and the
-    cache of the live requests."""
-    weights = cfg.num_hidden_layers * (matrix_params_per_layer(cfg) * element + 2 * cfg.hidden_size * 4
-                                       + 2 * cfg.head_dim * 4)
-    weights += cfg.vocab_size * cfg.hidden_size * element + cfg.hidden_size * 4     # head and final norm
-    weights += batch * cfg.hidden_size * element                                     # embedding rows
-    kv = batch * context * cfg.num_hidden_layers * 2 * cfg.num_key_value_heads * cfg.head_dim * element
-    return weights + kv
+def _numel(shape) -> int:
+    n = 1
+    for size in shape:
+        n *= int(size)
+    return n
 
 
 def random_prompts(n: int, length: int, vocab: int, seed: int):
@@ -223,7 +250,7 @@ def contexts_record(args, model, cfg, full_layers: int) -> dict:
     rows = {}
     for context in [int(c) for c in args.contexts.split(",")]:
         seconds = measure_prefill_portions(model, cfg, context, portion, args.page_size)
-        flops = sum(step_flops(cfg, min(portion, context - lo), lo, 0) for lo in range(0, context, portion))
+        flops = sum(Workload(model).step_flops(min(portion, context - lo), lo, 0) for lo in range(0, context, portion))
         row = {"prefill_tok_s": round(context / seconds, 1), "prefill_ms": round(1e3 * seconds, 2),
                "prefill_frac": round(flops / seconds / PEAK_FLOPS[args.dtype], 4)}
         for batch in (1, 8, 64):
@@ -237,7 +264,7 @@ def contexts_record(args, model, cfg, full_layers: int) -> dict:
             step_s = t[0] / args.steps
             row[f"decode_b{batch}_tok_s"] = round(batch / step_s, 1)
             row[f"decode_b{batch}_ms"] = round(1e3 * step_s, 3)
-            row[f"decode_b{batch}_hbm_frac"] = round(decode_bytes(cfg, batch, mean_context, element) / step_s
+            row[f"decode_b{batch}_hbm_frac"] = round(Workload(model).decode_bytes(batch, mean_context, element) / step_s
                                                      / PEAK_HBM, 4)
             torch.cuda.empty_cache()
         rows[str(context)] = row
@@ -417,7 +444,7 @@ def main(argv=None) -> int:
     elapsed = statistics.median(times)
     ms_per_step = 1e3 * elapsed / args.steps
     value = args.batch * args.steps / elapsed
-    bytes_step = decode_bytes(cfg, args.batch, context, element)
+    bytes_step = Workload(model).decode_bytes(args.batch, context, element)
     achieved = bytes_step / (elapsed / args.steps)
 
     record = {
@@ -452,7 +479,7 @@ def main(argv=None) -> int:
 
     if not args.no_points:
         seconds = measure_prefill(model, cfg, args.prefill_len, args.page_size)
-        flops = step_flops(cfg, args.prefill_len, 0, 1)
+        flops = Workload(model).step_flops(args.prefill_len, 0, 1)
         record["prefill"] = {"value": round(args.prefill_len / seconds, 1), "tokens": args.prefill_len,
                              "ms": round(1e3 * seconds, 3),
                              "frac": round(flops / seconds / PEAK_FLOPS[args.dtype], 4)}

@@ -207,6 +207,45 @@ __global__ __launch_bounds__(256) void swiglu_kernel(const T* __restrict__ gu, T
 }
 
 // ---------------------------------------------------------------------------
+// Bias and activation on float rows (the output of a product stored in float):
+//   out[m][n] = act(x[m][n] + bias[n])                              plain
+//   out[m][n] = act(x[m][n] + bias[n]) * (x[m][N + n] + bias[N + n])  gated (x has 2N columns)
+// for parts with biases or with another activation than the product's own SwiGLU epilogue: a
+// pass of its own over the rows, slower than an epilogue, but it keeps every such part out of the
+// product kernels.  `out` may be `x` itself (plain, float output).  All arithmetic in float.
+// ---------------------------------------------------------------------------
+enum Activation { kActNone = 0, kActSilu = 1, kActGeluTanh = 2, kActGelu = 3, kActRelu = 4 };
+
+__device__ __forceinline__ float activate(float v, int act) {
+  switch (act) {
+    case kActSilu: return v * (1.0f / (1.0f + expf(-v)));
+    case kActGeluTanh: return 0.5f * v * (1.0f + tanhf(0.7978845608028654f * (v + 0.044715f * v * v * v)));
+    case kActGelu: return 0.5f * v * (1.0f + erff(v * 0.7071067811865476f));
+    case kActRelu: return fmaxf(v, 0.0f);
+    default: return v;
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void bias_act_kernel(const float* __restrict__ x, long ldx,
+                                                       const float* __restrict__ bias, T* __restrict__ out, long ldo,
+                                                       int rows, int width, int act, int gated) {
+  const long idx = (long)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (long)rows * width) return;
+  const long r = idx / width;
+  const int c = (int)(idx % width);
+  float v = x[r * ldx + c];
+  if (bias) v = v + bias[c];
+  v = activate(v, act);
+  if (gated) {
+    float u = x[r * ldx + width + c];
+    if (bias) u = u + bias[width + c];
+    v = v * u;
+  }
+  out[r * ldo + c] = from_f32<T>(v);
+}
+
+// ---------------------------------------------------------------------------
 // Residual add of a product left as slice sums, then RMSNorm of the new row:
 //   h[row] += (P[0][row] + P[1][row] + ...)   (slices ascending, from +0)
 //   out[r] = rmsnorm(h[row]) * weight         (skipped when out == nullptr)
@@ -575,6 +614,29 @@ extern "C" int ls_swiglu(int dtype, const void* gu, void* out, int rows, int int
   else
     return fail("swiglu: unknown dtype %d", dtype);
   return check_launch("swiglu");
+}
+
+// out_dtype: 0 float32, 1 bfloat16.  act: 0 none, 1 SiLU, 2 GELU (tanh form), 3 GELU (erf form), 4 ReLU.
+// x float [rows][ldx] with `width` columns (2 * width when gated), bias float [width] ([2 * width] when
+// gated) or null, out [rows][ldo] of out_dtype; out may be x (not gated, float32).
+extern "C" int ls_bias_act(int out_dtype, const float* x, long ldx, const float* bias, void* out, long ldo, int rows,
+                           int width, int act, int gated, void* stream) {
+  using namespace ls;
+  LS_REQUIRE(rows > 0 && width > 0 && ldo >= width && ldx >= (gated ? 2 * width : width), "bias_act: bad sizes");
+  LS_REQUIRE(act >= 0 && act <= 4, "bias_act: unknown activation %d", act);
+  LS_REQUIRE(!(gated && (const void*)x == out), "bias_act: a gated pass cannot work in place");
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  const long total = (long)rows * width;
+  dim3 grid((unsigned)((total + 255) / 256));
+  if (out_dtype == kF32)
+    hipLaunchKernelGGL(bias_act_kernel<float>, grid, dim3(256), 0, s, x, ldx, bias, (float*)out, ldo, rows, width, act,
+                       gated);
+  else if (out_dtype == kBF16)
+    hipLaunchKernelGGL(bias_act_kernel<bf16_t>, grid, dim3(256), 0, s, x, ldx, bias, (bf16_t*)out, ldo, rows, width,
+                       act, gated);
+  else
+    return fail("bias_act: unknown dtype %d", out_dtype);
+  return check_launch("bias_act");
 }
 
 // Chunks a row of this width is cut into; scratch must hold 2 * rows * chunks 4-byte words when chunks > 1.

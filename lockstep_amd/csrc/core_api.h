@@ -26,6 +26,11 @@ int ls_qk_rope_kv(int dtype, void* qkv, long ld, int n_tokens, int nq, int nkv, 
                   int table_stride, void* k_pages, void* v_pages, int page_size, int write_kv, void* stream);
 int ls_swiglu(int dtype, const void* gu, void* out, int rows, int inter, long ld_in, long ld_out, void* stream);
 
+// Bias and activation on float rows: out = act(x + bias), times (x[:, width:] + bias[width:]) when gated.
+// out_dtype 0 float32, 1 bfloat16; act 0 none, 1 SiLU, 2 GELU (tanh), 3 GELU (erf), 4 ReLU.
+int ls_bias_act(int out_dtype, const float* x, long ldx, const float* bias, void* out, long ldo, int rows, int width,
+                int act, int gated, void* stream);
+
 // Arg-max of float rows, lowest index among equal maxima.  Rows wider than one chunk leave the
 // chunks' winners in `scratch` (2 * rows * ls_argmax_chunks(width) 4-byte words, device memory
 // the caller brings) for a second small launch.

@@ -310,6 +310,29 @@ class Kernels:
             c_int(DTYPE_CODE[out.dtype]), _ptr(gate_up), _ptr(out), c_int(rows), c_int(inter),
             c_long(gate_up.stride(0)), c_long(out.stride(0)), _stream()))
 
+    ACTIVATIONS = {"none": 0, "silu": 1, "gelu_tanh": 2, "gelu": 3, "relu": 4}
+
+    def bias_act(self, x: torch.Tensor, bias, out: torch.Tensor, activation: str = "none", gated: bool = False) -> None:
+        """``out = act(x + bias)`` on float32 rows ``x``; gated: ``x`` holds gates then ups and
+        ``out = act(gate + bias_gate) * (up + bias_up)``.  ``bias`` float32 or None; ``out`` float32
+        or bfloat16, and may be ``x`` itself when not gated."""
+        _rows_ok(x, "bias_act x"); _rows_ok(out, "bias_act out")
+        if activation not in self.ACTIVATIONS:
+            raise KernelError(f"activation {activation!r} is not built; known: {', '.join(self.ACTIVATIONS)}")
+        rows, width = out.shape
+        if not (x.dtype == torch.float32 and x.shape == (rows, 2 * width if gated else width) and out.dtype in DTYPE_CODE):
+            raise KernelError(f"bias_act reads float32 [{rows},{2 * width if gated else width}], got {tuple(x.shape)} {x.dtype}")
+        if bias is not None:
+            if not (bias.is_cuda and bias.dtype == torch.float32 and bias.is_contiguous() and bias.shape == (x.shape[1],)):
+                raise KernelError(f"bias_act bias must be float32 [{x.shape[1]}]")
+        if gated and x.data_ptr() == out.data_ptr():
+            raise KernelError("a gated bias_act cannot work in place")
+        if rows == 0:
+            return
+        self._launch(self.core, self.core.ls_bias_act, (
+            c_int(DTYPE_CODE[out.dtype]), _ptr(x), c_long(x.stride(0)), _ptr(bias), _ptr(out), c_long(out.stride(0)),
+            c_int(rows), c_int(width), c_int(self.ACTIVATIONS[activation]), c_int(1 if gated else 0), _stream()))
+
     #: (row, chunk) pairs the library's static arg-max scratch holds (LS_ARGMAX_STATIC_PAIRS)
     ARGMAX_STATIC_PAIRS = 16384
 

@@ -200,7 +200,8 @@ class Attention(Mixer):
     """Parameters: ``hidden_size``, ``num_heads``, ``num_kv_heads``,
     ``head_dim``, ``qk_norm`` (a norm ``PartSpec`` or None), ``position`` (a
     position-encoding ``PartSpec``), ``window`` (keys visible to a query,
-    None for all), ``bias`` (must be False), ``scale`` (score multiplier)."""
+    None for all), ``bias`` (biases of the q, k and v projections), ``out_bias`` (optional, a
+    bias of the output projection), ``scale`` (score multiplier)."""
 
     graph_safe = True
     repeatable = True
@@ -217,8 +218,8 @@ class Attention(Mixer):
         self.d = int(p["head_dim"])
         self.window = p.get("window")
         self.scale = float(p["scale"])
-        if p.get("bias"):
-            raise ValueError("attention with projection biases is not built")
+        self.bias = bool(p.get("bias"))              # q_proj.bias, k_proj.bias, v_proj.bias
+        self.out_bias = bool(p.get("out_bias"))      # o_proj.bias
         if self.nq % self.nkv:
             raise ValueError(f"{self.nq} query heads are not a multiple of {self.nkv} kv heads")
         if self.d % 16 or not 16 <= self.d <= 256:
@@ -231,6 +232,7 @@ class Attention(Mixer):
         if self.position.rotary_dim > self.d:
             raise ValueError(f"rotary_dim {self.position.rotary_dim} exceeds head size {self.d}")
         self.w_qkv = self.w_q = self.w_o = self.q_norm = self.k_norm = None
+        self.b_qkv = self.b_q = self.b_o = None
         self.norm_eps = float(self.qk_norm_spec["eps"]) if self.qk_norm_spec else 0.0
         if self.qk_norm_spec is not None:
             if self.qk_norm_spec.kind != "rmsnorm" or int(self.qk_norm_spec["size"]) != self.d:
@@ -249,6 +251,12 @@ class Attention(Mixer):
         if p.get("qk_norm") is not None:
             out += [WeightSpec(f"{prefix}.q_norm.weight", (d,), kind="vector", init="norm"),
                     WeightSpec(f"{prefix}.k_norm.weight", (d,), kind="vector", init="norm")]
+        if p.get("bias"):
+            out += [WeightSpec(f"{prefix}.q_proj.bias", (nq * d,), kind="vector"),
+                    WeightSpec(f"{prefix}.k_proj.bias", (nkv * d,), kind="vector"),
+                    WeightSpec(f"{prefix}.v_proj.bias", (nkv * d,), kind="vector")]
+        if p.get("out_bias"):
+            out.append(WeightSpec(f"{prefix}.o_proj.bias", (h,), kind="vector"))
         return out
 
     def cache_spec(self):
@@ -258,13 +266,32 @@ class Attention(Mixer):
         q = weights.get(f"{self.prefix}.q_proj.weight")
         k = weights.get(f"{self.prefix}.k_proj.weight")
         v = weights.get(f"{self.prefix}.v_proj.weight")
+        order = self.position.dim_order(self.d) if hasattr(self.position, "dim_order") else None
+        if order is not None:
+            order = torch.as_tensor(list(order), dtype=torch.long)
+            if sorted(order.tolist()) != list(range(self.d)):
+                raise ValueError(f"the position encoding's dim_order is no permutation of range({self.d})")
+            q = q.view(self.nq, self.d, -1)[:, order].reshape(q.shape)       # every head's dimensions alike
+            k = k.view(self.nkv, self.d, -1)[:, order].reshape(k.shape)
         self.w_qkv = rt.matrix(torch.cat([q.to(torch.float32), k.to(torch.float32), v.to(torch.float32)], dim=0)
                                if len({q.dtype, k.dtype, v.dtype}) > 1 else torch.cat([q, k, v], dim=0))
         self.w_q = self.w_qkv[: self.nq * self.d]
         self.w_o = rt.matrix(weights.get(f"{self.prefix}.o_proj.weight"))
+        if self.bias:
+            bq, bk, bv = (weights.get(f"{self.prefix}.{n}_proj.bias").to(torch.float32) for n in "qkv")
+            if order is not None:
+                bq = bq.view(self.nq, self.d)[:, order].reshape(-1)
+                bk = bk.view(self.nkv, self.d)[:, order].reshape(-1)
+            self.b_qkv = rt.vector(torch.cat([bq, bk, bv]))
+            self.b_q = self.b_qkv[: self.nq * self.d]
+        if self.out_bias:
+            self.b_o = rt.vector(weights.get(f"{self.prefix}.o_proj.bias"))
         if self.qk_norm_spec is not None:
-            self.q_norm = rt.vector(weights.get(f"{self.prefix}.q_norm.weight"))
-            self.k_norm = rt.vector(weights.get(f"{self.prefix}.k_norm.weight"))
+            q_norm, k_norm = weights.get(f"{self.prefix}.q_norm.weight"), weights.get(f"{self.prefix}.k_norm.weight")
+            if order is not None:
+                q_norm, k_norm = q_norm[order], k_norm[order]
+            self.q_norm = rt.vector(q_norm)
+            self.k_norm = rt.vector(k_norm)
         rt.kernels.attention_lib(self.d)
         if hasattr(self.position, "bind"):
             self.position.bind(rt)      # layers with equal constants share their tables
@@ -301,7 +328,16 @@ class Attention(Mixer):
         width = (nq + 2 * nkv) * d
         qkv = ctx.buf("attention.qkv", (t, width), rt.dtype)
         fused = {} if norm is None else {"norm_weight": norm.weight, "eps": norm.eps}
-        if run.writes_cache:
+        if self.b_qkv is not None:
+            # biases: the product in float32, then a pass that adds them and rounds to the compute dtype
+            raw = ctx.buf("attention.qkv_f32", (t, width), torch.float32)
+            if run.writes_cache:
+                k.gemm(x, self.w_qkv, raw, STORE_F32, **fused)
+                k.bias_act(raw, self.b_qkv, qkv)
+            else:
+                k.gemm(x, self.w_q, raw[:, : nq * d], STORE_F32, **fused)
+                k.bias_act(raw[:, : nq * d], self.b_q, qkv[:, : nq * d])
+        elif run.writes_cache:
             k.gemm(x, self.w_qkv, qkv, **fused)
         else:
             k.gemm(x, self.w_q, qkv[:, : nq * d], **fused)
@@ -348,6 +384,11 @@ class Attention(Mixer):
 
     def _project_out(self, ctx, attn, out, accumulate: bool, defer: bool):
         k = ctx.rt.kernels
+        if self.b_o is not None:
+            # (stream + product) + bias, at once: the order of the additions must not depend on the batch
+            k.gemm(attn, self.w_o, out, ADD_F32 if accumulate else STORE_F32)
+            k.bias_act(out, self.b_o, out)
+            return None
         if defer and accumulate and 0 < ctx.n_tokens <= deferred_rows(ctx, self.nq * self.d, out.shape[1]):
             slices = k.gemm_slices_count(self.nq * self.d)
             partials = ctx.buf("attention.out_slices", (slices * ctx.n_tokens, out.shape[1]), torch.float32)

@@ -135,6 +135,15 @@ class PositionEncoding(Part):
     cos = None
     sin = None
 
+    def dim_order(self, head_dim: int):
+        """An encoding that pairs other dimensions than ``i`` with ``i + rotary_dim/2`` (neighbours,
+        for instance) says here in which order a head's dimensions have to stand for its pairs to be
+        those: a permutation of ``range(head_dim)``, ``order[j]`` being the dimension that comes to
+        place ``j``.  The mixer reorders the rows of its query and key projections (and the
+        per-head norm weights) that way when it loads them; scores do not change, because queries
+        and keys are reordered alike.  None: as they are."""
+        return None
+
     def ensure(self, max_position: int, rt) -> None:
         """Make the tables cover positions ``< max_position``; a part that replaces a table
         a captured graph may hold calls ``bump_device_epoch()``."""

@@ -141,6 +141,35 @@ def test_gemm_refuses_mismatched_operands():
         K().gemm(x, w, torch.zeros(4, 8, device="cuda"))
 
 
+@pytest.mark.parametrize("out_dtype", DTYPES)
+@pytest.mark.parametrize("activation", ["none", "silu", "gelu_tanh", "gelu", "relu"])
+@pytest.mark.parametrize("rows,width", [(1, 40), (7, 1000), (70, 3072)])
+def test_bias_and_activation_pass_against_torch(out_dtype, activation, rows, width):
+    """``act(x + bias)`` and its gated form ``act(gate + b) * (up + b)``, with and without a bias, also in place."""
+    g = torch.Generator().manual_seed(rows + width)
+    acts = {"none": lambda v: v, "silu": torch.nn.functional.silu, "relu": torch.relu,
+            "gelu": torch.nn.functional.gelu, "gelu_tanh": lambda v: torch.nn.functional.gelu(v, approximate="tanh")}
+    tol = 2e-6 if out_dtype is torch.float32 else 5e-3
+    for gated in (False, True):
+        x = torch.randn(rows, width * (2 if gated else 1) + 8, generator=g).cuda()[:, : width * (2 if gated else 1)]
+        for bias in (None, torch.randn(x.shape[1], generator=g).cuda()):
+            out = torch.full((rows, width), float("nan"), dtype=out_dtype, device="cuda")
+            K().bias_act(x, bias, out, activation, gated=gated)
+            v = x.double() + (bias.double() if bias is not None else 0.0)
+            want = acts[activation](v[:, :width]) * (v[:, width:] if gated else 1.0)
+            assert rel_err(out, want) < tol, (activation, gated, bias is not None)
+    x = torch.randn(rows, width, generator=g).cuda()
+    bias = torch.randn(width, generator=g).cuda()
+    want = acts[activation](x.double() + bias.double())
+    K().bias_act(x, bias, x, activation)                        # in place
+    assert rel_err(x, want) < 2e-6
+    from lockstep_amd.ops import KernelError
+    with pytest.raises(KernelError, match="not built"):
+        K().bias_act(x, None, x, "swish7")
+    with pytest.raises(KernelError, match="float32 \\["):
+        K().bias_act(x, None, torch.empty(rows, width + 1, device="cuda"), "none")
+
+
 # -- norm --------------------------------------------------------------------------
 
 @pytest.mark.parametrize("dtype", DTYPES)

@@ -130,6 +130,165 @@ def test_attention_part_alone_in_portions(dtype, tol):
     assert rel_err(torch.cat(got), want) < tol
 
 
+def test_a_position_encoding_that_pairs_neighbours_registers_without_a_kernel_of_its_own():
+    """A toy rotary encoding whose pairs are the neighbours (2i, 2i + 1) of the first 32 of 48
+    dimensions: it states the order that brings its pairs to (i, i + rotary_dim/2), the attention
+    part reorders its query and key rows (and norm weights) at load, and the result equals a plain
+    attention that rotates neighbours -- in portions, in float32."""
+    from lockstep_amd.config import PartSpec
+    from lockstep_amd.parts import build_part, register_part, unregister_part
+    from lockstep_amd.parts.rope import RotaryHalf
+
+    @register_part("toy_rope_neighbours")
+    class NeighbourRotary(RotaryHalf):
+        def share_key(self):
+            return ("toy_rope_neighbours",) + super().share_key()
+
+        def bind(self, rt):                       # tables of its own, not the half rotation's
+            self._store = self.__dict__.setdefault("_own_tables", [None, None])
+
+        def dim_order(self, head_dim):
+            rot = self.rotary_dim
+            return list(range(0, rot, 2)) + list(range(1, rot, 2)) + list(range(rot, head_dim))
+
+    hidden, nq, nkv, d, rot, theta, eps = 40, 6, 2, 48, 32, 1e4, 1e-5
+    try:
+        spec = PartSpec("attention", {
+            "hidden_size": hidden, "num_heads": nq, "num_kv_heads": nkv, "head_dim": d,
+            "qk_norm": PartSpec("rmsnorm", {"size": d, "eps": eps}),
+            "position": PartSpec("toy_rope_neighbours", {"rotary_dim": rot, "theta": theta}),
+            "window": None, "bias": False, "scale": d ** -0.5})
+        part = build_part(spec, "att")
+        g = torch.Generator().manual_seed(4)
+        w = {"att.q_proj.weight": torch.randn(nq * d, hidden, generator=g) * 0.3,
+             "att.k_proj.weight": torch.randn(nkv * d, hidden, generator=g) * 0.3,
+             "att.v_proj.weight": torch.randn(nkv * d, hidden, generator=g) * 0.3,
+             "att.o_proj.weight": torch.randn(hidden, nq * d, generator=g) * 0.3,
+             "att.q_norm.weight": 1 + 0.2 * torch.randn(d, generator=g),
+             "att.k_norm.weight": 1 + 0.2 * torch.randn(d, generator=g)}
+        w = {k: v.to(torch.bfloat16) for k, v in w.items()}
+        h = Harness("float32", unit_specs=(part.cache_spec(),))
+        part.load(store(w), h.rt)
+        t = 27
+        x = torch.randn(t, hidden, generator=g).to(torch.bfloat16)
+
+        # the plain form: rotate neighbours of the first `rot` dimensions, in the checkpoint's own order
+        w64 = {k: v.double() for k, v in w.items()}
+        x64 = x.double()
+        q = P.rmsnorm((x64 @ w64["att.q_proj.weight"].T).view(t, nq, d), w64["att.q_norm.weight"], eps)
+        k = P.rmsnorm((x64 @ w64["att.k_proj.weight"].T).view(t, nkv, d), w64["att.k_norm.weight"], eps)
+        v = (x64 @ w64["att.v_proj.weight"].T).view(t, nkv, d)
+        inv_freq = theta ** (-torch.arange(0, rot, 2, dtype=torch.float64) / rot)
+        angles = torch.arange(t, dtype=torch.float64)[:, None] * inv_freq[None, :]
+
+        def rotate(z):
+            out = z.clone()
+            even, odd = z[..., 0:rot:2], z[..., 1:rot:2]
+            c, s_ = angles.cos()[:, None, :], angles.sin()[:, None, :]
+            out[..., 0:rot:2] = even * c - odd * s_
+            out[..., 1:rot:2] = odd * c + even * s_
+            return out
+
+        attn = P.causal_attention(rotate(q), rotate(k), v, q_positions=torch.arange(t))
+        want = attn.reshape(t, nq * d) @ w64["att.o_proj.weight"].T
+        # a half rotation of the same weights is something else: the order matters
+        cos, sin = P.rope_tables(rot, theta, torch.arange(t))
+        assert rel_err(P.apply_rope(q[..., :rot], cos, sin), rotate(q)[..., :rot]) > 0.1
+
+        got, pos = [], 0
+        for n in (9, 2, 15, 1):
+            ctx = h.context({"a": n}, mixers=[part])
+            out = torch.zeros(n, hidden, device="cuda")
+            part.forward(ctx, Run(), x[pos:pos + n].float().cuda(), out, accumulate=False)
+            h.commit(ctx)
+            got.append(out.cpu())
+            pos += n
+        assert rel_err(torch.cat(got), want) < 2e-5
+    finally:
+        unregister_part("toy_rope_neighbours")
+
+
+@pytest.mark.parametrize("dtype,tol", [("float32", 2e-5), ("bfloat16", 3e-2)])
+def test_parts_with_biases_and_another_activation(dtype, tol):
+    """Attention with biases on all four projections and a gated feed-forward with the tanh form
+    of GELU and biases, each alone in portions against the formulas in float64; the same rows in
+    one step and in portions give the same bits."""
+    from lockstep_amd.config import PartSpec
+    from lockstep_amd.parts import build_part
+
+    hidden, nq, nkv, d, inter, eps = 72, 6, 3, 32, 200, 1e-5
+    g = torch.Generator().manual_seed(8)
+    rnd = lambda *shape, scale=0.3: (torch.randn(*shape, generator=g) * scale).to(torch.bfloat16)
+    att = build_part(PartSpec("attention", {
+        "hidden_size": hidden, "num_heads": nq, "num_kv_heads": nkv, "head_dim": d,
+        "qk_norm": PartSpec("rmsnorm", {"size": d, "eps": eps}),
+        "position": PartSpec("rope_half", {"rotary_dim": d, "theta": 1e4}),
+        "window": None, "bias": True, "out_bias": True, "scale": d ** -0.5}), "att")
+    names = [w.name for w in att.weight_specs(att.spec, "att")]
+    assert {"att.q_proj.bias", "att.k_proj.bias", "att.v_proj.bias", "att.o_proj.bias"} <= set(names)
+    w = {"att.q_proj.weight": rnd(nq * d, hidden), "att.k_proj.weight": rnd(nkv * d, hidden),
+         "att.v_proj.weight": rnd(nkv * d, hidden), "att.o_proj.weight": rnd(hidden, nq * d),
+         "att.q_norm.weight": (1 + 0.2 * torch.randn(d, generator=g)).to(torch.bfloat16),
+         "att.k_norm.weight": (1 + 0.2 * torch.randn(d, generator=g)).to(torch.bfloat16),
+         "att.q_proj.bias": rnd(nq * d), "att.k_proj.bias": rnd(nkv * d), "att.v_proj.bias": rnd(nkv * d),
+         "att.o_proj.bias": rnd(hidden)}
+    h = Harness(dtype, unit_specs=(att.cache_spec(),))
+    att.load(store(w), h.rt)
+    t = 30
+    x = rnd(t, hidden, scale=1.0)
+    w64, x64 = {k: v.double() for k, v in w.items()}, x.double()
+    q = P.rmsnorm((x64 @ w64["att.q_proj.weight"].T + w64["att.q_proj.bias"]).view(t, nq, d), w64["att.q_norm.weight"], eps)
+    k = P.rmsnorm((x64 @ w64["att.k_proj.weight"].T + w64["att.k_proj.bias"]).view(t, nkv, d), w64["att.k_norm.weight"], eps)
+    v = (x64 @ w64["att.v_proj.weight"].T + w64["att.v_proj.bias"]).view(t, nkv, d)
+    cos, sin = P.rope_tables(d, 1e4, torch.arange(t))
+    attn = P.causal_attention(P.apply_rope(q, cos, sin), P.apply_rope(k, cos, sin), v, q_positions=torch.arange(t))
+    want = attn.reshape(t, nq * d) @ w64["att.o_proj.weight"].T + w64["att.o_proj.bias"]
+
+    def run_attention(rid, cuts):
+        got, pos = [], 0
+        for n in cuts:
+            ctx = h.context({rid: n}, mixers=[att])
+            out = torch.zeros(n, hidden, device="cuda")
+            att.forward(ctx, Run(), x[pos:pos + n].to(h.rt.dtype).cuda(), out, accumulate=False)
+            h.commit(ctx)
+            got.append(out.cpu())
+            pos += n
+        return torch.cat(got)
+
+    whole, cut = run_attention("whole", (t,)), run_attention("cut", (11, 2, 16, 1))
+    assert rel_err(whole, want) < tol and torch.equal(whole, cut)
+
+    ff = build_part(PartSpec("gated_mlp", {"hidden_size": hidden, "intermediate_size": inter,
+                                           "activation": "gelu_tanh", "bias": True}), "ff")
+    wf = {"ff.gate_proj.weight": rnd(inter, hidden), "ff.up_proj.weight": rnd(inter, hidden),
+          "ff.down_proj.weight": rnd(hidden, inter), "ff.gate_proj.bias": rnd(inter), "ff.up_proj.bias": rnd(inter),
+          "ff.down_proj.bias": rnd(hidden)}
+    ff.load(store(wf), h.rt)
+    f64 = {k: v.double() for k, v in wf.items()}
+    gate = x64 @ f64["ff.gate_proj.weight"].T + f64["ff.gate_proj.bias"]
+    up = x64 @ f64["ff.up_proj.weight"].T + f64["ff.up_proj.bias"]
+    stream = torch.randn(t, hidden, generator=g)
+    want = stream.double() + (torch.nn.functional.gelu(gate, approximate="tanh") * up) @ f64["ff.down_proj.weight"].T \
+        + f64["ff.down_proj.bias"]
+
+    def run_ff(cuts):
+        got, pos = [], 0
+        for n in cuts:
+            ctx = h.context({f"f{len(cuts)}": n})
+            out = stream[pos:pos + n].cuda().clone()
+            left = ff.forward(ctx, x[pos:pos + n].to(h.rt.dtype).cuda(), out, accumulate=True, defer=True)
+            assert left is None                      # with biases the addition is not left to the next norm
+            h.commit(ctx)
+            got.append(out.cpu())
+            pos += n
+        return torch.cat(got)
+
+    whole, cut = run_ff((t,)), run_ff((3, 20, 7))
+    assert rel_err(whole, want) < tol and torch.equal(whole, cut)
+    with pytest.raises(ValueError, match="not built"):
+        build_part(PartSpec("gated_mlp", {"hidden_size": 8, "intermediate_size": 8, "activation": "swish7"}), "x")
+
+
 def test_feed_forward_part_and_block_alone():
     from lockstep_amd.config import LayerSpec, PartSpec
     from lockstep_amd.parts import build_part, part_class
@@ -150,7 +309,7 @@ def test_feed_forward_part_and_block_alone():
     want = 1 + P.mlp_block({k: v.double() for k, v in w.items()}, "L.mlp", x.double())
     assert rel_err(out.cpu(), want) < 2e-5
     with pytest.raises(ValueError):
-        build_part(PartSpec("gated_mlp", {"hidden_size": 8, "intermediate_size": 8, "activation": "gelu"}), "m")
+        build_part(PartSpec("gated_mlp", {"hidden_size": 8, "intermediate_size": 8, "activation": "softsign"}), "m")
 
     # the whole arrangement: h += attn(norm(h)); h += mlp(norm(h))
     nq, nkv, d = 4, 4, 16
