@@ -1644,10 +1644,13 @@ __global__ __launch_bounds__(256) void combine_kernel(const SeqMeta* __restrict_
 }
 
 // The fold for requests of at most 16 rows a kv head (decoded tokens), where a request far away has dozens
-// of splits: the fold of one split has to wait for the one before, so what takes time is the loads.  Here
-// the four waves share the columns (wave w has the column blocks w, w + 4, ..., as in the cooperative
-// kernel), so a lane holds a quarter of a row's sums and can ask for sixteen splits at a time.  Every
-// element goes through the operations of fold_split in the same order: the same bits.
+// of splits.  The fold of one split has to wait for the one before, and with two rows a request only eight
+// lanes of a wave have anything to load, so loads straight into the folding lanes cost a memory round
+// trip every few splits.  Here all 256 threads bring the partial results of a batch of splits into LDS in
+// whole lines (a row's splits lie one after the other), the next batch's loads are in flight while this one
+// is folded, and the four waves share the columns (wave w has the column blocks w, w + 4, ..., as in the
+// cooperative kernel).  Every element goes through the operations of fold_split in the same order: the same
+// bits.
 template <typename T>
 __global__ __launch_bounds__(256) void combine_few_rows_kernel(const SeqMeta* __restrict__ seqs,
                                                                const CombineItem* __restrict__ items,
@@ -1655,23 +1658,29 @@ __global__ __launch_bounds__(256) void combine_few_rows_kernel(const SeqMeta* __
                                                                const float* __restrict__ part_ml,
                                                                T* __restrict__ out, long ldo, int G) {
   constexpr int MYDB = (DB + 3) / 4;
-  constexpr int BATCH = MYDB <= 2 ? 16 : 8;
+  constexpr int STAGE = 6144;           // floats of sums a buffer holds
+  constexpr int ROW_PAD = 4;            // floats between rows: spreads the rows over the banks
+  constexpr int PIECES = STAGE / 4 / 256;  // 16-byte pieces a thread moves per batch
+  __shared__ __attribute__((aligned(16))) float stage_acc[2][STAGE];
+  __shared__ float stage_ml[2][2 * 512];
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const CombineItem item = items[blockIdx.x];
   const int kvh = blockIdx.y;
   const int rows_total = item.q_len * G;  // <= 16, checked on the host
+  if (rows_total <= 0) return;
   const int r = lane & 15;
-  if (r >= rows_total) return;
   const int g = lane >> 4;
-  const int qi = r / G;
-  const int head = kvh * G + r % G;
+  const bool mine = r < rows_total;
+  const int qi = mine ? r / G : 0;
+  const int head = kvh * G + (mine ? r % G : 0);
+  const int n_splits = item.n_splits;
+  const long pr_base = item.part_base + (long)kvh * rows_total * n_splits;  // row r, split s: pr_base + r * n_splits + s
 
   f32x4 run_acc[MYDB];
   float run_m = kNegSentinel, run_l = 0.f;
 #pragma unroll
   for (int j = 0; j < MYDB; ++j) run_acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
-  const long pr0 = item.part_base + ((long)kvh * rows_total + r) * item.n_splits;
   auto fold = [&](const f32x4 (&acc)[MYDB], float m, float l) {  // fold_split on this wave's blocks
     if (!(l > 0.f)) return;
     const float m_new = fmaxf(run_m, m);
@@ -1684,33 +1693,85 @@ __global__ __launch_bounds__(256) void combine_few_rows_kernel(const SeqMeta* __
     run_l = run_l * a + l * b;
     run_m = m_new;
   };
-  auto load = [&](f32x4 (&acc)[MYDB], float& m, float& l, long pr) {
-#pragma unroll
-    for (int j = 0; j < MYDB; ++j) {
-      const int blk = min(wave + 4 * j, DB - 1);
-      acc[j] = *reinterpret_cast<const f32x4*>(part_acc + pr * D + blk * 16 + 4 * g);
-    }
-    m = part_ml[pr * 2];
-    l = part_ml[pr * 2 + 1];
-  };
+
   if (LS_MUTANT_DEVICE(kMutantReversedFold)) {
-    for (int s = item.n_splits - 1; s >= 0; --s) {
+    for (int s = n_splits - 1; s >= 0 && mine; --s) {
+      const long pr = pr_base + (long)r * n_splits + s;
       f32x4 acc[MYDB];
-      float m, l;
-      load(acc, m, l, pr0 + s);
-      fold(acc, m, l);
+#pragma unroll
+      for (int j = 0; j < MYDB; ++j)
+        acc[j] = *reinterpret_cast<const f32x4*>(part_acc + pr * D + min(wave + 4 * j, DB - 1) * 16 + 4 * g);
+      fold(acc, part_ml[pr * 2], part_ml[pr * 2 + 1]);
     }
   } else {
-    for (int s0 = 0; s0 < item.n_splits; s0 += BATCH) {
-      f32x4 acc[BATCH][MYDB];
-      float m[BATCH], l[BATCH];
+    // splits a batch: what fits the buffer, at most 32
+    const int row_floats_max = STAGE / rows_total - ROW_PAD;
+    const int batch = max(1, min(32, row_floats_max / D));
+    const int row_stride = batch * D + ROW_PAD;      // floats
+    const int per_row = batch * (D / 4);             // 16-byte pieces of a row's batch
+    const int total = rows_total * per_row;          // <= STAGE / 4
+    f32x4 moved[PIECES];
+    float2 moved_ml[2] = {float2{0.f, 0.f}, float2{0.f, 0.f}};  // up to 16 rows x 32 splits over 256 threads
+    auto request = [&](int s0) {  // the loads of the batch that starts at split s0, into registers
 #pragma unroll
-      for (int u = 0; u < BATCH; ++u) load(acc[u], m[u], l[u], pr0 + min(s0 + u, item.n_splits - 1));  // clamped: loaded, not used
+      for (int i = 0; i < PIECES; ++i) {
+        const int idx = i * 256 + (int)threadIdx.x;
+        const int row = min(idx / per_row, rows_total - 1);
+        const int rest = idx - (idx / per_row) * per_row;
+        const int u = rest / (D / 4);
+        const int piece = rest - u * (D / 4);
+        const long pr = pr_base + (long)row * n_splits + min(s0 + u, n_splits - 1);  // clamped: loaded, not used
+        moved[i] = *reinterpret_cast<const f32x4*>(part_acc + pr * D + piece * 4);
+      }
 #pragma unroll
-      for (int u = 0; u < BATCH; ++u)
-        if (s0 + u < item.n_splits) fold(acc[u], m[u], l[u]);
+      for (int i = 0; i < 2; ++i) {
+        const int e = i * 256 + (int)threadIdx.x;
+        if (e < rows_total * batch) {
+          const int row = e / batch;
+          const int u = e - row * batch;
+          const long pr = pr_base + (long)row * n_splits + min(s0 + u, n_splits - 1);
+          moved_ml[i] = *reinterpret_cast<const float2*>(part_ml + pr * 2);
+        }
+      }
+    };
+    auto put = [&](int buf) {  // ... and from the registers to their place in LDS
+#pragma unroll
+      for (int i = 0; i < PIECES; ++i) {
+        const int idx = i * 256 + (int)threadIdx.x;
+        if (idx >= total) continue;
+        const int row = idx / per_row;
+        const int rest = idx - row * per_row;
+        *reinterpret_cast<f32x4*>(&stage_acc[buf][row * row_stride + rest * 4]) = moved[i];
+      }
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const int e = i * 256 + (int)threadIdx.x;
+        if (e < rows_total * batch) {
+          stage_ml[buf][2 * e] = moved_ml[i].x;
+          stage_ml[buf][2 * e + 1] = moved_ml[i].y;
+        }
+      }
+    };
+    request(0);
+    int buf = 0;
+    for (int s0 = 0; s0 < n_splits; s0 += batch, buf ^= 1) {
+      put(buf);
+      __syncthreads();  // the batch is in its buffer; the other buffer has been folded by every wave
+      if (s0 + batch < n_splits) request(s0 + batch);
+      if (mine) {
+        const int count = min(batch, n_splits - s0);
+        for (int u = 0; u < count; ++u) {
+          f32x4 acc[MYDB];
+#pragma unroll
+          for (int j = 0; j < MYDB; ++j)
+            acc[j] = *reinterpret_cast<const f32x4*>(
+                &stage_acc[buf][r * row_stride + u * D + min(wave + 4 * j, DB - 1) * 16 + 4 * g]);
+          fold(acc, stage_ml[buf][2 * (r * batch + u)], stage_ml[buf][2 * (r * batch + u) + 1]);
+        }
+      }
     }
   }
+  if (!mine) return;
   T* dst = out + (long)(item.q_off + qi) * ldo + (long)head * D;
 #pragma unroll
   for (int j = 0; j < MYDB; ++j) {
