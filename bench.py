@@ -60,7 +60,9 @@ def build_model(args):
         overrides["num_hidden_layers"] = args.layers
     config = preset(args.model, **overrides)
     full_layers = preset(args.model).num_hidden_layers
+    print(f"[bench] drawing random weights for {args.model}", file=sys.stderr, flush=True)
     tensors = random_tensors(config, seed=0, std=0.02, norm_std=0.0, dtype=torch.bfloat16)
+    print("[bench] weights drawn; loading them onto the GPU", file=sys.stderr, flush=True)
     model = model_from_tensors(config, tensors, dtype="bfloat16" if args.dtype == "bf16" else "float32")
     del tensors
     return model, config, full_layers
@@ -128,7 +130,7 @@ def random_prompts(n: int, length: int, vocab: int, seed: int):
 
 
 def measure_decode(model, cfg, batch: int, prompt_len: int, steps: int, warmup: int, page_size: int,
-                   device_loop: bool = True, repeats: int = 1):
+                   device_loop: bool = True, repeats: int = 1, progress: bool = False):
     """(seconds of the timed steps of every repeat, mean context length during them).  Every
     repeat starts from freshly prefilled requests and times exactly ``steps`` decode steps."""
     import torch
@@ -153,6 +155,8 @@ def measure_decode(model, cfg, batch: int, prompt_len: int, steps: int, warmup: 
                 cache.open(r.uid)
             logits = model.step(cache, [StepEntry(r.uid, r.prompt, [len(r.prompt) - 1]) for r in group])
             tokens += sampler.sample(logits, group)
+            if progress:
+                print(f"[bench] prompts of {lo + len(group)} of {batch} requests are in", file=sys.stderr, flush=True)
         return tokens
 
     def decode(tokens, n):
@@ -249,6 +253,7 @@ def contexts_record(args, model, cfg, full_layers: int) -> dict:
     portion = args.prefill_chunk or 2048
     rows = {}
     for context in [int(c) for c in args.contexts.split(",")]:
+        print(f"[bench] context {context}: prefill in portions of {portion}", file=sys.stderr, flush=True)
         seconds = measure_prefill_portions(model, cfg, context, portion, args.page_size)
         flops = sum(Workload(model).step_flops(min(portion, context - lo), lo, 0) for lo in range(0, context, portion))
         row = {"prefill_tok_s": round(context / seconds, 1), "prefill_ms": round(1e3 * seconds, 2),
@@ -259,8 +264,9 @@ def contexts_record(args, model, cfg, full_layers: int) -> dict:
             free, _ = torch.cuda.mem_get_info()
             if cache_bytes > free - (12 << 30):
                 continue
+            print(f"[bench] context {context}: decode at batch {batch}", file=sys.stderr, flush=True)
             t, mean_context = measure_decode(model, cfg, batch, context, args.steps, 2, args.page_size,
-                                             not args.host_sampling, 1)
+                                             not args.host_sampling, 1, progress=True)
             step_s = t[0] / args.steps
             row[f"decode_b{batch}_tok_s"] = round(batch / step_s, 1)
             row[f"decode_b{batch}_ms"] = round(1e3 * step_s, 3)

@@ -1644,71 +1644,72 @@ __global__ __launch_bounds__(256) void combine_kernel(const SeqMeta* __restrict_
 }
 
 // The fold for requests of at most 16 rows a kv head (decoded tokens), where a request far away has dozens
-// of splits.  The fold of one split has to wait for the one before, and with two rows a request only eight
-// lanes of a wave have anything to load, so loads straight into the folding lanes cost a memory round
-// trip every few splits.  Here all 256 threads bring the partial results of a batch of splits into LDS in
-// whole lines (a row's splits lie one after the other), the next batch's loads are in flight while this one
-// is folded, and the four waves share the columns (wave w has the column blocks w, w + 4, ..., as in the
-// cooperative kernel).  Every element goes through the operations of fold_split in the same order: the same
-// bits.
+// of splits.  The fold of one split has to wait for the one before, so what counts is how long one fold
+// takes and that its operands are there.  All 256 threads bring the partial results of a batch of splits
+// into LDS in whole lines (a row's splits lie one after the other), the next batch's loads are in flight
+// while this one is folded, and the folding itself is dealt out by elements: a thread owns four
+// neighbouring columns of one row (with two rows of 128 columns one wave does all of it, every lane busy,
+// a fold is some twenty instructions).  Every element goes through the operations of fold_split in the
+// same order: the same bits.
 template <typename T>
 __global__ __launch_bounds__(256) void combine_few_rows_kernel(const SeqMeta* __restrict__ seqs,
                                                                const CombineItem* __restrict__ items,
                                                                const float* __restrict__ part_acc,
                                                                const float* __restrict__ part_ml,
                                                                T* __restrict__ out, long ldo, int G) {
-  constexpr int MYDB = (DB + 3) / 4;
-  constexpr int STAGE = 6144;           // floats of sums a buffer holds
-  constexpr int ROW_PAD = 4;            // floats between rows: spreads the rows over the banks
-  constexpr int PIECES = STAGE / 4 / 256;  // 16-byte pieces a thread moves per batch
+  constexpr int QUADS = D / 4;                       // groups of four columns in a row
+  constexpr int MAXQ = (16 * QUADS + 255) / 256;     // such groups a thread owns at most (16 rows)
+  constexpr int STAGE = 6144;                        // floats of sums a buffer holds
+  constexpr int ROW_PAD = 4;                         // floats between rows: spreads the rows over the banks
+  constexpr int PIECES = STAGE / 4 / 256;            // 16-byte pieces a thread moves per batch
   __shared__ __attribute__((aligned(16))) float stage_acc[2][STAGE];
   __shared__ float stage_ml[2][2 * 512];
-  const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
   const CombineItem item = items[blockIdx.x];
   const int kvh = blockIdx.y;
   const int rows_total = item.q_len * G;  // <= 16, checked on the host
   if (rows_total <= 0) return;
-  const int r = lane & 15;
-  const int g = lane >> 4;
-  const bool mine = r < rows_total;
-  const int qi = mine ? r / G : 0;
-  const int head = kvh * G + (mine ? r % G : 0);
   const int n_splits = item.n_splits;
   const long pr_base = item.part_base + (long)kvh * rows_total * n_splits;  // row r, split s: pr_base + r * n_splits + s
+  const int owned = rows_total * QUADS;   // groups of four columns to fold
 
-  f32x4 run_acc[MYDB];
-  float run_m = kNegSentinel, run_l = 0.f;
+  f32x4 run_acc[MAXQ];
+  float run_m[MAXQ], run_l[MAXQ];
+  int row_of[MAXQ], quad_of[MAXQ];
 #pragma unroll
-  for (int j = 0; j < MYDB; ++j) run_acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
-  auto fold = [&](const f32x4 (&acc)[MYDB], float m, float l) {  // fold_split on this wave's blocks
+  for (int q = 0; q < MAXQ; ++q) {
+    run_acc[q] = f32x4{0.f, 0.f, 0.f, 0.f};
+    run_m[q] = kNegSentinel;
+    run_l[q] = 0.f;
+    const int it = min(q * 256 + (int)threadIdx.x, owned - 1);
+    row_of[q] = it / QUADS;
+    quad_of[q] = it - row_of[q] * QUADS;
+  }
+  auto fold = [&](int q, const f32x4& acc, float m, float l) {  // fold_split on these four columns
     if (!(l > 0.f)) return;
-    const float m_new = fmaxf(run_m, m);
-    const float a = softmax_exp<T>(run_m - m_new);
+    const float m_new = fmaxf(run_m[q], m);
+    const float a = softmax_exp<T>(run_m[q] - m_new);
     const float b = softmax_exp<T>(m - m_new);
 #pragma unroll
-    for (int j = 0; j < MYDB; ++j)
-#pragma unroll
-      for (int e = 0; e < 4; ++e) run_acc[j][e] = run_acc[j][e] * a + acc[j][e] * b;
-    run_l = run_l * a + l * b;
-    run_m = m_new;
+    for (int e = 0; e < 4; ++e) run_acc[q][e] = run_acc[q][e] * a + acc[e] * b;
+    run_l[q] = run_l[q] * a + l * b;
+    run_m[q] = m_new;
   };
 
   if (LS_MUTANT_DEVICE(kMutantReversedFold)) {
-    for (int s = n_splits - 1; s >= 0 && mine; --s) {
-      const long pr = pr_base + (long)r * n_splits + s;
-      f32x4 acc[MYDB];
+    for (int s = n_splits - 1; s >= 0; --s) {
 #pragma unroll
-      for (int j = 0; j < MYDB; ++j)
-        acc[j] = *reinterpret_cast<const f32x4*>(part_acc + pr * D + min(wave + 4 * j, DB - 1) * 16 + 4 * g);
-      fold(acc, part_ml[pr * 2], part_ml[pr * 2 + 1]);
+      for (int q = 0; q < MAXQ; ++q) {
+        if (q * 256 + (int)threadIdx.x >= owned) continue;
+        const long pr = pr_base + (long)row_of[q] * n_splits + s;
+        fold(q, *reinterpret_cast<const f32x4*>(part_acc + pr * D + quad_of[q] * 4), part_ml[pr * 2], part_ml[pr * 2 + 1]);
+      }
     }
   } else {
     // splits a batch: what fits the buffer, at most 32
     const int row_floats_max = STAGE / rows_total - ROW_PAD;
     const int batch = max(1, min(32, row_floats_max / D));
     const int row_stride = batch * D + ROW_PAD;      // floats
-    const int per_row = batch * (D / 4);             // 16-byte pieces of a row's batch
+    const int per_row = batch * QUADS;               // 16-byte pieces of a row's batch
     const int total = rows_total * per_row;          // <= STAGE / 4
     f32x4 moved[PIECES];
     float2 moved_ml[2] = {float2{0.f, 0.f}, float2{0.f, 0.f}};  // up to 16 rows x 32 splits over 256 threads
@@ -1718,8 +1719,8 @@ __global__ __launch_bounds__(256) void combine_few_rows_kernel(const SeqMeta* __
         const int idx = i * 256 + (int)threadIdx.x;
         const int row = min(idx / per_row, rows_total - 1);
         const int rest = idx - (idx / per_row) * per_row;
-        const int u = rest / (D / 4);
-        const int piece = rest - u * (D / 4);
+        const int u = rest / QUADS;
+        const int piece = rest - u * QUADS;
         const long pr = pr_base + (long)row * n_splits + min(s0 + u, n_splits - 1);  // clamped: loaded, not used
         moved[i] = *reinterpret_cast<const f32x4*>(part_acc + pr * D + piece * 4);
       }
@@ -1758,29 +1759,25 @@ __global__ __launch_bounds__(256) void combine_few_rows_kernel(const SeqMeta* __
       put(buf);
       __syncthreads();  // the batch is in its buffer; the other buffer has been folded by every wave
       if (s0 + batch < n_splits) request(s0 + batch);
-      if (mine) {
-        const int count = min(batch, n_splits - s0);
-        for (int u = 0; u < count; ++u) {
-          f32x4 acc[MYDB];
+      const int count = min(batch, n_splits - s0);
 #pragma unroll
-          for (int j = 0; j < MYDB; ++j)
-            acc[j] = *reinterpret_cast<const f32x4*>(
-                &stage_acc[buf][r * row_stride + u * D + min(wave + 4 * j, DB - 1) * 16 + 4 * g]);
-          fold(acc, stage_ml[buf][2 * (r * batch + u)], stage_ml[buf][2 * (r * batch + u) + 1]);
-        }
+      for (int q = 0; q < MAXQ; ++q) {
+        if (q * 256 + (int)threadIdx.x >= owned) continue;
+        const float* mine = &stage_acc[buf][row_of[q] * row_stride + quad_of[q] * 4];
+        const float* ml = &stage_ml[buf][2 * row_of[q] * batch];
+        for (int u = 0; u < count; ++u)
+          fold(q, *reinterpret_cast<const f32x4*>(mine + u * D), ml[2 * u], ml[2 * u + 1]);
       }
     }
   }
-  if (!mine) return;
-  T* dst = out + (long)(item.q_off + qi) * ldo + (long)head * D;
 #pragma unroll
-  for (int j = 0; j < MYDB; ++j) {
-    const int blk = wave + 4 * j;
-    if (blk >= DB) continue;
+  for (int q = 0; q < MAXQ; ++q) {
+    if (q * 256 + (int)threadIdx.x >= owned) continue;
+    const int r = row_of[q];
+    T* p = out + (long)(item.q_off + r / G) * ldo + (long)(kvh * G + r % G) * D + quad_of[q] * 4;
     float o[4];
 #pragma unroll
-    for (int e = 0; e < 4; ++e) o[e] = run_l > 0.f ? run_acc[j][e] / run_l : 0.f;
-    T* p = dst + blk * 16 + 4 * g;
+    for (int e = 0; e < 4; ++e) o[e] = run_l[q] > 0.f ? run_acc[q][e] / run_l[q] : 0.f;
     if (sizeof(T) == 2) {
       bf16x4 v;
       v[0] = (bf16_t)o[0]; v[1] = (bf16_t)o[1]; v[2] = (bf16_t)o[2]; v[3] = (bf16_t)o[3];
@@ -1854,13 +1851,16 @@ static bool coop_kernel_ready() {
 // where they fit; when the grid brings at least two workgroups per CU, with
 // one buffer instead, so that two workgroups share a CU and overlap each
 // other's loads.
+#ifndef LS_COOP_CROWDED_FROM
+#define LS_COOP_CROWDED_FROM 512  // from this many workgroups on: one tile buffer each, two workgroups a CU
+#endif
 template <typename T, bool FUSE, bool SPANS>
 static int launch_coop_as(dim3 grid, hipStream_t s, const void* q, long ldq, const void* k_pages, const void* v_pages,
                           int nkv, int page_size, int page_shift, const int* table, int table_stride, const void* seqs,
                           const void* items, void* out, long ldo, float* part_acc, float* part_ml, int G, float scale,
                           int window, DecodeFuse<T> fz) {
   constexpr int BUFS = coop_bufs(sizeof(T));
-  const bool crowded = (long)grid.x * grid.y >= 512;
+  const bool crowded = (long)grid.x * grid.y >= LS_COOP_CROWDED_FROM;
 #define LS_COOP(NBUF_)                                                                                              \
   hipLaunchKernelGGL((attention_coop_kernel<T, NBUF_, FUSE, SPANS>), grid, dim3(256), (coop_kernel_lds<T, NBUF_>()), s, \
                      (const T*)q, ldq, (const T*)k_pages, (const T*)v_pages, nkv, page_size, page_shift, table,        \

@@ -28,8 +28,10 @@ from .base import Mixer, PagedKVSpec, PendingAdd, WeightSpec, build_part, deferr
 # Steps of single decoded tokens run norm, rotation and cache write inside the
 # attention kernel (one launch less per layer); "0" keeps the separate kernel.
 FUSE_DECODE = os.environ.get("LOCKSTEP_FUSE_DECODE", "1") not in ("", "0")
-# From this many attention workgroups on (two a CU: the kernel is then bound by the cache it streams) the
-# prologue of the fused kernel costs more than the separate norm/rotation launch; measured +2 % at batch 64.
+# From this many (request, kv head) pairs on, the prologue of the fused kernel costs more than the separate
+# norm/rotation launch (measured +2 % at batch 64, 8 kv heads).  Pairs, not workgroups: a request that is cut
+# into many items repeats only the query's part of the prologue in each, and one launch less still pays
+# (eight requests of 16,384 tokens: 4.23 -> 4.13 ms a step).
 FUSE_DECODE_BELOW = int(os.environ.get("LOCKSTEP_FUSE_DECODE_BELOW", "512"))
 # The most splits (of 256 keys) one cooperative workgroup walks when a request is cut over several.
 MAX_SPAN = 4               # splits of a work item where requests of a ragged batch are cut
@@ -73,7 +75,7 @@ class AttentionPlan:
                 self.wide_variant, self.spans)
 
 
-def _round_up(n: int, buckets=(1, 2, 4, 8, 16, 32, 64), step: int = 64) -> int:
+def _round_up(n: int, buckets=(1, 2, 4, 8, 12, 16, 24, 32, 40, 48, 56, 64), step: int = 16) -> int:
     """``n`` rounded up to one of a few sizes (then to a multiple of ``step``): list sizes of
     graph-replayed steps, so that one graph serves many steps."""
     for b in buckets:
@@ -353,7 +355,7 @@ class Attention(Mixer):
         if plan.part_rows:
             part_acc = ctx.buf(f"attention.part_acc.{d}", (plan.part_rows, d), torch.float32)
             part_ml = ctx.buf("attention.part_ml", (plan.part_rows, 2), torch.float32)
-        if plan.decode_fused and FUSE_DECODE and plan.n_coop * nkv < FUSE_DECODE_BELOW:
+        if plan.decode_fused and FUSE_DECODE and ctx.n_seqs * nkv < FUSE_DECODE_BELOW:
             # single decoded tokens: norm, rotation and cache write happen inside the attention kernel
             k.attention_decode(qkv, nq, nkv, d, key_pages, value_pages, group.page_size, group.table, ctx.seqs,
                                coop_items, plan.n_coop, attn, part_acc, part_ml, self.scale, window,
