@@ -28,6 +28,9 @@ namespace ls {
 #ifndef LS_GEMM_BIG
 #define LS_GEMM_BIG 256       // from this many 128 x 128 tiles on (one for every CU), use them; fewer leave CUs idle and 64 x 64 tiles win
 #endif
+#ifndef LS_GEMM_BIG_ROWS
+#define LS_GEMM_BIG_ROWS 64   // ... and only with more rows than this: up to 64 rows half of a 128-row tile would be idle
+#endif
 #ifndef LS_GEMM_PD_BIG
 #define LS_GEMM_PD_BIG 1      // register prefetch depth (stages) of the 128 x 128 kernel (2: registers run out, a third slower)
 #endif
@@ -999,7 +1002,7 @@ int launch_gemm(const void* X, const void* W, void* C, int M, int N, int K, long
     // (operands that are not 16-byte aligned take the small tiles, element by element: every tile
     // shape gives the same bits)
     if (!aligned) LS_TILED(64, 64, LS_GEMM_PD_SMALL, false)
-    else if (big_tiles >= LS_GEMM_BIG) LS_TILED(128, 128, LS_GEMM_PD_BIG, true)
+    else if (big_tiles >= LS_GEMM_BIG && M > LS_GEMM_BIG_ROWS) LS_TILED(128, 128, LS_GEMM_PD_BIG, true)
     else LS_TILED(64, 64, LS_GEMM_PD_SMALL, true)
 #undef LS_TILED
   }
