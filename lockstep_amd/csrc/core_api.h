@@ -31,6 +31,13 @@ int ls_swiglu(int dtype, const void* gu, void* out, int rows, int inter, long ld
 int ls_bias_act(int out_dtype, const float* x, long ldx, const float* bias, void* out, long ldo, int rows, int width,
                 int act, int gated, void* stream);
 
+// Temperature / nucleus sampling of n rows.  requests: n records of 32 bytes on the device (int row of logits,
+// float temperature > 0, double top_p, unsigned key0, key1 (halves of seed XOR k(uid)), unsigned position low, high:
+// the draw is Philox-4x32-10 of them); token ids to out[i].  scratch: n * vocab * 12 bytes of device memory, 8-byte
+// aligned.
+int ls_sample_top_p(const float* logits, long ld, const void* requests, int* out, void* scratch, int n, int vocab,
+                    void* stream);
+
 // Arg-max of float rows, lowest index among equal maxima.  Rows wider than one chunk leave the
 // chunks' winners in `scratch` (2 * rows * ls_argmax_chunks(width) 4-byte words, device memory
 // the caller brings) for a second small launch.

@@ -36,7 +36,7 @@ FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-shared", "-fPIC",
 ]
-CORE_SOURCES = ("core.hip", "gemm.hip")
+CORE_SOURCES = ("core.hip", "gemm.hip", "sample.hip")
 ATTENTION_SOURCES = ("attention.hip",)
 
 

@@ -79,6 +79,7 @@ class Kernels:
         self._attention: dict[int, ctypes.CDLL] = {}
         self.attention_paths: dict[int, str] = {}
         self._argmax_scratch: dict = {}
+        self._sample_scratch: dict = {}
         self._capabilities: dict = {}
         #: while this is a list, every launch is noted on it as (library, entry point, arguments):
         #: the engine repeats the launches of one layer for the next layers that are alike
@@ -363,6 +364,41 @@ class Kernels:
         self._launch(self.core, self.core.ls_argmax, (
             _ptr(logits), _ptr(out), c_int(logits.shape[0]), c_int(logits.shape[1]), c_long(logits.stride(0)),
             _ptr(scratch), c_long(scratch.numel()), _stream()))
+
+    #: one row's request as ``sample_top_p`` takes it (32 bytes; csrc/sample.hip: SampleRow)
+    SAMPLE_ROW = [("row", "<i4"), ("temperature", "<f4"), ("top_p", "<f8"), ("key0", "<u4"), ("key1", "<u4"),
+                  ("pos_lo", "<u4"), ("pos_hi", "<u4")]
+
+    def sample_top_p(self, logits: torch.Tensor, requests, out: torch.Tensor) -> None:
+        """One token for each request: ``requests`` is a sequence of (row of the float32 ``logits``,
+        temperature > 0, top_p, seed XOR k(uid) as an int of 64 bits, position); ``out`` int32 on the GPU.
+        The host sampler's procedure in float64 (sampling/sampler.py) without its sort, the draw included
+        (Philox-4x32-10 keyed as sampling/philox.py keys it)."""
+        import numpy as np
+
+        _rows_ok(logits, "sample logits")
+        n = len(requests)
+        if not (out.is_cuda and out.dtype == torch.int32 and out.is_contiguous() and out.shape == (n,)):
+            raise KernelError(f"sample out must be int32 [{n}] on the GPU")
+        if not (logits.dtype == torch.float32):
+            raise KernelError("sample reads float32 logits")
+        if n == 0:
+            return
+        packed = np.zeros(n, dtype=self.SAMPLE_ROW)
+        for i, (row, temperature, top_p, mixed, position) in enumerate(requests):
+            if not (0 <= row < logits.shape[0] and temperature > 0):
+                raise KernelError(f"sample: row {row} of {logits.shape[0]} at temperature {temperature}")
+            packed[i] = (row, temperature, top_p, mixed & 0xFFFFFFFF, (mixed >> 32) & 0xFFFFFFFF,
+                         position & 0xFFFFFFFF, (position >> 32) & 0xFFFFFFFF)
+        on_device = torch.from_numpy(packed.view(np.uint8)).to(logits.device)
+        vocab = logits.shape[1]
+        scratch = self._sample_scratch.get(logits.device)
+        if scratch is None or scratch.numel() * 8 < n * vocab * 12:      # weights (8 bytes) and order keys (4) a token
+            scratch = self._sample_scratch[logits.device] = torch.empty((n * vocab * 12 + 7) // 8, dtype=torch.float64,
+                                                                        device=logits.device)
+        self._launch(self.core, self.core.ls_sample_top_p, (
+            _ptr(logits), c_long(logits.stride(0)), _ptr(on_device), _ptr(out), _ptr(scratch), c_int(n), c_int(vocab),
+            _stream()))
 
     def advance_decode(self, meta: torch.Tensor, n_seqs: int, off_tokens: int, picked: torch.Tensor,
                        ring: torch.Tensor, counter: torch.Tensor, off_runs: int, n_runs: int) -> None:

@@ -10,12 +10,14 @@ output word times 2^-32 (reference engine/sampler/philox.py:9-61).
 
 from __future__ import annotations
 
+import functools
 import hashlib
 
 _MASK = 0xFFFFFFFF
 _ROUNDS = 10
 
 
+@functools.lru_cache(maxsize=65536)
 def uid_key(uid: str) -> int:
     return int.from_bytes(hashlib.sha256(uid.encode("utf-8")).digest()[:8], "big")
 

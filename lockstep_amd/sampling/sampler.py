@@ -3,7 +3,10 @@
 ``greedy`` takes the lowest token id among the maxima of the row in float32
 (reference engine/sampler/philox.py:64-68); on the GPU it is one arg-max
 kernel over all rows of the step.  ``top_p`` follows the reference's
-procedure on the host in float64 (engine/sampler/philox.py:71-98):
+procedure in float64 (engine/sampler/philox.py:71-98), here on the host and,
+for logits on the GPU, in a kernel that finds the same token without sorting
+(``Kernels.sample_top_p``; the two can part only where a draw lands within
+rounding of a token's boundary):
 temperature <= 0 is greedy; else softmax of float32(row)/T, tokens ordered by
 (-probability, id), the shortest head whose cumulative sum reaches ``p`` is
 kept, and the draw ``u * sum(head)`` picks the first token whose cumulative
@@ -66,7 +69,18 @@ class Sampler:
             else:
                 for i in greedy_rows:
                     out[i] = greedy(logits[i])
-        for i, r in enumerate(requests):
-            if out[i] is None:
-                out[i] = top_p(logits[i], r.seed, r.uid, r.total_tokens() - 1, r.top_p, r.temperature)
+        drawn = [i for i in range(n) if out[i] is None]
+        if drawn and logits.is_cuda and self.kernels is not None:
+            # the same procedure on the device, the draw included (csrc/sample.hip)
+            picked = torch.empty(len(drawn), dtype=torch.int32, device=logits.device)
+            self.kernels.sample_top_p(
+                logits, [(i, float(requests[i].temperature), float(requests[i].top_p),
+                          int(requests[i].seed) ^ philox.uid_key(requests[i].uid), requests[i].total_tokens() - 1)
+                         for i in drawn], picked)
+            for i, token in zip(drawn, picked.cpu().tolist()):
+                out[i] = int(token)
+            return out  # type: ignore[return-value]
+        for i in drawn:
+            r = requests[i]
+            out[i] = top_p(logits[i], r.seed, r.uid, r.total_tokens() - 1, r.top_p, r.temperature)
         return out  # type: ignore[return-value]

@@ -132,6 +132,56 @@ def test_swiglu_with_few_rows_and_many_columns_has_the_same_bits(dtype, inter, k
         assert torch.equal(part, full[:rows]), f"rows={rows}"
 
 
+@pytest.mark.parametrize("vocab", [7, 1000, 4099, 151936])
+def test_the_sampling_kernel_picks_the_host_samplers_token(vocab):
+    """Temperature and nucleus sampling on the device against the host procedure (float64, sorted): the same
+    token for every row, with spread-out and with quantised logits (many equal values: the order among
+    equals is the order of the ids), small and large nuclei, several temperatures; twice the same."""
+    from lockstep_amd.sampling import philox
+    from lockstep_amd.sampling.sampler import top_p as host_top_p
+
+    n = 48 if vocab < 100000 else 12
+    g = torch.Generator().manual_seed(vocab)
+    logits = torch.randn(n + 3, vocab, generator=g) * (0.5 + 3 * torch.rand(n + 3, 1, generator=g))
+    logits[::5] = torch.round(logits[::5] * 2) / 2
+    logits[1, : vocab // 2] = logits[1, 0]                          # half of the row is one value
+    rows = torch.randperm(n + 3, generator=g)[:n].to(torch.int32)
+    temperature = [[0.3, 0.8, 1.0, 1.7][i % 4] for i in range(n)]
+    nucleus = [[1.0, 0.9, 0.5, 0.05, 0.999, 0.0][i % 6] for i in range(n)]
+    seed = 7 + (1 << 40)                          # both halves of the key in use
+    # the host procedure with the same seed, uid and position (positions beyond 32 bits too)
+    positions = [i if i % 7 else (5 << 32) + i for i in range(n)]
+    want = [host_top_p(logits[int(rows[i])], seed, "kernel", positions[i], nucleus[i], temperature[i]) for i in range(n)]
+    dev = logits.cuda()
+    requests = [(int(rows[i]), temperature[i], nucleus[i], seed ^ philox.uid_key("kernel"), positions[i]) for i in range(n)]
+    out = torch.full((n,), -1, dtype=torch.int32, device="cuda")
+    K().sample_top_p(dev, requests, out)
+    assert out.cpu().tolist() == want
+    again = torch.full((n,), -1, dtype=torch.int32, device="cuda")
+    K().sample_top_p(dev, requests, again)
+    assert torch.equal(out, again)
+    assert len(set(want)) > 1
+
+
+def test_the_sampler_takes_greedy_and_drawn_rows_of_one_step_together():
+    from lockstep_amd.sampling import Sampler
+    from lockstep_amd.sampling.sampler import top_p as host_top_p
+
+    class Row:
+        def __init__(self, uid, seed, temperature, nucleus, total):
+            self.uid, self.seed, self.temperature, self.top_p, self._total = uid, seed, temperature, nucleus, total
+
+        def total_tokens(self):
+            return self._total
+
+    g = torch.Generator().manual_seed(3)
+    logits = torch.randn(6, 5003, generator=g) * 2
+    requests = [Row("a", 1, 0.0, 1.0, 5), Row("b", 2, 0.7, 0.9, 9), Row("c", 3, 0.0, 1.0, 2), Row("d", 4, 1.3, 1.0, 40),
+                Row("e", 5, 0.2, 0.3, 7), Row("f", 6, 1.0, 0.95, 1)]
+    want = [host_top_p(logits[i], r.seed, r.uid, r.total_tokens() - 1, r.top_p, r.temperature) for i, r in enumerate(requests)]
+    assert Sampler(K()).sample(logits.cuda(), requests) == want
+
+
 def test_gemm_refuses_mismatched_operands():
     from lockstep_amd.ops import KernelError
 
