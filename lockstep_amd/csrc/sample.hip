@@ -16,177 +16,38 @@
 // can fall to the neighbour; nothing else differs.  Distinct float values whose weights round to the
 // same double (values below 1e-16 of each other, next to zero) are ordered by value here, by id there.
 //
-// One workgroup of 1,024 threads a row; the weights and the order keys of a row are kept in a scratch
-// buffer the caller brings (12 bytes a token and row).  In a pass a thread adds each of its tokens' weights
-// to the thread's own slot of the token's candidate in LDS (sixteen slots a thread, no two threads share
-// one, so no atomics and a fixed order); the slots of a candidate are then summed over the block.
+// A row is cut into kChunks runs of neighbouring tokens, each with a workgroup of its own, and every step
+// of the walk is a launch of its own: a launch reads the sums the launch before left for every chunk, adds
+// them up in chunk order (every workgroup of the row does the same arithmetic, so they agree without
+// talking to each other), and leaves its own chunk's sums.  The weights and the order keys of a row are
+// kept in a scratch buffer the caller brings.  In a pass a thread adds each of its tokens' weights to the
+// thread's own slot of the token's candidate in LDS (sixteen slots a thread, no two threads share one, so
+// no atomics and a fixed order); the slots of a candidate are then summed over the workgroup.
 
 #include <hip/hip_runtime.h>
 
 #include "common.h"
 #include "core_api.h"
 
+#include <algorithm>
+
+#ifndef LS_SAMPLE_WORKGROUPS
+#define LS_SAMPLE_WORKGROUPS 1024  // workgroups of a launch that the rows of a call are cut for
+#endif
+#ifndef LS_SAMPLE_MIN_CHUNKS
+#define LS_SAMPLE_MIN_CHUNKS 2
+#endif
+
 namespace ls {
 
-constexpr int kSampleThreads = 1024;
+constexpr int kSampleThreads = 256;
 constexpr int kSampleWaves = kSampleThreads / 64;
-constexpr int kBatch = 8;  // loads a thread has in flight in the passes over a row
+constexpr int kChunks = 32;  // the most workgroups a row (few rows); many rows take fewer each
+constexpr int kBatch = 8;    // loads a thread has in flight in the passes over its chunk
 
 __device__ __forceinline__ unsigned int order_key(float f) {  // ascending in f; -0 counts as +0
   const unsigned int b = __float_as_uint(f + 0.0f);
   return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
-}
-
-// The same total in every thread: butterfly over the wave, then the waves' sums in wave order.
-__device__ __forceinline__ double block_sum(double v, double* __restrict__ wave_sums) {
-#pragma unroll
-  for (int off = 32; off >= 1; off >>= 1) v = v + __shfl_xor(v, off);
-  __syncthreads();  // wave_sums may still be read from the call before
-  if ((threadIdx.x & 63) == 0) wave_sums[threadIdx.x >> 6] = v;
-  __syncthreads();
-  double total = 0.0;
-#pragma unroll
-  for (int w = 0; w < kSampleWaves; ++w) total = total + wave_sums[w];
-  return total;
-}
-
-struct Found {
-  int token;       // the first token, in the order of the sort, whose cumulative weight reaches the target
-  double reached;  // that cumulative weight
-};
-
-// `slots`: 16 * kSampleThreads doubles (candidate b of thread t at slots[b * kSampleThreads + t]: a wave's lanes
-// fall on different banks whatever their candidates are); `shared_d`: 16 * kSampleWaves doubles; `shared_i`:
-// kSampleThreads + 8 ints.
-__device__ Found first_reaching(const unsigned int* __restrict__ keys, const double* __restrict__ weights, int vocab,
-                                double target, double* __restrict__ slots, double* __restrict__ shared_d,
-                                int* __restrict__ shared_i) {
-  const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
-  unsigned int prefix = 0;   // the bits of the key that are known, in their place
-  double above = 0.0;        // weights of the keys that are larger than every key with this prefix
-  for (int shift = 28; shift >= 0; shift -= 4) {
-#pragma unroll
-    for (int b = 0; b < 16; ++b) slots[b * kSampleThreads + threadIdx.x] = 0.0;
-    const unsigned int known = shift == 28 ? 0u : (0xffffffffu << (shift + 4));
-    // eight tokens' loads at a time, unconditional, so that they are in flight together; the additions
-    // keep the order of the ids
-    for (int i0 = threadIdx.x; i0 < vocab; i0 += kBatch * kSampleThreads) {
-      unsigned int key[kBatch];
-      double w[kBatch];
-#pragma unroll
-      for (int u = 0; u < kBatch; ++u) {
-        const int i = min(i0 + u * kSampleThreads, vocab - 1);
-        key[u] = keys[i];
-        w[u] = weights[i];
-      }
-#pragma unroll
-      for (int u = 0; u < kBatch; ++u) {
-        if (i0 + u * kSampleThreads >= vocab || (key[u] & known) != prefix) continue;
-        double* slot = &slots[((key[u] >> shift) & 15) * kSampleThreads + threadIdx.x];
-        *slot = *slot + w[u];
-      }
-    }
-    double sums[16];
-#pragma unroll
-    for (int b = 0; b < 16; ++b) {
-      sums[b] = slots[b * kSampleThreads + threadIdx.x];
-#pragma unroll
-      for (int off = 32; off >= 1; off >>= 1) sums[b] = sums[b] + __shfl_xor(sums[b], off);
-    }
-    __syncthreads();  // shared_d may still be read from the level before
-    if (lane == 0) {
-#pragma unroll
-      for (int b = 0; b < 16; ++b) shared_d[wave * 16 + b] = sums[b];
-    }
-    __syncthreads();
-    // every thread walks the sixteen sums from the top (the same arithmetic in all of them)
-    int chosen = -1, lowest = 0;
-    double passed = above;
-    for (int b = 15; b >= 0; --b) {
-      double s = 0.0;
-#pragma unroll
-      for (int w = 0; w < kSampleWaves; ++w) s = s + shared_d[w * 16 + b];
-      if (!(s > 0.0)) continue;
-      lowest = b;
-      if (passed + s >= target) {
-        chosen = b;
-        break;
-      }
-      passed = passed + s;
-    }
-    if (chosen < 0) {
-      // rounding left the target just above the last sum: the end of the range is meant.  `passed` counts
-      // the lowest candidate in; take it out again by walking once more (the same in every thread).
-      chosen = lowest;
-      passed = above;
-      for (int b = 15; b > lowest; --b) {
-        double s = 0.0;
-#pragma unroll
-        for (int w = 0; w < kSampleWaves; ++w) s = s + shared_d[w * 16 + b];
-        if (s > 0.0) passed = passed + s;
-      }
-    }
-    above = passed;
-    prefix |= (unsigned int)chosen << shift;
-  }
-  // Tokens whose key is `prefix` share one weight; count them off in the order of their ids.  A thread
-  // takes a run of neighbouring ids.
-  const int per = (vocab + kSampleThreads - 1) / kSampleThreads;
-  const int begin = min(vocab, (int)threadIdx.x * per), end = min(vocab, begin + per);
-  int mine = 0, last_tie = -1;
-  for (int i0 = begin; i0 < end; i0 += kBatch) {
-    unsigned int key[kBatch];
-#pragma unroll
-    for (int u = 0; u < kBatch; ++u) key[u] = keys[min(i0 + u, vocab - 1)];
-#pragma unroll
-    for (int u = 0; u < kBatch; ++u)
-      if (i0 + u < end && key[u] == prefix) {
-        ++mine;
-        last_tie = i0 + u;
-      }
-  }
-  double tie_weight = last_tie >= 0 ? weights[last_tie] : 0.0;
-  __syncthreads();
-  shared_i[threadIdx.x] = mine;
-  // any tie's weight (they are equal): the largest over the block, zero where a thread has none
-#pragma unroll
-  for (int off = 32; off >= 1; off >>= 1) tie_weight = fmax(tie_weight, __shfl_xor(tie_weight, off));
-  if (lane == 0) shared_d[wave] = tie_weight;
-  __syncthreads();
-  double w_tie = 0.0;
-#pragma unroll
-  for (int w = 0; w < kSampleWaves; ++w) w_tie = fmax(w_tie, shared_d[w]);
-  int before = 0, ties = 0;
-  for (int t = 0; t < kSampleThreads; ++t) {
-    const int c = shared_i[t];
-    if (t < (int)threadIdx.x) before += c;
-    ties += c;
-  }
-  // the m-th tie is the first whose cumulative weight above + m * w reaches the target
-  int m = 1;
-  if (w_tie > 0.0 && target > above + w_tie) {
-    const double need = ceil((target - above) / w_tie);
-    m = need >= (double)ties ? ties : (int)need;
-    if (m < 1) m = 1;
-  }
-  if (m > ties) m = ties;
-  __syncthreads();
-  if (mine > 0 && before < m && m <= before + mine) {
-    int seen = before;
-    for (int i = begin; i < end; ++i)
-      if (keys[i] == prefix && ++seen == m) {
-        shared_i[kSampleThreads] = i;
-        break;
-      }
-  }
-  if (ties == 0 && threadIdx.x == 0) shared_i[kSampleThreads] = 0;  // an empty row cannot happen; stay in range
-  __syncthreads();
-  Found found;
-  found.token = shared_i[kSampleThreads];
-  found.reached = above + (double)m * w_tie;
-  __syncthreads();
-  return found;
 }
 
 // One row's request: which row of the logits, its temperature and nucleus, and the key and counter of
@@ -197,6 +58,34 @@ struct SampleRow {
   double top_p;
   unsigned int key0, key1;   // the two halves of seed XOR k(uid)
   unsigned int pos_lo, pos_hi;
+};
+
+// Where a walk stands: the bits of the key that are known (in their place), the weights of all keys above
+// every key with these bits, and what the walk looks for.
+struct SearchState {
+  double target, above;
+  unsigned int prefix;
+  int pad;
+};
+
+struct Found {
+  double reached;  // the cumulative weight of the token that was found
+  int token;
+  int pad;
+};
+
+// What the launches of one call leave for each other, per row (and per chunk where it says so).
+struct SampleScratch {
+  int chunks;             // workgroups a row in this call (at most kChunks)
+  double* weights;        // [n][vocab]
+  unsigned int* keys;     // [n][vocab]
+  float* part_max;        // [n][kChunks]
+  double* part_sum;       // [n][kChunks]
+  double* part_level;     // [2][n][kChunks][16]: the candidates' sums of a chunk, by the parity of the level
+  SearchState* state;     // [2 walks][2 parities][n]
+  int* tie_count;         // [n][kChunks]
+  double* tie_weight;     // [n][kChunks]
+  Found* found;           // [2 walks][n]
 };
 
 // Philox-4x32 with ten rounds; the draw is the first output word times 2^-32 (reference
@@ -220,90 +109,361 @@ __device__ __forceinline__ double philox_uniform(unsigned int k0, unsigned int k
   return (double)c0 * 2.3283064365386963e-10;  // 2^-32, exact
 }
 
-__global__ __launch_bounds__(kSampleThreads) void sample_top_p_kernel(
-    const float* __restrict__ logits, long ld, const SampleRow* __restrict__ requests, int* __restrict__ out,
-    double* __restrict__ scratch_weights, unsigned int* __restrict__ scratch_keys, int vocab) {
-  extern __shared__ __attribute__((aligned(16))) double slots[];  // [16][kSampleThreads]
-  __shared__ double shared_d[16 * kSampleWaves];
-  __shared__ int shared_i[kSampleThreads + 8];
+// The same total in every thread: butterfly over the wave, then the waves' sums in wave order.
+__device__ __forceinline__ double block_sum(double v, double* __restrict__ wave_sums) {
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) v = v + __shfl_xor(v, off);
+  __syncthreads();  // wave_sums may still be read from the call before
+  if ((threadIdx.x & 63) == 0) wave_sums[threadIdx.x >> 6] = v;
+  __syncthreads();
+  double total = 0.0;
+#pragma unroll
+  for (int w = 0; w < kSampleWaves; ++w) total = total + wave_sums[w];
+  return total;
+}
+
+// grid (kChunks, n): the largest float(logit) / T of a chunk
+__global__ __launch_bounds__(kSampleThreads) void sample_max_kernel(const float* __restrict__ logits, long ld,
+                                                                    const SampleRow* __restrict__ requests,
+                                                                    SampleScratch sc, int vocab, int chunk_len) {
   __shared__ float wave_max[kSampleWaves];
-  const int r = blockIdx.x;
+  const int r = blockIdx.y, c = blockIdx.x;
   const SampleRow request = requests[r];
   const float* row = logits + (long)request.row * ld;
-  const float t = request.temperature;
-  double* weights = scratch_weights + (long)r * vocab;
-  unsigned int* keys = scratch_keys + (long)r * vocab;
-
+  const int begin = min(vocab, c * chunk_len), end = min(vocab, begin + chunk_len);
   float top = -INFINITY;
-  for (int i0 = threadIdx.x; i0 < vocab; i0 += kBatch * kSampleThreads) {
+  for (int i0 = begin + threadIdx.x; i0 < end; i0 += kBatch * kSampleThreads) {
     float x[kBatch];
 #pragma unroll
-    for (int u = 0; u < kBatch; ++u) x[u] = row[min(i0 + u * kSampleThreads, vocab - 1)];  // (a repeated token changes no maximum)
+    for (int u = 0; u < kBatch; ++u) x[u] = row[min(i0 + u * kSampleThreads, end - 1)];  // (a repeated token changes no maximum)
 #pragma unroll
-    for (int u = 0; u < kBatch; ++u) top = fmaxf(top, x[u] / t);
+    for (int u = 0; u < kBatch; ++u) top = fmaxf(top, x[u] / request.temperature);
   }
 #pragma unroll
   for (int off = 32; off >= 1; off >>= 1) top = fmaxf(top, __shfl_xor(top, off));
   if ((threadIdx.x & 63) == 0) wave_max[threadIdx.x >> 6] = top;
   __syncthreads();
+  if (threadIdx.x == 0) {
 #pragma unroll
-  for (int w = 0; w < kSampleWaves; ++w) top = fmaxf(top, wave_max[w]);
-  const double v_max = (double)top;
+    for (int w = 0; w < kSampleWaves; ++w) top = fmaxf(top, wave_max[w]);
+    sc.part_max[r * sc.chunks + c] = top;
+  }
+}
 
+// grid (kChunks, n): weights and order keys of a chunk, and the sum of its weights
+__global__ __launch_bounds__(kSampleThreads) void sample_exp_kernel(const float* __restrict__ logits, long ld,
+                                                                    const SampleRow* __restrict__ requests,
+                                                                    SampleScratch sc, int vocab, int chunk_len) {
+  __shared__ double wave_sums[kSampleWaves];
+  const int r = blockIdx.y, c = blockIdx.x;
+  const SampleRow request = requests[r];
+  const float* row = logits + (long)request.row * ld;
+  double* weights = sc.weights + (long)r * vocab;
+  unsigned int* keys = sc.keys + (long)r * vocab;
+  float top = -INFINITY;
+  for (int k = 0; k < sc.chunks; ++k) top = fmaxf(top, sc.part_max[r * sc.chunks + k]);
+  const double v_max = (double)top;
+  const int begin = min(vocab, c * chunk_len), end = min(vocab, begin + chunk_len);
   double part = 0.0;
-  for (int i0 = threadIdx.x; i0 < vocab; i0 += kBatch * kSampleThreads) {
+  for (int i0 = begin + threadIdx.x; i0 < end; i0 += kBatch * kSampleThreads) {
     float x[kBatch];
 #pragma unroll
-    for (int u = 0; u < kBatch; ++u) x[u] = row[min(i0 + u * kSampleThreads, vocab - 1)];
+    for (int u = 0; u < kBatch; ++u) x[u] = row[min(i0 + u * kSampleThreads, end - 1)];
 #pragma unroll
     for (int u = 0; u < kBatch; ++u) {
       const int i = i0 + u * kSampleThreads;
-      if (i >= vocab) continue;
-      const float f = x[u] / t;
+      if (i >= end) continue;
+      const float f = x[u] / request.temperature;
       const double w = exp((double)f - v_max);
       weights[i] = w;
       keys[i] = order_key(f);
       part = part + w;
     }
   }
-  const double total = block_sum(part, shared_d);  // (its barriers also publish weights and keys to the block)
+  const double total = block_sum(part, wave_sums);
+  if (threadIdx.x == 0) sc.part_sum[r * sc.chunks + c] = total;
+}
 
-  double head = total;
-  const double p = request.top_p;
-  if (p < 1.0) head = first_reaching(keys, weights, vocab, p * total, slots, shared_d, shared_i).reached;
-  // the draw in the word of the counter that the third counter word 0 names (index 0 of the host's uniform())
-  const double u = philox_uniform(request.key0, request.key1, request.pos_lo, request.pos_hi);
-  const Found pick = first_reaching(keys, weights, vocab, u * head, slots, shared_d, shared_i);
-  if (threadIdx.x == 0) out[r] = pick.token;
+// The state of walk `walk` of row r after level `level - 1`, from the state after level `level - 2` (which
+// the launch before left, or the start of the walk) and the sums of level `level - 1`.  Every thread of
+// every workgroup of the row computes it with the same arithmetic.
+// `staged`: kChunks * 16 doubles of LDS; all threads of the workgroup call this together.
+__device__ SearchState state_before_level(const SampleScratch& sc, const SampleRow& request, int n, int r, int walk,
+                                          int level, double* __restrict__ staged) {
+  SearchState st;
+  if (level == 0) {
+    double total = 0.0;
+    for (int k = 0; k < sc.chunks; ++k) total = total + sc.part_sum[r * sc.chunks + k];
+    if (walk == 0) {
+      st.target = request.top_p * total;  // the nucleus: the shortest head that reaches top_p
+    } else {
+      const double head = request.top_p < 1.0 ? sc.found[0 * n + r].reached : total;
+      st.target = philox_uniform(request.key0, request.key1, request.pos_lo, request.pos_hi) * head;
+    }
+    st.above = 0.0;
+    st.prefix = 0u;
+    st.pad = 0;
+    return st;
+  }
+  st = sc.state[(walk * 2 + (level & 1)) * n + r];  // after level - 2 (parity of level - 2 = parity of level)
+  const int shift = 28 - 4 * (level - 1);
+  // the chunks' sums of level - 1 into LDS with one round of loads, then every thread walks them
+  const double* from = sc.part_level + ((long)((level - 1) & 1) * n + r) * sc.chunks * 16;
+  for (int i = threadIdx.x; i < sc.chunks * 16; i += kSampleThreads) staged[i] = from[i];
+  __syncthreads();
+  const double* sums = staged;
+  int chosen = -1, lowest = 0;
+  double passed = st.above;
+  for (int b = 15; b >= 0; --b) {
+    double s = 0.0;
+    for (int k = 0; k < sc.chunks; ++k) s = s + sums[k * 16 + b];
+    if (!(s > 0.0)) continue;
+    lowest = b;
+    if (passed + s >= st.target) {
+      chosen = b;
+      break;
+    }
+    passed = passed + s;
+  }
+  if (chosen < 0) {
+    // rounding left the target just above the last sum: the end of the range is meant.  `passed` counts
+    // the lowest candidate in; take it out again by walking once more.
+    chosen = lowest;
+    passed = st.above;
+    for (int b = 15; b > lowest; --b) {
+      double s = 0.0;
+      for (int k = 0; k < sc.chunks; ++k) s = s + sums[k * 16 + b];
+      if (s > 0.0) passed = passed + s;
+    }
+  }
+  st.above = passed;
+  st.prefix |= (unsigned int)chosen << shift;
+  return st;
+}
+
+// grid (kChunks, n), levels 0 to 7: the sums of a chunk's weights for the sixteen candidates of this level's
+// four bits, among the tokens whose known bits fit.
+__global__ __launch_bounds__(kSampleThreads) void sample_level_kernel(const SampleRow* __restrict__ requests,
+                                                                      SampleScratch sc, int n, int vocab, int chunk_len,
+                                                                      int walk, int level) {
+  __shared__ double slots[16 * kSampleThreads];  // candidate b of thread t at slots[b * kSampleThreads + t]
+  __shared__ double wave_sums[kSampleWaves * 16];
+  const int r = blockIdx.y, c = blockIdx.x;
+  const SampleRow request = requests[r];
+  if (walk == 0 && !(request.top_p < 1.0)) return;  // the whole row is the head
+  __shared__ double staged[kChunks * 16];
+  const SearchState st = state_before_level(sc, request, n, r, walk, level, staged);
+  if (c == 0 && threadIdx.x == 0) sc.state[(walk * 2 + ((level + 1) & 1)) * n + r] = st;  // parity of level - 1
+  const unsigned int* keys = sc.keys + (long)r * vocab;
+  const double* weights = sc.weights + (long)r * vocab;
+  const int shift = 28 - 4 * level;
+  const unsigned int known = level == 0 ? 0u : (0xffffffffu << (shift + 4));
+#pragma unroll
+  for (int b = 0; b < 16; ++b) slots[b * kSampleThreads + threadIdx.x] = 0.0;
+  const int begin = min(vocab, c * chunk_len), end = min(vocab, begin + chunk_len);
+  // eight tokens' keys at a time, unconditional, so that the loads are in flight together; then the weights
+  // of those whose known bits fit (from the second level on these are few, and the others' weights are
+  // never fetched); the additions keep the order of the ids
+  for (int i0 = begin + threadIdx.x; i0 < end; i0 += kBatch * kSampleThreads) {
+    unsigned int key[kBatch];
+    double w[kBatch];
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) key[u] = keys[min(i0 + u * kSampleThreads, end - 1)];
+    bool fits[kBatch];
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) fits[u] = i0 + u * kSampleThreads < end && (key[u] & known) == st.prefix;
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) w[u] = fits[u] ? weights[i0 + u * kSampleThreads] : 0.0;
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) {
+      if (!fits[u]) continue;
+      double* slot = &slots[((key[u] >> shift) & 15) * kSampleThreads + threadIdx.x];
+      *slot = *slot + w[u];
+    }
+  }
+  double sums[16];
+#pragma unroll
+  for (int b = 0; b < 16; ++b) {
+    sums[b] = slots[b * kSampleThreads + threadIdx.x];
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) sums[b] = sums[b] + __shfl_xor(sums[b], off);
+  }
+  if ((threadIdx.x & 63) == 0) {
+#pragma unroll
+    for (int b = 0; b < 16; ++b) wave_sums[(threadIdx.x >> 6) * 16 + b] = sums[b];
+  }
+  __syncthreads();
+  if (threadIdx.x < 16) {
+    double s = 0.0;
+#pragma unroll
+    for (int w = 0; w < kSampleWaves; ++w) s = s + wave_sums[w * 16 + threadIdx.x];
+    sc.part_level[(((long)(level & 1) * n + r) * sc.chunks + c) * 16 + threadIdx.x] = s;
+  }
+}
+
+// grid (kChunks, n), after level 7: the key is known; how many tokens of the chunk have it, and their weight
+__global__ __launch_bounds__(kSampleThreads) void sample_tie_count_kernel(const SampleRow* __restrict__ requests,
+                                                                          SampleScratch sc, int n, int vocab,
+                                                                          int chunk_len, int walk) {
+  __shared__ int wave_count[kSampleWaves];
+  __shared__ double wave_weight[kSampleWaves];
+  const int r = blockIdx.y, c = blockIdx.x;
+  const SampleRow request = requests[r];
+  if (walk == 0 && !(request.top_p < 1.0)) return;
+  __shared__ double staged[kChunks * 16];
+  const SearchState st = state_before_level(sc, request, n, r, walk, 8, staged);
+  if (c == 0 && threadIdx.x == 0) sc.state[(walk * 2 + 1) * n + r] = st;  // after level 7
+  const unsigned int* keys = sc.keys + (long)r * vocab;
+  const double* weights = sc.weights + (long)r * vocab;
+  const int begin = min(vocab, c * chunk_len), end = min(vocab, begin + chunk_len);
+  int mine = 0, last_tie = -1;
+  for (int i0 = begin + threadIdx.x; i0 < end; i0 += kBatch * kSampleThreads) {
+    unsigned int key[kBatch];
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) key[u] = keys[min(i0 + u * kSampleThreads, end - 1)];
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u)
+      if (i0 + u * kSampleThreads < end && key[u] == st.prefix) {
+        ++mine;
+        last_tie = i0 + u * kSampleThreads;
+      }
+  }
+  double weight = last_tie >= 0 ? weights[last_tie] : 0.0;  // they are equal: any of them
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) {
+    mine += __shfl_xor(mine, off);
+    weight = fmax(weight, __shfl_xor(weight, off));
+  }
+  if ((threadIdx.x & 63) == 0) {
+    wave_count[threadIdx.x >> 6] = mine;
+    wave_weight[threadIdx.x >> 6] = weight;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int count = 0;
+    double w = 0.0;
+#pragma unroll
+    for (int k = 0; k < kSampleWaves; ++k) {
+      count += wave_count[k];
+      w = fmax(w, wave_weight[k]);
+    }
+    sc.tie_count[r * sc.chunks + c] = count;
+    sc.tie_weight[r * sc.chunks + c] = w;
+  }
+}
+
+// grid (kChunks, n): tokens that share the key are counted off in the order of their ids; the chunk that
+// holds the one that is meant finds it.
+__global__ __launch_bounds__(kSampleThreads) void sample_tie_pick_kernel(const SampleRow* __restrict__ requests,
+                                                                         SampleScratch sc, int n, int vocab,
+                                                                         int chunk_len, int walk, int* __restrict__ out) {
+  __shared__ int counts[kSampleThreads];
+  __shared__ int picked;
+  const int r = blockIdx.y, c = blockIdx.x;
+  const SampleRow request = requests[r];
+  if (walk == 0 && !(request.top_p < 1.0)) return;
+  const SearchState st = sc.state[(walk * 2 + 1) * n + r];
+  int before = 0, ties = 0;
+  double w_tie = 0.0;
+  for (int k = 0; k < sc.chunks; ++k) {
+    const int count = sc.tie_count[r * sc.chunks + k];
+    if (k < c) before += count;
+    ties += count;
+    w_tie = fmax(w_tie, sc.tie_weight[r * sc.chunks + k]);
+  }
+  // the m-th tie is the first whose cumulative weight above + m * w reaches the target
+  int m = 1;
+  if (w_tie > 0.0 && st.target > st.above + w_tie) {
+    const double need = ceil((st.target - st.above) / w_tie);
+    m = need >= (double)ties ? ties : (int)need;
+    if (m < 1) m = 1;
+  }
+  if (m > ties) m = ties;
+  const int mine_total = sc.tie_count[r * sc.chunks + c];
+  if (!(before < m && m <= before + mine_total)) return;  // another chunk holds it (uniform for the workgroup)
+  // a thread takes a run of neighbouring ids of the chunk
+  const unsigned int* keys = sc.keys + (long)r * vocab;
+  const int begin = min(vocab, c * chunk_len), end = min(vocab, begin + chunk_len);
+  const int per = (chunk_len + kSampleThreads - 1) / kSampleThreads;
+  const int lo = min(end, begin + (int)threadIdx.x * per), hi = min(end, lo + per);
+  int mine = 0;
+  for (int i = lo; i < hi; ++i) mine += keys[i] == st.prefix ? 1 : 0;
+  counts[threadIdx.x] = mine;
+  __syncthreads();
+  int ahead = before;
+  for (int t = 0; t < (int)threadIdx.x; ++t) ahead += counts[t];
+  if (mine > 0 && ahead < m && m <= ahead + mine) {
+    int seen = ahead;
+    for (int i = lo; i < hi; ++i)
+      if (keys[i] == st.prefix && ++seen == m) {
+        picked = i;
+        break;
+      }
+    Found found;
+    found.reached = st.above + (double)m * w_tie;
+    found.token = picked;
+    found.pad = 0;
+    sc.found[walk * n + r] = found;
+    if (walk == 1) out[r] = picked;
+  }
 }
 
 }  // namespace ls
 
+static size_t align_up(size_t bytes) { return (bytes + 255) / 256 * 256; }
+
+// Bytes of scratch that ls_sample_top_p needs for n rows of a vocabulary.
+extern "C" long ls_sample_scratch_bytes(int n, int vocab) {
+  using namespace ls;
+  if (n <= 0 || vocab <= 0) return 0;
+  size_t total = align_up((size_t)n * vocab * sizeof(double)) + align_up((size_t)n * vocab * sizeof(unsigned int));
+  total += align_up((size_t)n * kChunks * sizeof(float)) + align_up((size_t)n * kChunks * sizeof(double));
+  total += align_up((size_t)2 * n * kChunks * 16 * sizeof(double)) + align_up((size_t)4 * n * sizeof(SearchState));
+  total += align_up((size_t)n * kChunks * sizeof(int)) + align_up((size_t)n * kChunks * sizeof(double));
+  total += align_up((size_t)2 * n * sizeof(Found));
+  return (long)total;
+}
+
 // Sample one token for each of `n` rows.  `requests`: n records of 32 bytes on the device (int row of `logits`,
 // float temperature > 0, double top_p, then four unsigned words: the two halves of seed XOR k(uid) and the two
-// halves of the position); token ids to out[i].  `logits`: float [.][ld], `vocab` columns.  `scratch`: n * vocab * 12
-// bytes, 8-byte aligned (the rows' weights as doubles, then their order keys).
-extern "C" int ls_sample_top_p(const float* logits, long ld, const void* requests, int* out, void* scratch, int n,
-                               int vocab, void* stream) {
+// halves of the position); token ids to out[i].  `logits`: float [.][ld], `vocab` columns.  `scratch`:
+// ls_sample_scratch_bytes(n, vocab) bytes, 256-byte aligned.  `any_nucleus`: 0 if every top_p is >= 1 (the
+// launches that look for the nucleus are then left out).
+extern "C" int ls_sample_top_p(const float* logits, long ld, const void* requests, int* out, void* scratch,
+                               long scratch_bytes, int n, int vocab, int any_nucleus, void* stream) {
   using namespace ls;
   static_assert(sizeof(SampleRow) == 32, "the host packs 32 bytes a row");
   LS_REQUIRE(n > 0 && vocab > 0 && ld >= vocab, "sample: bad sizes (n=%d vocab=%d ld=%ld)", n, vocab, ld);
   LS_REQUIRE(logits && requests && out && scratch, "sample: null operand");
-  LS_REQUIRE(reinterpret_cast<uintptr_t>(scratch) % 8 == 0 && reinterpret_cast<uintptr_t>(requests) % 8 == 0,
-             "sample: the scratch buffer and the requests must be 8-byte aligned");
-  constexpr size_t lds = (size_t)16 * kSampleThreads * sizeof(double);  // 128 KB: granted per kernel, once
-  static int granted = 0;                                              // 0 unknown, 1 yes, -1 no
-  if (granted == 0) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&sample_top_p_kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) (void)hipGetLastError();
-    granted = e == hipSuccess ? 1 : -1;
-  }
-  if (granted != 1) return fail("sample: the device does not grant %zu bytes of LDS to a workgroup", lds);
+  LS_REQUIRE(reinterpret_cast<uintptr_t>(scratch) % 256 == 0 && reinterpret_cast<uintptr_t>(requests) % 8 == 0,
+             "sample: the scratch buffer must be 256-byte aligned, the requests 8-byte aligned");
+  LS_REQUIRE(scratch_bytes >= ls_sample_scratch_bytes(n, vocab), "sample: %ld bytes of scratch, %ld are needed",
+             scratch_bytes, ls_sample_scratch_bytes(n, vocab));
+  SampleScratch sc;
+  char* at = reinterpret_cast<char*>(scratch);
+  auto take = [&](size_t bytes) { char* here = at; at += align_up(bytes); return here; };
+  sc.weights = reinterpret_cast<double*>(take((size_t)n * vocab * sizeof(double)));
+  sc.keys = reinterpret_cast<unsigned int*>(take((size_t)n * vocab * sizeof(unsigned int)));
+  sc.part_max = reinterpret_cast<float*>(take((size_t)n * kChunks * sizeof(float)));
+  sc.part_sum = reinterpret_cast<double*>(take((size_t)n * kChunks * sizeof(double)));
+  sc.part_level = reinterpret_cast<double*>(take((size_t)2 * n * kChunks * 16 * sizeof(double)));
+  sc.state = reinterpret_cast<SearchState*>(take((size_t)4 * n * sizeof(SearchState)));
+  sc.tie_count = reinterpret_cast<int*>(take((size_t)n * kChunks * sizeof(int)));
+  sc.tie_weight = reinterpret_cast<double*>(take((size_t)n * kChunks * sizeof(double)));
+  sc.found = reinterpret_cast<Found*>(take((size_t)2 * n * sizeof(Found)));
+  const SampleRow* rows = reinterpret_cast<const SampleRow*>(requests);
+  // few rows are cut into many chunks (a row alone would keep one CU busy); many rows fill the GPU with fewer
+  sc.chunks = std::max(LS_SAMPLE_MIN_CHUNKS, std::min(kChunks, LS_SAMPLE_WORKGROUPS / n));
+  const int chunk_len = (vocab + sc.chunks - 1) / sc.chunks;
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-  double* weights = reinterpret_cast<double*>(scratch);
-  unsigned int* keys = reinterpret_cast<unsigned int*>(weights + (size_t)n * vocab);
-  hipLaunchKernelGGL(sample_top_p_kernel, dim3(n), dim3(kSampleThreads), lds, s, logits, ld,
-                     reinterpret_cast<const SampleRow*>(requests), out, weights, keys, vocab);
+  const dim3 grid(sc.chunks, n), block(kSampleThreads);
+  hipLaunchKernelGGL(sample_max_kernel, grid, block, 0, s, logits, ld, rows, sc, vocab, chunk_len);
+  hipLaunchKernelGGL(sample_exp_kernel, grid, block, 0, s, logits, ld, rows, sc, vocab, chunk_len);
+  for (int walk = any_nucleus ? 0 : 1; walk < 2; ++walk) {
+    for (int level = 0; level < 8; ++level)
+      hipLaunchKernelGGL(sample_level_kernel, grid, block, 0, s, rows, sc, n, vocab, chunk_len, walk, level);
+    hipLaunchKernelGGL(sample_tie_count_kernel, grid, block, 0, s, rows, sc, n, vocab, chunk_len, walk);
+    hipLaunchKernelGGL(sample_tie_pick_kernel, grid, block, 0, s, rows, sc, n, vocab, chunk_len, walk, out);
+  }
   return check_launch("sample");
 }

@@ -76,6 +76,7 @@ class Kernels:
         self.core_path = _build.build_core_mutants() if mutants else _build.build_core()
         self.core = ctypes.CDLL(str(self.core_path))
         self.core.ls_last_error.restype = ctypes.c_char_p
+        self.core.ls_sample_scratch_bytes.restype = ctypes.c_long
         self._attention: dict[int, ctypes.CDLL] = {}
         self.attention_paths: dict[int, str] = {}
         self._argmax_scratch: dict = {}
@@ -392,13 +393,14 @@ class Kernels:
                          position & 0xFFFFFFFF, (position >> 32) & 0xFFFFFFFF)
         on_device = torch.from_numpy(packed.view(np.uint8)).to(logits.device)
         vocab = logits.shape[1]
+        need = int(self.core.ls_sample_scratch_bytes(c_int(n), c_int(vocab)))
         scratch = self._sample_scratch.get(logits.device)
-        if scratch is None or scratch.numel() * 8 < n * vocab * 12:      # weights (8 bytes) and order keys (4) a token
-            scratch = self._sample_scratch[logits.device] = torch.empty((n * vocab * 12 + 7) // 8, dtype=torch.float64,
-                                                                        device=logits.device)
+        if scratch is None or scratch.numel() < need:
+            scratch = self._sample_scratch[logits.device] = torch.empty(need, dtype=torch.uint8, device=logits.device)
+        any_nucleus = any(top_p < 1.0 for _, _, top_p, _, _ in requests)
         self._launch(self.core, self.core.ls_sample_top_p, (
-            _ptr(logits), c_long(logits.stride(0)), _ptr(on_device), _ptr(out), _ptr(scratch), c_int(n), c_int(vocab),
-            _stream()))
+            _ptr(logits), c_long(logits.stride(0)), _ptr(on_device), _ptr(out), _ptr(scratch), c_long(scratch.numel()),
+            c_int(n), c_int(vocab), c_int(1 if any_nucleus else 0), _stream()))
 
     def advance_decode(self, meta: torch.Tensor, n_seqs: int, off_tokens: int, picked: torch.Tensor,
                        ring: torch.Tensor, counter: torch.Tensor, off_runs: int, n_runs: int) -> None:
