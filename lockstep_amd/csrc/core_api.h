@@ -34,10 +34,11 @@ int ls_bias_act(int out_dtype, const float* x, long ldx, const float* bias, void
 // Temperature / nucleus sampling of n rows.  requests: n records of 32 bytes on the device (int row of logits,
 // float temperature > 0, double top_p, unsigned key0, key1 (halves of seed XOR k(uid)), unsigned position low, high:
 // the draw is Philox-4x32-10 of them); token ids to out[i].  scratch: ls_sample_scratch_bytes(n, vocab) bytes of
-// device memory, 256-byte aligned.  any_nucleus: 0 if every top_p is >= 1.
+// device memory, 256-byte aligned.  any_nucleus: 0 if every top_p is >= 1.  scatter: token ids go to out[row of the
+// record] instead of out[i].
 long ls_sample_scratch_bytes(int n, int vocab);
 int ls_sample_top_p(const float* logits, long ld, const void* requests, int* out, void* scratch, long scratch_bytes,
-                    int n, int vocab, int any_nucleus, void* stream);
+                    int n, int vocab, int any_nucleus, int scatter, void* stream);
 
 // Arg-max of float rows, lowest index among equal maxima.  Rows wider than one chunk leave the
 // chunks' winners in `scratch` (2 * rows * ls_argmax_chunks(width) 4-byte words, device memory

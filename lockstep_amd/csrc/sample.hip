@@ -55,9 +55,10 @@ __device__ __forceinline__ unsigned int order_key(float f) {  // ascending in f;
 struct SampleRow {
   int row;
   float temperature;
-  double top_p;
-  unsigned int key0, key1;   // the two halves of seed XOR k(uid)
-  unsigned int pos_lo, pos_hi;
+  unsigned int top_p_lo, top_p_hi;  // the double, in two words: records may lie at any multiple of four bytes
+  unsigned int key0, key1;          // the two halves of seed XOR k(uid)
+  unsigned int pos_lo, pos_hi;      // (pos_lo moves on by one a token where steps run without the host)
+  __device__ __forceinline__ double top_p() const { return __hiloint2double((int)top_p_hi, (int)top_p_lo); }
 };
 
 // Where a walk stands: the bits of the key that are known (in their place), the weights of all keys above
@@ -195,9 +196,9 @@ __device__ SearchState state_before_level(const SampleScratch& sc, const SampleR
     double total = 0.0;
     for (int k = 0; k < sc.chunks; ++k) total = total + sc.part_sum[r * sc.chunks + k];
     if (walk == 0) {
-      st.target = request.top_p * total;  // the nucleus: the shortest head that reaches top_p
+      st.target = request.top_p() * total;  // the nucleus: the shortest head that reaches top_p
     } else {
-      const double head = request.top_p < 1.0 ? sc.found[0 * n + r].reached : total;
+      const double head = request.top_p() < 1.0 ? sc.found[0 * n + r].reached : total;
       st.target = philox_uniform(request.key0, request.key1, request.pos_lo, request.pos_hi) * head;
     }
     st.above = 0.0;
@@ -250,7 +251,7 @@ __global__ __launch_bounds__(kSampleThreads) void sample_level_kernel(const Samp
   __shared__ double wave_sums[kSampleWaves * 16];
   const int r = blockIdx.y, c = blockIdx.x;
   const SampleRow request = requests[r];
-  if (walk == 0 && !(request.top_p < 1.0)) return;  // the whole row is the head
+  if (walk == 0 && !(request.top_p() < 1.0)) return;  // the whole row is the head
   __shared__ double staged[kChunks * 16];
   const SearchState st = state_before_level(sc, request, n, r, walk, level, staged);
   if (c == 0 && threadIdx.x == 0) sc.state[(walk * 2 + ((level + 1) & 1)) * n + r] = st;  // parity of level - 1
@@ -309,7 +310,7 @@ __global__ __launch_bounds__(kSampleThreads) void sample_tie_count_kernel(const 
   __shared__ double wave_weight[kSampleWaves];
   const int r = blockIdx.y, c = blockIdx.x;
   const SampleRow request = requests[r];
-  if (walk == 0 && !(request.top_p < 1.0)) return;
+  if (walk == 0 && !(request.top_p() < 1.0)) return;
   __shared__ double staged[kChunks * 16];
   const SearchState st = state_before_level(sc, request, n, r, walk, 8, staged);
   if (c == 0 && threadIdx.x == 0) sc.state[(walk * 2 + 1) * n + r] = st;  // after level 7
@@ -356,12 +357,13 @@ __global__ __launch_bounds__(kSampleThreads) void sample_tie_count_kernel(const 
 // holds the one that is meant finds it.
 __global__ __launch_bounds__(kSampleThreads) void sample_tie_pick_kernel(const SampleRow* __restrict__ requests,
                                                                          SampleScratch sc, int n, int vocab,
-                                                                         int chunk_len, int walk, int* __restrict__ out) {
+                                                                         int chunk_len, int walk, int* __restrict__ out,
+                                                                         int scatter) {
   __shared__ int counts[kSampleThreads];
   __shared__ int picked;
   const int r = blockIdx.y, c = blockIdx.x;
   const SampleRow request = requests[r];
-  if (walk == 0 && !(request.top_p < 1.0)) return;
+  if (walk == 0 && !(request.top_p() < 1.0)) return;
   const SearchState st = sc.state[(walk * 2 + 1) * n + r];
   int before = 0, ties = 0;
   double w_tie = 0.0;
@@ -404,7 +406,7 @@ __global__ __launch_bounds__(kSampleThreads) void sample_tie_pick_kernel(const S
     found.token = picked;
     found.pad = 0;
     sc.found[walk * n + r] = found;
-    if (walk == 1) out[r] = picked;
+    if (walk == 1) out[scatter ? request.row : r] = picked;
   }
 }
 
@@ -425,18 +427,18 @@ extern "C" long ls_sample_scratch_bytes(int n, int vocab) {
 }
 
 // Sample one token for each of `n` rows.  `requests`: n records of 32 bytes on the device (int row of `logits`,
-// float temperature > 0, double top_p, then four unsigned words: the two halves of seed XOR k(uid) and the two
-// halves of the position); token ids to out[i].  `logits`: float [.][ld], `vocab` columns.  `scratch`:
-// ls_sample_scratch_bytes(n, vocab) bytes, 256-byte aligned.  `any_nucleus`: 0 if every top_p is >= 1 (the
-// launches that look for the nucleus are then left out).
+// float temperature > 0, double top_p (low word first), then four unsigned words: the two halves of seed XOR k(uid) and the two
+// halves of the position); token ids to out[i], or with `scatter` to out[row of the record].  `logits`: float
+// [.][ld], `vocab` columns.  `scratch`: ls_sample_scratch_bytes(n, vocab) bytes, 256-byte aligned.  `any_nucleus`:
+// 0 if every top_p is >= 1 (the launches that look for the nucleus are then left out).
 extern "C" int ls_sample_top_p(const float* logits, long ld, const void* requests, int* out, void* scratch,
-                               long scratch_bytes, int n, int vocab, int any_nucleus, void* stream) {
+                               long scratch_bytes, int n, int vocab, int any_nucleus, int scatter, void* stream) {
   using namespace ls;
   static_assert(sizeof(SampleRow) == 32, "the host packs 32 bytes a row");
   LS_REQUIRE(n > 0 && vocab > 0 && ld >= vocab, "sample: bad sizes (n=%d vocab=%d ld=%ld)", n, vocab, ld);
   LS_REQUIRE(logits && requests && out && scratch, "sample: null operand");
-  LS_REQUIRE(reinterpret_cast<uintptr_t>(scratch) % 256 == 0 && reinterpret_cast<uintptr_t>(requests) % 8 == 0,
-             "sample: the scratch buffer must be 256-byte aligned, the requests 8-byte aligned");
+  LS_REQUIRE(reinterpret_cast<uintptr_t>(scratch) % 256 == 0 && reinterpret_cast<uintptr_t>(requests) % 4 == 0,
+             "sample: the scratch buffer must be 256-byte aligned, the requests 4-byte aligned");
   LS_REQUIRE(scratch_bytes >= ls_sample_scratch_bytes(n, vocab), "sample: %ld bytes of scratch, %ld are needed",
              scratch_bytes, ls_sample_scratch_bytes(n, vocab));
   SampleScratch sc;
@@ -463,7 +465,7 @@ extern "C" int ls_sample_top_p(const float* logits, long ld, const void* request
     for (int level = 0; level < 8; ++level)
       hipLaunchKernelGGL(sample_level_kernel, grid, block, 0, s, rows, sc, n, vocab, chunk_len, walk, level);
     hipLaunchKernelGGL(sample_tie_count_kernel, grid, block, 0, s, rows, sc, n, vocab, chunk_len, walk);
-    hipLaunchKernelGGL(sample_tie_pick_kernel, grid, block, 0, s, rows, sc, n, vocab, chunk_len, walk, out);
+    hipLaunchKernelGGL(sample_tie_pick_kernel, grid, block, 0, s, rows, sc, n, vocab, chunk_len, walk, out, scatter);
   }
   return check_launch("sample");
 }

@@ -302,6 +302,36 @@ class Model:
             n_steps -= chunk
         return np.concatenate(out)
 
+    def decode_sampled(self, cache: CacheManager, requests: Sequence, tokens: Sequence[int], n_steps: int,
+                       sampling: Sequence):
+        """``decode_greedy`` where some requests draw their tokens: ``sampling[i]`` is None (greedy) or
+        ``(temperature > 0, top_p, seed XOR k(uid))``; the draw of a step is keyed on the position of the
+        step's input token, as the host sampler keys it.  The sampling kernels run inside the captured
+        step and the positions in their records move on with every token, so the tokens equal those of
+        step-by-step sampling.  Returns None where the steps cannot run from a captured graph (the caller
+        then takes single steps)."""
+        if not any(s is not None for s in sampling):
+            return self.decode_greedy(cache, requests, tokens, n_steps)
+        n = len(requests)
+        if n == 0 or n_steps <= 0:
+            return np.zeros((0, n), dtype=np.int64)
+        if len(set(requests)) != n or len(sampling) != n:
+            raise ValueError("a request appears twice, or the sampling list has another length")
+        vocab = self.spec.vocab_size
+        if any(not 0 <= int(t) < vocab for t in tokens):
+            raise ValueError(f"a token id lies outside [0, {vocab})")
+        if not (self.use_graphs and self._graph_safe):
+            return None
+        out = []
+        tokens = [int(t) for t in tokens]
+        while n_steps > 0:
+            chunk = min(n_steps, self.LOOP_CAPACITY)
+            picked = self._decode_loop(cache, requests, tokens, chunk, sampling)
+            out.append(picked)
+            tokens = picked[-1].tolist()
+            n_steps -= chunk
+        return np.concatenate(out)
+
     def _decode_greedy_stepwise(self, cache, requests, tokens, n_steps):
         picked = torch.empty(len(requests), dtype=torch.int32, device=self.rt.device)
         out = np.zeros((n_steps, len(requests)), dtype=np.int64)
@@ -313,7 +343,7 @@ class Model:
             out[i] = tokens
         return out
 
-    def _decode_loop(self, cache, requests, tokens, n_steps):
+    def _decode_loop(self, cache, requests, tokens, n_steps, sampling=None):
         n = len(requests)
         starts = [cache.length(r) for r in requests]
         limit = self.spec.max_positions
@@ -332,9 +362,19 @@ class Model:
         ctx = StepContext(self.rt, cache, self.workspace, entries, fixed_shape=True, horizon=max(n_steps - 1, 1))
         for mixer in self._preparers:
             mixer.prepare(ctx)
+        kernels = self.rt.kernels
+        drawn = [i for i in range(n) if sampling is not None and sampling[i] is not None]
+        any_nucleus = any(sampling[i][1] < 1.0 for i in drawn)
+        if drawn:
+            # the sampling kernels' records travel with the step's metadata; the position a draw is keyed on
+            # is that of the step's input token and moves on with it
+            records = kernels.pack_sample_requests([(i, float(sampling[i][0]), float(sampling[i][1]), int(sampling[i][2]),
+                                                     starts[i]) for i in drawn], n)
+            ctx.declare(("loop", "sampling"), records,
+                        advance=[(kernels.SAMPLE_POSITION_AT, kernels.SAMPLE_ROW_INTS, len(drawn))],
+                        signature=("sampling", len(drawn), any_nucleus))
         ctx.upload()
         layout = ctx.meta_layout()
-        kernels = self.rt.kernels
         ring = self.workspace.get("loop.ring", (self.LOOP_CAPACITY * max(n, 64),), torch.int32)
         counter = self.workspace.get("loop.counter", (1,), torch.int32)
         picked = self.workspace.get("loop.picked", (max(n, 64),), torch.int32)
@@ -343,6 +383,9 @@ class Model:
         def one_step(logits):
             self._forward(ctx, logits)
             kernels.argmax(logits, picked[:n])
+            if drawn:                                     # the drawn rows' picks replace their arg-max
+                kernels.sample_top_p(logits, None, picked, records=ctx.block(("loop", "sampling")),
+                                     any_nucleus=any_nucleus, scatter=True)
             kernels.advance_decode(layout["meta"], n, layout["tokens"], picked, ring, counter, *layout["runs"])
 
         graphs = cache.step_graphs

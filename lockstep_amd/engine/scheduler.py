@@ -126,9 +126,10 @@ class Scheduler:
         """``num_blocks`` pages of ``block_size`` tokens, ``eos_token_ids``, ``audit`` and
         ``enable_prefix_cache`` carry the reference's names (engine/sched/scheduler.py:51-60).
         ``max_batched_tokens`` bounds the tokens of one step (None: no bound).  ``decode_burst`` > 1:
-        while nothing waits, every running request decodes greedily and no answer of the policy can
-        change from step to step, up to that many decode steps run as one call of the model's
-        device-side loop (``decode_greedy``); tokens, counters and marks are those of single steps."""
+        while nothing waits, every running request decodes and no answer of the policy can change
+        from step to step, up to that many decode steps run as one call of the model's device-side
+        loop (``decode_greedy``, or ``decode_sampled`` where requests draw their tokens); tokens,
+        counters and marks are those of single steps."""
         if reserve not in ("full", "lazy"):
             raise ValueError("reserve must be 'full' or 'lazy'")
         self.model = model
@@ -432,13 +433,24 @@ class Scheduler:
             return False
         if self.max_batched_tokens is not None and self.max_batched_tokens < len(self.running):
             return False
-        if any(s.temperature > 0 or not s.decoding for s in self.running):
+        if any(not s.decoding for s in self.running):
             return False
         steps = min(self.decode_burst, max_steps - self.step_index, min(s.budget_left for s in self.running))
         if steps <= 1:
             return False
-        picked = self.model.decode_greedy(self.cache, [s.uid for s in self.running],
-                                          [s.tokens[-1] for s in self.running], steps)
+        uids, last = [s.uid for s in self.running], [s.tokens[-1] for s in self.running]
+        if any(s.temperature > 0 for s in self.running):
+            if not hasattr(self.model, "decode_sampled"):
+                return False
+            from ..sampling import philox
+
+            picked = self.model.decode_sampled(self.cache, uids, last, steps, [
+                None if s.temperature <= 0 else (s.temperature, s.top_p, int(s.request.seed) ^ philox.uid_key(s.uid))
+                for s in self.running])
+            if picked is None:
+                return False
+        else:
+            picked = self.model.decode_greedy(self.cache, uids, last, steps)
         for row in picked:
             for seq, token in zip(self.running, row):
                 seq.tokens.append(int(token))

@@ -81,6 +81,7 @@ class Kernels:
         self.attention_paths: dict[int, str] = {}
         self._argmax_scratch: dict = {}
         self._sample_scratch: dict = {}
+        self._sample_scratch_kept: list = []
         self._capabilities: dict = {}
         #: while this is a list, every launch is noted on it as (library, entry point, arguments):
         #: the engine repeats the launches of one layer for the next layers that are alike
@@ -366,41 +367,65 @@ class Kernels:
             _ptr(logits), _ptr(out), c_int(logits.shape[0]), c_int(logits.shape[1]), c_long(logits.stride(0)),
             _ptr(scratch), c_long(scratch.numel()), _stream()))
 
-    #: one row's request as ``sample_top_p`` takes it (32 bytes; csrc/sample.hip: SampleRow)
+    #: one row's request as ``sample_top_p`` takes it (eight 4-byte words; csrc/sample.hip: SampleRow)
     SAMPLE_ROW = [("row", "<i4"), ("temperature", "<f4"), ("top_p", "<f8"), ("key0", "<u4"), ("key1", "<u4"),
                   ("pos_lo", "<u4"), ("pos_hi", "<u4")]
+    SAMPLE_ROW_INTS = 8
+    SAMPLE_POSITION_AT = 6          # the word of a record that holds the low half of the position
 
-    def sample_top_p(self, logits: torch.Tensor, requests, out: torch.Tensor) -> None:
-        """One token for each request: ``requests`` is a sequence of (row of the float32 ``logits``,
-        temperature > 0, top_p, seed XOR k(uid) as an int of 64 bits, position); ``out`` int32 on the GPU.
-        The host sampler's procedure in float64 (sampling/sampler.py) without its sort, the draw included
-        (Philox-4x32-10 keyed as sampling/philox.py keys it)."""
+    @classmethod
+    def pack_sample_requests(cls, requests, rows: int):
+        """``requests``: (row of the logits, temperature > 0, top_p, seed XOR k(uid) as an int of 64 bits,
+        position) each; the records as int32 words, eight a request."""
         import numpy as np
 
-        _rows_ok(logits, "sample logits")
-        n = len(requests)
-        if not (out.is_cuda and out.dtype == torch.int32 and out.is_contiguous() and out.shape == (n,)):
-            raise KernelError(f"sample out must be int32 [{n}] on the GPU")
-        if not (logits.dtype == torch.float32):
-            raise KernelError("sample reads float32 logits")
-        if n == 0:
-            return
-        packed = np.zeros(n, dtype=self.SAMPLE_ROW)
+        packed = np.zeros(len(requests), dtype=cls.SAMPLE_ROW)
         for i, (row, temperature, top_p, mixed, position) in enumerate(requests):
-            if not (0 <= row < logits.shape[0] and temperature > 0):
-                raise KernelError(f"sample: row {row} of {logits.shape[0]} at temperature {temperature}")
+            if not (0 <= row < rows and temperature > 0):
+                raise KernelError(f"sample: row {row} of {rows} at temperature {temperature}")
             packed[i] = (row, temperature, top_p, mixed & 0xFFFFFFFF, (mixed >> 32) & 0xFFFFFFFF,
                          position & 0xFFFFFFFF, (position >> 32) & 0xFFFFFFFF)
-        on_device = torch.from_numpy(packed.view(np.uint8)).to(logits.device)
+        return packed.view(np.int32)
+
+    def sample_top_p(self, logits: torch.Tensor, requests, out: torch.Tensor, records: torch.Tensor | None = None,
+                     any_nucleus: bool | None = None, scatter: bool = False) -> None:
+        """One token for each request: ``requests`` is a sequence of (row of the float32 ``logits``,
+        temperature > 0, top_p, seed XOR k(uid) as an int of 64 bits, position); ``out`` int32 on the GPU
+        gets request i's token at ``out[i]`` (with ``scatter`` at ``out[row]``).  Or ``records``: the same
+        packed by ``pack_sample_requests`` and already on the GPU (int32, eight words a request), with
+        ``any_nucleus`` saying whether any top_p is below one.  The host sampler's procedure in float64
+        (sampling/sampler.py) without its sort, the draw included (Philox-4x32-10 keyed as
+        sampling/philox.py keys it)."""
+        _rows_ok(logits, "sample logits")
+        if not (logits.dtype == torch.float32):
+            raise KernelError("sample reads float32 logits")
+        if records is None:
+            n = len(requests)
+            if n == 0:
+                return
+            records = torch.from_numpy(self.pack_sample_requests(requests, logits.shape[0])).to(logits.device)
+            any_nucleus = any(top_p < 1.0 for _, _, top_p, _, _ in requests)
+        else:
+            if not (records.is_cuda and records.dtype == torch.int32 and records.is_contiguous()
+                    and records.numel() % self.SAMPLE_ROW_INTS == 0 and any_nucleus is not None):
+                raise KernelError("sample records: contiguous int32 on the GPU, eight words a request, and any_nucleus")
+            n = records.numel() // self.SAMPLE_ROW_INTS
+            if n == 0:
+                return
+        if not (out.is_cuda and out.dtype == torch.int32 and out.is_contiguous()
+                and out.numel() >= (logits.shape[0] if scatter else n)):
+            raise KernelError("sample out must be int32 on the GPU, one for every request (with scatter: every row)")
         vocab = logits.shape[1]
         need = int(self.core.ls_sample_scratch_bytes(c_int(n), c_int(vocab)))
         scratch = self._sample_scratch.get(logits.device)
         if scratch is None or scratch.numel() < need:
-            scratch = self._sample_scratch[logits.device] = torch.empty(need, dtype=torch.uint8, device=logits.device)
-        any_nucleus = any(top_p < 1.0 for _, _, top_p, _, _ in requests)
+            # (a buffer that was outgrown is kept: a captured graph may still write into it)
+            scratch = torch.empty(need, dtype=torch.uint8, device=logits.device)
+            self._sample_scratch_kept.append(self._sample_scratch.get(logits.device))
+            self._sample_scratch[logits.device] = scratch
         self._launch(self.core, self.core.ls_sample_top_p, (
-            _ptr(logits), c_long(logits.stride(0)), _ptr(on_device), _ptr(out), _ptr(scratch), c_long(scratch.numel()),
-            c_int(n), c_int(vocab), c_int(1 if any_nucleus else 0), _stream()))
+            _ptr(logits), c_long(logits.stride(0)), _ptr(records), _ptr(out), _ptr(scratch), c_long(scratch.numel()),
+            c_int(n), c_int(vocab), c_int(1 if any_nucleus else 0), c_int(1 if scatter else 0), _stream()))
 
     def advance_decode(self, meta: torch.Tensor, n_seqs: int, off_tokens: int, picked: torch.Tensor,
                        ring: torch.Tensor, counter: torch.Tensor, off_runs: int, n_runs: int) -> None:

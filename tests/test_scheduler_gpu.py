@@ -145,6 +145,38 @@ def test_lazy_reservation_preempts_for_pages_and_gives_the_same_bits(tiny_dirs, 
     check(model, wave, out, s, page_size, plain_for(folder, dtype))
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_bursts_of_decode_steps_draw_the_tokens_of_single_steps(tiny_dirs, dtype):
+    """Requests that sample (different temperatures and nuclei, one greedy among them) decode in bursts
+    on the GPU: the draws are keyed on positions that move on inside the captured step, and the tokens
+    are those of one step at a time with the sampler called from the host."""
+    from lockstep_amd import Request, Scheduler
+
+    model = load(tiny_dirs[("B", "gen")], dtype)
+    vocab = model.spec.vocab_size
+
+    def requests():
+        return [Request(uid="t0", prompt=random_tokens(9, vocab, seed=71), max_new_tokens=40, temperature=0.8, seed=3),
+                Request(uid="t1", prompt=random_tokens(30, vocab, seed=72), max_new_tokens=33, temperature=1.3, top_p=0.9,
+                        seed=1 << 35),
+                Request(uid="t2", prompt=random_tokens(4, vocab, seed=73), max_new_tokens=40),
+                Request(uid="t3", prompt=random_tokens(17, vocab, seed=74), max_new_tokens=25, temperature=0.5, top_p=0.5,
+                        seed=9)]
+
+    results = {}
+    for burst in (1, 7, 32):
+        replays = model.graph_replays
+        s = Scheduler(model, num_blocks=64, block_size=8, audit=False, decode_burst=burst)
+        for r in requests():
+            s.submit(r)
+        results[burst] = s.run()
+        assert s.counters["decode_step"] == 39 + 32 + 39 + 24
+        if burst > 1:
+            assert model.graph_replays - replays >= 30
+    assert results[7] == results[1] and results[32] == results[1]
+    assert len({tuple(v) for v in results[1].values()}) == 4
+
+
 def test_replayed_decode_steps_are_checked_against_eager_ones(tiny_dirs, monkeypatch):
     """With LOCKSTEP_VERIFY_GRAPHS every replayed step graph is followed by the same step run
     eagerly and the two sets of logits must be equal bit for bit; a serving run passes it."""
