@@ -425,7 +425,7 @@ class Scheduler:
     def _burst(self, max_steps: int) -> bool:
         """Run decode steps through the model's device-side loop while every decision of those
         steps is known beforehand (see ``decode_burst``).  Returns whether any ran."""
-        if self.decode_burst <= 1 or self.waiting or not self.running or self.eos or self.audit_enabled:
+        if self.decode_burst <= 1 or self.waiting or not self.running or self.audit_enabled:
             return False
         if self.keep_logits or self.lazy or not hasattr(self.model, "decode_greedy"):
             return False
@@ -451,13 +451,22 @@ class Scheduler:
                 return False
         else:
             picked = self.model.decode_greedy(self.cache, uids, last, steps)
+        # A request that draws an end-of-sequence id stops there: the steps the loop ran for it beyond that
+        # are dropped (its pages go back when it retires below; the others' tokens do not depend on it).
+        stopped = set()
         for row in picked:
             for seq, token in zip(self.running, row):
+                if seq.uid in stopped:
+                    continue
                 seq.tokens.append(int(token))
                 seq.cached += 1
                 self.counters.hit("decode_step")
                 self._mark(seq.uid, Event.DECODE)
+                if int(token) in self.eos:
+                    stopped.add(seq.uid)
             self.step_index += 1
+            if len(stopped) == len(self.running):
+                break                              # single steps would have stopped here as well
         self._retire()
         return True
 

@@ -281,7 +281,8 @@ def test_lifecycle_follows_the_state_machine():
 def test_decode_bursts_change_neither_tokens_nor_counts():
     """With decode_burst > 1 runs of decode steps go through the model's device-side loop: same
     tokens, same counters, same number of steps, same life cycle; a burst never runs past a
-    request's last token, and not while something waits, samples, or may stop at an end token."""
+    request's last token, and not while something waits or samples (this stand-in model has no loop for
+    that); a request that draws an end-of-sequence id inside a burst stops there."""
     ps = prompts(3, 20, 41)
     lengths = (5, 9, 14)
 
@@ -295,11 +296,20 @@ def test_decode_bursts_change_neither_tokens_nor_counts():
     assert not hasattr(m1, "bursts")
     assert s1.counters.counts == s2.counters.counts
     assert s1.step_index == s2.step_index and s1.lifecycle == s2.lifecycle
-    # conditions that keep single steps: audit on, an end token, sampling, a waiting request
-    for kw, requests in (({"audit": True}, build()), ({"audit": False, "eos_token_ids": [7]}, build()),
+    # conditions that keep single steps: audit on, sampling with a model that has no loop for it, a waiting request
+    for kw, requests in (({"audit": True}, build()),
                          ({"audit": False}, [Request(uid="t", prompt=ps[0], max_new_tokens=6, temperature=0.8, seed=3)])):
         _, _, m = run(requests, decode_burst=4, **kw)
         assert not hasattr(m, "bursts"), kw
+    # end-of-sequence ids inside a burst: the request stops where single steps would stop it, the steps the
+    # loop ran for it beyond that are dropped, and counters, steps and life cycles agree
+    eos = [single["r1"][3], single["r2"][9]]
+    stopped, s4, _ = run(build(), audit=False, eos_token_ids=eos)
+    assert stopped == {f"r{i}": expected_greedy(p, n, eos) for i, (p, n) in enumerate(zip(ps, lengths))}
+    assert any(len(stopped[u]) < len(single[u]) for u in stopped)
+    bursting, s5, m5 = run(build(), audit=False, eos_token_ids=eos, decode_burst=4)
+    assert bursting == stopped and getattr(m5, "bursts", [])
+    assert s4.counters.counts == s5.counters.counts and s4.lifecycle == s5.lifecycle and s4.step_index == s5.step_index
     many = [Request(uid=f"w{i}", prompt=ps[0], max_new_tokens=8) for i in range(3)]
     out, s3, m3 = run(many, audit=False, decode_burst=16, policy=None, num_blocks=2)   # pages for two at a time
     assert out == {f"w{i}": expected_greedy(ps[0], 8) for i in range(3)}

@@ -177,6 +177,40 @@ def test_bursts_of_decode_steps_draw_the_tokens_of_single_steps(tiny_dirs, dtype
     assert len({tuple(v) for v in results[1].values()}) == 4
 
 
+def test_end_of_sequence_ids_inside_a_burst_stop_a_request_where_single_steps_would(tiny_dirs):
+    """End-of-sequence ids picked from the requests' own continuations, so that they stop in the middle
+    of bursts, at different steps, one of them at once: the same tokens, finishes and counters as with
+    one step at a time."""
+    from lockstep_amd import Request, Scheduler
+
+    model = load(tiny_dirs[("B", "gen")], "bfloat16")
+    vocab = model.spec.vocab_size
+
+    def requests():
+        return [Request(uid=f"e{i}", prompt=random_tokens(n, vocab, seed=80 + i), max_new_tokens=36,
+                        temperature=0.9 if i == 2 else 0.0, seed=i) for i, n in enumerate((6, 21, 3, 40))]
+
+    def serve(burst, eos):
+        s = Scheduler(model, num_blocks=64, block_size=8, audit=False, decode_burst=burst, eos_token_ids=eos)
+        for r in requests():
+            s.submit(r)
+        return s.run(), s
+
+    free, _ = serve(1, None)
+    eos = [free["e0"][11], free["e1"][20], free["e2"][0]]          # e2 stops with its first token
+    single, s1 = serve(1, eos)
+    assert len(single["e0"]) <= 12 and len(single["e1"]) <= 21 and len(single["e2"]) == 1
+    assert any(len(single[u]) < 36 for u in ("e0", "e1")) and s1.counters["finish_eos"] >= 2
+    for burst in (5, 32):
+        replays = model.graph_replays
+        got, s = serve(burst, eos)
+        assert got == single and model.graph_replays > replays
+        for name in ("finish_eos", "finish_limit", "decode_step"):
+            assert s.counters[name] == s1.counters[name], name
+        s.cache.audit()
+        assert s.cache.free_slots == s.cache.max_requests
+
+
 def test_replayed_decode_steps_are_checked_against_eager_ones(tiny_dirs, monkeypatch):
     """With LOCKSTEP_VERIFY_GRAPHS every replayed step graph is followed by the same step run
     eagerly and the two sets of logits must be equal bit for bit; a serving run passes it."""
