@@ -311,7 +311,8 @@ def serve_trace(kind: str, model_name: str, vocab: int, n_requests: int = 0):
     return [torch.randint(0, vocab, (n,), generator=g).tolist() for n in lengths], new, chunk
 
 
-def measure_serve(model, prompts, new_tokens: int, chunk, page_size: int, max_batched_tokens, repeats: int):
+def measure_serve(model, prompts, new_tokens: int, chunk, page_size: int, max_batched_tokens, repeats: int,
+                  temperature: float = 0.0, top_p: float = 1.0):
     """Run the workload ``repeats`` + 1 times through the scheduler (the first pass untimed).
     Returns per timed pass (seconds, seconds until no prompt token was left, scheduler steps,
     steps of the decode-only phase)."""
@@ -330,7 +331,8 @@ def measure_serve(model, prompts, new_tokens: int, chunk, page_size: int, max_ba
         scheduler = Scheduler(model, num_blocks=pages, policy=policy, audit=False, block_size=page_size,
                               max_batched_tokens=max_batched_tokens, cache=cache, decode_burst=32)
         for j, prompt in enumerate(prompts):
-            scheduler.submit(Request(uid=f"r{j:02d}", prompt=prompt, seed=j, max_new_tokens=new_tokens))
+            scheduler.submit(Request(uid=f"r{j:02d}", prompt=prompt, seed=j, max_new_tokens=new_tokens,
+                                     temperature=temperature, top_p=top_p))
         torch.cuda.synchronize()
         started = time.perf_counter()
         prompts_done_at, steps_at = None, 0
@@ -355,8 +357,10 @@ def serve_record(args, model, cfg, full_layers) -> dict:
     prompts, new_tokens, chunk = serve_trace(args.workload, args.model, cfg.vocab_size, args.requests)
     if args.prefill_chunk is not None:
         chunk = args.prefill_chunk or None
+    if args.new_tokens:
+        new_tokens = args.new_tokens
     passes = measure_serve(model, prompts, new_tokens, chunk, args.page_size, args.max_batched_tokens,
-                           args.repeats)
+                           args.repeats, args.temperature, args.top_p)
     order = sorted(passes, key=lambda t: t[0])
     elapsed, prompts_done, steps, decode_steps = order[len(order) // 2]
     prompt_tokens = sum(len(p) for p in prompts)
@@ -392,6 +396,7 @@ def serve_record(args, model, cfg, full_layers) -> dict:
             "until_prompts_done_s": round(prompts_done, 4), "decode_only_s": round(decode_seconds, 4),
             "decode_only_steps": decode_steps,
             "decode_only_step_ms": round(1e3 * decode_seconds / decode_steps, 4) if decode_steps else None,
+            "sampling": "greedy" if args.temperature <= 0 else f"temperature {args.temperature}, top_p {args.top_p}",
         },
     }
 
@@ -419,6 +424,10 @@ def main(argv=None) -> int:
     p.add_argument("--requests", type=int, default=0, help="serve: only the first N requests of the workload")
     p.add_argument("--prefill-chunk", type=int, default=None, help="serve: prompt portion (0: whole prompts)")
     p.add_argument("--max-batched-tokens", type=int, default=8192, help="serve: token budget of a step (0: none)")
+    p.add_argument("--temperature", type=float, default=0.0,
+                   help="serve: requests draw their tokens at this temperature (0: greedy), a seed a request")
+    p.add_argument("--top-p", type=float, default=1.0, help="serve: nucleus of the requests that draw their tokens")
+    p.add_argument("--new-tokens", type=int, default=0, help="serve: new tokens a request (0: the workload's own)")
     p.add_argument("--only-prefill", action="store_true",
                    help="run the prefill measurement alone and print its record (for profiling)")
     args = p.parse_args(argv)
