@@ -49,6 +49,15 @@ namespace ls {
 #ifndef LS_GEMM_GROUP_M
 #define LS_GEMM_GROUP_M 4     // row tiles per band of the tile numbering (0: column-major numbering)
 #endif
+#ifndef LS_GEMM_WIDE
+#define LS_GEMM_WIDE 1        // 0: never the 128 x 256 tiles of eight waves
+#endif
+#ifndef LS_GEMM_WIDE_FILL
+#define LS_GEMM_WIDE_FILL 85  // ... which need whole rounds of the CUs (one workgroup a CU): at least this share, in percent,
+#endif                        // of the last round's CUs busy, or eight rounds and more
+#ifndef LS_GEMM_PD_WIDE
+#define LS_GEMM_PD_WIDE 2     // their register prefetch depth (2 is 1 to 4 % ahead of 1)
+#endif
 #ifndef LS_GEMM_PD_SMALL
 #define LS_GEMM_PD_SMALL 4    // ... and of the 64 x 64 kernel (measured 1 to 4: 4 is 2 to 10 % ahead of 2)
 #endif
@@ -694,30 +703,38 @@ __global__ __launch_bounds__(256) void gemm_slices_stream_kernel(const T* __rest
 }
 
 // ---------------------------------------------------------------------------
-// Tiled kernel: BM x BN outputs per workgroup, four waves in a 2 x 2 grid,
-// each (BM/2) x (BN/2).  Both operands go through LDS in stages of 128 bytes
+// Tiled kernel: BM x BN outputs per workgroup, NWM x NWN waves, each
+// (BM/NWM) x (BN/NWN).  Both operands go through LDS in stages of 128 bytes
 // of K per row, double buffered: while stage i is multiplied, stage i+1 is
 // written to the other buffer and the global loads of stage i+2 are in
-// flight.  Accumulators are small enough for two or three workgroups a CU,
-// which is what hides the LDS and barrier latency.  Workgroups are numbered
-// so that those that share a weight tile run on the same XCD (each XCD has
-// its own L2).
+// flight.  A wave's accumulators (at most 64 x 64 outputs, twice: the slice
+// sum and the total) leave room for two waves a SIMD, which is what hides
+// the LDS and barrier latency.  Workgroups are numbered so that those that
+// share a weight tile run on the same XCD (each XCD has its own L2).
+//
+// What bounds the kernel is the rate at which a CU gets operand bytes from
+// L2 (measured: every tile shape runs at 45 to 48 GB/s a CU), so the bytes a
+// workgroup loads per MFMA decide: (BM + BN) / (BM BN).  Hence eight waves
+// with 128 x 256 outputs where that many tiles fill the CUs, and the 2 x 2
+// grids of waves below that.
 // ---------------------------------------------------------------------------
 constexpr int kRowBytes = 128;               // bytes of K per row per stage (two chunks)
 constexpr int kRowStride = kRowBytes + 16;   // padded LDS row
 
-template <typename T, int EPI, int BM, int BN, int PD, bool AL>
-__global__ __launch_bounds__(256) void gemm_tiled_kernel(const T* __restrict__ X, const T* __restrict__ W,
+template <typename T, int EPI, int BM, int BN, int PD, bool AL, int NWM = 2, int NWN = 2>
+__global__ __launch_bounds__(64 * NWM * NWN) void gemm_tiled_kernel(const T* __restrict__ X, const T* __restrict__ W,
                                                          void* __restrict__ C, int M, int N, int K, long ldx,
                                                          long ldc, int kslice, int vec_ok, int tiles_m, int tiles_n,
                                                          int out_cols) {
   typedef Atom<T> A;
   typedef typename A::vec_t vec_t;
   constexpr int BK = kRowBytes / sizeof(T);  // elements of K per stage
-  constexpr int TI = BN / 32;                // weight tiles (16 columns) per wave
-  constexpr int TJ = BM / 32;                // row tiles per wave
-  constexpr int WP = BN / 32;                // staging passes over the weight tile (32 rows each)
-  constexpr int XP = BM / 32;
+  constexpr int TI = BN / (16 * NWN);        // weight tiles (16 columns) per wave
+  constexpr int TJ = BM / (16 * NWM);        // row tiles per wave
+  constexpr int PASS = 8 * NWM * NWN;        // rows per staging pass: 8 threads a row
+  constexpr int WP = BN / PASS;              // staging passes over the weight tile
+  constexpr int XP = BM / PASS;
+  static_assert(BN % PASS == 0 && BM % PASS == 0 && TI * 16 * NWN == BN && TJ * 16 * NWM == BM, "tile shape");
   constexpr int STAGE_BYTES = (BM + BN) * kRowStride;
   __shared__ __attribute__((aligned(16))) unsigned char lds[2 * STAGE_BYTES];
 
@@ -742,11 +759,11 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const T* __restrict__ X
 
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
-  const int wn = (wave & 1) * (BN / 2);
-  const int wm = (wave >> 1) * (BM / 2);
+  const int wn = (wave % NWN) * (BN / NWN);
+  const int wm = (wave / NWN) * (BM / NWM);
   const int row16 = lane & 15;
   const int g = lane >> 4;
-  const int st_row = threadIdx.x >> 3;             // staging: 8 threads per row, 32 rows per pass
+  const int st_row = threadIdx.x >> 3;             // staging: 8 threads per row, PASS rows per pass
   const int st_col = (threadIdx.x & 7) * A::VEC;
 
   f32x4 total[TI][TJ];
@@ -771,9 +788,9 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const T* __restrict__ X
   const T* x_src[XP];
   if (AL) {
 #pragma unroll
-    for (int p = 0; p < WP; ++p) w_src[p] = W + (long)min(n_base + st_row + 32 * p, N - 1) * K;
+    for (int p = 0; p < WP; ++p) w_src[p] = W + (long)min(n_base + st_row + PASS * p, N - 1) * K;
 #pragma unroll
-    for (int p = 0; p < XP; ++p) x_src[p] = X + (long)min(m_base + st_row + 32 * p, M - 1) * ldx;
+    for (int p = 0; p < XP; ++p) x_src[p] = X + (long)min(m_base + st_row + PASS * p, M - 1) * ldx;
   }
   auto fetch = [&](int slot, int k0) {
     if (AL) {
@@ -786,12 +803,12 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const T* __restrict__ X
     }
 #pragma unroll
     for (int p = 0; p < WP; ++p) {
-      const int r = st_row + 32 * p;
+      const int r = st_row + PASS * p;
       wv[slot][p] = load_vec<T>(W, n_base + r, k0 + st_col, K, K, n_base + r < N, false);
     }
 #pragma unroll
     for (int p = 0; p < XP; ++p) {
-      const int r = st_row + 32 * p;
+      const int r = st_row + PASS * p;
       xv[slot][p] = load_vec<T>(X, m_base + r, k0 + st_col, K, ldx, m_base + r < M, false);
     }
   };
@@ -800,18 +817,18 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const T* __restrict__ X
     unsigned char* x_lds = w_lds + BN * kRowStride;
 #pragma unroll
     for (int p = 0; p < WP; ++p)
-      *reinterpret_cast<vec_t*>(&w_lds[(st_row + 32 * p) * kRowStride + st_col * sizeof(T)]) = wv[slot][p];
+      *reinterpret_cast<vec_t*>(&w_lds[(st_row + PASS * p) * kRowStride + st_col * sizeof(T)]) = wv[slot][p];
 #pragma unroll
     for (int p = 0; p < XP; ++p)
-      *reinterpret_cast<vec_t*>(&x_lds[(st_row + 32 * p) * kRowStride + st_col * sizeof(T)]) = xv[slot][p];
+      *reinterpret_cast<vec_t*>(&x_lds[(st_row + PASS * p) * kRowStride + st_col * sizeof(T)]) = xv[slot][p];
     if (AL && k0 + BK > K) {  // uniform: the last stage where K is no multiple of BK; its columns from K on are cleared
       if (k0 + st_col >= K) {
 #pragma unroll
         for (int p = 0; p < WP; ++p)
-          *reinterpret_cast<vec_t*>(&w_lds[(st_row + 32 * p) * kRowStride + st_col * sizeof(T)]) = A::zero();
+          *reinterpret_cast<vec_t*>(&w_lds[(st_row + PASS * p) * kRowStride + st_col * sizeof(T)]) = A::zero();
 #pragma unroll
         for (int p = 0; p < XP; ++p)
-          *reinterpret_cast<vec_t*>(&x_lds[(st_row + 32 * p) * kRowStride + st_col * sizeof(T)]) = A::zero();
+          *reinterpret_cast<vec_t*>(&x_lds[(st_row + PASS * p) * kRowStride + st_col * sizeof(T)]) = A::zero();
       }
     }
   };
@@ -992,19 +1009,32 @@ int launch_gemm(const void* X, const void* W, void* C, int M, int N, int K, long
     // Large products take 128 x 128 tiles (least LDS traffic per MFMA); smaller ones take
     // 64 x 64 tiles so that every CU has several workgroups, with a deeper register prefetch.
     const long big_tiles = (long)((M + 127) / 128) * ((N + 127) / 128);
-#define LS_TILED(BM_, BN_, PD_, AL_)                                                                           \
+#define LS_TILED_WAVES(BM_, BN_, PD_, AL_, NWM_, NWN_)                                                         \
   {                                                                                                             \
     const int tiles_m = (M + BM_ - 1) / BM_, tiles_n = (N + BN_ - 1) / BN_;                                       \
-    hipLaunchKernelGGL((gemm_tiled_kernel<T, EPI, BM_, BN_, PD_, AL_>), dim3(tiles_m * tiles_n), dim3(256), 0,   \
-                       stream, reinterpret_cast<const T*>(X), w, C, M, N, K, ldx, ldc, kslice, vec_ok, tiles_m,   \
-                       tiles_n, out_cols);                                                                      \
+    hipLaunchKernelGGL((gemm_tiled_kernel<T, EPI, BM_, BN_, PD_, AL_, NWM_, NWN_>), dim3(tiles_m * tiles_n),      \
+                       dim3(64 * NWM_ * NWN_), 0, stream, reinterpret_cast<const T*>(X), w, C, M, N, K, ldx, ldc, \
+                       kslice, vec_ok, tiles_m, tiles_n, out_cols);                                             \
   }
+#define LS_TILED(BM_, BN_, PD_, AL_) LS_TILED_WAVES(BM_, BN_, PD_, AL_, 2, 2)
+    // 128 x 256 tiles load a quarter fewer operand bytes per MFMA (measured at 2,048 rows: gate and up of
+    // Qwen3-8B sizes 511 -> 446 us, down 246 -> 211 us), but a CU holds one such workgroup, so a last
+    // round that leaves CUs idle costs more than it does with the smaller tiles, two of which share a CU
+    const long wide_tiles = (long)((M + 127) / 128) * ((N + 255) / 256);
+    const long cus = compute_units();
+    const long wide_rounds = (wide_tiles + cus - 1) / cus;
+    const bool wide_fills = LS_GEMM_WIDE && sizeof(T) == 2 && M > LS_GEMM_BIG_ROWS && wide_tiles >= cus &&
+                            (wide_rounds >= 8 || wide_tiles * 100 >= wide_rounds * cus * LS_GEMM_WIDE_FILL);
     // (operands that are not 16-byte aligned take the small tiles, element by element: every tile
     // shape gives the same bits)
     if (!aligned) LS_TILED(64, 64, LS_GEMM_PD_SMALL, false)
+    else if (wide_fills) {
+      if constexpr (sizeof(T) == 2) LS_TILED_WAVES(128, 256, LS_GEMM_PD_WIDE, true, 2, 4)
+    }
     else if (big_tiles >= LS_GEMM_BIG && M > LS_GEMM_BIG_ROWS) LS_TILED(128, 128, LS_GEMM_PD_BIG, true)
     else LS_TILED(64, 64, LS_GEMM_PD_SMALL, true)
 #undef LS_TILED
+#undef LS_TILED_WAVES
   }
   return check_launch("gemm");
 }

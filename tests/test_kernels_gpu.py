@@ -113,6 +113,44 @@ def test_gemm_with_few_rows_and_many_columns_has_the_same_bits(dtype, k, n):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("k", [264, 1088])
+def test_gemm_with_many_rows_and_columns_has_the_bits_of_few_rows(dtype, k):
+    """2,050 rows by 3,740 columns: 17 x 15 tiles of 128 x 256 outputs fill one round of 256 CUs, so
+    bfloat16 takes the workgroups of eight waves; rows, columns and (with 264) K end inside a tile.
+    Every epilogue; rows from all over the product have the bits they have in a product of 40 rows,
+    which the skinny kernel computes."""
+    from lockstep_amd.ops import ADD_F32, STORE, STORE_F32, SWIGLU, interleave_gate_up
+
+    g = torch.Generator().manual_seed(k)
+    m, n = 2050, 3740
+    x = torch.randn(m, k, generator=g).to(dtype).cuda()
+    w = (torch.randn(n, k, generator=g) * 0.1).to(dtype).cuda()
+    full = torch.empty(m, n, dtype=torch.float32, device="cuda")
+    K().gemm(x, w, full, STORE_F32)
+    want = x[-3:].double().cpu() @ w.double().cpu().T
+    assert rel_err(full[-3:], want) < 2e-5
+    stored = torch.empty(m, n, dtype=dtype, device="cuda")
+    K().gemm(x, w, stored, STORE)
+    assert torch.equal(stored, full.to(dtype))
+    base = torch.randn(m, n, generator=g).cuda()
+    acc = base.clone()
+    K().gemm(x, w, acc, ADD_F32)
+    assert torch.equal(acc, base + full)
+    inter = n // 2
+    wi = interleave_gate_up(w[:inter].cpu(), w[inter:].cpu()).cuda()
+    gated = torch.empty(m, inter, dtype=dtype, device="cuda")
+    K().gemm(x, wi, gated, SWIGLU)
+    for first in (0, 100, 1000, 2010):
+        rows = slice(first, first + 40)
+        part = torch.empty(40, n, dtype=torch.float32, device="cuda")
+        K().gemm(x[rows], w, part, STORE_F32)
+        assert torch.equal(part, full[rows]), f"rows from {first}"
+        part = torch.empty(40, inter, dtype=dtype, device="cuda")
+        K().gemm(x[rows], wi, part, SWIGLU)
+        assert torch.equal(part, gated[rows]), f"rows from {first}, SwiGLU"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("inter,k", [(4096 + 40, 4096), (16384 + 72, 1024)])
 def test_swiglu_with_few_rows_and_many_columns_has_the_same_bits(dtype, inter, k):
     from lockstep_amd.ops import SWIGLU, interleave_gate_up
