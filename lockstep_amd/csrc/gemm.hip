@@ -8,9 +8,10 @@
 // The skinny kernel (M <= 64, decode) gives each slice to a wave, so the
 // weights stream from HBM with many waves in flight; the streaming kernel
 // does the same for products with many columns, one workgroup walking many
-// column blocks; the slice kernel leaves the slice sums to its consumer; the
+// column blocks; the slice kernels leave the slice sums to their consumer; the
 // tiled kernel (prefill) walks the slices one after the other with both
-// operands staged in LDS.  All produce the same bits for a row, so a token's
+// operands staged in LDS, or (slice sums of 17 rows and more) a group of them
+// a workgroup.  All produce the same bits for a row, so a token's
 // projections do not depend on how many tokens share its step.
 //
 // The MFMA runs "swapped": W rows are the first operand, X rows the second,
@@ -58,6 +59,15 @@ namespace ls {
 #ifndef LS_GEMM_PD_WIDE
 #define LS_GEMM_PD_WIDE 2     // their register prefetch depth (2 is 1 to 4 % ahead of 1)
 #endif
+#ifndef LS_GEMM_READ_AHEAD
+#define LS_GEMM_READ_AHEAD 1  // the tiled kernel reads a stage's second chunk of fragments from LDS before it multiplies the first
+#endif
+#ifndef LS_GEMM_SLICES_TILED
+#define LS_GEMM_SLICES_TILED 1      // 0: never the tiled kernel for slice sums
+#endif
+#ifndef LS_GEMM_NARROW
+#define LS_GEMM_NARROW 1      // 0: never the 64 x 32 tiles
+#endif
 #ifndef LS_GEMM_PD_SMALL
 #define LS_GEMM_PD_SMALL 4    // ... and of the 64 x 64 kernel (measured 1 to 4: 4 is 2 to 10 % ahead of 2)
 #endif
@@ -68,6 +78,8 @@ enum Epilogue : int {
   kAddF32 = 2,    // C[m][n] += total, float (residual stream)
   kSwiGLU = 3,    // W holds gate and up rows interleaved in tiles of 16 (gate rows 16t.., then up rows 16t..);
                   // C[m][16t + i] = (g * 1/(1 + exp(-g))) * u in float, stored in the compute dtype
+  kSliceSums = 4, // the tiled kernel only: C is float [slices][M][N] and gets the sums of the K slices, not their
+                  // total; the workgroups with blockIdx.y = y take the slices [y * out_cols, (y + 1) * out_cols)
 };
 
 __host__ __device__ inline int kslice_for(int K) { return 256 * ((K + 4095) / 4096); }
@@ -833,22 +845,38 @@ __global__ __launch_bounds__(64 * NWM * NWN) void gemm_tiled_kernel(const T* __r
     }
   };
 
-  const int stages = (K + BK - 1) / BK;
+  // the stages of this workgroup: all of K, or (kSliceSums) those of its group of slices
+  constexpr bool SLICES = EPI == kSliceSums;
+  const int all_stages = (K + BK - 1) / BK;
+  const int first_stage = SLICES ? (int)blockIdx.y * out_cols * (kslice / BK) : 0;
+  const int stages = SLICES ? min(all_stages - first_stage, out_cols * (kslice / BK)) : all_stages;
+  auto k_of = [&](int st) { return (first_stage + st) * BK; };
+  auto store_slice = [&](int slice) {  // the sums of one slice to their place among the slice sums
+    float* sums = reinterpret_cast<float*>(C) + (long)slice * M * N;
+#pragma unroll
+    for (int i = 0; i < TI; ++i)
+#pragma unroll
+      for (int j = 0; j < TJ; ++j) {
+        float t[4] = {acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]};
+        epilogue4<T, kStoreF32>(sums, ldc, m_base + wm + j * 16 + row16, n_base + wn + i * 16 + g * 4, M, N, t, vec_ok);
+      }
+  };
   // stage s lives in register slot s % PD until it is written to LDS buffer s % 2
-  fetch(0, 0);
-  stash(0, 0, 0);
+  fetch(0, k_of(0));
+  stash(0, 0, k_of(0));
   // (AL: stages past the end are fetched too, from clamped addresses: with no condition around a
   // fetch the compiler can count which loads are still in flight when a stage goes to LDS)
 #pragma unroll
   for (int u = 1; u <= PD; ++u)
-    if (AL || u < stages) fetch(u % PD, u * BK);
+    if (AL || u < stages) fetch(u % PD, k_of(u));
   for (int base = 0; base < stages; base += PD) {
 #pragma unroll
     for (int u = 0; u < PD; ++u) {  // unrolled so that the register slots are static
       const int st = base + u;
       if (st >= stages) break;
-      const int k0 = st * BK;
-      if (k0 > 0 && k0 % kslice == 0) {  // a stage never straddles a slice: kslice is a multiple of BK
+      const int k0 = k_of(st);
+      if (st > 0 && k0 % kslice == 0) {  // a stage never straddles a slice: kslice is a multiple of BK
+        if (SLICES) store_slice(k0 / kslice - 1);
 #pragma unroll
         for (int i = 0; i < TI; ++i)
 #pragma unroll
@@ -860,56 +888,66 @@ __global__ __launch_bounds__(64 * NWM * NWN) void gemm_tiled_kernel(const T* __r
       }
       __syncthreads();  // stage st is in its buffer; the other buffer has been read by every wave
       if (AL || st + 1 < stages) {  // (AL: past the last stage too, into the buffer that nobody reads any more)
-        stash((u + 1) % PD, (st + 1) & 1, (st + 1) * BK);
-        if (AL || st + 1 + PD < stages) fetch((u + 1) % PD, (st + 1 + PD) * BK);
+        stash((u + 1) % PD, (st + 1) & 1, k_of(st + 1));
+        if (AL || st + 1 + PD < stages) fetch((u + 1) % PD, k_of(st + 1 + PD));
       }
       const unsigned char* w_lds = lds + (st & 1) * STAGE_BYTES;
       const unsigned char* x_lds = w_lds + BN * kRowStride;
+      // the fragments of the second chunk are read while the first is multiplied
+      vec_t a[2][TI], b[2][TJ];
+      auto fragments = [&](int c) {
+#pragma unroll
+        for (int i = 0; i < TI; ++i)
+          a[c][i] = *reinterpret_cast<const vec_t*>(&w_lds[(wn + i * 16 + row16) * kRowStride + c * 64 + g * 16]);
+#pragma unroll
+        for (int j = 0; j < TJ; ++j)
+          b[c][j] = *reinterpret_cast<const vec_t*>(&x_lds[(wm + j * 16 + row16) * kRowStride + c * 64 + g * 16]);
+      };
+      fragments(0);
 #pragma unroll
       for (int c = 0; c < 2; ++c) {
         // The skinny kernel visits a chunk iff it starts below K; do the same.
         if (k0 + c * A::KCHUNK >= K) break;
-        vec_t a[TI], b[TJ];
-#pragma unroll
-        for (int i = 0; i < TI; ++i)
-          a[i] = *reinterpret_cast<const vec_t*>(&w_lds[(wn + i * 16 + row16) * kRowStride + c * 64 + g * 16]);
-#pragma unroll
-        for (int j = 0; j < TJ; ++j)
-          b[j] = *reinterpret_cast<const vec_t*>(&x_lds[(wm + j * 16 + row16) * kRowStride + c * 64 + g * 16]);
+        if (c == 0 && LS_GEMM_READ_AHEAD) fragments(1);
+        if (c == 1 && !LS_GEMM_READ_AHEAD) fragments(1);
 #pragma unroll
         for (int i = 0; i < TI; ++i)
 #pragma unroll
-          for (int j = 0; j < TJ; ++j) A::mma(acc[i][j], a[i], b[j]);
+          for (int j = 0; j < TJ; ++j) A::mma(acc[i][j], a[c][i], b[c][j]);
       }
     }
   }
+  if constexpr (SLICES) {
+    if (stages > 0) store_slice(k_of(stages - 1) / kslice);
+  } else {
 #pragma unroll
-  for (int i = 0; i < TI; ++i)
+    for (int i = 0; i < TI; ++i)
 #pragma unroll
-    for (int j = 0; j < TJ; ++j)
+      for (int j = 0; j < TJ; ++j)
 #pragma unroll
-      for (int r = 0; r < 4; ++r) total[i][j][r] = total[i][j][r] + acc[i][j][r];
+        for (int r = 0; r < 4; ++r) total[i][j][r] = total[i][j][r] + acc[i][j][r];
 
-  if (EPI == kSwiGLU) {
-    // the wave's weight tiles come in pairs (gate t, up t)
+    if (EPI == kSwiGLU) {
+      // the wave's weight tiles come in pairs (gate t, up t)
 #pragma unroll
-    for (int i = 0; i < TI; i += 2)
+      for (int i = 0; i < TI; i += 2)
+#pragma unroll
+        for (int j = 0; j < TJ; ++j) {
+          float gate[4] = {total[i][j][0], total[i][j][1], total[i][j][2], total[i][j][3]};
+          float up[4] = {total[i + 1][j][0], total[i + 1][j][1], total[i + 1][j][2], total[i + 1][j][3]};
+          epilogue_swiglu4<T>(C, ldc, m_base + wm + j * 16 + row16, (n_base + wn + i * 16) / 2 + g * 4, M, out_cols,
+                              gate, up, vec_ok);
+        }
+      return;
+    }
+#pragma unroll
+    for (int i = 0; i < TI; ++i)
 #pragma unroll
       for (int j = 0; j < TJ; ++j) {
-        float gate[4] = {total[i][j][0], total[i][j][1], total[i][j][2], total[i][j][3]};
-        float up[4] = {total[i + 1][j][0], total[i + 1][j][1], total[i + 1][j][2], total[i + 1][j][3]};
-        epilogue_swiglu4<T>(C, ldc, m_base + wm + j * 16 + row16, (n_base + wn + i * 16) / 2 + g * 4, M, out_cols, gate,
-                            up, vec_ok);
+        float t[4] = {total[i][j][0], total[i][j][1], total[i][j][2], total[i][j][3]};
+        epilogue4<T, EPI>(C, ldc, m_base + wm + j * 16 + row16, n_base + wn + i * 16 + g * 4, M, N, t, vec_ok);
       }
-    return;
   }
-#pragma unroll
-  for (int i = 0; i < TI; ++i)
-#pragma unroll
-    for (int j = 0; j < TJ; ++j) {
-      float t[4] = {total[i][j][0], total[i][j][1], total[i][j][2], total[i][j][3]};
-      epilogue4<T, EPI>(C, ldc, m_base + wm + j * 16 + row16, n_base + wn + i * 16 + g * 4, M, N, t, vec_ok);
-    }
 }
 
 // Compute units of the current device (asked once per device).
@@ -983,6 +1021,20 @@ int launch_gemm(const void* X, const void* W, void* C, int M, int N, int K, long
     else launched = false;
 #undef LS_STREAM
     if (launched) return check_launch("gemm");
+  }
+  // 32 to 64 rows over a product that neither fills the CUs with 64-column tiles nor has a streaming kernel
+  // for its slice length (QKV of Qwen3-14B and 32B sizes: slices of 512): the skinny kernel re-reads all
+  // rows of X for 16 columns a workgroup; tiles of 64 x 32 outputs where they give most CUs a workgroup
+  // (measured at 64 rows: N = 10,240, K = 5,120 83 -> 49 us; N = 7,168 56 -> 35 us; at 17 rows no gain).
+  if constexpr (EPI != kSwiGLU) {
+    if (LS_GEMM_NARROW && !norm_w && aligned && M >= 32 && M <= 64 && !tiled_fills && N < 32768 &&
+        (N + 31) / 32 >= compute_units() * 7 / 10) {
+      const int tiles_n = (N + 31) / 32;
+      hipLaunchKernelGGL((gemm_tiled_kernel<T, EPI, 64, 32, LS_GEMM_PD_SMALL, true, 2, 2>), dim3(tiles_n), dim3(256), 0,
+                         stream, reinterpret_cast<const T*>(X), w, C, M, N, K, ldx, ldc, kslice, vec_ok, 1, tiles_n,
+                         out_cols);
+      return check_launch("gemm");
+    }
   }
   if (M <= 64 && !tiled_fills && !(M > 16 && N >= 32768)) {
     const int mt = (M + 15) / 16;
@@ -1123,6 +1175,32 @@ extern "C" int ls_gemm_slices(int dtype, const void* X, const void* W, float* P,
   int rounds =
       (int)std::min<long>(4, (long)col_blocks * groups * std::max(row_groups, 1) / (2L * compute_units()));
   if (mt > 4 && rounds < 1) rounds = 1;  // more than 64 rows: this kernel only, if with one column block a workgroup
+  // Enough rows over weights large enough that 64 x 64 tiles times groups of slices give every CU a
+  // workgroup: the tiled kernel, which stages both operands in LDS four stages ahead and so keeps twice the
+  // bytes of the wide kernel in flight (measured at 64 rows, Qwen3-8B and 32B sizes: O 18.3 -> 12.4 and
+  // 44.9 -> 27.8 us, down 42.3 -> 30.3 and 119.9 -> 68.0 us; at 256 rows O 44.5 -> 30.4 and 147.9 -> 68.1 us).
+  // A workgroup takes as many slices as give it eight stages, fewer where that leaves CUs without one.
+  // From 17 rows on in bfloat16 (from 8 over weights of 64 MB and more, where the kernels of a wave a slice
+  // fall to 3.7 TB/s and this one holds 4.2 to 4.6; below that and over smaller weights those are ahead),
+  // from 33 rows on in float32.
+  const long weight_bytes = (long)N * K * (dtype == kF32 ? 4 : 2);
+  const int tiled_from = dtype == kF32 ? 33 : (weight_bytes >= (64L << 20) ? 8 : 17);
+  if (LS_GEMM_SLICES_TILED && aligned && M >= tiled_from && N % 4 == 0) {
+    const int stages_a_slice = kslice / (128 / (dtype == kF32 ? 4 : 2));
+    int per = std::min(nslices, std::max(1, (8 + stages_a_slice - 1) / stages_a_slice));
+    const int tiles_m = (M + 63) / 64, tiles_n = (N + 63) / 64;
+    auto workgroups = [&](int p) { return (long)tiles_m * tiles_n * ((nslices + p - 1) / p); };
+    while (per > 1 && workgroups(per) < compute_units()) per = (per + 1) / 2;
+    if (workgroups(per) >= compute_units()) {
+      dim3 tiled_grid(tiles_m * tiles_n, (nslices + per - 1) / per);
+#define LS_TILED_SLICES(T_)                                                                                          \
+  hipLaunchKernelGGL((gemm_tiled_kernel<T_, kSliceSums, 64, 64, LS_GEMM_PD_SMALL, true, 2, 2>), tiled_grid, dim3(256), \
+                     0, s, (const T_*)X, (const T_*)W, (void*)P, M, N, K, ldx, (long)N, kslice, 1, tiles_m, tiles_n, per)
+      if (dtype == kF32) { LS_TILED_SLICES(float); } else if (dtype == kBF16) { LS_TILED_SLICES(bf16_t); } else return fail("gemm_slices: unknown dtype %d", dtype);
+#undef LS_TILED_SLICES
+      return check_launch("gemm_slices");
+    }
+  }
   // More than 16 rows and enough columns that workgroups of 64 columns fill the GPU: the wide kernel.
   {
     const int wide_blocks = (N + 63) / 64;

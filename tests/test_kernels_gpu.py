@@ -81,6 +81,8 @@ def test_gemm_row_does_not_depend_on_the_batch(dtype):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("k,n", [(4096, 4096 + 24), (1000, 16384 + 24), (5120, 4096 + 104), (260, 32768 + 40),
+                                 # slices of 512 and some 7,000 columns: from 32 rows on tiles of 64 x 32 outputs
+                                 (5120, 7168 + 24), (1000, 6144 + 8),
                                  (2048, 8192 + 8), (96, 65536 + 48)])
 def test_gemm_with_few_rows_and_many_columns_has_the_same_bits(dtype, k, n):
     """With up to 64 rows and more column blocks than the GPU holds workgroups, a workgroup walks
