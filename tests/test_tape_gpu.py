@@ -66,7 +66,7 @@ def test_the_decode_loop_and_captured_steps_repeat_layers_too(deep_dirs):
 
     tokens = {}
     for flags in ({}, {"use_tapes": False}):
-        model = load(deep_dirs["B"], "bfloat16", **flags)
+        model = load(deep_dirs["B"], "bfloat16", **(flags or {"use_tapes": True, "verify_tapes": False}))
         cache = model.make_cache(num_pages=64, page_size=8, max_requests=3)
         firsts = []
         for i, n in enumerate((5, 33, 18)):
