@@ -68,6 +68,9 @@ namespace ls {
 #ifndef LS_GEMM_NARROW
 #define LS_GEMM_NARROW 1      // 0: never the 64 x 32 tiles
 #endif
+#ifndef LS_GEMM_ROWS64_WIDE
+#define LS_GEMM_ROWS64_WIDE 1 // 0: never 64 x 128 tiles for products of up to 64 rows
+#endif
 #ifndef LS_GEMM_PD_SMALL
 #define LS_GEMM_PD_SMALL 4    // ... and of the 64 x 64 kernel (measured 1 to 4: 4 is 2 to 10 % ahead of 2)
 #endif
@@ -1084,6 +1087,11 @@ int launch_gemm(const void* X, const void* W, void* C, int M, int N, int K, long
       if constexpr (sizeof(T) == 2) LS_TILED_WAVES(128, 256, LS_GEMM_PD_WIDE, true, 2, 4)
     }
     else if (big_tiles >= LS_GEMM_BIG && M > LS_GEMM_BIG_ROWS) LS_TILED(128, 128, LS_GEMM_PD_BIG, true)
+    // up to 64 rows over so many columns that tiles of 128 columns still give every CU a workgroup (the
+    // logits head, gate and up of 32B sizes): every workgroup reads all rows of X, so half as many
+    // workgroups halve that traffic (gate and up of 32B sizes at 64 rows 135 -> 112 us, the head 82 -> 77 us)
+    else if (LS_GEMM_ROWS64_WIDE && M <= 64 && (N + 127) / 128 >= cus)
+      LS_TILED_WAVES(64, 128, LS_GEMM_PD_SMALL, true, 2, 4)
     else LS_TILED(64, 64, LS_GEMM_PD_SMALL, true)
 #undef LS_TILED
 #undef LS_TILED_WAVES
@@ -1192,7 +1200,8 @@ extern "C" int ls_gemm_slices(int dtype, const void* X, const void* W, float* P,
     auto workgroups = [&](int p) { return (long)tiles_m * tiles_n * ((nslices + p - 1) / p); };
     while (per > 1 && workgroups(per) < compute_units()) per = (per + 1) / 2;
     if (workgroups(per) >= compute_units()) {
-      dim3 tiled_grid(tiles_m * tiles_n, (nslices + per - 1) / per);
+      const int groups_y = (nslices + per - 1) / per;
+      dim3 tiled_grid(tiles_m * tiles_n, groups_y);
 #define LS_TILED_SLICES(T_)                                                                                          \
   hipLaunchKernelGGL((gemm_tiled_kernel<T_, kSliceSums, 64, 64, LS_GEMM_PD_SMALL, true, 2, 2>), tiled_grid, dim3(256), \
                      0, s, (const T_*)X, (const T_*)W, (void*)P, M, N, K, ldx, (long)N, kslice, 1, tiles_m, tiles_n, per)
