@@ -249,3 +249,128 @@ def test_hidden_keys_state_what_a_dropped_key_would_give():
     keep = [0, 2, 3, 4]
     want = P.causal_attention(q[3:], k[keep], v[keep], q_positions=torch.tensor([2, 3]))
     assert torch.allclose(out[3:], want, atol=1e-14)
+
+
+# --------------------------------------------------------------------------
+# the wiring of a layer, composed by hand from library routines only
+# --------------------------------------------------------------------------
+
+def _one_layer(tmp_path, zero=()):
+    """A one-layer model whose norm weights are far from one and from each other, so that a norm
+    in the wrong place changes the logits; ``zero`` names projections whose weights are zeros."""
+    import json
+    from safetensors.torch import save_file
+
+    cfg = dict(model_type="qwen3", hidden_size=24, intermediate_size=40, num_hidden_layers=1,
+               num_attention_heads=6, num_key_value_heads=2, head_dim=8, vocab_size=37, rms_norm_eps=1e-5,
+               rope_theta=100.0, max_position_embeddings=64, tie_word_embeddings=False)
+    g = torch.Generator().manual_seed(5)
+    p = "model.layers.0"
+    w = {"model.embed_tokens.weight": torch.randn(37, 24, generator=g),
+         "model.norm.weight": 1 + 0.5 * torch.rand(24, generator=g),
+         "lm_head.weight": torch.randn(37, 24, generator=g) * 0.5,
+         f"{p}.input_layernorm.weight": 0.5 + torch.rand(24, generator=g),
+         f"{p}.post_attention_layernorm.weight": 1.5 + torch.rand(24, generator=g),
+         f"{p}.self_attn.q_proj.weight": torch.randn(48, 24, generator=g) * 0.4,
+         f"{p}.self_attn.k_proj.weight": torch.randn(16, 24, generator=g) * 0.4,
+         f"{p}.self_attn.v_proj.weight": torch.randn(16, 24, generator=g) * 0.4,
+         f"{p}.self_attn.o_proj.weight": torch.randn(24, 48, generator=g) * 0.4,
+         f"{p}.self_attn.q_norm.weight": 0.5 + torch.rand(8, generator=g),
+         f"{p}.self_attn.k_norm.weight": 1.5 + torch.rand(8, generator=g),
+         f"{p}.mlp.gate_proj.weight": torch.randn(40, 24, generator=g) * 0.4,
+         f"{p}.mlp.up_proj.weight": torch.randn(40, 24, generator=g) * 0.4,
+         f"{p}.mlp.down_proj.weight": torch.randn(24, 40, generator=g) * 0.4}
+    for name in zero:
+        w[f"{p}.{name}.weight"] = torch.zeros_like(w[f"{p}.{name}.weight"])
+    (tmp_path / "config.json").write_text(json.dumps(cfg))
+    save_file(w, str(tmp_path / "model.safetensors"))
+    return tmp_path
+
+
+def _rotate_by_complex_product(x, theta):
+    """The rotation as a product of complex numbers (no code of the plain implementation):
+    dimension i of a head is the real part and dimension i + d/2 the imaginary part of one number,
+    which turns by position * theta^(-2i/d)."""
+    t, heads, d = x.shape
+    half = d // 2
+    freq = torch.tensor([theta ** (-2.0 * i / d) for i in range(half)], dtype=torch.float64)
+    turn = torch.polar(torch.ones(t, half, dtype=torch.float64), torch.arange(t, dtype=torch.float64)[:, None] * freq)
+    z = torch.complex(x[..., :half], x[..., half:]) * turn[:, None, :]
+    return torch.cat([z.real, z.imag], dim=-1)
+
+
+def _layer_by_hand(model, ids, norms=("input_layernorm", "post_attention_layernorm"), parallel=False):
+    """One layer as the reference wires it (engine/model/qwen3.py:319-373), from library routines:
+    ``h = E[ids]; h = h + O(attn(norm_1(h))); h = h + down(silu(gate(norm_2(h))) * up(norm_2(h)));
+    logits = head(norm(h))``.  ``norms`` and ``parallel`` state the two plausible misreadings."""
+    cfg, w = model.cfg, model.w
+    p = "model.layers.0"
+    eps = cfg["rms_norm_eps"]
+    nq, nkv, d = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
+    hidden = cfg["hidden_size"]
+    t = len(ids)
+    h = F.embedding(torch.tensor(ids), w["model.embed_tokens.weight"])
+    x = F.rms_norm(h, (hidden,), w[f"{p}.{norms[0]}.weight"], eps)
+    q = F.linear(x, w[f"{p}.self_attn.q_proj.weight"]).view(t, nq, d)
+    k = F.linear(x, w[f"{p}.self_attn.k_proj.weight"]).view(t, nkv, d)
+    v = F.linear(x, w[f"{p}.self_attn.v_proj.weight"]).view(t, nkv, d)
+    q = _rotate_by_complex_product(F.rms_norm(q, (d,), w[f"{p}.self_attn.q_norm.weight"], eps), cfg["rope_theta"])
+    k = _rotate_by_complex_product(F.rms_norm(k, (d,), w[f"{p}.self_attn.k_norm.weight"], eps), cfg["rope_theta"])
+    g = nq // nkv
+    attn = F.scaled_dot_product_attention(
+        q.transpose(0, 1)[None], k.repeat_interleave(g, 1).transpose(0, 1)[None],
+        v.repeat_interleave(g, 1).transpose(0, 1)[None], is_causal=True, scale=d ** -0.5)[0].transpose(0, 1)
+    after_attention = h + F.linear(attn.reshape(t, nq * d), w[f"{p}.self_attn.o_proj.weight"])
+    x = F.rms_norm(h if parallel else after_attention, (hidden,), w[f"{p}.{norms[1]}.weight"], eps)
+    mlp = F.linear(F.silu(F.linear(x, w[f"{p}.mlp.gate_proj.weight"])) * F.linear(x, w[f"{p}.mlp.up_proj.weight"]),
+                   w[f"{p}.mlp.down_proj.weight"])
+    out = after_attention + mlp
+    return F.linear(F.rms_norm(out, (hidden,), w["model.norm.weight"], eps), w["lm_head.weight"])
+
+
+IDS = [3, 30, 7, 7, 19, 0, 36, 11, 2]
+
+
+def test_one_layer_equals_its_composition_from_library_routines(tmp_path):
+    """Pins the wiring: which norm feeds which part, and that the feed-forward reads the stream
+    after the attention's addition.  The two misreadings are computed too and must differ."""
+    model = P.PlainModel(_one_layer(tmp_path))
+    got = model.logits(IDS)
+    want = _layer_by_hand(model, IDS)
+    assert torch.allclose(got, want, atol=1e-10)
+    scale = float(want.abs().max())
+    swapped = _layer_by_hand(model, IDS, norms=("post_attention_layernorm", "input_layernorm"))
+    side_by_side = _layer_by_hand(model, IDS, parallel=True)
+    assert float((swapped - got).abs().max()) > 1e-2 * scale
+    assert float((side_by_side - got).abs().max()) > 1e-2 * scale
+
+
+@pytest.mark.parametrize("zeroed", ["self_attn.o_proj", "mlp.down_proj"])
+def test_half_zeroed_layers(tmp_path, zeroed):
+    """Only the attention's output projection zero: the layer is the feed-forward on the embedding,
+    under the second norm.  Only the down projection zero: the layer is the attention alone."""
+    model = P.PlainModel(_one_layer(tmp_path, zero=(zeroed,)))
+    cfg, w = model.cfg, model.w
+    p = "model.layers.0"
+    eps, hidden = cfg["rms_norm_eps"], cfg["hidden_size"]
+    got = model.logits(IDS)
+    assert torch.allclose(got, _layer_by_hand(model, IDS), atol=1e-10)
+    h = F.embedding(torch.tensor(IDS), w["model.embed_tokens.weight"])
+    if zeroed == "self_attn.o_proj":
+        x = F.rms_norm(h, (hidden,), w[f"{p}.post_attention_layernorm.weight"], eps)
+        h = h + F.linear(F.silu(F.linear(x, w[f"{p}.mlp.gate_proj.weight"])) * F.linear(x, w[f"{p}.mlp.up_proj.weight"]),
+                         w[f"{p}.mlp.down_proj.weight"])
+    else:
+        x = F.rms_norm(h, (hidden,), w[f"{p}.input_layernorm.weight"], eps)
+        h = h + P.attention_block(cfg, w, f"{p}.self_attn", x, torch.arange(len(IDS)))
+    want = F.linear(F.rms_norm(h, (hidden,), w["model.norm.weight"], eps), w["lm_head.weight"])
+    assert torch.allclose(got, want, atol=1e-10)
+    if zeroed == "self_attn.o_proj":
+        # the first norm's weight in the second one's place would show
+        x2 = F.rms_norm(F.embedding(torch.tensor(IDS), w["model.embed_tokens.weight"]), (hidden,),
+                        w[f"{p}.input_layernorm.weight"], eps)
+        h2 = F.embedding(torch.tensor(IDS), w["model.embed_tokens.weight"]) + F.linear(
+            F.silu(F.linear(x2, w[f"{p}.mlp.gate_proj.weight"])) * F.linear(x2, w[f"{p}.mlp.up_proj.weight"]),
+            w[f"{p}.mlp.down_proj.weight"])
+        wrong = F.linear(F.rms_norm(h2, (hidden,), w["model.norm.weight"], eps), w["lm_head.weight"])
+        assert float((wrong - got).abs().max()) > 1e-2 * float(got.abs().max())
