@@ -83,7 +83,9 @@ def test_gemm_row_does_not_depend_on_the_batch(dtype):
 @pytest.mark.parametrize("k,n", [(4096, 4096 + 24), (1000, 16384 + 24), (5120, 4096 + 104), (260, 32768 + 40),
                                  # slices of 512 and some 7,000 columns: from 32 rows on tiles of 64 x 32 outputs
                                  (5120, 7168 + 24), (1000, 6144 + 8),
-                                 (2048, 8192 + 8), (96, 65536 + 48)])
+                                 (2048, 8192 + 8), (96, 65536 + 48),
+                                 # K of 5,120 over so many columns that tiles of 64 x 128 give every CU one
+                                 (5120, 36864 + 72)])
 def test_gemm_with_few_rows_and_many_columns_has_the_same_bits(dtype, k, n):
     """With up to 64 rows and more column blocks than the GPU holds workgroups, a workgroup walks
     several column blocks with its rows of X in registers (the streaming kernel; beyond 32 rows two
@@ -153,7 +155,7 @@ def test_gemm_with_many_rows_and_columns_has_the_bits_of_few_rows(dtype, k):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("inter,k", [(4096 + 40, 4096), (16384 + 72, 1024)])
+@pytest.mark.parametrize("inter,k", [(4096 + 40, 4096), (16384 + 72, 1024), (25600, 5120)])
 def test_swiglu_with_few_rows_and_many_columns_has_the_same_bits(dtype, inter, k):
     from lockstep_amd.ops import SWIGLU, interleave_gate_up
 
@@ -170,6 +172,31 @@ def test_swiglu_with_few_rows_and_many_columns_has_the_same_bits(dtype, inter, k
         part = torch.empty(rows, inter, dtype=dtype, device="cuda")
         K().gemm(x[:rows], w, part, SWIGLU)
         assert torch.equal(part, full[:rows]), f"rows={rows}"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("k", [1024, 4096, 5120])
+def test_the_full_vocabulary_head_against_double_precision(dtype, k):
+    """151,936 columns (the streaming kernel for few rows, tiles of 64 x 128 up to 64 rows, large tiles
+    beyond) at 1, 8, 64 and 200 rows: every row equals the double-precision product and has the
+    same bits at every number of rows."""
+    from lockstep_amd.ops import STORE_F32
+
+    vocab = 151936
+    g = torch.Generator(device="cuda").manual_seed(k)
+    x = torch.randn(200, k, generator=g, device="cuda").to(dtype)
+    w = (torch.randn(vocab, k, generator=g, device="cuda") * 0.05).to(dtype)
+    want = torch.cat([x.double() @ w[lo:lo + 16384].double().T for lo in range(0, vocab, 16384)], dim=1)
+    full = None
+    for rows in (200, 1, 8, 64):
+        out = torch.full((rows, vocab), float("nan"), device="cuda")
+        K().gemm(x[:rows], w, out, STORE_F32)
+        assert rel_err(out, want[:rows]) < 2e-5, rows
+        if full is None:
+            full = out
+        assert torch.equal(out, full[:rows]), rows
+    del w, want, full
+    torch.cuda.empty_cache()
 
 
 @pytest.mark.parametrize("vocab", [7, 1000, 4099, 151936])
@@ -484,7 +511,7 @@ ATT_TOL = {torch.float32: 2e-5, torch.bfloat16: 2e-2}
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("nq,nkv,d,ps", [(16, 8, 128, 16), (4, 4, 16, 8), (8, 1, 64, 32), (6, 2, 48, 16),
-                                         (32, 4, 80, 64), (2, 2, 256, 128)])
+                                         (32, 4, 80, 64), (2, 2, 256, 128), (64, 8, 128, 16)])
 @pytest.mark.parametrize("kv_len", [1, 5, 64, 129, 257, 600])
 def test_prefill_attention_matches_naive(dtype, nq, nkv, d, ps, kv_len):
     qkv = rand_qkv(kv_len, nq, nkv, d, dtype, seed=kv_len + d)
@@ -650,7 +677,7 @@ def test_norm_rotation_and_cache_write(dtype):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("nq,nkv,d,ps", [(16, 8, 128, 16), (4, 4, 16, 8), (8, 1, 64, 32), (6, 2, 48, 16),
-                                         (32, 2, 80, 64), (2, 2, 256, 128), (3, 3, 32, 8)])
+                                         (32, 2, 80, 64), (2, 2, 256, 128), (3, 3, 32, 8), (64, 8, 128, 16)])
 def test_decode_attention_is_the_same_in_every_kernel(dtype, nq, nkv, d, ps):
     """The last one or two tokens of a sequence through the staged, the direct
     and the cooperative kernel, split or not: same bits, and right."""
@@ -678,7 +705,8 @@ def test_decode_attention_is_the_same_in_every_kernel(dtype, nq, nkv, d, ps):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("nq,nkv,d,ps", [(16, 8, 128, 16), (4, 4, 16, 8), (6, 2, 48, 16), (3, 3, 32, 8)])
+@pytest.mark.parametrize("nq,nkv,d,ps", [(16, 8, 128, 16), (4, 4, 16, 8), (6, 2, 48, 16), (3, 3, 32, 8),
+                                         (64, 8, 128, 16)])
 def test_cooperative_items_of_several_splits_leave_the_same_partial_results(dtype, nq, nkv, d, ps):
     """A long request cut into work items of one, two, three or four splits each (a partial result a
     split, folded by the combine kernel), laid out for more splits than it has, with and without
@@ -701,7 +729,8 @@ def test_cooperative_items_of_several_splits_leave_the_same_partial_results(dtyp
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("nq,nkv,d,ps", [(16, 8, 128, 16), (4, 4, 16, 8), (6, 2, 48, 16), (2, 1, 256, 16)])
+@pytest.mark.parametrize("nq,nkv,d,ps", [(16, 8, 128, 16), (4, 4, 16, 8), (6, 2, 48, 16), (2, 1, 256, 16),
+                                         (64, 8, 128, 16)])
 def test_the_fold_for_few_rows_has_the_bits_of_the_general_fold_over_many_splits(dtype, nq, nkv, d, ps):
     """Forty-one splits (more than two of the fold's rounds of sixteen), one and three tokens."""
     if not K().coop_supported(d, dtype, ps):
@@ -724,7 +753,7 @@ def test_the_fold_for_few_rows_has_the_bits_of_the_general_fold_over_many_splits
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("nq,nkv,d,ps,rot,normed,window", [
-    (16, 8, 128, 16, 128, True, 0), (8, 1, 64, 32, 64, True, 0), (4, 4, 16, 8, 16, True, 0),
+    (16, 8, 128, 16, 128, True, 0), (64, 8, 128, 16, 128, True, 0), (8, 1, 64, 32, 64, True, 0), (4, 4, 16, 8, 16, True, 0),
     (6, 2, 48, 16, 32, False, 0), (4, 2, 32, 8, 0, True, 0), (4, 2, 64, 16, 64, True, 200)])
 def test_fused_decode_attention_equals_the_separate_kernels(dtype, nq, nkv, d, ps, rot, normed, window):
     """A decoded token through qk_rope_kv + cooperative attention, and through the one fused launch:
@@ -850,7 +879,9 @@ def test_gemm_with_fused_norm_equals_norm_then_gemm(dtype, m, n, k):
 @pytest.mark.parametrize("n,k", [(1024, 3072), (96, 520), (1024, 2048), (40, 64), (4096, 1024), (5120, 96),
                                  (1028, 4096), (16384, 64), (16388, 64),
                                  # enough column blocks and slices that workgroups walk several blocks
-                                 (4104, 4096), (4104, 12288), (4200, 8192), (8200, 2048)])
+                                 (4104, 4096), (4104, 12288), (4200, 8192), (8200, 2048),
+                                 # K of 25,600: fifteen slices of 1,792 (the last one shorter)
+                                 (5120, 25600), (1032, 25600)])
 def test_slice_sums_and_fused_add_norm_equal_the_separate_kernels(dtype, m, n, k):
     """gemm_slices + add_rmsnorm give the bits of gemm(ADD_F32) + rmsnorm: the residual row and the
     normalised row; also for a list of rows and for the plain addition.  More than 64 rows (several

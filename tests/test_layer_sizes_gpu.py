@@ -1,5 +1,5 @@
 """The engine at the layer sizes of real models (one or two layers of them):
-head size 128, widths of 1,024 to 4,096, K cut into 4 to 16 slices.  These
+head size 128, widths of 1,024 to 5,120, K cut into 4 to 100 slices.  These
 sizes take other kernels and other paths inside the kernels than the tiny
 configurations do (128 x 128 tiles, the streaming and the walking products,
 the cooperative and the wide attention kernel at their full tile sizes), so
@@ -23,6 +23,11 @@ SIZES = {
     "8b-like": dict(hidden_size=4096, num_attention_heads=32, num_key_value_heads=8, head_dim=128,
                     intermediate_size=12288, num_hidden_layers=1, vocab_size=5003, tie_word_embeddings=False,
                     rms_norm_eps=1e-6, rope_theta=1000000.0, max_position_embeddings=2048),
+    # width 5,120 (K slices of 512), eight query heads a kv head (eight rows a decoded token), a feed-forward
+    # width of 25,600 (gate/up over 51,200 columns; the down product over 100 K slices of 256 = 15 of 1,792)
+    "32b-like": dict(hidden_size=5120, num_attention_heads=64, num_key_value_heads=8, head_dim=128,
+                     intermediate_size=25600, num_hidden_layers=1, vocab_size=5011, tie_word_embeddings=False,
+                     rms_norm_eps=1e-6, rope_theta=1000000.0, max_position_embeddings=2048),
 }
 
 
@@ -101,7 +106,7 @@ def test_many_requests_decode_with_the_bits_of_one(models, name):
     folder, config = models[name]
     model = load(folder, "bfloat16")
     vocab = config.vocab_size
-    n_req, n_decode = {"0.6b-like": 66, "8b-like": 40}[name], 3
+    n_req, n_decode = {"0.6b-like": 66, "8b-like": 40, "32b-like": 64}[name], 3
     lengths = [5 + (61 * i) % 400 for i in range(n_req)]
     prompts = [random_tokens(m + n_decode, vocab, seed=50 + i) for i, m in enumerate(lengths)]
     cache = model.make_cache(num_pages=sum(-(-(m + n_decode) // 16) for m in lengths) + 4, page_size=16,
@@ -219,21 +224,43 @@ def test_few_long_requests_are_cut_so_that_every_cu_has_work(tmp_path):
         assert token == int(picked[k][1]), k
 
 
-def test_the_32_bit_path_matches_plain_at_real_layer_sizes(models):
-    """float32 against the plain float64 implementation, and bfloat16 within its tolerance, on the
-    two-layer configuration (whole prompt and decoded tail)."""
+@pytest.mark.parametrize("name", list(SIZES))
+def test_both_paths_match_plain_at_real_layer_sizes(models, name):
+    """float32 against the plain float64 implementation, and bfloat16 within its tolerance: a whole
+    prompt and a decoded tail; then the last rows again out of a step of 40 requests (the kernels
+    that 17 to 64 rows take) and out of a portion of 200 tokens beside them."""
+    from lockstep_amd.engine.batch import StepEntry
     from plain.qwen3_plain import PlainModel
 
-    folder, config = models["0.6b-like"]
-    tokens = random_tokens(300, config.vocab_size, seed=9)
+    folder, config = models[name]
+    n = 300 if name == "0.6b-like" else 130
+    tokens = random_tokens(n, config.vocab_size, seed=9)
     want = PlainModel(folder).logits(tokens)
+    others = [random_tokens(3 + (7 * i) % 30, config.vocab_size, seed=200 + i) for i in range(39)]
     for dtype, tol in (("float32", FP32_TOL_SOFT), ("bfloat16", BF16_TOL)):
         model = load(folder, dtype)
-        cache = model.make_cache(num_pages=40, page_size=16)
-        got = feed(model, cache, "a", tokens, [270] + [1] * 30)
+        cache = model.make_cache(num_pages=40 + 3 * 40, page_size=16, max_requests=42)
+        got = feed(model, cache, "a", tokens, [n - 30] + [1] * 30)
         err = rel_err(got, want)
-        print(f"0.6b-like {dtype}: rel err {err:.3e}")
+        print(f"{name} {dtype}: rel err {err:.3e}")
         assert err < tol
+        # the last two tokens again, decoded in a step of 40 requests
+        cache.close("a")
+        for i, toks in enumerate(others):
+            cache.open(f"o{i}")
+        model.step(cache, [StepEntry(f"o{i}", toks[:-2], []) for i, toks in enumerate(others)])
+        cache.open("b")
+        model.step(cache, [StepEntry("b", tokens[:n - 2], [])])
+        rows = []
+        for k in range(2):
+            entries = [StepEntry(f"o{i}", [toks[len(toks) - 2 + k]], []) for i, toks in enumerate(others)]
+            entries.insert(17, StepEntry("b", [tokens[n - 2 + k]], [0]))
+            rows.append(model.step(cache, entries).cpu())
+        together = torch.cat(rows)
+        assert rel_err(together, want[n - 2:]) < tol
+        assert torch.equal(together, got[n - 2:]), "decoded among 40 requests: the bits of the request alone"
+        del model, cache
+        torch.cuda.empty_cache()
 
 
 def test_the_device_side_loop_at_real_layer_sizes(models):
