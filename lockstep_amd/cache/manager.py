@@ -324,7 +324,17 @@ class CacheManager:
     def shareable(self) -> bool:
         """Whole pages of a prefix can stand for the prefix only when every unit
         keeps all keys in pages: one group without a window and no state."""
-        return len(self.groups) == 1 and self.groups[0].spec.window is None and not self.state_units
+        return self.why_not_shareable() is None
+
+    def why_not_shareable(self):
+        """None if pages can be shared between requests, else the reason in words."""
+        if self.state_units:
+            return "a mixer keeps per-request state, which no page of keys and values stands for"
+        if len(self.groups) != 1:
+            return f"the layers' caches form {len(self.groups)} groups with page tables of their own"
+        if self.groups[0].spec.window is not None:
+            return "the layers keep a window of keys only, so early pages of a prefix are gone"
+        return None
 
     def adopt(self, request_id: Hashable, pages: Sequence[int]) -> None:
         """Map shared ``pages`` as the request's first logical pages."""

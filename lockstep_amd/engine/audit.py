@@ -18,28 +18,46 @@ import hashlib
 from collections import Counter
 from dataclasses import dataclass
 
+#: every path a run can be asked to prove it took: name -> what one count of it stands for.
+#: The names follow the reference's counters (engine/audit/counters.py:8-37) where it has the
+#: path, so that its relations can be stated against either engine.
 PATHS = {
-    "admit": "a waiting request was admitted",
-    "admit_refused": "the policy declined to admit a waiting request",
-    "admit_no_pages": "a request was admitted by the policy but its pages could not be reserved",
-    "resume": "a preempted request was admitted again",
-    "prefill_chunk": "a portion of a prompt (or of a recomputed context) ran",
-    "prefill_complete": "a prompt's last portion ran",
-    "decode_step": "a single decoded token ran",
-    "budget_deferred": "a request got no tokens this step because the token budget was spent",
-    "preempt_fired": "a running request was preempted for recompute",
-    "preempt_for_pages": "a running request was preempted because another could not grow",
-    "cache_hit": "a prefix hit was found and honoured",
-    "cache_hit_refused": "a prefix hit was found and the policy declined it",
-    "cache_miss": "a lookup found no usable prefix",
-    "cache_insert": "whole pages were indexed after a request finished",
-    "cache_full_prompt_trimmed": "a whole-prompt hit gave its last page back",
-    "eviction_taken": "an indexed page was reclaimed under pressure",
-    "finish": "a request finished and gave its pages back",
-    "finish_eos": "a request finished on an end-of-sequence token",
-    "finish_limit": "a request finished at max_new_tokens",
-    "out_of_pages": "nothing could run and nothing could be admitted",
-    "position_limit": "a request was refused because it would pass the model's last position",
+    # admission
+    "admit": "one request left the queue and got a slot and its pages",
+    "admit_refused": "the policy said no to a queued request (asked once per request and step)",
+    "admit_no_pages": "the policy said yes, but the pool could not cover the request even after evictions",
+    "resume": "the request admitted had been preempted before",
+    "position_limit": "submit turned a request down: prompt plus new tokens pass the model's last position",
+    "request_refused": "submit turned a request down for its fields (a uid in use, a value out of range)",
+    # what a step ran
+    "prefill_chunk": "a request ran more than its one newest token in a step (part of a prompt, or of a "
+                     "context that is computed again)",
+    "prefill_complete": "the step that cached the last prompt token of a request that has emitted nothing yet",
+    "decode_step": "a request ran exactly its newest token",
+    "budget_deferred": "the step's token budget was used up before this request's turn",
+    "chunk_boundary_mid_block": "a portion stopped short of its context's end at a position inside a page",
+    "chunk_boundary_on_block": "a portion stopped short of its context's end exactly where a page ends",
+    "chunk_boundary_mid_split": "a portion stopped short of its context's end inside an attention split",
+    "attention_multi_split": "a request's keys reached into a second attention split in this step",
+    "attention_single_split": "all keys of a request lay in the first attention split in this step",
+    # giving the cache up
+    "preempt_fired": "the policy asked for a running request's cache to be dropped",
+    "preempt_for_pages": "a request lost its cache so that another could take its next pages (lazy reservation)",
+    "preempt_depth_2": "the request preempted had been preempted once before",
+    "preempt_depth_3_plus": "the request preempted had been preempted at least twice before",
+    # prefix index
+    "cache_hit": "indexed pages matched a prompt's beginning and were mapped into the request",
+    "cache_hit_refused": "indexed pages matched, and the policy chose to compute them anyway",
+    "cache_miss": "no indexed page matched the prompt's beginning",
+    "cache_insert": "counts the pages a finished request added to the index",
+    "cache_full_prompt_trimmed": "the index held the whole prompt; its last page was left out so that the last "
+                                 "prompt token runs",
+    "eviction_taken": "a page that only the index held went back to the pool to make room",
+    # endings
+    "finish": "a request retired and its pages went back",
+    "finish_eos": "... because its newest token is an end-of-sequence id",
+    "finish_limit": "... because it has emitted max_new_tokens",
+    "out_of_pages": "a step found nothing running and nothing it could start",
 }
 
 
@@ -48,21 +66,32 @@ class VacuousRun(AssertionError):
 
 
 class Counters:
+    """How often a run took each declared path."""
+
     def __init__(self):
         self.counts: Counter = Counter()
 
     def hit(self, path: str, amount: int = 1) -> None:
-        if path not in PATHS:
-            raise KeyError(f"{path!r} is not a declared path; add it to PATHS with what firing it means")
-        self.counts[path] += amount
+        if path in PATHS:
+            self.counts[path] += amount
+            return
+        raise KeyError(f"{path!r} is not a declared path; add it to PATHS with what one count of it stands for")
 
     def __getitem__(self, path: str) -> int:
-        return self.counts.get(path, 0)
+        return self.counts[path]          # (a Counter answers 0 for what it never saw, without keeping it)
+
+    def never_taken(self, *paths: str) -> list:
+        """Those of ``paths`` (all declared ones if none are given) that the run did not take."""
+        return [p for p in (paths or PATHS) if self.counts[p] == 0]
 
     def require_fired(self, *paths: str) -> None:
-        missing = [p for p in paths if not self.counts.get(p)]
+        missing = self.never_taken(*paths) if paths else []
         if missing:
             raise VacuousRun(f"the run never took: {', '.join(missing)}")
+
+    def report(self) -> str:
+        """One line per path taken: count, name, what it stands for."""
+        return "\n".join(f"{n:8d}  {path}: {PATHS[path]}" for path, n in sorted(self.counts.items()) if n)
 
 
 def _digest(*chunks: bytes) -> bytes:

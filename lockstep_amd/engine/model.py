@@ -89,6 +89,13 @@ class Model:
         self._run_kinds = weakref.WeakKeyDictionary()      # cache manager -> (device epoch, RunKinds)
         self.layers_repeated = 0
 
+    @property
+    def split_keys(self):
+        """Keys of one attention split: the unit in which the mixers' kernels cut a request's keys
+        (the smallest, if mixers differ; None if no mixer cuts)."""
+        sizes = [layer.mixer.split_keys(self.rt) for layer in self.layers if hasattr(layer.mixer, "split_keys")]
+        return min(sizes) if sizes else None
+
     def _kinds_for(self, cache) -> RunKinds:
         held = self._run_kinds.get(cache)
         if held is None or held[0] != device_epoch():
@@ -149,11 +156,13 @@ class Model:
                 if not 0 <= w < len(e.tokens):
                     raise ValueError(f"request {e.request!r} wants logits at {w}, it brings {len(e.tokens)} tokens")
         limit = self.spec.max_positions
-        for e in entries:
+        for e in entries:                               # every request's bound before anything is taken for any
             start = cache.length(e.request)
             if limit is not None and start + len(e.tokens) > limit:
                 raise ValueError(f"request {e.request!r} would reach {start + len(e.tokens)} tokens; the model's "
                                  f"positions end at {limit}")
+        for e in entries:
+            start = cache.length(e.request)
             cache.reserve(e.request, start + len(e.tokens))
             if cache.ever_shared:
                 for gi in range(len(cache.groups)):
@@ -354,10 +363,11 @@ class Model:
         n = len(requests)
         starts = [cache.length(r) for r in requests]
         limit = self.spec.max_positions
-        for r, start in zip(requests, starts):
+        for r, start in zip(requests, starts):         # every request's bound before anything is taken for any
             if limit is not None and start + n_steps > limit:
                 raise ValueError(f"request {r!r} would reach {start + n_steps} tokens; the model's positions end "
                                  f"at {limit}")
+        for r, start in zip(requests, starts):
             cache.reserve(r, start + n_steps)          # every page the loop will write, now
             if cache.ever_shared:
                 for gi in range(len(cache.groups)):

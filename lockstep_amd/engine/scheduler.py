@@ -32,7 +32,10 @@ from __future__ import annotations
 
 from dataclasses import dataclass, field
 
+import math
+
 from ..cache import OutOfPages, PrefixIndex
+from . import lifecycle
 from .audit import Counters, StepLedger
 from .batch import StepEntry
 from .policy import DefaultPolicy, Event, Policy, View
@@ -101,6 +104,10 @@ class OversizedRequest(ValueError):
     """No state of the engine could ever run this request."""
 
 
+class InvalidRequest(ValueError):
+    """A field of the request is out of range, or its uid is already in use."""
+
+
 @dataclass
 class _Portion:
     seq: Sequence
@@ -149,6 +156,17 @@ class Scheduler:
         self.num_pages = min((g.pool.num_pages for g in cache.groups), default=num_blocks)
         self.max_positions = getattr(getattr(model, "spec", None), "max_positions", None)
         self.prefix = PrefixIndex(self.page_size) if enable_prefix_cache and cache.shareable() else None
+        #: why the prefix cache that was asked for is off (None: it is on, or was not asked for)
+        self.prefix_cache_refused = None
+        if enable_prefix_cache and self.prefix is None:
+            import warnings
+
+            self.prefix_cache_refused = cache.why_not_shareable()
+            warnings.warn(f"enable_prefix_cache was asked for, but this model's cache cannot share pages between "
+                          f"requests ({self.prefix_cache_refused}); requests are served without prefix reuse",
+                          RuntimeWarning, stacklevel=2)
+        #: keys of an attention split (None if the model does not say): the split counters are about these
+        self.split_keys = getattr(model, "split_keys", None)
         if sampler is None:
             from ..sampling import Sampler
 
@@ -163,6 +181,9 @@ class Scheduler:
         self.lifecycle: dict[str, list] = {}
         self.trajectory = StepLedger()
         self.emitted_logits: dict[str, list] = {}
+        self._known: set = set()                 # every uid this scheduler has accepted
+        self._states: dict = {}                  # uid -> lifecycle.State (kept while auditing)
+        self._steps_table = lifecycle.steps(self.lazy)
 
     @classmethod
     def from_config(cls, model, config, policy: Policy | None = None, **overrides) -> "Scheduler":
@@ -178,6 +199,13 @@ class Scheduler:
     # -- small helpers -----------------------------------------------------------------
     def _mark(self, uid: str, event: Event) -> None:
         self.lifecycle.setdefault(uid, []).append(event)
+        if self.audit_enabled:
+            state = self._states.get(uid, lifecycle.FIRST)
+            target = self._steps_table.get((state, event))
+            if target is None:
+                raise lifecycle.IllegalMark(f"step {self.step_index}: request {uid!r} is {state.value} and was "
+                                            f"marked {event.value}")
+            self._states[uid] = target
 
     def _pages_for(self, total_tokens: int) -> int:
         """Pages the neediest cache group takes for a request of that many tokens."""
@@ -198,9 +226,35 @@ class Scheduler:
                     reclaimable_pages=self.prefix.reclaimable(self.cache) if self.prefix else 0)
 
     # -- in ---------------------------------------------------------------------------------
+    def _refuse(self, message: str):
+        self.counters.hit("request_refused")
+        raise InvalidRequest(message)
+
     def submit(self, request: Request) -> None:
+        """Queue a request.  Everything that can be wrong with it is found here, before anything of
+        the scheduler has changed: a uid that this scheduler has seen before (waiting, running or
+        finished: records are kept by uid), an empty prompt, ``max_new_tokens`` below one, a negative
+        or non-finite ``temperature``, a ``top_p`` outside [0, 1], a size that no state of the engine
+        could hold."""
+        uid = request.uid
+        if uid in self._known:
+            where = ("waiting" if any(s.uid == uid for s in self.waiting) else
+                     "running" if any(s.uid == uid for s in self.running) else "finished")
+            self._refuse(f"a request with uid {uid!r} was submitted before (it is {where}); uids name the "
+                         "records of a run and the draws of its sampler, so each is used once")
         if not len(request.prompt):
-            raise ValueError(f"request {request.uid!r} has no prompt tokens")
+            self._refuse(f"request {uid!r} has no prompt tokens")
+        new = request.max_new_tokens
+        if isinstance(new, bool) or not isinstance(new, int) or new < 1:
+            self._refuse(f"request {uid!r}: max_new_tokens must be an integer of at least 1, got {new!r}")
+        for name, low, high in (("temperature", 0.0, math.inf), ("top_p", 0.0, 1.0)):
+            value = getattr(request, name)
+            if isinstance(value, bool) or not isinstance(value, (int, float)) or not low <= value <= high \
+                    or value == math.inf:
+                self._refuse(f"request {uid!r}: {name} must be a number in [{low}, {high}"
+                             f"{')' if high == math.inf else ']'}, got {value!r}")
+        if not isinstance(request.seed, int) or isinstance(request.seed, bool) or not 0 <= request.seed < 1 << 64:
+            self._refuse(f"request {uid!r}: seed must be an integer in [0, 2^64), got {request.seed!r}")
         total = len(request.prompt) + request.max_new_tokens
         if self.max_positions is not None and total > self.max_positions:
             self.counters.hit("position_limit")
@@ -213,6 +267,7 @@ class Scheduler:
                 f"request {request.uid!r} would hold {need} pages of {self.page_size} tokens for its {total} tokens; "
                 f"the pool has {self.num_pages} and a block table {self.cache.max_pages_per_request} columns, so it "
                 "could not run even alone")
+        self._known.add(uid)
         self.waiting.append(Sequence(request))
 
     # -- pages --------------------------------------------------------------------------
@@ -271,6 +326,10 @@ class Scheduler:
         self.running.remove(seq)
         self.waiting.insert(0, seq)
         self._mark(seq.uid, Event.PREEMPT)
+        if seq.preemptions == 2:
+            self.counters.hit("preempt_depth_2")
+        elif seq.preemptions > 2:
+            self.counters.hit("preempt_depth_3_plus")
 
     # -- the phases of a step -------------------------------------------------------------
     def _start_waiting(self) -> None:
@@ -279,7 +338,16 @@ class Scheduler:
             if self.cache.free_slots == 0 or not self.policy.admit(view, seq.uid, self._need(seq)):
                 self.counters.hit("admit_refused")
                 continue
+            # (the mark comes first: what starting does to the request -- a prefix hit, evictions -- follows it)
+            marks_before = len(self.lifecycle.get(seq.uid, ()))
+            state_before = self._states.get(seq.uid)
+            self._mark(seq.uid, Event.RESUME if seq.preemptions else Event.ADMIT)
             if not self._start(seq, view):
+                del self.lifecycle[seq.uid][marks_before:]          # it did not start after all
+                if state_before is None:
+                    self._states.pop(seq.uid, None)
+                else:
+                    self._states[seq.uid] = state_before
                 self.counters.hit("admit_no_pages")
                 continue
             self.waiting.remove(seq)
@@ -287,9 +355,6 @@ class Scheduler:
             self.counters.hit("admit")
             if seq.preemptions:
                 self.counters.hit("resume")
-                self._mark(seq.uid, Event.RESUME)
-            else:
-                self._mark(seq.uid, Event.ADMIT)
             view = self._view()
 
     def _preempt_on_request(self) -> None:
@@ -350,7 +415,19 @@ class Scheduler:
             else:
                 self.counters.hit("prefill_chunk")
                 self._mark(seq.uid, Event.DECODE if portion.samples else Event.CHUNK)
+            self._count_edges(seq.cached + count, portion.samples)
         return batch
+
+    def _count_edges(self, end: int, whole_context: bool) -> None:
+        """Where the tokens a request ran in this step end, relative to pages and attention splits
+        (the reference counts the same, engine/sched/scheduler.py:270-279)."""
+        hit = self.counters.hit
+        if not whole_context:
+            hit("chunk_boundary_mid_block" if end % self.page_size else "chunk_boundary_on_block")
+            if self.split_keys and end % self.split_keys:
+                hit("chunk_boundary_mid_split")
+        if self.split_keys:
+            hit("attention_multi_split" if end > self.split_keys else "attention_single_split")
 
     def _run_and_sample(self, batch: _Batch) -> None:
         entries = [StepEntry(p.seq.uid, p.seq.tokens[p.start:p.start + p.count], [p.count - 1] if p.samples else [])
@@ -462,6 +539,7 @@ class Scheduler:
                 seq.cached += 1
                 self.counters.hit("decode_step")
                 self._mark(seq.uid, Event.DECODE)
+                self._count_edges(seq.cached, True)
                 if int(token) in self.eos:
                     stopped.add(seq.uid)
             self.step_index += 1

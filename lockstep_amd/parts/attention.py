@@ -298,6 +298,10 @@ class Attention(Mixer):
         if hasattr(self.position, "bind"):
             self.position.bind(rt)      # layers with equal constants share their tables
 
+    def split_keys(self, rt) -> int:
+        """Keys of one split of the attention kernels for this head size."""
+        return int(rt.kernels.attention_geometry(self.d)[1])
+
     def prepare_group(self):
         share = getattr(self.position, "share_key", None)
         if share is None:

@@ -254,7 +254,13 @@ def test_sampled_tokens_depend_on_the_request_alone():
 
 
 def test_lifecycle_follows_the_state_machine():
-    legal = {
+    """Every life a run leaves walks the engine's own table (the scheduler checks each mark while
+    auditing; here the whole lives again), the table is the reference's under full reservation
+    (engine/sched/lifecycle.py:26-40), and a life that breaks it is refused."""
+    from lockstep_amd.engine import lifecycle
+    from lockstep_amd.engine.lifecycle import State
+
+    reference = {
         ("waiting", Event.ADMIT): "admitted", ("admitted", Event.EVICT): "admitted",
         ("admitted", Event.CACHE_HIT): "prefilling", ("admitted", Event.CHUNK): "prefilling",
         ("admitted", Event.DECODE): "decoding", ("prefilling", Event.CHUNK): "prefilling",
@@ -262,20 +268,199 @@ def test_lifecycle_follows_the_state_machine():
         ("prefilling", Event.EVICT): "prefilling", ("decoding", Event.DECODE): "decoding",
         ("decoding", Event.PREEMPT): "preempted", ("decoding", Event.FINISH): "done",
         ("preempted", Event.RESUME): "admitted",
-    }   # reference engine/sched/lifecycle.py:26-40
+    }
+    assert {(a.value, e): b.value for (a, e), b in lifecycle.STEPS.items()} == reference
+    assert lifecycle.reachable() == set(State) and lifecycle.reachable(lazy=True) == set(State)
     ps = prompts(9, 23, 40)
     _, s, _ = run(reqs(ps, n=8), policy=PreemptAtStepsPolicy("r1", (3, 6), chunk=7), max_batched_tokens=20)
     for uid, events in s.lifecycle.items():
-        state = "waiting"
-        for event in events:
-            assert (state, event) in legal, f"{uid}: {event} in state {state}"
-            state = legal[(state, event)]
-        assert state == "done"
+        assert lifecycle.follow(events) is State.DONE
+    # what the run's lives contain is among what the table allows, and the table allows more than one run takes
+    for n in (1, 2, 3):
+        seen = lifecycle.observed_runs(s.lifecycle, n)
+        assert seen and seen <= lifecycle.feasible_runs(n)
+    assert len(lifecycle.feasible_runs(1)) == len(Event)
+    assert (Event.PREEMPT, Event.RESUME) in lifecycle.feasible_runs(2)
+    assert (Event.FINISH, Event.ADMIT) not in lifecycle.feasible_runs(2)
+    assert lifecycle.feasible_runs(2) < lifecycle.feasible_runs(2, lazy=True)
+    with pytest.raises(lifecycle.IllegalMark, match="not allowed in state waiting"):
+        lifecycle.follow([Event.CHUNK])
+    with pytest.raises(lifecycle.IllegalMark, match="marks decode first"):
+        lifecycle.follow([Event.ADMIT, Event.FINISH])
+    with pytest.raises(lifecycle.IllegalMark):
+        lifecycle.follow([Event.ADMIT, Event.PREEMPT])                 # only lazy reservation does that
+    assert lifecycle.follow([Event.ADMIT, Event.PREEMPT], lazy=True) is State.PREEMPTED
     a = run(reqs(ps, n=8))[1].trajectory
     b = run(reqs(ps, n=8))[1].trajectory
     c = run(reqs(ps, n=8), policy=FixedChunkPolicy(7))[1].trajectory
     assert a.hexdigest() == b.hexdigest() and a.first_divergence(b) is None
     assert a.hexdigest() != c.hexdigest() and a.first_divergence(c) == 0
+
+
+def test_a_mark_the_table_forbids_stops_an_audited_run(monkeypatch):
+    """Positive control of the walk: a scheduler that marks a finished request once more is caught at
+    that mark when auditing, and not otherwise."""
+    from lockstep_amd.engine import lifecycle
+
+    original = Scheduler._retire
+
+    def retire_and_mark_again(self):
+        before = len(self.done)
+        original(self)
+        for seq in self.done[before:]:
+            self._mark(seq.uid, Event.DECODE)
+
+    monkeypatch.setattr(Scheduler, "_retire", retire_and_mark_again)
+    with pytest.raises(lifecycle.IllegalMark, match="is done and was marked decode"):
+        run(reqs(prompts(5), n=3))
+    run(reqs(prompts(5), n=3), audit=False)
+
+
+def test_lives_with_prefix_hits_evictions_and_lazy_preemption_follow_the_table():
+    """The marks around a start (admit, then the prefix hit and the evictions it causes), and under lazy
+    reservation the preemption of a request of which nothing has run yet."""
+    from lockstep_amd.engine import lifecycle
+
+    shared = prompts(32, seed=5)[0]
+    model = StandInModel()
+    s = Scheduler(model, num_blocks=12, block_size=8, enable_prefix_cache=True)
+
+    def serve(uid, prompt, n=4):
+        model.prompts[uid] = list(prompt)
+        s.submit(Request(uid=uid, prompt=list(prompt), max_new_tokens=n))
+        s.run()
+
+    serve("a", shared + [1, 2, 3])
+    serve("b", shared + [7, 8])
+    serve("d", prompts(80, seed=9)[0], n=8)                    # needs the indexed pages back
+    assert s.lifecycle["b"][:2] == [Event.ADMIT, Event.CACHE_HIT]
+    assert s.lifecycle["d"][:2] == [Event.ADMIT, Event.EVICT]
+    for events in s.lifecycle.values():
+        assert lifecycle.follow(events) is lifecycle.State.DONE
+
+    class Eager(DefaultPolicy):
+        def admit(self, state, uid, pages_needed):
+            return len(state.running) < self.max_running and state.free_pages >= 3
+
+    ps = prompts(20, 20, 20)
+    _, s, _ = run(reqs(ps, n=12), num_blocks=8, block_size=8, reserve="lazy", policy=Eager())
+    s.counters.require_fired("preempt_for_pages", "resume")
+    for events in s.lifecycle.values():
+        assert lifecycle.follow(events, lazy=True) is lifecycle.State.DONE
+
+
+def test_submit_refuses_before_anything_changes():
+    """A uid in use (waiting, running, finished), fields out of range: a typed error from ``submit``,
+    and the scheduler is as it was."""
+    from lockstep_amd.engine.scheduler import InvalidRequest
+
+    model = StandInModel()
+    s = Scheduler(model, num_blocks=16)
+
+    def state():
+        return ([q.uid for q in s.waiting], [q.uid for q in s.running], [q.uid for q in s.done],
+                s.cache.free_pages, s.cache.free_slots, dict(s.lifecycle))
+
+    model.prompts["a"] = [1, 2, 3]
+    s.submit(Request(uid="a", prompt=[1, 2, 3], max_new_tokens=3))
+    before = state()
+    with pytest.raises(InvalidRequest, match="it is waiting"):
+        s.submit(Request(uid="a", prompt=[4, 5]))
+    assert state() == before
+    s.step()
+    before = state()
+    with pytest.raises(InvalidRequest, match="it is running"):
+        s.submit(Request(uid="a", prompt=[4, 5]))
+    assert state() == before
+    s.run()
+    with pytest.raises(InvalidRequest, match="it is finished"):
+        s.submit(Request(uid="a", prompt=[4, 5]))
+    bad = [dict(max_new_tokens=0), dict(max_new_tokens=-3), dict(max_new_tokens=2.5), dict(max_new_tokens=True),
+           dict(temperature=-0.1), dict(temperature=float("nan")), dict(temperature=float("inf")),
+           dict(temperature="hot"), dict(top_p=1.5), dict(top_p=-0.01), dict(top_p=float("nan")),
+           dict(seed=-1), dict(seed=1 << 64), dict(seed=0.5), dict(prompt=[])]
+    before = state()
+    for i, fields in enumerate(bad):
+        with pytest.raises(InvalidRequest):
+            s.submit(Request(**{"uid": f"bad{i}", "prompt": [1, 2], **fields}))
+    assert state() == before and s.counters["request_refused"] == 3 + len(bad)
+    assert issubclass(InvalidRequest, ValueError)
+    # the edges that are allowed: greedy, a nucleus of nothing but the best token, the whole distribution
+    for i, fields in enumerate([dict(temperature=0), dict(temperature=0.0, top_p=0.0), dict(temperature=2.5, top_p=1),
+                                dict(seed=(1 << 64) - 1, max_new_tokens=1)]):
+        model.prompts[f"ok{i}"] = [1, 2]
+        s.submit(Request(**{"uid": f"ok{i}", "prompt": [1, 2], **fields}))
+    s.run()
+    # a uid that was refused for its size or fields was never taken: it may come again
+    with pytest.raises(OversizedRequest):
+        s.submit(Request(uid="big", prompt=[1] * 300, max_new_tokens=8))
+    model.prompts["big"] = [1] * 30
+    s.submit(Request(uid="big", prompt=[1] * 30, max_new_tokens=2))
+    s.submit(Request(uid="bad0", prompt=[1, 2]))
+    model.prompts["bad0"] = [1, 2]
+    assert set(s.run()) >= {"big", "bad0"}
+
+
+def test_edge_counters_say_where_portions_ended():
+    """Portions that end inside a page, on a page's edge and inside an attention split; contexts within one
+    split and beyond it; second and third preemptions of one request: the run can show that it
+    crossed them (the reference counts the same, engine/audit/counters.py:19-27)."""
+    model = StandInModel()
+    model.split_keys = 32
+    p = prompts(70, seed=4)[0]
+    model.prompts["r"] = p
+    s = Scheduler(model, num_blocks=16, block_size=8, policy=ScriptedPolicy(chunk_plan=[8, 5, 19, 3]))
+    s.submit(Request(uid="r", prompt=p, max_new_tokens=3))
+    out = s.run()
+    assert out["r"] == expected_greedy(p, 3)
+    c = s.counters
+    # ends at 8 (page edge), 13, 32 (page edge and split edge), 35, then the rest (the whole context: no edge)
+    assert c["chunk_boundary_on_block"] == 2 and c["chunk_boundary_mid_block"] == 2
+    assert c["chunk_boundary_mid_split"] == 3
+    assert c["attention_single_split"] == 3 and c["attention_multi_split"] == 2 + 2     # 35, 70, and two decoded tokens
+    c.require_fired("chunk_boundary_mid_block", "chunk_boundary_on_block", "chunk_boundary_mid_split",
+                    "attention_multi_split", "attention_single_split")
+    # a model that does not say how its attention is cut: the page counters only
+    quiet = run(reqs([p], n=2), policy=FixedChunkPolicy(20))[1].counters
+    assert quiet["chunk_boundary_mid_block"] == 3 and quiet["attention_multi_split"] == 0
+    with pytest.raises(AssertionError, match="never took: attention_multi_split"):
+        quiet.require_fired("chunk_boundary_mid_block", "attention_multi_split")
+    # preemption depth
+    ps = prompts(9, 23)
+    for steps, second, third in (((2,), 0, 0), ((2, 5), 1, 0), ((2, 4, 6, 9), 1, 2)):
+        _, s, _ = run(reqs(ps, n=10), policy=PreemptAtStepsPolicy("r0", steps, chunk=7))
+        assert (s.counters["preempt_depth_2"], s.counters["preempt_depth_3_plus"]) == (second, third)
+        assert s.counters["preempt_fired"] == len(steps)
+    assert "preempt_depth_2" in s.counters.report() and not s.counters.never_taken("resume")
+
+
+def test_a_prefix_cache_that_cannot_be_had_says_so():
+    """A cache with a window (or state) cannot share pages: asking for the prefix cache then warns once,
+    at construction, with the reason, and the scheduler records it."""
+    from lockstep_amd.parts import StateSpec
+
+    class Windowed(StandInModel):
+        def make_cache(self, num_pages, page_size=16, max_requests=64, max_tokens_per_request=None, **_):
+            return CacheManager([PagedKVSpec(1, 16, 24)], page_size, num_pages, max_requests,
+                                max_tokens_per_request or num_pages * page_size)
+
+    class Stateful(StandInModel):
+        def make_cache(self, num_pages, page_size=16, max_requests=64, max_tokens_per_request=None, **_):
+            return CacheManager([PagedKVSpec(1, 16, None), StateSpec((4,))], page_size, num_pages, max_requests,
+                                max_tokens_per_request or num_pages * page_size)
+
+    for model, reason in ((Windowed(), "window of keys"), (Stateful(), "per-request state")):
+        with pytest.warns(RuntimeWarning, match=reason):
+            s = Scheduler(model, num_blocks=16, block_size=8, enable_prefix_cache=True)
+        assert s.prefix is None and reason in s.prefix_cache_refused
+    import warnings
+
+    with warnings.catch_warnings():
+        warnings.simplefilter("error")
+        s = Scheduler(StandInModel(), num_blocks=16, block_size=8, enable_prefix_cache=True)
+        assert s.prefix is not None and s.prefix_cache_refused is None
+        s = Scheduler(Windowed(), num_blocks=16, block_size=8)
+        assert s.prefix_cache_refused is None
 
 
 def test_decode_bursts_change_neither_tokens_nor_counts():
