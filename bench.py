@@ -69,21 +69,21 @@ def build_model(args):
 
 
 class Workload:
-    """What a step costs, read from the model's own description (its parts' tensors and cache
-    units) rather than from one architecture's formulas: per run of a layer the elements of its
-    matrices and vectors, and for an attention mixer its heads; the head's matrix."""
+    """What a step costs, read from the model's own description rather than from one
+    architecture's formulas: per run of a layer the elements of its matrices and vectors; what
+    its mixer keeps between steps (``cache_spec()``: keys and values a token, or a state a
+    request) and what mixing costs beyond the matrices (``mixing_flops``); the head's matrix."""
 
     def __init__(self, model):
         from lockstep_amd.parts import part_class
 
         spec = model.spec
         per_layer = []
-        for layer in spec.layers:
-            tensors = part_class(layer.arrangement.kind).weight_specs(layer)
+        for layer_spec, layer in zip(spec.layers, model.layers):
+            tensors = part_class(layer_spec.arrangement.kind).weight_specs(layer_spec)
             matrices = sum(_numel(w.shape) for w in tensors if w.kind == "matrix")
             vectors = sum(_numel(w.shape) for w in tensors if w.kind != "matrix")
-            mixer = layer.mixer.params if layer.mixer.kind == "attention" else None
-            per_layer.append((matrices, vectors, mixer))
+            per_layer.append((matrices, vectors, layer.mixer))
         self.runs = [per_layer[run.layer] for run in spec.schedule]
         self.writers = [per_layer[run.layer][2] for run in spec.schedule if run.writes_cache]
         self.head = spec.vocab_size * spec.hidden_size
@@ -94,25 +94,31 @@ class Workload:
         one request with ``wanted`` logit rows."""
         total = 2.0 * wanted * self.head
         for matrices, _, mixer in self.runs:
-            total += 2.0 * tokens * matrices
-            if mixer is not None:
-                window = mixer.get("window")
-                pairs = sum(min(start + i + 1, window or start + i + 1) for i in range(tokens))   # visible (query, key) pairs
-                total += 4.0 * mixer["head_dim"] * mixer["num_heads"] * pairs
+            total += 2.0 * tokens * matrices + (mixer.mixing_flops(tokens, start) if mixer is not None else 0.0)
         return total
 
     def decode_bytes(self, batch: int, context: float, element: int) -> float:
-        """Bytes a decode step has to read: every weight it uses once, and the cache of the
-        live requests."""
+        """Bytes a decode step has to read: every weight it uses once, and what the mixers hold
+        of the live requests."""
         weights = sum(matrices * element + vectors * 4 for matrices, vectors, _ in self.runs)
         weights += self.head * element + self.hidden * 4                     # head and final norm
         weights += batch * self.hidden * element                             # embedding rows
-        kv = 0.0
-        for mixer in self.writers:
-            if mixer is not None:
-                held = min(context, mixer.get("window") or context)
-                kv += batch * held * 2 * mixer["num_kv_heads"] * mixer["head_dim"] * element
-        return weights + kv
+        held = sum(batch * cache_bytes(mixer.cache_spec(), context, element) for mixer in self.writers
+                   if mixer is not None)
+        return weights + held
+
+
+def cache_bytes(spec, context: float, element: int) -> float:
+    """Bytes one request of ``context`` tokens holds in a cache unit of this description."""
+    from lockstep_amd.parts import PagedKVSpec, StateSpec
+
+    if spec is None:
+        return 0.0
+    if isinstance(spec, PagedKVSpec):
+        return min(context, spec.window or context) * 2 * spec.num_kv_heads * spec.head_dim * element
+    if isinstance(spec, StateSpec):
+        return _numel(spec.shape) * {"float32": 4, "int32": 4, "bfloat16": 2}[spec.dtype]
+    raise TypeError(f"a cache unit described by {type(spec).__name__}: bench.py does not know its size")
 
 
 def _numel(shape) -> int:
@@ -120,6 +126,39 @@ def _numel(shape) -> int:
     for size in shape:
         n *= int(size)
     return n
+
+
+def gpu_state() -> dict:
+    """Clocks and temperatures of the GPU at this moment, as ``rocm-smi`` reports them (the
+    reference records the same beside its measurements, bench/throughput.py:88-104); empty if
+    the tool is missing or says nothing."""
+    import re
+    import subprocess
+
+    try:
+        out = subprocess.run(["rocm-smi", "--showclocks", "--showtemp", "--showpower", "--json"],
+                             capture_output=True, text=True, timeout=20).stdout
+        cards = json.loads(out[out.index("{"):])
+    except (OSError, ValueError, subprocess.SubprocessError):
+        return {}
+    card = cards.get("card0") or next(iter(cards.values()), {})
+    state = {}
+    for key, value in card.items():
+        number = re.search(r"-?\d+(\.\d+)?", str(value))
+        if number is None:
+            continue
+        low = key.lower()
+        for name, wanted in (("sclk_mhz", "sclk clock speed"), ("mclk_mhz", "mclk clock speed"),
+                             ("fclk_mhz", "fclk clock speed"), ("temp_junction_c", "sensor junction"),
+                             ("temp_memory_c", "sensor memory"), ("power_w", "power (w)")):
+            if wanted in low:
+                state[name] = float(number.group())
+    return state
+
+
+def states_record(before: dict, after: dict) -> dict:
+    """Two readings of ``gpu_state`` as one flat record."""
+    return {**{f"{k}_before": v for k, v in before.items()}, **{f"{k}_after": v for k, v in after.items()}}
 
 
 def random_prompts(n: int, length: int, vocab: int, seed: int):
@@ -359,8 +398,10 @@ def serve_record(args, model, cfg, full_layers) -> dict:
         chunk = args.prefill_chunk or None
     if args.new_tokens:
         new_tokens = args.new_tokens
+    state_before = gpu_state()
     passes = measure_serve(model, prompts, new_tokens, chunk, args.page_size, args.max_batched_tokens,
                            args.repeats, args.temperature, args.top_p)
+    state_after = gpu_state()
     order = sorted(passes, key=lambda t: t[0])
     elapsed, prompts_done, steps, decode_steps = order[len(order) // 2]
     prompt_tokens = sum(len(p) for p in prompts)
@@ -398,6 +439,7 @@ def serve_record(args, model, cfg, full_layers) -> dict:
             "decode_only_step_ms": round(1e3 * decode_seconds / decode_steps, 4) if decode_steps else None,
             "sampling": "greedy" if args.temperature <= 0 else f"temperature {args.temperature}, top_p {args.top_p}",
         },
+        "gpu_state": states_record(state_before, state_after),
     }
 
 
@@ -454,8 +496,10 @@ def main(argv=None) -> int:
                                       "ms": round(1e3 * seconds, 3)}}))
         return 0
 
+    state_before = gpu_state()
     times, context = measure_decode(model, cfg, args.batch, args.prompt_len, args.steps, args.warmup,
                                     args.page_size, not args.host_sampling, args.repeats)
+    state_after = gpu_state()
     elapsed = statistics.median(times)
     ms_per_step = 1e3 * elapsed / args.steps
     value = args.batch * args.steps / elapsed
@@ -490,6 +534,8 @@ def main(argv=None) -> int:
         "spread": spread(times, args.steps),
         "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": PEAK_HBM / 1e9,
                      "unit": "GB/s", "frac": round(achieved / PEAK_HBM, 4)},
+        # clocks and temperatures right before and right after the headline's timed runs
+        "gpu_state": states_record(state_before, state_after),
     }
 
     if not args.no_points:

@@ -38,18 +38,52 @@ class PartSpec:
 
 @dataclass(frozen=True)
 class LayerSpec:
-    """One layer: parts and the arrangement that wires them.
+    """One layer: an arrangement and the parts it wires.
 
     ``prefix`` is the layer's tensor-name prefix in the checkpoint, e.g.
     ``model.layers.3``; each part appends its own names to it.
+
+    The four named fields are the common case (one mixer, one feed-forward, a
+    norm in front of each) and are all optional: an arrangement reads the parts
+    it knows by name with ``part(name)`` and need not use these names at all.
+    Whatever else a layer is made of (a norm behind each part as well, a second
+    feed-forward, a gate) goes into ``parts``, an open mapping from names of the
+    arrangement's choosing to ``PartSpec``s.
     """
 
     prefix: str
     arrangement: PartSpec
-    mixer: PartSpec
-    feed_forward: PartSpec
-    mixer_norm: PartSpec
-    feed_forward_norm: PartSpec
+    mixer: PartSpec | None = None
+    feed_forward: PartSpec | None = None
+    mixer_norm: PartSpec | None = None
+    feed_forward_norm: PartSpec | None = None
+    parts: Mapping[str, PartSpec] = field(default_factory=dict)
+
+    COMMON = ("mixer", "feed_forward", "mixer_norm", "feed_forward_norm")
+
+    def __post_init__(self):
+        clash = [name for name in self.parts if name in self.COMMON or name in ("prefix", "arrangement", "parts")]
+        if clash:
+            raise ConfigError(f"layer {self.prefix!r}: the names {clash} in 'parts' are fields of the layer itself")
+        wrong = [name for name, spec in self.named_parts().items() if not isinstance(spec, PartSpec)]
+        if wrong:
+            raise ConfigError(f"layer {self.prefix!r}: the parts {wrong} are not PartSpecs")
+
+    def named_parts(self) -> dict:
+        """Every part of the layer by name: the common fields that are set, then ``parts``."""
+        out = {name: getattr(self, name) for name in self.COMMON if getattr(self, name) is not None}
+        out.update(self.parts)
+        return out
+
+    def part(self, name: str) -> PartSpec:
+        found = self.named_parts().get(name)
+        if found is None:
+            raise ConfigError(f"layer {self.prefix!r} has no part named {name!r}; it has: "
+                              f"{', '.join(self.named_parts()) or 'none'}")
+        return found
+
+    def has(self, name: str) -> bool:
+        return name in self.named_parts()
 
 
 @dataclass(frozen=True)

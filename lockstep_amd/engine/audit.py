@@ -35,6 +35,8 @@ PATHS = {
     "prefill_complete": "the step that cached the last prompt token of a request that has emitted nothing yet",
     "decode_step": "a request ran exactly its newest token",
     "budget_deferred": "the step's token budget was used up before this request's turn",
+    "decode_burst": "a run of decode steps went through the device-side loop in one call",
+    "burst_on_shared_prefix": "... while a request in it read pages adopted from the prefix index",
     "chunk_boundary_mid_block": "a portion stopped short of its context's end at a position inside a page",
     "chunk_boundary_on_block": "a portion stopped short of its context's end exactly where a page ends",
     "chunk_boundary_mid_split": "a portion stopped short of its context's end inside an attention split",

@@ -77,6 +77,8 @@ class Model:
         # one mixer of each group of equal ones is asked to prepare a step
         seen, self._preparers = set(), []
         for layer in self.layers:
+            if layer.mixer is None:                    # a layer without a mixer keeps and prepares nothing
+                continue
             group = layer.mixer.prepare_group()
             if group is None or group not in seen:
                 self._preparers.append(layer.mixer)
@@ -94,6 +96,7 @@ class Model:
         """Keys of one attention split: the unit in which the mixers' kernels cut a request's keys
         (the smallest, if mixers differ; None if no mixer cuts)."""
         sizes = [layer.mixer.split_keys(self.rt) for layer in self.layers if hasattr(layer.mixer, "split_keys")]
+        # (a layer without a mixer has ``mixer`` None, which has no such method)
         return min(sizes) if sizes else None
 
     def _kinds_for(self, cache) -> RunKinds:
@@ -121,8 +124,9 @@ class Model:
     def cache_unit_specs(self) -> list:
         units = [None] * self.spec.cache_units()
         for run in self.schedule:
-            if run.writes_cache:
-                units[run.cache] = self.layers[run.layer].mixer.cache_spec()
+            mixer = self.layers[run.layer].mixer
+            if run.writes_cache and mixer is not None:
+                units[run.cache] = mixer.cache_spec()
         return units
 
     def make_cache(self, num_pages: int, page_size: int = 16, max_requests: int = 64,

@@ -528,6 +528,9 @@ class Scheduler:
                 return False
         else:
             picked = self.model.decode_greedy(self.cache, uids, last, steps)
+        self.counters.hit("decode_burst")
+        if any(s.reused for s in self.running):
+            self.counters.hit("burst_on_shared_prefix")
         # A request that draws an end-of-sequence id stops there: the steps the loop ran for it beyond that
         # are dropped (its pages go back when it retires below; the others' tokens do not depend on it).
         stopped = set()

@@ -298,6 +298,12 @@ class Attention(Mixer):
         if hasattr(self.position, "bind"):
             self.position.bind(rt)      # layers with equal constants share their tables
 
+    def mixing_flops(self, tokens: int, start: int) -> float:
+        """Scores and value products over the (query, key) pairs a query sees."""
+        window = int(self.window) if self.window is not None else None
+        pairs = sum(min(start + i + 1, window or start + i + 1) for i in range(tokens))
+        return 4.0 * self.d * self.nq * pairs
+
     def split_keys(self, rt) -> int:
         """Keys of one split of the attention kernels for this head size."""
         return int(rt.kernels.attention_geometry(self.d)[1])

@@ -162,6 +162,11 @@ class Mixer(Part):
         (one of them is called); None: always call this one."""
         return None
 
+    def mixing_flops(self, tokens: int, start: int) -> float:
+        """Multiply-adds times two that mixing ``tokens`` new tokens of one request at positions
+        ``start``.. costs beyond the part's matrix products (measurements price a step with it)."""
+        return 0.0
+
     def forward(self, ctx, run, x, out, accumulate: bool) -> None:
         raise NotImplementedError
 
@@ -182,7 +187,9 @@ class Arrangement(Part):
         raise NotImplementedError
 
     @property
-    def mixer(self) -> Mixer:
+    def mixer(self):
+        """The part that owns the layer's unit of the cache and prepares its steps: a ``Mixer``,
+        or None for a layer that mixes nothing."""
         raise NotImplementedError
 
     def forward(self, ctx, run, h) -> None:

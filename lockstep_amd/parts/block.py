@@ -22,11 +22,11 @@ class PreNormResidual(Arrangement):
         super().__init__(layer_spec, build_part)
         p = layer_spec.arrangement.params
         base = layer_spec.prefix
-        self.mixer_norm = build_part(layer_spec.mixer_norm, self.join(base, p["mixer_norm_name"]))
-        self._mixer = build_part(layer_spec.mixer, self.join(base, p["mixer_prefix"]))
-        self.feed_forward_norm = build_part(layer_spec.feed_forward_norm,
+        self.mixer_norm = build_part(layer_spec.part("mixer_norm"), self.join(base, p["mixer_norm_name"]))
+        self._mixer = build_part(layer_spec.part("mixer"), self.join(base, p["mixer_prefix"]))
+        self.feed_forward_norm = build_part(layer_spec.part("feed_forward_norm"),
                                             self.join(base, p["feed_forward_norm_name"]))
-        self.feed_forward = build_part(layer_spec.feed_forward, self.join(base, p["feed_forward_prefix"]))
+        self.feed_forward = build_part(layer_spec.part("feed_forward"), self.join(base, p["feed_forward_prefix"]))
         self._fuse_mixer = self._fuses(self._mixer, self.mixer_norm)
         self._fuse_ff = self._fuses(self.feed_forward, self.feed_forward_norm)
         # parts that can leave their residual addition to the next norm (see PendingAdd)
@@ -42,10 +42,10 @@ class PreNormResidual(Arrangement):
         p = layer_spec.arrangement.params
         base = layer_spec.prefix
         out = []
-        for spec, name in ((layer_spec.mixer_norm, p["mixer_norm_name"]),
-                           (layer_spec.mixer, p["mixer_prefix"]),
-                           (layer_spec.feed_forward_norm, p["feed_forward_norm_name"]),
-                           (layer_spec.feed_forward, p["feed_forward_prefix"])):
+        for spec, name in ((layer_spec.part("mixer_norm"), p["mixer_norm_name"]),
+                           (layer_spec.part("mixer"), p["mixer_prefix"]),
+                           (layer_spec.part("feed_forward_norm"), p["feed_forward_norm_name"]),
+                           (layer_spec.part("feed_forward"), p["feed_forward_prefix"])):
             out += part_class(spec.kind).weight_specs(spec, cls.join(base, name))
         return out
 

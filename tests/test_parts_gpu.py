@@ -737,3 +737,184 @@ def test_toy_routed_feed_forward_and_toy_position_encoding(tmp_path, routed):
         unregister_part("toy_linear_angles")
         unregister_part("toy_top1_experts")
         unregister_architecture(RoutedToyConfig)
+
+
+# ---------------------------------------------------------------------------
+# a third toy, for the shape of a layer itself: an arrangement with a norm in
+# front of and behind each part (four norms), and one that is a feed-forward
+# and nothing else -- parts beyond the common four travel in ``LayerSpec.parts``
+# ---------------------------------------------------------------------------
+
+def _register_sandwich_toy():
+    from lockstep_amd.config import (LayerSpec, ModelConfig, ModelSpec, PartSpec, ScheduleEntry,
+                                     register_architecture)
+    from lockstep_amd.parts import Arrangement, build_part, part_class, register_part
+
+    @register_part("toy_sandwich")
+    class Sandwich(Arrangement):
+        """``h += after_mixer(mixer(before_mixer(h))); h += after_ff(ff(before_ff(h)))``."""
+
+        graph_safe = True
+        NAMES = ("before_mixer", "mixer", "after_mixer", "before_ff", "ff", "after_ff")
+
+        def __init__(self, layer_spec, prefix=""):
+            super().__init__(layer_spec, build_part)
+            for name in self.NAMES:
+                setattr(self, f"p_{name}", build_part(layer_spec.part(name), self.join(layer_spec.prefix, name)))
+
+        @classmethod
+        def weight_specs(cls, layer_spec, prefix=""):
+            return [w for name in cls.NAMES
+                    for w in part_class(layer_spec.part(name).kind).weight_specs(layer_spec.part(name),
+                                                                                 cls.join(layer_spec.prefix, name))]
+
+        def parts(self):
+            return tuple(getattr(self, f"p_{name}") for name in self.NAMES)
+
+        mixer = property(lambda self: self.p_mixer)
+
+        def load(self, weights, rt):
+            for part in self.parts():
+                part.load(weights, rt)
+
+        def forward(self, ctx, run, h):
+            rt, t, width = ctx.rt, ctx.n_tokens, h.shape[1]
+            x = ctx.buf("sandwich.x", (t, width), rt.dtype)
+            y = ctx.buf("sandwich.y", (t, width), torch.float32)
+            z = ctx.buf("sandwich.z", (t, width), torch.float32)
+            for before, part, after in ((self.p_before_mixer, self.p_mixer, self.p_after_mixer),
+                                        (self.p_before_ff, self.p_ff, self.p_after_ff)):
+                before.forward(ctx, h, x)
+                if part is self.p_mixer:
+                    part.forward(ctx, run, x, y, accumulate=False)
+                else:
+                    part.forward(ctx, x, y, accumulate=False)
+                after.forward(ctx, y, z)                  # normalised into float32: the stream's own dtype
+                h.add_(z)
+
+    @register_part("toy_ff_only")
+    class FeedForwardOnly(Arrangement):
+        """``h += ff(norm(h))``: a layer that mixes nothing and keeps nothing."""
+
+        graph_safe = True
+
+        def __init__(self, layer_spec, prefix=""):
+            super().__init__(layer_spec, build_part)
+            self.norm = build_part(layer_spec.part("feed_forward_norm"), self.join(layer_spec.prefix, "norm"))
+            self.ff = build_part(layer_spec.part("feed_forward"), self.join(layer_spec.prefix, "ff"))
+
+        @classmethod
+        def weight_specs(cls, layer_spec, prefix=""):
+            norm, ff = layer_spec.part("feed_forward_norm"), layer_spec.part("feed_forward")
+            return (part_class(norm.kind).weight_specs(norm, cls.join(layer_spec.prefix, "norm"))
+                    + part_class(ff.kind).weight_specs(ff, cls.join(layer_spec.prefix, "ff")))
+
+        def parts(self):
+            return (self.norm, self.ff)
+
+        mixer = property(lambda self: None)
+
+        def load(self, weights, rt):
+            self.norm.load(weights, rt)
+            self.ff.load(weights, rt)
+
+        def forward(self, ctx, run, h):
+            x = ctx.buf("ff_only.x", (ctx.n_tokens, h.shape[1]), ctx.rt.dtype)
+            self.norm.forward(ctx, h, x)
+            self.ff.forward(ctx, x, h, accumulate=True)
+
+    @register_architecture
+    @dataclass(frozen=True)
+    class SandwichConfig(ModelConfig):
+        hidden_size: int
+        vocab_size: int
+        architecture_names = ("toy-sandwich",)
+
+        def model_spec(self):
+            h = self.hidden_size
+
+            def norm(eps):
+                return PartSpec("rmsnorm", {"size": h, "eps": eps})
+
+            ff = PartSpec("gated_mlp", {"hidden_size": h, "intermediate_size": 3 * h, "activation": "silu"})
+            attn = PartSpec("attention", {"hidden_size": h, "num_heads": 4, "num_kv_heads": 2, "head_dim": 16,
+                                          "qk_norm": None,
+                                          "position": PartSpec("rope_half", {"rotary_dim": 16, "theta": 50.0}),
+                                          "window": None, "bias": False, "scale": 0.25})
+            sandwich = LayerSpec("layers.0", PartSpec("toy_sandwich"), mixer=attn,
+                                 parts={"before_mixer": norm(1e-5), "after_mixer": norm(1e-4), "before_ff": norm(1e-3),
+                                        "ff": ff, "after_ff": norm(1e-2)})
+            ff_only = LayerSpec("layers.1", PartSpec("toy_ff_only"), feed_forward=ff, feed_forward_norm=norm(1e-5))
+            return ModelSpec(
+                hidden_size=h, vocab_size=self.vocab_size,
+                embedding=PartSpec("token_embedding", {"name": "embed.weight", "vocab_size": self.vocab_size,
+                                                       "hidden_size": h}),
+                layers=(sandwich, ff_only),
+                # the layer without a mixer names a cache unit like every run; it keeps nothing in it
+                schedule=(ScheduleEntry(0, 0, True), ScheduleEntry(1, 1, True), ScheduleEntry(1, 1, True)),
+                final_norm=PartSpec("rmsnorm", {"size": h, "eps": 1e-5, "name": "final_norm.weight"}),
+                head=PartSpec("linear_head", {"name": "head.weight", "tied_to": None,
+                                              "vocab_size": self.vocab_size, "hidden_size": h}))
+
+    return SandwichConfig
+
+
+def _sandwich_plain(w, tokens, hidden):
+    t = len(tokens)
+    h = w["embed.weight"][torch.tensor(tokens)]
+    cos, sin = P.rope_tables(16, 50.0, torch.arange(t))
+    p = "layers.0"
+    x = P.rmsnorm(h, w[f"{p}.before_mixer.weight"], 1e-5)
+    q = P.apply_rope(P.linear(x, w[f"{p}.mixer.q_proj.weight"]).view(t, 4, 16), cos, sin)
+    k = P.apply_rope(P.linear(x, w[f"{p}.mixer.k_proj.weight"]).view(t, 2, 16), cos, sin)
+    v = P.linear(x, w[f"{p}.mixer.v_proj.weight"]).view(t, 2, 16)
+    attn = P.causal_attention(q * (0.25 * 4.0), k, v)
+    h = h + P.rmsnorm(P.linear(attn.reshape(t, 64), w[f"{p}.mixer.o_proj.weight"]), w[f"{p}.after_mixer.weight"], 1e-4)
+    h = h + P.rmsnorm(P.mlp_block(w, f"{p}.ff", P.rmsnorm(h, w[f"{p}.before_ff.weight"], 1e-3)),
+                      w[f"{p}.after_ff.weight"], 1e-2)
+    for _ in range(2):                                       # the layer without a mixer runs twice
+        h = h + P.mlp_block(w, "layers.1.ff", P.rmsnorm(h, w["layers.1.norm.weight"], 1e-5))
+    return P.linear(P.rmsnorm(h, w["final_norm.weight"], 1e-5), w["head.weight"])
+
+
+def test_layers_of_other_shapes_than_the_common_one(tmp_path):
+    """A layer with four norms (two of them in ``LayerSpec.parts``, as is its feed-forward) and a layer
+    that has no mixer at all, registered from outside: the weights are collected under the names the
+    arrangements give them, the cache has one unit, and steps in portions and from replayed graphs
+    equal the plain forward."""
+    from lockstep_amd.config import ConfigError, LayerSpec, PartSpec, unregister_architecture
+    from lockstep_amd.engine.model import load_model
+    from lockstep_amd.parts import unregister_part
+    from lockstep_amd.weights import write_random_model
+    from safetensors.torch import load_file
+
+    SandwichConfig = _register_sandwich_toy()
+    try:
+        cfg = SandwichConfig(hidden_size=48, vocab_size=90)
+        spec = cfg.model_spec()
+        assert set(spec.layers[0].named_parts()) == {"mixer", "before_mixer", "after_mixer", "before_ff", "ff", "after_ff"}
+        assert spec.layers[1].mixer is None and not spec.layers[1].has("mixer")
+        with pytest.raises(ConfigError, match="no part named 'gate'.*it has: feed_forward, feed_forward_norm"):
+            spec.layers[1].part("gate")
+        with pytest.raises(ConfigError, match="fields of the layer itself"):
+            LayerSpec("x", PartSpec("toy_sandwich"), parts={"mixer": PartSpec("attention")})
+        folder = write_random_model(cfg, tmp_path / "sandwich", seed=3, std=0.2, norm_std=0.2)
+        w = {k: v.double() for k, v in load_file(str(folder / "model.safetensors")).items()}
+        assert {"layers.0.after_ff.weight", "layers.0.before_mixer.weight", "layers.0.ff.down_proj.weight",
+                "layers.1.norm.weight", "layers.1.ff.gate_proj.weight"} <= set(w)
+        model = load_model(folder, dtype="float32")
+        assert [type(u).__name__ for u in model.cache_unit_specs()] == ["PagedKVSpec", "NoneType"]
+        tokens = random_tokens(50, 90, seed=6)
+        want = _sandwich_plain(w, tokens, 48)
+        cache = model.make_cache(num_pages=24, page_size=8, max_requests=3, poison_on_free=True)
+        assert len(cache.groups) == 1 and not cache.state_units and cache.shareable()
+        whole = feed(model, cache, "w", tokens, [])
+        assert rel_err(whole, want) < 5e-5
+        cut = feed(model, cache, "c", tokens, [7, 2, 21] + [1] * 20)
+        assert rel_err(cut, want) < 5e-5
+        assert model.graph_replays > 10
+        cache.audit()
+    finally:
+        unregister_part("toy_sandwich")
+        unregister_part("toy_ff_only")
+        unregister_architecture(SandwichConfig)
