@@ -1589,18 +1589,16 @@ struct CombineItem {  // 8 ints
   int reserved[2];
 };
 
+// The fold of one block of 64 rows of a request: a lane takes a row and a quarter of its columns.
 template <typename T>
-__global__ __launch_bounds__(256) void combine_kernel(const SeqMeta* __restrict__ seqs,
-                                                      const CombineItem* __restrict__ items,
-                                                      const float* __restrict__ part_acc,
-                                                      const float* __restrict__ part_ml, T* __restrict__ out,
-                                                      long ldo, int G) {
+__device__ __forceinline__ void combine_row_block(const CombineItem& item, int row_block, int kvh,
+                                                  const float* __restrict__ part_acc,
+                                                  const float* __restrict__ part_ml, T* __restrict__ out, long ldo,
+                                                  int G) {
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
-  const CombineItem item = items[blockIdx.x];
-  const int kvh = blockIdx.y;
   const int rows_total = item.q_len * G;
-  const int r = item.row_block * 64 + wave * 16 + (lane & 15);
+  const int r = row_block * 64 + wave * 16 + (lane & 15);
   if (r >= rows_total) return;
   const int g = lane >> 4;
   const int qi = r / G;
@@ -1643,6 +1641,16 @@ __global__ __launch_bounds__(256) void combine_kernel(const SeqMeta* __restrict_
   store_output<T>(run, out + (long)(item.q_off + qi) * ldo + (long)head * D, g);
 }
 
+template <typename T>
+__global__ __launch_bounds__(256) void combine_kernel(const SeqMeta* __restrict__ seqs,
+                                                      const CombineItem* __restrict__ items,
+                                                      const float* __restrict__ part_acc,
+                                                      const float* __restrict__ part_ml, T* __restrict__ out,
+                                                      long ldo, int G) {
+  const CombineItem item = items[blockIdx.x];
+  combine_row_block<T>(item, item.row_block, blockIdx.y, part_acc, part_ml, out, ldo, G);
+}
+
 // The fold for requests of at most 16 rows a kv head (decoded tokens), where a request far away has dozens
 // of splits.  The fold of one split has to wait for the one before, so what counts is how long one fold
 // takes and that its operands are there.  All 256 threads bring the partial results of a batch of splits
@@ -1666,8 +1674,15 @@ __global__ __launch_bounds__(256) void combine_few_rows_kernel(const SeqMeta* __
   __shared__ float stage_ml[2][2 * 512];
   const CombineItem item = items[blockIdx.x];
   const int kvh = blockIdx.y;
-  const int rows_total = item.q_len * G;  // <= 16, checked on the host
+  const int rows_total = item.q_len * G;
   if (rows_total <= 0) return;
+  if (rows_total > 16) {
+    // more rows than this kernel's threads own columns for (the caller promised otherwise): the general
+    // fold, block of rows by block of rows -- the same bits, only slower
+    for (int block = 0; block * 64 < rows_total; ++block)
+      combine_row_block<T>(item, block, kvh, part_acc, part_ml, out, ldo, G);
+    return;
+  }
   const int n_splits = item.n_splits;
   const long pr_base = item.part_base + (long)kvh * rows_total * n_splits;  // row r, split s: pr_base + r * n_splits + s
   const int owned = rows_total * QUADS;   // groups of four columns to fold

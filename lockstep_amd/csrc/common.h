@@ -334,6 +334,19 @@ inline int check_launch(const char* what) {
   if (e != hipSuccess) return fail("%s: %s", what, hipGetErrorString(e));
   return 0;
 }
+
+// Compute units of the current device (asked once per device).
+inline int compute_units() {
+  static int cached[64] = {0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (cached[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cached[dev] = n;
+  }
+  return cached[dev];
+}
 }  // namespace ls
 
 #define LS_DEFINE_ERROR_API \
@@ -349,6 +362,7 @@ namespace ls {
 // bits of the mask, core library
 constexpr int kMutantKsliceByRows = 1;  // the skinny product cuts K into other slices above 16 rows
 constexpr int kMutantNormByRows = 2;    // RMSNorm adds its wave sums in another order in launches of more than four rows
+constexpr int kMutantSampleChunksByRows = 4;  // the sampler cuts a row into fewer chunks when the call has many rows
 // bits of the mask, attention libraries
 constexpr int kMutantReversedFold = 1;  // the combine kernel folds the splits from the last to the first
 }  // namespace ls

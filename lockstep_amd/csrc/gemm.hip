@@ -27,7 +27,7 @@
 namespace ls {
 
 #ifndef LS_GEMM_BIG
-#define LS_GEMM_BIG 256       // from this many 128 x 128 tiles on (one for every CU), use them; fewer leave CUs idle and 64 x 64 tiles win
+#define LS_GEMM_BIG 0         // from this many 128 x 128 tiles on, use them; 0: one for every CU (fewer leave CUs idle and 64 x 64 tiles win)
 #endif
 #ifndef LS_GEMM_BIG_ROWS
 #define LS_GEMM_BIG_ROWS 64   // ... and only with more rows than this: up to 64 rows half of a 128-row tile would be idle
@@ -953,19 +953,6 @@ __global__ __launch_bounds__(64 * NWM * NWN) void gemm_tiled_kernel(const T* __r
   }
 }
 
-// Compute units of the current device (asked once per device).
-inline int compute_units() {
-  static int cached[64] = {0};
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
-  if (cached[dev] == 0) {
-    int n = 0;
-    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
-    cached[dev] = n;
-  }
-  return cached[dev];
-}
-
 template <typename T, int EPI>
 int launch_gemm(const void* X, const void* W, void* C, int M, int N, int K, long ldx, long ldc, const float* norm_w,
                 float eps, int out_cols, hipStream_t stream) {
@@ -1086,7 +1073,7 @@ int launch_gemm(const void* X, const void* W, void* C, int M, int N, int K, long
     else if (wide_fills) {
       if constexpr (sizeof(T) == 2) LS_TILED_WAVES(128, 256, LS_GEMM_PD_WIDE, true, 2, 4)
     }
-    else if (big_tiles >= LS_GEMM_BIG && M > LS_GEMM_BIG_ROWS) LS_TILED(128, 128, LS_GEMM_PD_BIG, true)
+    else if (big_tiles >= (LS_GEMM_BIG ? LS_GEMM_BIG : cus) && M > LS_GEMM_BIG_ROWS) LS_TILED(128, 128, LS_GEMM_PD_BIG, true)
     // up to 64 rows over so many columns that tiles of 128 columns still give every CU a workgroup (the
     // logits head, gate and up of 32B sizes): every workgroup reads all rows of X, so half as many
     // workgroups halve that traffic (gate and up of 32B sizes at 64 rows 135 -> 112 us, the head 82 -> 77 us)
@@ -1161,7 +1148,7 @@ extern "C" int ls_gemm_slices(int dtype, const void* X, const void* W, float* P,
   const int nslices = (K + kslice - 1) / kslice;
   const int col_blocks = (N + 15) / 16;
   // enough groups of slices to fill the GPU, at most four slices (waves) a workgroup
-  int groups = (256 + col_blocks - 1) / col_blocks;
+  int groups = (compute_units() + col_blocks - 1) / col_blocks;
   if (groups > nslices) groups = nslices;
   if (groups < (nslices + 3) / 4) groups = (nslices + 3) / 4;
   const int per_group = (nslices + groups - 1) / groups;

@@ -16,10 +16,13 @@
 // can fall to the neighbour; nothing else differs.  Distinct float values whose weights round to the
 // same double (values below 1e-16 of each other, next to zero) are ordered by value here, by id there.
 //
-// A row is cut into kChunks runs of neighbouring tokens, each with a workgroup of its own, and every step
+// A row is always cut into kChunks runs of neighbouring tokens, whatever else the call samples: which
+// elements a thread adds and how the chunks' sums are folded are functions of the vocabulary alone, so a
+// row gives the same token beside any number of other rows.  A workgroup takes one chunk, or (many rows)
+// several chunks of a row one after the other, each exactly as a workgroup of its own would.  Every step
 // of the walk is a launch of its own: a launch reads the sums the launch before left for every chunk, adds
 // them up in chunk order (every workgroup of the row does the same arithmetic, so they agree without
-// talking to each other), and leaves its own chunk's sums.  The weights and the order keys of a row are
+// talking to each other), and leaves its own chunks' sums.  The weights and the order keys of a row are
 // kept in a scratch buffer the caller brings.  In a pass a thread adds each of its tokens' weights to the
 // thread's own slot of the token's candidate in LDS (sixteen slots a thread, no two threads share one, so
 // no atomics and a fixed order); the slots of a candidate are then summed over the workgroup.
@@ -31,18 +34,15 @@
 
 #include <algorithm>
 
-#ifndef LS_SAMPLE_WORKGROUPS
-#define LS_SAMPLE_WORKGROUPS 1024  // workgroups of a launch that the rows of a call are cut for
-#endif
-#ifndef LS_SAMPLE_MIN_CHUNKS
-#define LS_SAMPLE_MIN_CHUNKS 2
+#ifndef LS_SAMPLE_WORKGROUPS_A_CU
+#define LS_SAMPLE_WORKGROUPS_A_CU 4  // workgroups a CU that a launch aims at: with more rows a workgroup walks several chunks
 #endif
 
 namespace ls {
 
 constexpr int kSampleThreads = 256;
 constexpr int kSampleWaves = kSampleThreads / 64;
-constexpr int kChunks = 32;  // the most workgroups a row (few rows); many rows take fewer each
+constexpr int kChunks = 32;  // chunks a row is cut into, always
 constexpr int kBatch = 8;    // loads a thread has in flight in the passes over its chunk
 
 __device__ __forceinline__ unsigned int order_key(float f) {  // ascending in f; -0 counts as +0
@@ -77,7 +77,7 @@ struct Found {
 
 // What the launches of one call leave for each other, per row (and per chunk where it says so).
 struct SampleScratch {
-  int chunks;             // workgroups a row in this call (at most kChunks)
+  int chunks;             // chunks a row (kChunks; a mutant of the tests' control library makes it follow the rows)
   double* weights;        // [n][vocab]
   unsigned int* keys;     // [n][vocab]
   float* part_max;        // [n][kChunks]
@@ -123,40 +123,46 @@ __device__ __forceinline__ double block_sum(double v, double* __restrict__ wave_
   return total;
 }
 
-// grid (kChunks, n): the largest float(logit) / T of a chunk
+// All kernels below: grid (g, n) with g <= chunks; the workgroup (x, r) takes the chunks x, x + g, ... of row r,
+// one after the other, each as if it were alone.
+
+// the largest float(logit) / T of a chunk
 __global__ __launch_bounds__(kSampleThreads) void sample_max_kernel(const float* __restrict__ logits, long ld,
                                                                     const SampleRow* __restrict__ requests,
                                                                     SampleScratch sc, int vocab, int chunk_len) {
   __shared__ float wave_max[kSampleWaves];
-  const int r = blockIdx.y, c = blockIdx.x;
+  const int r = blockIdx.y;
   const SampleRow request = requests[r];
   const float* row = logits + (long)request.row * ld;
-  const int begin = min(vocab, c * chunk_len), end = min(vocab, begin + chunk_len);
-  float top = -INFINITY;
-  for (int i0 = begin + threadIdx.x; i0 < end; i0 += kBatch * kSampleThreads) {
-    float x[kBatch];
+  for (int c = blockIdx.x; c < sc.chunks; c += gridDim.x) {
+    const int begin = min(vocab, c * chunk_len), end = min(vocab, begin + chunk_len);
+    float top = -INFINITY;
+    for (int i0 = begin + threadIdx.x; i0 < end; i0 += kBatch * kSampleThreads) {
+      float x[kBatch];
 #pragma unroll
-    for (int u = 0; u < kBatch; ++u) x[u] = row[min(i0 + u * kSampleThreads, end - 1)];  // (a repeated token changes no maximum)
+      for (int u = 0; u < kBatch; ++u) x[u] = row[min(i0 + u * kSampleThreads, end - 1)];  // (a repeated token changes no maximum)
 #pragma unroll
-    for (int u = 0; u < kBatch; ++u) top = fmaxf(top, x[u] / request.temperature);
-  }
+      for (int u = 0; u < kBatch; ++u) top = fmaxf(top, x[u] / request.temperature);
+    }
 #pragma unroll
-  for (int off = 32; off >= 1; off >>= 1) top = fmaxf(top, __shfl_xor(top, off));
-  if ((threadIdx.x & 63) == 0) wave_max[threadIdx.x >> 6] = top;
-  __syncthreads();
-  if (threadIdx.x == 0) {
+    for (int off = 32; off >= 1; off >>= 1) top = fmaxf(top, __shfl_xor(top, off));
+    __syncthreads();  // wave_max may still be read for the chunk before
+    if ((threadIdx.x & 63) == 0) wave_max[threadIdx.x >> 6] = top;
+    __syncthreads();
+    if (threadIdx.x == 0) {
 #pragma unroll
-    for (int w = 0; w < kSampleWaves; ++w) top = fmaxf(top, wave_max[w]);
-    sc.part_max[r * sc.chunks + c] = top;
+      for (int w = 0; w < kSampleWaves; ++w) top = fmaxf(top, wave_max[w]);
+      sc.part_max[r * sc.chunks + c] = top;
+    }
   }
 }
 
-// grid (kChunks, n): weights and order keys of a chunk, and the sum of its weights
+// weights and order keys of a chunk, and the sum of its weights
 __global__ __launch_bounds__(kSampleThreads) void sample_exp_kernel(const float* __restrict__ logits, long ld,
                                                                     const SampleRow* __restrict__ requests,
                                                                     SampleScratch sc, int vocab, int chunk_len) {
   __shared__ double wave_sums[kSampleWaves];
-  const int r = blockIdx.y, c = blockIdx.x;
+  const int r = blockIdx.y;
   const SampleRow request = requests[r];
   const float* row = logits + (long)request.row * ld;
   double* weights = sc.weights + (long)r * vocab;
@@ -164,25 +170,27 @@ __global__ __launch_bounds__(kSampleThreads) void sample_exp_kernel(const float*
   float top = -INFINITY;
   for (int k = 0; k < sc.chunks; ++k) top = fmaxf(top, sc.part_max[r * sc.chunks + k]);
   const double v_max = (double)top;
-  const int begin = min(vocab, c * chunk_len), end = min(vocab, begin + chunk_len);
-  double part = 0.0;
-  for (int i0 = begin + threadIdx.x; i0 < end; i0 += kBatch * kSampleThreads) {
-    float x[kBatch];
+  for (int c = blockIdx.x; c < sc.chunks; c += gridDim.x) {
+    const int begin = min(vocab, c * chunk_len), end = min(vocab, begin + chunk_len);
+    double part = 0.0;
+    for (int i0 = begin + threadIdx.x; i0 < end; i0 += kBatch * kSampleThreads) {
+      float x[kBatch];
 #pragma unroll
-    for (int u = 0; u < kBatch; ++u) x[u] = row[min(i0 + u * kSampleThreads, end - 1)];
+      for (int u = 0; u < kBatch; ++u) x[u] = row[min(i0 + u * kSampleThreads, end - 1)];
 #pragma unroll
-    for (int u = 0; u < kBatch; ++u) {
-      const int i = i0 + u * kSampleThreads;
-      if (i >= end) continue;
-      const float f = x[u] / request.temperature;
-      const double w = exp((double)f - v_max);
-      weights[i] = w;
-      keys[i] = order_key(f);
-      part = part + w;
+      for (int u = 0; u < kBatch; ++u) {
+        const int i = i0 + u * kSampleThreads;
+        if (i >= end) continue;
+        const float f = x[u] / request.temperature;
+        const double w = exp((double)f - v_max);
+        weights[i] = w;
+        keys[i] = order_key(f);
+        part = part + w;
+      }
     }
+    const double total = block_sum(part, wave_sums);
+    if (threadIdx.x == 0) sc.part_sum[r * sc.chunks + c] = total;
   }
-  const double total = block_sum(part, wave_sums);
-  if (threadIdx.x == 0) sc.part_sum[r * sc.chunks + c] = total;
 }
 
 // The state of walk `walk` of row r after level `level - 1`, from the state after level `level - 2` (which
@@ -242,135 +250,139 @@ __device__ SearchState state_before_level(const SampleScratch& sc, const SampleR
   return st;
 }
 
-// grid (kChunks, n), levels 0 to 7: the sums of a chunk's weights for the sixteen candidates of this level's
-// four bits, among the tokens whose known bits fit.
+// levels 0 to 7: the sums of a chunk's weights for the sixteen candidates of this level's four bits, among the
+// tokens whose known bits fit.
 __global__ __launch_bounds__(kSampleThreads) void sample_level_kernel(const SampleRow* __restrict__ requests,
                                                                       SampleScratch sc, int n, int vocab, int chunk_len,
                                                                       int walk, int level) {
   __shared__ double slots[16 * kSampleThreads];  // candidate b of thread t at slots[b * kSampleThreads + t]
   __shared__ double wave_sums[kSampleWaves * 16];
-  const int r = blockIdx.y, c = blockIdx.x;
+  const int r = blockIdx.y;
   const SampleRow request = requests[r];
   if (walk == 0 && !(request.top_p() < 1.0)) return;  // the whole row is the head
   __shared__ double staged[kChunks * 16];
   const SearchState st = state_before_level(sc, request, n, r, walk, level, staged);
-  if (c == 0 && threadIdx.x == 0) sc.state[(walk * 2 + ((level + 1) & 1)) * n + r] = st;  // parity of level - 1
+  if (blockIdx.x == 0 && threadIdx.x == 0) sc.state[(walk * 2 + ((level + 1) & 1)) * n + r] = st;  // parity of level - 1
   const unsigned int* keys = sc.keys + (long)r * vocab;
   const double* weights = sc.weights + (long)r * vocab;
   const int shift = 28 - 4 * level;
   const unsigned int known = level == 0 ? 0u : (0xffffffffu << (shift + 4));
+  for (int c = blockIdx.x; c < sc.chunks; c += gridDim.x) {
 #pragma unroll
-  for (int b = 0; b < 16; ++b) slots[b * kSampleThreads + threadIdx.x] = 0.0;
-  const int begin = min(vocab, c * chunk_len), end = min(vocab, begin + chunk_len);
-  // eight tokens' keys at a time, unconditional, so that the loads are in flight together; then the weights
-  // of those whose known bits fit (from the second level on these are few, and the others' weights are
-  // never fetched); the additions keep the order of the ids
-  for (int i0 = begin + threadIdx.x; i0 < end; i0 += kBatch * kSampleThreads) {
-    unsigned int key[kBatch];
-    double w[kBatch];
+    for (int b = 0; b < 16; ++b) slots[b * kSampleThreads + threadIdx.x] = 0.0;
+    const int begin = min(vocab, c * chunk_len), end = min(vocab, begin + chunk_len);
+    // eight tokens' keys at a time, unconditional, so that the loads are in flight together; then the weights
+    // of those whose known bits fit (from the second level on these are few, and the others' weights are
+    // never fetched); the additions keep the order of the ids
+    for (int i0 = begin + threadIdx.x; i0 < end; i0 += kBatch * kSampleThreads) {
+      unsigned int key[kBatch];
+      double w[kBatch];
 #pragma unroll
-    for (int u = 0; u < kBatch; ++u) key[u] = keys[min(i0 + u * kSampleThreads, end - 1)];
-    bool fits[kBatch];
+      for (int u = 0; u < kBatch; ++u) key[u] = keys[min(i0 + u * kSampleThreads, end - 1)];
+      bool fits[kBatch];
 #pragma unroll
-    for (int u = 0; u < kBatch; ++u) fits[u] = i0 + u * kSampleThreads < end && (key[u] & known) == st.prefix;
+      for (int u = 0; u < kBatch; ++u) fits[u] = i0 + u * kSampleThreads < end && (key[u] & known) == st.prefix;
 #pragma unroll
-    for (int u = 0; u < kBatch; ++u) w[u] = fits[u] ? weights[i0 + u * kSampleThreads] : 0.0;
+      for (int u = 0; u < kBatch; ++u) w[u] = fits[u] ? weights[i0 + u * kSampleThreads] : 0.0;
 #pragma unroll
-    for (int u = 0; u < kBatch; ++u) {
-      if (!fits[u]) continue;
-      double* slot = &slots[((key[u] >> shift) & 15) * kSampleThreads + threadIdx.x];
-      *slot = *slot + w[u];
+      for (int u = 0; u < kBatch; ++u) {
+        if (!fits[u]) continue;
+        double* slot = &slots[((key[u] >> shift) & 15) * kSampleThreads + threadIdx.x];
+        *slot = *slot + w[u];
+      }
     }
-  }
-  double sums[16];
+    double sums[16];
 #pragma unroll
-  for (int b = 0; b < 16; ++b) {
-    sums[b] = slots[b * kSampleThreads + threadIdx.x];
+    for (int b = 0; b < 16; ++b) {
+      sums[b] = slots[b * kSampleThreads + threadIdx.x];
 #pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) sums[b] = sums[b] + __shfl_xor(sums[b], off);
-  }
-  if ((threadIdx.x & 63) == 0) {
+      for (int off = 32; off >= 1; off >>= 1) sums[b] = sums[b] + __shfl_xor(sums[b], off);
+    }
+    __syncthreads();  // wave_sums may still be read for the chunk before
+    if ((threadIdx.x & 63) == 0) {
 #pragma unroll
-    for (int b = 0; b < 16; ++b) wave_sums[(threadIdx.x >> 6) * 16 + b] = sums[b];
-  }
-  __syncthreads();
-  if (threadIdx.x < 16) {
-    double s = 0.0;
+      for (int b = 0; b < 16; ++b) wave_sums[(threadIdx.x >> 6) * 16 + b] = sums[b];
+    }
+    __syncthreads();
+    if (threadIdx.x < 16) {
+      double s = 0.0;
 #pragma unroll
-    for (int w = 0; w < kSampleWaves; ++w) s = s + wave_sums[w * 16 + threadIdx.x];
-    sc.part_level[(((long)(level & 1) * n + r) * sc.chunks + c) * 16 + threadIdx.x] = s;
+      for (int w = 0; w < kSampleWaves; ++w) s = s + wave_sums[w * 16 + threadIdx.x];
+      sc.part_level[(((long)(level & 1) * n + r) * sc.chunks + c) * 16 + threadIdx.x] = s;
+    }
   }
 }
 
-// grid (kChunks, n), after level 7: the key is known; how many tokens of the chunk have it, and their weight
+// after level 7: the key is known; how many tokens of the chunk have it, and their weight
 __global__ __launch_bounds__(kSampleThreads) void sample_tie_count_kernel(const SampleRow* __restrict__ requests,
                                                                           SampleScratch sc, int n, int vocab,
                                                                           int chunk_len, int walk) {
   __shared__ int wave_count[kSampleWaves];
   __shared__ double wave_weight[kSampleWaves];
-  const int r = blockIdx.y, c = blockIdx.x;
+  const int r = blockIdx.y;
   const SampleRow request = requests[r];
   if (walk == 0 && !(request.top_p() < 1.0)) return;
   __shared__ double staged[kChunks * 16];
   const SearchState st = state_before_level(sc, request, n, r, walk, 8, staged);
-  if (c == 0 && threadIdx.x == 0) sc.state[(walk * 2 + 1) * n + r] = st;  // after level 7
+  if (blockIdx.x == 0 && threadIdx.x == 0) sc.state[(walk * 2 + 1) * n + r] = st;  // after level 7
   const unsigned int* keys = sc.keys + (long)r * vocab;
   const double* weights = sc.weights + (long)r * vocab;
-  const int begin = min(vocab, c * chunk_len), end = min(vocab, begin + chunk_len);
-  int mine = 0, last_tie = -1;
-  for (int i0 = begin + threadIdx.x; i0 < end; i0 += kBatch * kSampleThreads) {
-    unsigned int key[kBatch];
+  for (int c = blockIdx.x; c < sc.chunks; c += gridDim.x) {
+    const int begin = min(vocab, c * chunk_len), end = min(vocab, begin + chunk_len);
+    int mine = 0, last_tie = -1;
+    for (int i0 = begin + threadIdx.x; i0 < end; i0 += kBatch * kSampleThreads) {
+      unsigned int key[kBatch];
 #pragma unroll
-    for (int u = 0; u < kBatch; ++u) key[u] = keys[min(i0 + u * kSampleThreads, end - 1)];
+      for (int u = 0; u < kBatch; ++u) key[u] = keys[min(i0 + u * kSampleThreads, end - 1)];
 #pragma unroll
-    for (int u = 0; u < kBatch; ++u)
-      if (i0 + u * kSampleThreads < end && key[u] == st.prefix) {
-        ++mine;
-        last_tie = i0 + u * kSampleThreads;
-      }
-  }
-  double weight = last_tie >= 0 ? weights[last_tie] : 0.0;  // they are equal: any of them
-#pragma unroll
-  for (int off = 32; off >= 1; off >>= 1) {
-    mine += __shfl_xor(mine, off);
-    weight = fmax(weight, __shfl_xor(weight, off));
-  }
-  if ((threadIdx.x & 63) == 0) {
-    wave_count[threadIdx.x >> 6] = mine;
-    wave_weight[threadIdx.x >> 6] = weight;
-  }
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    int count = 0;
-    double w = 0.0;
-#pragma unroll
-    for (int k = 0; k < kSampleWaves; ++k) {
-      count += wave_count[k];
-      w = fmax(w, wave_weight[k]);
+      for (int u = 0; u < kBatch; ++u)
+        if (i0 + u * kSampleThreads < end && key[u] == st.prefix) {
+          ++mine;
+          last_tie = i0 + u * kSampleThreads;
+        }
     }
-    sc.tie_count[r * sc.chunks + c] = count;
-    sc.tie_weight[r * sc.chunks + c] = w;
+    double weight = last_tie >= 0 ? weights[last_tie] : 0.0;  // they are equal: any of them
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+      mine += __shfl_xor(mine, off);
+      weight = fmax(weight, __shfl_xor(weight, off));
+    }
+    __syncthreads();  // the wave values may still be read for the chunk before
+    if ((threadIdx.x & 63) == 0) {
+      wave_count[threadIdx.x >> 6] = mine;
+      wave_weight[threadIdx.x >> 6] = weight;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      int count = 0;
+      double w = 0.0;
+#pragma unroll
+      for (int k = 0; k < kSampleWaves; ++k) {
+        count += wave_count[k];
+        w = fmax(w, wave_weight[k]);
+      }
+      sc.tie_count[r * sc.chunks + c] = count;
+      sc.tie_weight[r * sc.chunks + c] = w;
+    }
   }
 }
 
-// grid (kChunks, n): tokens that share the key are counted off in the order of their ids; the chunk that
-// holds the one that is meant finds it.
+// tokens that share the key are counted off in the order of their ids; the chunk that holds the one that is
+// meant finds it.
 __global__ __launch_bounds__(kSampleThreads) void sample_tie_pick_kernel(const SampleRow* __restrict__ requests,
                                                                          SampleScratch sc, int n, int vocab,
                                                                          int chunk_len, int walk, int* __restrict__ out,
                                                                          int scatter) {
   __shared__ int counts[kSampleThreads];
   __shared__ int picked;
-  const int r = blockIdx.y, c = blockIdx.x;
+  const int r = blockIdx.y;
   const SampleRow request = requests[r];
   if (walk == 0 && !(request.top_p() < 1.0)) return;
   const SearchState st = sc.state[(walk * 2 + 1) * n + r];
-  int before = 0, ties = 0;
+  int ties = 0;
   double w_tie = 0.0;
   for (int k = 0; k < sc.chunks; ++k) {
-    const int count = sc.tie_count[r * sc.chunks + k];
-    if (k < c) before += count;
-    ties += count;
+    ties += sc.tie_count[r * sc.chunks + k];
     w_tie = fmax(w_tie, sc.tie_weight[r * sc.chunks + k]);
   }
   // the m-th tie is the first whose cumulative weight above + m * w reaches the target
@@ -381,32 +393,37 @@ __global__ __launch_bounds__(kSampleThreads) void sample_tie_pick_kernel(const S
     if (m < 1) m = 1;
   }
   if (m > ties) m = ties;
-  const int mine_total = sc.tie_count[r * sc.chunks + c];
-  if (!(before < m && m <= before + mine_total)) return;  // another chunk holds it (uniform for the workgroup)
-  // a thread takes a run of neighbouring ids of the chunk
   const unsigned int* keys = sc.keys + (long)r * vocab;
-  const int begin = min(vocab, c * chunk_len), end = min(vocab, begin + chunk_len);
-  const int per = (chunk_len + kSampleThreads - 1) / kSampleThreads;
-  const int lo = min(end, begin + (int)threadIdx.x * per), hi = min(end, lo + per);
-  int mine = 0;
-  for (int i = lo; i < hi; ++i) mine += keys[i] == st.prefix ? 1 : 0;
-  counts[threadIdx.x] = mine;
-  __syncthreads();
-  int ahead = before;
-  for (int t = 0; t < (int)threadIdx.x; ++t) ahead += counts[t];
-  if (mine > 0 && ahead < m && m <= ahead + mine) {
-    int seen = ahead;
-    for (int i = lo; i < hi; ++i)
-      if (keys[i] == st.prefix && ++seen == m) {
-        picked = i;
-        break;
-      }
-    Found found;
-    found.reached = st.above + (double)m * w_tie;
-    found.token = picked;
-    found.pad = 0;
-    sc.found[walk * n + r] = found;
-    if (walk == 1) out[scatter ? request.row : r] = picked;
+  for (int c = blockIdx.x; c < sc.chunks; c += gridDim.x) {
+    int before = 0;
+    for (int k = 0; k < c; ++k) before += sc.tie_count[r * sc.chunks + k];
+    const int mine_total = sc.tie_count[r * sc.chunks + c];
+    if (!(before < m && m <= before + mine_total)) continue;  // another chunk holds it (uniform for the workgroup)
+    // a thread takes a run of neighbouring ids of the chunk
+    const int begin = min(vocab, c * chunk_len), end = min(vocab, begin + chunk_len);
+    const int per = (chunk_len + kSampleThreads - 1) / kSampleThreads;
+    const int lo = min(end, begin + (int)threadIdx.x * per), hi = min(end, lo + per);
+    int mine = 0;
+    for (int i = lo; i < hi; ++i) mine += keys[i] == st.prefix ? 1 : 0;
+    counts[threadIdx.x] = mine;
+    __syncthreads();
+    int ahead = before;
+    for (int t = 0; t < (int)threadIdx.x; ++t) ahead += counts[t];
+    if (mine > 0 && ahead < m && m <= ahead + mine) {
+      int seen = ahead;
+      for (int i = lo; i < hi; ++i)
+        if (keys[i] == st.prefix && ++seen == m) {
+          picked = i;
+          break;
+        }
+      Found found;
+      found.reached = st.above + (double)m * w_tie;
+      found.token = picked;
+      found.pad = 0;
+      sc.found[walk * n + r] = found;
+      if (walk == 1) out[scatter ? request.row : r] = picked;
+    }
+    return;  // one chunk holds it: nothing is left to look for
   }
 }
 
@@ -454,11 +471,15 @@ extern "C" int ls_sample_top_p(const float* logits, long ld, const void* request
   sc.tie_weight = reinterpret_cast<double*>(take((size_t)n * kChunks * sizeof(double)));
   sc.found = reinterpret_cast<Found*>(take((size_t)2 * n * sizeof(Found)));
   const SampleRow* rows = reinterpret_cast<const SampleRow*>(requests);
-  // few rows are cut into many chunks (a row alone would keep one CU busy); many rows fill the GPU with fewer
-  sc.chunks = std::max(LS_SAMPLE_MIN_CHUNKS, std::min(kChunks, LS_SAMPLE_WORKGROUPS / n));
+  // A row's cut is the same in every call.  Few rows get a workgroup a chunk (a row alone would keep one CU
+  // busy); with many rows a workgroup walks several chunks of its row, so that the launch has some
+  // LS_SAMPLE_WORKGROUPS_A_CU workgroups a CU instead of thousands of short ones.
+  sc.chunks = kChunks;
+  if (LS_MUTANT_HOST(kMutantSampleChunksByRows)) sc.chunks = std::max(2, std::min(kChunks, 1024 / n));  // the mutant: a cut that depends on the rows of the call
   const int chunk_len = (vocab + sc.chunks - 1) / sc.chunks;
+  const int per_row = std::max(2, std::min(sc.chunks, LS_SAMPLE_WORKGROUPS_A_CU * compute_units() / n));
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-  const dim3 grid(sc.chunks, n), block(kSampleThreads);
+  const dim3 grid(per_row, n), block(kSampleThreads);
   hipLaunchKernelGGL(sample_max_kernel, grid, block, 0, s, logits, ld, rows, sc, vocab, chunk_len);
   hipLaunchKernelGGL(sample_exp_kernel, grid, block, 0, s, logits, ld, rows, sc, vocab, chunk_len);
   for (int walk = any_nucleus ? 0 : 1; walk < 2; ++walk) {

@@ -25,7 +25,7 @@ from ..parts.base import device_epoch, graph_safe_tree, takes
 from ..weights.store import load_weights, weights_from_dict
 from .batch import StepContext, StepEntry, Workspace
 from .runtime import Runtime
-from .tape import LayerTape, RunKinds
+from .tape import LayerTape, RunKinds, TapeMismatch, TapeRefused
 
 
 def collect_weight_specs(spec: ModelSpec) -> list[WeightSpec]:
@@ -90,6 +90,7 @@ class Model:
         self.verify_tapes = os.environ.get("LOCKSTEP_VERIFY_TAPE", "") not in ("", "0")
         self._run_kinds = weakref.WeakKeyDictionary()      # cache manager -> (device epoch, RunKinds)
         self.layers_repeated = 0
+        self.tapes_refused = 0
 
     @property
     def split_keys(self):
@@ -202,7 +203,7 @@ class Model:
                 situation = (self.workspace.version,
                              None if pending is None else (pending.partials.data_ptr(), tuple(pending.partials.shape)))
                 held = met.get(kind)
-                if held is not None and held[1] == situation and not self.verify_tapes:
+                if held is not None and held[1] == situation and kind in kinds.verified and not self.verify_tapes:
                     held[0].repeat(kinds.addresses[index])
                     pending = held[2]
                     self.layers_repeated += 1
@@ -230,10 +231,24 @@ class Model:
                 met[kind] = None
                 continue
             held = met[kind]
-            if held is not None and held[1] == situation:          # only with verify_tapes
-                held[0].compare(launches, kinds.addresses[index], f"layer run {index}")
+            if held is not None and held[1] == situation:
+                # The first layer of a kind that a tape could have stood for (once per model and cache; every
+                # one with verify_tapes) ran in Python as well: its launches must be what the tape would launch.
+                try:
+                    held[0].compare(launches, kinds.addresses[index], f"layer run {index}")
+                    kinds.verified.add(kind)
+                except TapeMismatch:
+                    if self.verify_tapes:
+                        raise
+                    kinds.refuse(kind)                             # these layers run in Python from now on
+                    self.tapes_refused += 1
+                    continue
             if situation[0] == self.workspace.version:             # the run did not move the workspace
-                met[kind] = (LayerTape(launches, kinds.addresses[index]), situation, pending)
+                try:
+                    met[kind] = (LayerTape(launches, kinds.addresses[index], kinds.foreign[index]), situation, pending)
+                except TapeRefused:
+                    kinds.refuse(kind)
+                    self.tapes_refused += 1
         if ctx.n_want:
             x = ctx.buf("final.normed", (ctx.n_want, self.spec.hidden_size), self.rt.dtype)
             if pending is not None and self._final_takes_pending:

@@ -14,12 +14,21 @@ cache units in the same group of the cache.  The first run of a kind is never no
 may do once a step what later layers find done.  A noted run stands for later ones only while they
 arrive in the same situation: the same pending addition (or none) and an unchanged workspace.
 
-``LOCKSTEP_VERIFY_TAPE=1`` runs every layer in Python all the same and compares its launches,
-argument by argument, with what the tape would have launched.
+A tape is refused (``TapeRefused``; the layers of that kind then run their ``forward`` every time)
+when a launch of the noted layer passes an address that lies inside a tensor of *another* layer and
+is not among the noted layer's own: the part holds a per-layer tensor where ``device_constants``
+does not find it, and repeating the launch would run every later layer on that one tensor.
+
+The first layer that a tape of its kind could stand for (once per model and cache) runs in Python all
+the same and its launches are compared, argument by argument, with what the tape would have launched;
+only when they agree do later layers repeat the tape, and a disagreement (a per-layer tensor that
+neither walk finds, a per-layer number passed to a kernel) switches the repetition off for the kind.
+``LOCKSTEP_VERIFY_TAPE=1`` does the same for every layer of every step, and raises.
 """
 
 from __future__ import annotations
 
+import bisect
 import dataclasses
 from ctypes import c_void_p
 
@@ -75,6 +84,7 @@ class RunKinds:
 
     def __init__(self, model, cache):
         self.kind: list = []            # per schedule entry: a small int, or None (always run in Python)
+        self.verified: set = set()      # kinds whose tape was once compared with a layer run in Python, and agreed
         self.addresses: list = []       # per schedule entry: name -> (address, bytes)
         seen: list = []
         for run in model.schedule:
@@ -96,17 +106,38 @@ class RunKinds:
             else:
                 seen.append(key)
                 self.kind.append(len(seen) - 1)
+        # per schedule entry: the address ranges of tensors that belong to other entries and not to this one
+        owners: dict = {}
+        for index, names in enumerate(self.addresses):
+            for base, size in names.values():
+                owners.setdefault((base, base + size), set()).add(index)
+        self.foreign: list = [sorted(r for r, who in owners.items() if index not in who)
+                              for index in range(len(self.addresses))]
+
+    def refuse(self, kind) -> None:
+        """Layers of this kind run their ``forward`` every time from now on."""
+        self.kind = [None if k == kind else k for k in self.kind]
 
 
 def _value(arg):
     return getattr(arg, "value", arg)
 
 
+class TapeMismatch(RuntimeError):
+    """A layer run in Python launched something else than the tape of its kind would have."""
+
+
+class TapeRefused(RuntimeError):
+    """A noted launch names a tensor of another layer that the noted layer is not known to hold."""
+
+
 class LayerTape:
     """The launches of one layer run, with the places marked where an address of that layer stands."""
 
-    def __init__(self, launches, addresses: dict):
+    def __init__(self, launches, addresses: dict, foreign=()):
+        """``foreign``: sorted (first, end) address ranges of the other layers' own tensors."""
         ranges = sorted((base, base + size, name) for name, (base, size) in addresses.items())
+        starts = [lo for lo, _ in foreign]
         self.calls = []
         for lib, entry, args in launches:
             marks = []
@@ -116,6 +147,12 @@ class LayerTape:
                         if lo <= a.value < hi:
                             marks.append((i, name, a.value - lo))
                             break
+                    else:
+                        at = bisect.bisect_right(starts, a.value) - 1
+                        if at >= 0 and a.value < foreign[at][1]:
+                            raise TapeRefused(
+                                f"argument {i} of {getattr(entry, '__name__', entry)} points into a tensor of "
+                                "another layer that this layer's parts do not list among their own")
             self.calls.append((lib, entry, args, tuple(marks)))
 
     def arguments(self, addresses: dict):
@@ -136,10 +173,10 @@ class LayerTape:
         """Raise unless ``launches`` (of a layer run in Python) are what ``repeat`` would launch."""
         mine = list(self.arguments(addresses))
         if len(mine) != len(launches):
-            raise RuntimeError(f"{what}: the layer launched {len(launches)} kernels, the tape holds {len(mine)}")
+            raise TapeMismatch(f"{what}: the layer launched {len(launches)} kernels, the tape holds {len(mine)}")
         for n, ((_, entry, args), (_, entry2, args2)) in enumerate(zip(mine, launches)):
             same = entry == entry2 and len(args) == len(args2) and all(
                 _value(a) == _value(b) for a, b in zip(args, args2))
             if not same:
-                raise RuntimeError(f"{what}: launch {n} ({getattr(entry2, '__name__', entry2)}) differs from the "
+                raise TapeMismatch(f"{what}: launch {n} ({getattr(entry2, '__name__', entry2)}) differs from the "
                                    f"tape's: {[_value(a) for a in args2]} against {[_value(a) for a in args]}")

@@ -114,7 +114,7 @@ class Kernels:
         return lib
 
     #: bits of ``set_mutants`` (csrc/common.h)
-    MUTANT_KSLICE_BY_ROWS, MUTANT_NORM_BY_ROWS = 1, 2      # core library
+    MUTANT_KSLICE_BY_ROWS, MUTANT_NORM_BY_ROWS, MUTANT_SAMPLE_CHUNKS_BY_ROWS = 1, 2, 4      # core library
     MUTANT_REVERSED_FOLD = 1                               # attention libraries
 
     def set_mutants(self, core: int = 0, attention: int = 0) -> None:
@@ -344,7 +344,11 @@ class Kernels:
         scratch array go through the entry point that allocates nothing: that array never moves, so
         a captured graph that contains the launch stays valid whatever runs in between.  Larger
         calls bring a scratch buffer; a buffer that was outgrown is kept until the process ends,
-        because a captured graph may still write into it."""
+        because a captured graph may still write into it.
+
+        The static array is one per GPU and process: calls that overlap on one GPU (two streams, two
+        engines in one process that do not order their work) race on it.  This engine launches
+        everything on one stream, which orders them."""
         _rows_ok(logits, "argmax logits")
         if not (logits.dtype == torch.float32):
             raise KernelError("argmax reads float32 logits")

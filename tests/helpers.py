@@ -3,6 +3,8 @@ request in portions and compare logits with the plain implementation."""
 
 from __future__ import annotations
 
+import math
+
 import numpy as np
 import torch
 
@@ -125,3 +127,27 @@ def max_live_tokens(steps, round_to: int = 64) -> int:
         for rid in step["end"]:
             held.pop(rid, None)
     return worst
+
+
+def sampling_rows_on_boundaries(vocab: int, rows: int = 24, seed: int = 0):
+    """Logits rows and sampling requests on which a change in the order of any of the sampler's sums
+    shows as another token.  A row takes four values a quarter apart, so its weights are a few long
+    runs of equal, irrational addends; the nucleus is put exactly on the boundary between two tokens
+    (top_p = the cumulative weight up to a token / the total, both summed here without rounding
+    error, so that the quotient is off by its own rounding only), so whether that token is still
+    inside is decided in the last bit of the kernel's own sums, and the head it leaves scales the draw.  Returns (float32 logits [rows, vocab], requests as ``sample_top_p`` takes them)."""
+    from lockstep_amd.sampling import philox
+
+    g = torch.Generator().manual_seed(seed + vocab)
+    logits = torch.randint(0, 4, (rows, vocab), generator=g).float() * -0.25
+    key = philox.uid_key("boundaries")
+    requests = []
+    for i in range(rows):
+        temperature = [0.7, 1.0, 1.9, 0.45][i % 4]
+        values = (logits[i] / torch.tensor(temperature, dtype=torch.float32)).double()
+        weights = (values - values.max()).exp()
+        ordered = torch.sort(weights, descending=True, stable=True)[0].tolist()
+        at = int(vocab * (0.15 + 0.7 * (i + 1) / (rows + 1)))
+        top_p = math.fsum(ordered[: at + 1]) / math.fsum(ordered)
+        requests.append((i, temperature, top_p, (31 + i) ^ key, 2000 + 13 * i))
+    return logits, requests

@@ -6,7 +6,7 @@ and shows that it holds again once the breakage is taken out.
 Device-side breakages are wrong variants compiled into control libraries (``-DLS_MUTANTS``,
 files of their own beside the product libraries) and switched on by a mask: K blocking that
 depends on the rows of a launch, a norm whose summation order depends on the rows of a launch,
-the fold over the attention splits reversed.  Host-side breakages are patched in from here: a
+a sampler whose cut of a row depends on the rows of a call, the fold over the attention splits reversed.  Host-side breakages are patched in from here: a
 block table that is not refreshed when a slot is used again, a recomputation that skips a token,
 a prefix match rounded up past a page, a draw keyed on the step instead of the position, a page
 given back without its holder count going down.  The list follows the reference's seeded faults
@@ -103,6 +103,24 @@ def test_a_norm_whose_order_depends_on_the_rows_of_a_launch_is_caught(control_ke
         return all(torch.equal(normed(lo, lo + 4), together[lo:lo + 4]) for lo in range(0, 40, 4))
 
     holds_breaks_holds(rows_alone_equal_rows_in_a_batch, lambda: mutant(k, core=k.MUTANT_NORM_BY_ROWS))
+
+
+def test_a_sampler_whose_cut_depends_on_the_rows_of_a_call_is_caught(control_kernels):
+    """Rows whose nucleus lies exactly on the boundary between two tokens get the same tokens alone
+    and among 200 rows; a sampler that cuts a row into fewer chunks when the call has many rows adds
+    its sums in another order there, and some boundary falls the other way."""
+    from helpers import sampling_rows_on_boundaries
+    from test_kernels_gpu import sample_among
+
+    k = control_kernels
+    logits, requests = sampling_rows_on_boundaries(151936, rows=24)
+    dev = logits.cuda()
+
+    def same_tokens_alone_and_in_company():
+        alone = [sample_among(k, dev, [r], 1, 0)[0] for r in requests]
+        return all(sample_among(k, dev, requests, n, n) == alone for n in (64, 200))
+
+    holds_breaks_holds(same_tokens_alone_and_in_company, lambda: mutant(k, core=k.MUTANT_SAMPLE_CHUNKS_BY_ROWS))
 
 
 # -- device side: through the model ---------------------------------------------------------------

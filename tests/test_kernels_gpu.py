@@ -230,6 +230,51 @@ def test_the_sampling_kernel_picks_the_host_samplers_token(vocab):
     assert len(set(want)) > 1
 
 
+def sample_among(kernels, dev, requests, n_rows: int, order_seed: int):
+    """The tokens of ``requests`` when they are sampled in one call of ``n_rows`` rows (the others
+    being further draws from the same logits rows), in a shuffled order."""
+    base = len(requests)
+    extra = [(i % base, 0.5 + (i % 7) / 4, [1.0, 0.8][i % 2], 900 + i, 50000 + i) for i in range(max(0, n_rows - base))]
+    every = list(requests[:n_rows]) + extra
+    order = torch.randperm(len(every), generator=torch.Generator().manual_seed(order_seed)).tolist()
+    out = torch.full((len(every),), -1, dtype=torch.int32, device="cuda")
+    kernels.sample_top_p(dev, [every[j] for j in order], out)
+    picked = out.cpu().tolist()
+    tokens = [None] * len(every)
+    for place, j in enumerate(order):
+        tokens[j] = picked[place]
+    return tokens[:min(n_rows, base)]
+
+
+@pytest.mark.parametrize("vocab", [1000, 151936])
+def test_a_sampled_row_gets_the_same_token_beside_any_number_of_other_rows(vocab):
+    """The same logits rows sampled alone and in calls of 24, 33, 64 and 200 rows: the same tokens.
+    Half of the rows are spread-out logits with random nuclei; the other half are made so that a
+    change in the order of any sum would show (``sampling_rows_on_boundaries``: the positive
+    control of this test runs them against a sampler whose cut depends on the rows of the call)."""
+    from helpers import sampling_rows_on_boundaries
+    from lockstep_amd.sampling import philox
+
+    g = torch.Generator().manual_seed(vocab + 1)
+    spread = torch.randn(12, vocab, generator=g) * 2.0
+    spread[::2] = torch.round(spread[::2] * 4) / 4
+    spread[3, : vocab // 3] = 1.25
+    spread[5] = 0.0                                                 # one value only: the draw counts ties off
+    sharp, on_boundaries = sampling_rows_on_boundaries(vocab, rows=12)
+    dev = torch.cat([spread, sharp]).cuda()
+    key = philox.uid_key("same-row")
+    requests = [(i, [0.7, 1.0, 1.9][i % 3], [1.0, 0.9, 0.3, 0.999][i % 4], (11 + i) ^ key, 1000 + 17 * i) for i in range(12)]
+    requests += [(12 + row, t, p, k, pos) for row, t, p, k, pos in on_boundaries]
+    alone = []
+    for request in requests:                                        # every request in a call of its own
+        out = torch.full((1,), -1, dtype=torch.int32, device="cuda")
+        K().sample_top_p(dev, [request], out)
+        alone.append(int(out.item()))
+    assert all(0 <= t < vocab for t in alone)
+    for n_rows in (len(requests), 33, 64, 200):
+        assert sample_among(K(), dev, requests, n_rows, n_rows) == alone, f"{n_rows} rows in the call"
+
+
 def test_the_sampler_takes_greedy_and_drawn_rows_of_one_step_together():
     from lockstep_amd.sampling import Sampler
     from lockstep_amd.sampling.sampler import top_p as host_top_p
@@ -749,6 +794,23 @@ def test_the_fold_for_few_rows_has_the_bits_of_the_general_fold_over_many_splits
             general = case.attend(dev[start:], start, d ** -0.5, variant=3, force_split=True, span=span)
             few = case.attend(dev[start:], start, d ** -0.5, variant=3, force_split=True, span=span, few_rows=True)
             assert torch.equal(general, ref) and torch.equal(few, ref), f"tokens={tokens} span={span}"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_the_fold_for_few_rows_is_right_when_it_is_handed_more_rows_than_it_was_promised(dtype):
+    """The caller says "at most 16 rows" and a request brings 24 and 40: the fold notices and takes the
+    general way (it used to leave the rows beyond the sixteenth unwritten)."""
+    nq, nkv, d, ps = 8, 1, 64, 16
+    kv_len = 900
+    qkv = rand_qkv(kv_len, nq, nkv, d, dtype, seed=77, sharp=(40,))
+    case = PagedCase(dtype, nq, nkv, d, ps, kv_len, shuffle_seed=2)
+    dev = qkv.cuda()
+    case.write(dev, 0)
+    for tokens in (3, 5):
+        start = kv_len - tokens
+        ref = case.attend(dev[start:], start, d ** -0.5, variant=0, force_split=False)
+        lied = case.attend(dev[start:], start, d ** -0.5, variant=0, force_split=True, few_rows=True)
+        assert not torch.isnan(lied).any() and torch.equal(lied, ref), tokens
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

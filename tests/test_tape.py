@@ -77,3 +77,18 @@ def test_compare_accepts_the_same_launches_and_names_the_first_other_one():
     stale[0] = launches_of(lib, 0x100000, 0xA00000)[0]
     with pytest.raises(RuntimeError, match="launch 0"):
         tape.compare(stale, addresses(0x300000, 0xA00000), "layer run 2")
+
+
+def test_an_address_inside_another_layers_tensor_refuses_the_tape():
+    """A launch of the noted layer names a tensor that is listed for another layer only: the noted
+    layer holds it somewhere the walk over its attributes does not reach."""
+    from lockstep_amd.engine.tape import TapeRefused
+
+    lib = FakeLibrary()
+    foreign = sorted([(0x300000, 0x300000 + 4096), (0xA00000, 0xA00000 + (1 << 20))])
+    LayerTape(launches_of(lib, 0x100000, 0x800000), addresses(0x100000, 0x800000), foreign)      # all its own: fine
+    odd = launches_of(lib, 0x100000, 0x800000)
+    odd[0] = (lib, lib.entry, (c_int(3), c_void_p(0x9000), c_void_p(0x300000 + 128), c_void_p(0), c_float(1e-6)))
+    with pytest.raises(TapeRefused, match="argument 2 .* another layer"):
+        LayerTape(odd, addresses(0x100000, 0x800000), foreign)
+    LayerTape(odd, addresses(0x100000, 0x800000))                                                # not asked to look

@@ -47,8 +47,9 @@ def test_repeated_launches_give_the_bits_of_every_layer_run_in_python(deep_dirs,
     for model in (taped, checked, plainly):
         cache = model.make_cache(num_pages=60, page_size=page_size, max_requests=4, poison_on_free=True)
         results.append(replay_in_process(model, cache, steps))
-    # four of six layers a step are repeated; graph-replayed decode steps launch nothing from the host
-    assert taped.layers_repeated >= 4 * (len(steps) - taped.graph_replays) > 0
+    # four of six layers a step are repeated (three in the very first step, whose third layer runs in Python
+    # once more to be compared with the tape); graph-replayed decode steps launch nothing from the host
+    assert taped.layers_repeated >= 4 * (len(steps) - taped.graph_replays) - 1 > 0 and taped.tapes_refused == 0
     assert checked.layers_repeated == 0 and plainly.layers_repeated == 0
     for rid in requests:
         assert torch.equal(results[0][rid], results[2][rid]), rid
@@ -75,7 +76,7 @@ def test_the_decode_loop_and_captured_steps_repeat_layers_too(deep_dirs):
             firsts.append(int(logits[0].argmax()))
         tokens[bool(flags)] = model.decode_greedy(cache, [0, 1, 2], firsts, 24)
         if not flags:
-            assert model.graph_replays > 0 and model.layers_repeated >= 5 * 4     # three prompts, first step, capture
+            assert model.graph_replays > 0 and model.layers_repeated >= 5 * 4 - 1   # three prompts, first step, capture
     assert (tokens[False] == tokens[True]).all()
 
 
@@ -91,3 +92,43 @@ def test_the_check_mode_notices_a_number_that_differs_from_layer_to_layer(deep_d
     cache.open("r")
     with pytest.raises(RuntimeError, match="layer run 4: launch 0 .* differs from the tape"):
         model.step(cache, [StepEntry("r", random_tokens(20, 512, seed=1), [19])])
+
+
+def test_a_tensor_that_the_walk_does_not_find_switches_the_repetition_off(deep_dirs):
+    """A part that says ``repeatable`` but keeps a per-layer tensor where the walk over its attributes
+    does not look: the first layer a tape could stand for runs in Python as well, its launches name
+    another tensor than the tape would, and the layers of that kind run in Python from then on --
+    with the right logits, where repeating the tape would have run every layer on one layer's weight."""
+    import types
+
+    from lockstep_amd.parts.norm import RMSNorm
+
+    class HiddenWeight(RMSNorm):
+        weight = property(lambda self: self.box.tensor, lambda self, value: None)
+
+    def hide(model):
+        for layer in model.layers:
+            norm = layer.mixer_norm
+            box = types.SimpleNamespace(tensor=norm.__dict__.pop("weight"))
+            norm.__class__, norm.box = HiddenWeight, box
+        return model
+
+    folder = deep_dirs["B"]
+    hidden = hide(load(folder, "float32", use_tapes=True, verify_tapes=False))
+    plainly = load(folder, "float32", use_tapes=False)
+    requests, steps = trace_for(hidden.spec.vocab_size)
+    results = []
+    for model in (hidden, plainly):
+        cache = model.make_cache(num_pages=60, page_size=8, max_requests=4, poison_on_free=True)
+        results.append(replay_in_process(model, cache, steps))
+    assert hidden.tapes_refused == 1 and hidden.layers_repeated == 0
+    for rid in requests:
+        assert torch.equal(results[0][rid], results[1][rid]), rid
+    # under the check mode the same model raises, and says where
+    checked = hide(load(folder, "float32", verify_tapes=True))
+    cache = checked.make_cache(num_pages=8, page_size=8, max_requests=1)
+    cache.open("r")
+    from lockstep_amd.engine.batch import StepEntry
+
+    with pytest.raises(RuntimeError, match="layer run 2: launch 0 .* differs from the tape"):
+        checked.step(cache, [StepEntry("r", random_tokens(20, 1000, seed=1), [19])])
