@@ -54,7 +54,7 @@ constexpr int D = LS_HEAD_DIM;
 #endif
 static_assert(D % 16 == 0 && D >= 16 && D <= 256, "head size must be a multiple of 16 up to 256");
 constexpr int kTileKeys = 128;
-constexpr int kSplitKeys = 256;
+constexpr int kSplitKeys = 128;
 #ifndef LS_ATTN_RING
 #define LS_ATTN_RING 8
 #endif
@@ -125,10 +125,6 @@ __device__ __forceinline__ constexpr int row_rotation(int row) {
   return sizeof(T) == 2 ? (row & 3) + 4 * ((row >> 3) & 3) : row;
 }
 
-template <typename T> __device__ __forceinline__ float softmax_exp(float x);
-template <> __device__ __forceinline__ float softmax_exp<float>(float x) { return expf(x); }
-template <> __device__ __forceinline__ float softmax_exp<bf16_t>(float x) { return __expf(x); }
-
 // Keep elements n_lo <= e < n_hi of a vector of VEC consecutive keys, zero the others.
 __device__ __forceinline__ bf16x8 mask_keys(bf16x8 v, int n_lo, int n_hi) {
   typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
@@ -145,6 +141,25 @@ __device__ __forceinline__ f32x4 mask_keys(f32x4 v, int n_lo, int n_hi) {
 #pragma unroll
   for (int e = 0; e < 4; ++e) v[e] = (e >= n_lo && e < n_hi) ? v[e] : 0.f;
   return v;
+}
+
+// All bits set in every element (the operand of mask_keys that turns it into a mask), and the bitwise AND.
+template <typename T> __device__ __forceinline__ typename Atom<T>::vec_t ones_vec();
+template <> __device__ __forceinline__ bf16x8 ones_vec<bf16_t>() {
+  typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
+  return __builtin_bit_cast(bf16x8, u32x4{0xFFFFFFFFu, 0xFFFFFFFFu, 0xFFFFFFFFu, 0xFFFFFFFFu});
+}
+template <> __device__ __forceinline__ f32x4 ones_vec<float>() {
+  typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
+  return __builtin_bit_cast(f32x4, u32x4{0xFFFFFFFFu, 0xFFFFFFFFu, 0xFFFFFFFFu, 0xFFFFFFFFu});
+}
+__device__ __forceinline__ bf16x8 and_vec(bf16x8 a, bf16x8 b) {
+  typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
+  return __builtin_bit_cast(bf16x8, __builtin_bit_cast(u32x4, a) & __builtin_bit_cast(u32x4, b));
+}
+__device__ __forceinline__ f32x4 and_vec(f32x4 a, f32x4 b) {
+  typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
+  return __builtin_bit_cast(f32x4, __builtin_bit_cast(u32x4, a) & __builtin_bit_cast(u32x4, b));
 }
 
 struct RowState {
@@ -1242,10 +1257,13 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
   // Sixteen lanes a head (head16_finish): the workgroup's sixteen groups take the heads vi = group, group + 16.
   constexpr int PASSES = D > 128 ? 2 : 1;
   const int gl = threadIdx.x & 15;
-  const int grp = threadIdx.x >> 4;
+  // the head a group of sixteen lanes takes: the first four heads go to the first group of each wave, the next
+  // four to the second groups, ... (a step has mostly four heads a workgroup: two query heads, the key and the
+  // value; in one wave their different branches would run one after the other)
+  const int grp = ((threadIdx.x >> 4) & 3) * 4 + (threadIdx.x >> 6);
   long page_new = -1;
-  float hx[8 * PASSES];
-  HeadFactors<PASSES> hf;
+  float hx[8 * PASSES] = {};
+  HeadFactors<PASSES> hf = {};
   auto head_src = [&](int vi) -> const T* {
     return new_row + (long)(vi < G ? kvh * G + vi : vi == G ? fz.nq + kvh : fz.nq + nkv + kvh) * D;
   };
@@ -1255,12 +1273,57 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
       head16_load_factors<PASSES>(hf, D, vi < G ? fz.q_weight : fz.k_weight, fz.cos_table, fz.sin_table, p_new,
                                   fz.rot, gl);
   };
+  T* qrot = reinterpret_cast<T*>(prob);  // FUSE: [16][D] rotated query heads; the exchange buffers are free until the loop
+  // norm and rotation of head vi from hx / hf: a query head to qrot, the new key and value to LDS and to the cache
+  auto finish_head = [&](int vi) {
+    const int slot_new = p_new & (page_size - 1);
+    if (vi < G) {
+      head16_finish<T, PASSES>(hx, hf, D, fz.q_weight != nullptr, fz.eps, rotated, fz.rot, gl,
+                               [&](int e0, const T (&v)[8]) { store8<T>(qrot + vi * D + e0, v); });
+    } else if (vi == G) {
+      T* dst = fz.k_out + ((max(page_new, 0L) * nkv + kvh) * page_size + slot_new) * D;
+      head16_finish<T, PASSES>(hx, hf, D, fz.k_weight != nullptr, fz.eps, rotated, fz.rot, gl,
+                               [&](int e0, const T (&v)[8]) {
+                                 store8<T>(knew + e0, v);
+                                 if (page_new >= 0) store8<T>(dst + e0, v);
+                               });
+    } else {
+      T* dst = fz.v_out + ((max(page_new, 0L) * nkv + kvh) * D) * page_size + slot_new;
+#pragma unroll
+      for (int p = 0; p < PASSES; ++p) {
+        const int e0 = 128 * p + 8 * gl;
+        if (e0 >= D) continue;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const T v = from_f32<T>(hx[8 * p + j]);
+          vnew[e0 + j] = v;
+          if (page_new >= 0) dst[(long)(e0 + j) * page_size] = v;
+        }
+      }
+    }
+  };
   if (FUSE) {
     if (owner) page_new = tbl[p_new >> page_shift];
     if (grp < n_vec) head_fetch(grp);
   }
   if (ti_lo < ti_hi) fill_pages(ti_lo);
   __syncthreads();
+  if (FUSE) {
+    // The head's operands are awaited here, before the tile loads go out: a wait placed after them would also
+    // wait for the tiles (loads complete in the order of their issue, and the compiler does not count the tile
+    // loads), and the norm, the rotation and the cache write below would start only when the tiles are in.
+#pragma unroll
+    for (int i = 0; i < 8 * PASSES; ++i) __asm__ volatile("" ::"v"(hx[i]), "v"(hf.w[i]), "v"(hf.c[i]), "v"(hf.s[i]));
+    __asm__ volatile("" ::"v"((int)page_new));
+    if (n_vec > 16) {  // more heads than groups of sixteen lanes (fifteen query heads a kv head and more): all of
+      finish_head(grp);  // them now, so that no load of a head stands behind the tile loads
+      if (grp + 16 < n_vec) {
+        head_fetch(grp + 16);
+        finish_head(grp + 16);
+      }
+    }
+  }
+  PROBE(1)
   auto issue_tile = [&](int ti) {
     if (NBUF == 2) {
       issue(ti);
@@ -1270,36 +1333,14 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
     }
   };
   if (ti_lo < ti_hi) issue_tile(ti_lo);
+  // two buffers: both are free now, so the second tile is requested at once as well and its wait overlaps the
+  // first one's (a workgroup of a decode step mostly has two tiles, and a miss takes longer than a tile's work)
+  constexpr bool CAN_PRIME = NBUF == 2 && 2 * PER <= 63;  // (the wait names the loads of one tile: a 6-bit count)
+  const bool primed = CAN_PRIME && ti_lo + 1 < ti_hi && !window_start(ti_lo + 1);
+  if (primed) issue(ti_lo + 1);
+  PROBE(2)
   if (FUSE) {
-    T* qrot = reinterpret_cast<T*>(prob);  // [16][D]: the exchange buffers are free until the loop
-    const int slot_new = p_new & (page_size - 1);
-    for (int vi = grp; vi < n_vec; vi += 16) {  // uniform for the group
-      if (vi != grp) head_fetch(vi);
-      if (vi < G) {
-        head16_finish<T, PASSES>(hx, hf, D, fz.q_weight != nullptr, fz.eps, rotated, fz.rot, gl,
-                                 [&](int e0, const T (&v)[8]) { store8<T>(qrot + vi * D + e0, v); });
-      } else if (vi == G) {
-        T* dst = fz.k_out + ((max(page_new, 0L) * nkv + kvh) * page_size + slot_new) * D;
-        head16_finish<T, PASSES>(hx, hf, D, fz.k_weight != nullptr, fz.eps, rotated, fz.rot, gl,
-                                 [&](int e0, const T (&v)[8]) {
-                                   store8<T>(knew + e0, v);
-                                   if (page_new >= 0) store8<T>(dst + e0, v);
-                                 });
-      } else {
-        T* dst = fz.v_out + ((max(page_new, 0L) * nkv + kvh) * D) * page_size + slot_new;
-#pragma unroll
-        for (int p = 0; p < PASSES; ++p) {
-          const int e0 = 128 * p + 8 * gl;
-          if (e0 >= D) continue;
-#pragma unroll
-          for (int j = 0; j < 8; ++j) {
-            const T v = from_f32<T>(hx[8 * p + j]);
-            vnew[e0 + j] = v;
-            if (page_new >= 0) dst[(long)(e0 + j) * page_size] = v;
-          }
-        }
-      }
-    }
+    if (n_vec <= 16 && grp < n_vec) finish_head(grp);  // (more heads than groups: done above, before the tile loads)
     lds_barrier();
 #pragma unroll
     for (int c = 0; c < NC; ++c) {
@@ -1311,6 +1352,7 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
 #pragma unroll
     for (int c = 0; c < NC; ++c) __asm__ volatile("" ::"v"(qv[c]));
   }
+  PROBE(3)
   for (int ti = ti_lo; ti < ti_hi; ++ti) {
     const int t0 = ti * kTileKeys;
     const unsigned char* k_lds = lds + (NBUF == 2 ? (ti & 1) : 0) * BUF_BYTES;
@@ -1324,7 +1366,13 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
       issue_tile(ti);
     }
     if (NBUF == 2) {
-      __asm__ volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this thread's pieces of the tile have landed
+      // this thread's pieces of the tile have landed (loads complete in the order of their issue: behind the
+      // first tile only the 2 * PER loads of the second one, and stores, may still be on their way)
+      if (primed && ti == ti_lo) {
+        if constexpr (CAN_PRIME) __asm__ volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * PER) : "memory");
+      } else {
+        __asm__ volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      }
     } else {
       // this thread's pieces of the K tile have landed; its PER loads of the V tile, issued later, may be in flight
       __asm__ volatile("s_waitcnt vmcnt(%0)" ::"n"(PER) : "memory");
@@ -1334,7 +1382,7 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
     PROBE(5)
     const bool patch = owner && ti == tile_new;  // the new key and value go into this tile
     const bool clean = t0 + kTileKeys > sm.kv_len || t0 < lo_valid || patch;  // uniform
-    if (NBUF == 1 && FUSE && patch) {  // the new key goes into the K tile now, the V tile is dealt with when it is there
+    if (FUSE && patch) {  // the new key goes into the K tile now; the values are dealt with where they are read
 #pragma unroll
       for (int i = 0; i < PER; ++i) {
         const int p = i * NT + (int)threadIdx.x;
@@ -1347,31 +1395,7 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
       }
       lds_barrier();
     }
-    auto clean_values = [&](bool with_key) {  // clean the values of keys that are not held, place the new ones
-#pragma unroll
-      for (int i = 0; i < PER; ++i) {
-        const int p = i * NT + (int)threadIdx.x;
-        if (PER * NT != TOTAL && p >= TOTAL) break;
-        const int key0 = t0 + (p / D) * VEC;
-        vec_t* at = reinterpret_cast<vec_t*>(v_lds + p * 16);
-        vec_t v = mask_keys(*at, lo_valid - key0, sm.kv_len - key0);
-        if (FUSE && patch) {
-          const T fresh = vnew[p % D];
-#pragma unroll
-          for (int e = 0; e < VEC; ++e) v[e] = key0 + e == p_new ? fresh : v[e];
-          const int row = p / KPIECES;
-          if (with_key && t0 + row == p_new) {
-            const int piece = (p % KPIECES - row_rotation<T>(row) % KPIECES + KPIECES) % KPIECES;
-            *reinterpret_cast<vec_t*>(const_cast<unsigned char*>(k_lds) + p * 16) =
-                *reinterpret_cast<const vec_t*>(knew + piece * VEC);
-          }
-        }
-        *at = v;
-      }
-      lds_barrier();
-    };
-    if (NBUF == 2 && clean) clean_values(true);
-    if (NBUF == 2 && ahead) issue(ti + 1);
+    if (NBUF == 2 && ahead && !(primed && ti == ti_lo)) issue(ti + 1);
 
     // score blocks 2w and 2w+1
     PROBE(6)
@@ -1425,7 +1449,7 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
     }
     // this wave's value operands do not depend on the probabilities: with two buffers they are read before the
     // barrier; with one buffer the V tile is only now awaited (the K loads of the next tile, issued after it,
-    // may stay in flight), complete for every thread after the barrier, and cleaned then
+    // may stay in flight) and complete for every thread after the barrier
     constexpr int KB16 = VEC / 4;
     constexpr int NPAIR = NB / KB16;
     vec_t vop[NPAIR][MYDB];
@@ -1454,8 +1478,37 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
         vop[kp][j] = vv;
       }
     };
+    // The values of keys that are not held become zeros and the new token's value takes its place: in the
+    // operands as they were read (a lane's VEC values of a column belong to VEC consecutive keys), not in LDS.
+    auto fix_values = [&]() {
+#pragma unroll
+      for (int kp = 0; kp < NPAIR; ++kp) {
+        const int key0 = t0 + key_of_row<T>(kp * KB16, 4 * g);
+        const int n_lo = lo_valid - key0, n_hi = sm.kv_len - key0;
+        if (t0 + kp * (16 * KB16) + 16 * KB16 <= sm.kv_len && t0 + kp * (16 * KB16) >= lo_valid && !(FUSE && patch))
+          continue;  // uniform: every key of this pair of blocks is held
+        if (n_lo > 0 || n_hi < VEC) {
+          // one mask for the lane's VEC keys, used for all of its columns
+          const vec_t keep = mask_keys(ones_vec<T>(), n_lo, n_hi);
+#pragma unroll
+          for (int j = 0; j < MYDB; ++j) vop[kp][j] = and_vec(vop[kp][j], keep);
+        }
+        if (FUSE && patch && p_new >= key0 && p_new < key0 + VEC) {
+#pragma unroll
+          for (int j = 0; j < MYDB; ++j) {
+            const int blk = wave + 4 * j;
+            const T fresh = vnew[(blk < DB ? blk : 0) * 16 + row16];
+            vec_t v = vop[kp][j];
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) v[e] = key0 + e == p_new ? fresh : v[e];
+            vop[kp][j] = v;
+          }
+        }
+      }
+    };
     if (NBUF == 2) {
       read_values();
+      if (clean) fix_values();
     } else if (ahead) {
       __asm__ volatile("s_waitcnt vmcnt(%0)" ::"n"(PER) : "memory");
     } else {
@@ -1465,8 +1518,8 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
     lds_barrier();
     PROBE(10)
     if (NBUF == 1) {
-      if (clean) clean_values(false);
       read_values();
+      if (clean) fix_values();
     }
     float p_sum = 0.f;
 #pragma unroll
@@ -1873,9 +1926,11 @@ template <typename T, bool FUSE, bool SPANS>
 static int launch_coop_as(dim3 grid, hipStream_t s, const void* q, long ldq, const void* k_pages, const void* v_pages,
                           int nkv, int page_size, int page_shift, const int* table, int table_stride, const void* seqs,
                           const void* items, void* out, long ldo, float* part_acc, float* part_ml, int G, float scale,
-                          int window, DecodeFuse<T> fz) {
+                          int window, DecodeFuse<T> fz, bool single_tile) {
   constexpr int BUFS = coop_bufs(sizeof(T));
-  const bool crowded = (long)grid.x * grid.y >= LS_COOP_CROWDED_FROM;
+  // one tile buffer (two workgroups a CU) where a second one could not be used: many workgroups, or items of
+  // one tile each, which have no next tile to request ahead
+  const bool crowded = (long)grid.x * grid.y >= LS_COOP_CROWDED_FROM || single_tile;
 #define LS_COOP(NBUF_)                                                                                              \
   hipLaunchKernelGGL((attention_coop_kernel<T, NBUF_, FUSE, SPANS>), grid, dim3(256), (coop_kernel_lds<T, NBUF_>()), s, \
                      (const T*)q, ldq, (const T*)k_pages, (const T*)v_pages, nkv, page_size, page_shift, table,        \
@@ -1895,15 +1950,19 @@ static int launch_coop_as(dim3 grid, hipStream_t s, const void* q, long ldq, con
 // ``spans``: items may hold several splits and leave a partial result for each (an instance of its own, so
 // that the usual one-split items keep their code).
 template <typename T, bool FUSE>
-static int launch_coop(bool spans, dim3 grid, hipStream_t s, const void* q, long ldq, const void* k_pages,
+static int launch_coop(int spans, dim3 grid, hipStream_t s, const void* q, long ldq, const void* k_pages,
                        const void* v_pages, int nkv, int page_size, int page_shift, const int* table, int table_stride,
                        const void* seqs, const void* items, void* out, long ldo, float* part_acc, float* part_ml, int G,
                        float scale, int window, DecodeFuse<T> fz) {
-  if (spans)
+  // spans: bit 0, items that leave partial results may hold several splits; bit 1, every item holds one tile
+  const bool single_tile = (spans & 2) != 0;
+  if (spans & 1)
     return launch_coop_as<T, FUSE, true>(grid, s, q, ldq, k_pages, v_pages, nkv, page_size, page_shift, table,
-                                         table_stride, seqs, items, out, ldo, part_acc, part_ml, G, scale, window, fz);
+                                         table_stride, seqs, items, out, ldo, part_acc, part_ml, G, scale, window, fz,
+                                         false);
   return launch_coop_as<T, FUSE, false>(grid, s, q, ldq, k_pages, v_pages, nkv, page_size, page_shift, table,
-                                        table_stride, seqs, items, out, ldo, part_acc, part_ml, G, scale, window, fz);
+                                        table_stride, seqs, items, out, ldo, part_acc, part_ml, G, scale, window, fz,
+                                        single_tile);
 }
 
 static bool coop_supported(int dtype) {
@@ -1964,12 +2023,12 @@ extern "C" int ls_attention_decode(int dtype, const void* qkv, long ld, void* k_
   int rc = 0;
   if (dtype == kF32) {
     DecodeFuse<float> fz{q_weight, k_weight, eps, cos_table, sin_table, rot, nq, write_kv, (float*)k_pages, (float*)v_pages};
-    rc = launch_coop<float, true>(spans != 0, grid, s, qkv, ld, k_pages, v_pages, nkv, page_size, page_shift, table, table_stride,
+    rc = launch_coop<float, true>(spans, grid, s, qkv, ld, k_pages, v_pages, nkv, page_size, page_shift, table, table_stride,
                                   seqs, items, out, ldo, part_acc, part_ml, G, scale, window, fz);
   } else if (dtype == kBF16) {
     DecodeFuse<bf16_t> fz{q_weight, k_weight, eps, cos_table, sin_table, rot, nq, write_kv, (bf16_t*)k_pages,
                           (bf16_t*)v_pages};
-    rc = launch_coop<bf16_t, true>(spans != 0, grid, s, qkv, ld, k_pages, v_pages, nkv, page_size, page_shift, table, table_stride,
+    rc = launch_coop<bf16_t, true>(spans, grid, s, qkv, ld, k_pages, v_pages, nkv, page_size, page_shift, table, table_stride,
                                    seqs, items, out, ldo, part_acc, part_ml, G, scale, window, fz);
   } else {
     return fail("decode attention: unknown dtype %d", dtype);
@@ -2041,10 +2100,10 @@ extern "C" int ls_attention(int dtype, const void* q, long ldq, const void* k_pa
     LS_REQUIRE(page_size >= 8, "attention: the cooperative variant needs pages of at least 8 keys, got %d", page_size);
     int rc = 0;
     if (dtype == kF32)
-      rc = launch_coop<float, false>(spans != 0, grid, s, q, ldq, k_pages, v_pages, nkv, page_size, page_shift, table, table_stride,
+      rc = launch_coop<float, false>(spans, grid, s, q, ldq, k_pages, v_pages, nkv, page_size, page_shift, table, table_stride,
                                      seqs, items, out, ldo, part_acc, part_ml, G, scale, window, DecodeFuse<float>{});
     else if (dtype == kBF16)
-      rc = launch_coop<bf16_t, false>(spans != 0, grid, s, q, ldq, k_pages, v_pages, nkv, page_size, page_shift, table,
+      rc = launch_coop<bf16_t, false>(spans, grid, s, q, ldq, k_pages, v_pages, nkv, page_size, page_shift, table,
                                       table_stride, seqs, items, out, ldo, part_acc, part_ml, G, scale, window,
                                       DecodeFuse<bf16_t>{});
     else

@@ -99,6 +99,12 @@ __device__ __forceinline__ typename Atom<T>::vec_t load_vec(const T* __restrict_
   return v;
 }
 
+// The exponential of the softmax and of the fold over attention splits: the library routine on the
+// 32-bit path, the hardware's on the bfloat16 path.  One definition for every kernel that folds.
+template <typename T> __device__ __forceinline__ float softmax_exp(float x);
+template <> __device__ __forceinline__ float softmax_exp<float>(float x) { return expf(x); }
+template <> __device__ __forceinline__ float softmax_exp<bf16_t>(float x) { return __expf(x); }
+
 // Sum / max over the four lanes {l, l^16, l^32, l^48}; every lane of the
 // four ends with the same bits because each step adds a pair commutatively.
 __device__ __forceinline__ float quad16_sum(float v) {
@@ -363,6 +369,7 @@ namespace ls {
 constexpr int kMutantKsliceByRows = 1;  // the skinny product cuts K into other slices above 16 rows
 constexpr int kMutantNormByRows = 2;    // RMSNorm adds its wave sums in another order in launches of more than four rows
 constexpr int kMutantSampleChunksByRows = 4;  // the sampler cuts a row into fewer chunks when the call has many rows
+constexpr int kMutantReversedFoldInProduct = 8;  // the product that folds attention splits itself folds them from the last to the first
 // bits of the mask, attention libraries
 constexpr int kMutantReversedFold = 1;  // the combine kernel folds the splits from the last to the first
 }  // namespace ls

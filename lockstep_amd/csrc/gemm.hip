@@ -551,6 +551,133 @@ __global__ __launch_bounds__(256) void gemm_slices_kernel(const T* __restrict__ 
   }
 }
 
+// The slice kernel for an operand that is still the per-split sums of an attention launch (decoded tokens,
+// at most 16 rows): X [m][k] is the output of token m, head k / head_dim, column k % head_dim, which the fold
+// over the token's `splits` partial results (acc, m, l), ascending from the empty state, skipping empty ones,
+// then acc / l rounded to T, would give.  A workgroup takes one K slice and 64 output columns: its four waves
+// fold the slice's elements into LDS together first (every group of 64 columns repeats that, which costs
+// little while rows times splits are few), then each wave multiplies its 16 columns from there.  The launch
+// that would fold them into an output, and the round trip of that output, are saved.  Partial row of (token
+// m, head h, split s): (m * heads + h) * splits + s, as the attention kernels lay single decoded tokens out.
+// The fold is the attention library's fold_split operation by operation, and the chain of a slice is
+// gemm_slices_kernel's: the same bits as fold, then product.
+// UNITS, SPLITS: a thread's groups of four elements whose sums are requested together, and the most splits
+// each has (instances for few and for more of either; splits <= SPLITS and the host's choice of UNITS
+// change nothing in the arithmetic).  REVERSED: a wrong variant for the tests' control library (descending fold).
+template <typename T, bool REVERSED, int UNITS, int SPLITS>
+__global__ __launch_bounds__(256) void gemm_slices_folded_kernel(const float* __restrict__ part_acc,
+                                                                 const float* __restrict__ part_ml, int splits,
+                                                                 int head_dim, const T* __restrict__ W,
+                                                                 float* __restrict__ P, int M, int N, int K, int kslice) {
+  typedef Atom<T> A;
+  typedef typename A::vec_t vec_t;
+  extern __shared__ __attribute__((aligned(16))) unsigned char folded_lds[];
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int n0 = blockIdx.x * 64 + wave * 16;
+  const int row16 = lane & 15;
+  const int g = lane >> 4;
+  const int s = blockIdx.y;
+  const int k_begin = s * kslice;
+  const int k_end = min(K, k_begin + kslice);
+  const int row_stride = kslice + 16 / (int)sizeof(T);  // elements; the pad spreads the rows over the banks
+  T* xs = reinterpret_cast<T*>(folded_lds);             // [M][row_stride]
+  const int heads = K / head_dim;
+
+  // The weights of the slice's first round are requested before the sums: both are on their way together, and
+  // the fold runs while the weights arrive.
+  constexpr int UNR = 8;  // a slice of 256 elements in one round of loads
+  vec_t w_first[UNR];
+#pragma unroll
+  for (int u = 0; u < UNR; ++u) {
+    const int k = k_begin + u * A::KCHUNK + g * A::VEC;
+    w_first[u] = load_vec<T>(W, n0 + row16, k, K, K, n0 + row16 < N && k_begin + u * A::KCHUNK < k_end, true);
+  }
+  __builtin_amdgcn_sched_barrier(0);  // (the scheduler would move these loads down to their use, behind the fold)
+
+  // A unit is four neighbouring elements of one row; thread t takes the units t, t + 256, ...  A unit's
+  // splits are folded one after the other; the sums of UNITS units are requested together.
+  const int quads = kslice / 4;
+  const int units = M * quads;
+  for (int u0 = threadIdx.x; u0 < units; u0 += 256 * UNITS) {
+    f32x4 acc[UNITS][SPLITS];
+    float2 ml[UNITS][SPLITS];
+#pragma unroll
+    for (int j = 0; j < UNITS; ++j) {
+      const int unit = min(u0 + 256 * j, units - 1);                 // (clamped: loaded, not used)
+      const int m = unit / quads;
+      const int k = min(k_begin + 4 * (unit - m * quads), K - 4);
+      const int head = k / head_dim;
+      const long pr0 = ((long)m * heads + head) * splits;
+      const float* from = part_acc + (k - head * head_dim);
+#pragma unroll
+      for (int sp = 0; sp < SPLITS; ++sp) {
+        const int at = min(sp, splits - 1);
+        const long pr = pr0 + (REVERSED ? splits - 1 - at : at);
+        acc[j][sp] = *reinterpret_cast<const f32x4*>(from + pr * head_dim);
+        ml[j][sp] = *reinterpret_cast<const float2*>(part_ml + pr * 2);
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);  // every request is made before the first sum is used
+#pragma unroll
+    for (int j = 0; j < UNITS; ++j) {
+      f32x4 run_acc = f32x4{0.f, 0.f, 0.f, 0.f};
+      float run_m = kNegSentinel, run_l = 0.f;
+#pragma unroll
+      for (int sp = 0; sp < SPLITS; ++sp) {
+        if (sp < splits && ml[j][sp].y > 0.f) {  // fold_split on these four columns
+          const float m_new = fmaxf(run_m, ml[j][sp].x);
+          const float fa = softmax_exp<T>(run_m - m_new);
+          const float fb = softmax_exp<T>(ml[j][sp].x - m_new);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) run_acc[e] = run_acc[e] * fa + acc[j][sp][e] * fb;
+          run_l = run_l * fa + ml[j][sp].y * fb;
+          run_m = m_new;
+        }
+      }
+      const int unit = u0 + 256 * j;
+      const int m = unit / quads;
+      const int k = k_begin + 4 * (unit - m * quads);
+      if (unit < units && k < k_end) {  // the unit is folded: acc / l, rounded as the attention output is
+        T* dst = xs + (long)m * row_stride + (k - k_begin);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) dst[e] = from_f32<T>(run_l > 0.f ? run_acc[e] / run_l : 0.f);
+      }
+    }
+  }
+  __syncthreads();
+  if (n0 >= N) return;
+
+  f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int k0 = k_begin; k0 < k_end; k0 += UNR * A::KCHUNK) {
+    vec_t w[UNR], x[UNR];
+#pragma unroll
+    for (int u = 0; u < UNR; ++u) {
+      const int k = k0 + u * A::KCHUNK + g * A::VEC;
+      const bool in = k0 + u * A::KCHUNK < k_end;
+      w[u] = k0 == k_begin ? w_first[u] : load_vec<T>(W, n0 + row16, k, K, K, n0 + row16 < N && in, true);
+      x[u] = (row16 < M && in && k < k_end) ? *reinterpret_cast<const vec_t*>(xs + (long)row16 * row_stride + (k - k_begin))
+                                            : A::zero();
+    }
+#pragma unroll
+    for (int u = 0; u < UNR; ++u) {
+      if (k0 + u * A::KCHUNK >= k_end) break;  // uniform: a chunk is visited iff it starts inside the slice
+      A::mma(acc, w[u], x[u]);
+    }
+  }
+  const int n = n0 + g * 4;
+  if (row16 < M && n < N) {
+    float* dst = P + ((long)s * M + row16) * N + n;
+    if (n + 3 < N && (N & 3) == 0) {
+      *reinterpret_cast<f32x4*>(dst) = acc;
+    } else {
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        if (n + r < N) dst[r] = acc[r];
+    }
+  }
+}
+
 // The slice kernel for many rows and many columns: a wave takes one K slice of NTL column tiles (16 * NTL
 // columns) and all the rows, so a chunk of X that it has loaded meets NTL chunks of weights and a chunk of
 // weights MT chunks of X: at 64 rows and 64 columns the rows of X are read once for every byte of weights,
@@ -1253,4 +1380,66 @@ extern "C" int ls_gemm_slices(int dtype, const void* X, const void* W, float* P,
 #undef LS_SLICES_MT
 #undef LS_SLICES
   return check_launch("gemm_slices");
+}
+
+// Whether ls_gemm_slices_folded takes this product: at most 16 rows, whole heads of a size that is a
+// multiple of four, K a multiple of the load width, at most 32 splits, the folded rows of a slice within
+// 64 KB of LDS -- and the plain slice kernel is what ls_gemm_slices itself would run for these sizes (over
+// large weights it prefers the tiled kernel from eight rows on, which reads its operand from memory).
+extern "C" int ls_gemm_slices_folded_ok(int dtype, int M, int N, int K, int head_dim, int splits) {
+  using namespace ls;
+  if (dtype != kF32 && dtype != kBF16) return 0;
+  if (M < 1 || M > 16 || N < 1 || K < 1 || head_dim < 4 || head_dim % 4 || K % head_dim) return 0;
+  if (splits < 1 || splits > 32 || K % (dtype == kF32 ? 4 : 8)) return 0;
+  const long weight_bytes = (long)N * K * (dtype == kF32 ? 4 : 2);
+  const int tiled_from = dtype == kF32 ? 33 : (weight_bytes >= (64L << 20) ? 8 : 17);
+  if (LS_GEMM_SLICES_TILED && M >= tiled_from && N % 4 == 0) return 0;
+  const size_t element = dtype == kF32 ? 4 : 2;
+  return (size_t)M * (kslice_for(K) + 16 / element) * element <= 64 * 1024;
+}
+
+// ls_gemm_slices for an operand that is still `splits` per-split sums a (token, head) of an attention
+// launch over single decoded tokens (see gemm_slices_folded_kernel): part_acc [(M * heads) * splits][head_dim],
+// part_ml [(M * heads) * splits][2], heads = K / head_dim.  P as ls_gemm_slices leaves it, bit for bit what
+// it leaves for the folded and rounded operand.
+extern "C" int ls_gemm_slices_folded(int dtype, const float* part_acc, const float* part_ml, int splits, int head_dim,
+                                     const void* W, float* P, int M, int N, int K, void* stream) {
+  using namespace ls;
+  LS_REQUIRE(ls_gemm_slices_folded_ok(dtype, M, N, K, head_dim, splits),
+             "gemm_slices_folded: not for M=%d N=%d K=%d head_dim=%d splits=%d (see ls_gemm_slices_folded_ok)", M, N, K,
+             head_dim, splits);
+  LS_REQUIRE(part_acc && part_ml && W && P, "gemm_slices_folded: null operand");
+  LS_REQUIRE(reinterpret_cast<uintptr_t>(P) % 16 == 0 && reinterpret_cast<uintptr_t>(W) % 16 == 0 &&
+                 reinterpret_cast<uintptr_t>(part_acc) % 16 == 0 && reinterpret_cast<uintptr_t>(part_ml) % 8 == 0,
+             "gemm_slices_folded: operands must be 16-byte aligned");
+  const int kslice = kslice_for(K);
+  const int nslices = (K + kslice - 1) / kslice;
+  const size_t element = dtype == kF32 ? 4 : 2;
+  const size_t lds = (size_t)M * (kslice + 16 / element) * element;
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  dim3 grid((N + 63) / 64, nslices);
+#define LS_FOLDED_N(T_, REV_, UNITS_, SPLITS_)                                                                       \
+  hipLaunchKernelGGL((gemm_slices_folded_kernel<T_, REV_, UNITS_, SPLITS_>), grid, dim3(256), lds, s, part_acc, part_ml, \
+                     splits, head_dim, (const T_*)W, P, M, N, K, kslice)
+  // units of a thread whose sums are in flight together: all of them up to four
+  const int mine = (M * (kslice / 4) + 255) / 256;
+#define LS_FOLDED_S(T_, REV_, SPLITS_)                       \
+  if (mine <= 1) LS_FOLDED_N(T_, REV_, 1, SPLITS_);          \
+  else if (mine <= 2) LS_FOLDED_N(T_, REV_, 2, SPLITS_);     \
+  else LS_FOLDED_N(T_, REV_, 4, SPLITS_)
+#define LS_FOLDED(T_, REV_)                                  \
+  if (splits <= 4) { LS_FOLDED_S(T_, REV_, 4); }             \
+  else if (splits <= 8) { LS_FOLDED_S(T_, REV_, 8); }        \
+  else LS_FOLDED_N(T_, REV_, 1, 32)
+#ifdef LS_MUTANTS
+  if (LS_MUTANT_HOST(kMutantReversedFoldInProduct)) {
+    if (dtype == kF32) { LS_FOLDED(float, true); } else { LS_FOLDED(bf16_t, true); }
+    return check_launch("gemm_slices_folded");
+  }
+#endif
+  if (dtype == kF32) { LS_FOLDED(float, false); } else { LS_FOLDED(bf16_t, false); }
+#undef LS_FOLDED_S
+#undef LS_FOLDED_N
+#undef LS_FOLDED
+  return check_launch("gemm_slices_folded");
 }

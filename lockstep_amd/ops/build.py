@@ -98,8 +98,21 @@ def find_hipcc() -> str:
     raise BuildError("hipcc was not found (looked at $HIPCC, PATH and /opt/rocm/bin); the kernels cannot be built")
 
 
+def _run(cmd, what: str) -> None:
+    env = dict(os.environ)
+    env.setdefault("TMPDIR", tempfile.gettempdir())
+    if not env.get("HOME") or not os.access(env["HOME"], os.W_OK):
+        env["HOME"] = tempfile.gettempdir()
+    proc = subprocess.run(cmd, capture_output=True, text=True, env=env)
+    if proc.returncode != 0:
+        raise BuildError(f"hipcc failed for {what}:\n{' '.join(cmd)}\n{proc.stderr[-4000:]}")
+
+
 def _compile(kind: str, sources, defines, out: Path) -> None:
-    cmd = [find_hipcc(), *FLAGS, *defines, "-o", str(out), *[str(CSRC / s) for s in sources]]
+    """Compile ``sources`` into the shared library ``out``: every source to an object file of its own,
+    side by side, then one link (a library of several sources takes as long as its slowest one)."""
+    hipcc = find_hipcc()
+    compile_flags = [f for f in FLAGS if f != "-shared"]
     started = time.time()
     print(f"[lockstep_amd] compiling {kind} kernels for {ARCH} -> {out.name}", file=sys.stderr, flush=True)
     done = threading.Event()
@@ -111,16 +124,32 @@ def _compile(kind: str, sources, defines, out: Path) -> None:
 
     thread = threading.Thread(target=ticker, daemon=True)
     thread.start()
+    objects = [out.with_name(f"{out.name}.{Path(s).stem}.o") for s in sources]
     try:
-        env = dict(os.environ)
-        env.setdefault("TMPDIR", tempfile.gettempdir())
-        if not env.get("HOME") or not os.access(env["HOME"], os.W_OK):
-            env["HOME"] = tempfile.gettempdir()
-        proc = subprocess.run(cmd, capture_output=True, text=True, env=env)
+        if len(sources) == 1:
+            _run([hipcc, *FLAGS, *defines, "-o", str(out), str(CSRC / sources[0])], kind)
+        else:
+            errors: list = []
+
+            def one(source, obj):
+                try:
+                    _run([hipcc, *compile_flags, *defines, "-c", "-o", str(obj), str(CSRC / source)], f"{kind} ({source})")
+                except Exception as exc:  # noqa: BLE001 - reported below
+                    errors.append(exc)
+
+            workers = [threading.Thread(target=one, args=pair) for pair in zip(sources, objects)]
+            for w in workers:
+                w.start()
+            for w in workers:
+                w.join()
+            if errors:
+                raise errors[0]
+            _run([hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", str(out), *[str(o) for o in objects]], kind)
     finally:
         done.set()
-    if proc.returncode != 0:
-        raise BuildError(f"hipcc failed for {kind}:\n{' '.join(cmd)}\n{proc.stderr[-4000:]}")
+        for obj in objects:
+            if obj.exists():
+                obj.unlink()
     print(f"[lockstep_amd] compiled {kind} in {time.time() - started:.1f} s", file=sys.stderr, flush=True)
 
 

@@ -115,6 +115,7 @@ class Kernels:
 
     #: bits of ``set_mutants`` (csrc/common.h)
     MUTANT_KSLICE_BY_ROWS, MUTANT_NORM_BY_ROWS, MUTANT_SAMPLE_CHUNKS_BY_ROWS = 1, 2, 4      # core library
+    MUTANT_REVERSED_FOLD_IN_PRODUCT = 8
     MUTANT_REVERSED_FOLD = 1                               # attention libraries
 
     def set_mutants(self, core: int = 0, attention: int = 0) -> None:
@@ -231,6 +232,37 @@ class Kernels:
         self._launch(self.core, self.core.ls_gemm_slices, (
             c_int(DTYPE_CODE[w.dtype]), _ptr(x), _ptr(w), _ptr(partials), c_int(m), c_int(n), c_int(k),
             c_long(x.stride(0)), _stream()))
+
+    def gemm_slices_folded_ok(self, dtype: torch.dtype, m: int, n: int, k: int, head_dim: int, splits: int) -> bool:
+        """Whether ``gemm_slices_folded`` takes a product of these sizes."""
+        return self._memo(("slices_folded", dtype, m, n, k, head_dim, splits), lambda: bool(
+            self.core.ls_gemm_slices_folded_ok(c_int(DTYPE_CODE[dtype]), c_int(m), c_int(n), c_int(k), c_int(head_dim),
+                                               c_int(splits))))
+
+    def gemm_slices_folded(self, part_acc: torch.Tensor, part_ml: torch.Tensor, splits: int, head_dim: int,
+                           w: torch.Tensor, partials: torch.Tensor) -> None:
+        """``gemm_slices`` for an operand that still lies as the per-split sums of an attention launch over
+        single decoded tokens: row ``(m * heads + h) * splits + s`` of ``part_acc [., head_dim]`` and
+        ``part_ml [., 2]`` holds split ``s`` of token ``m``, head ``h``.  The kernel folds them (ascending,
+        from the empty state, then sum / weight rounded to the compute dtype: what the combine launch
+        would write) on its way; ``partials [slices, M, N]`` gets the bits ``gemm_slices`` would leave."""
+        slices, m, n = partials.shape
+        k = w.shape[1]
+        if not (w.is_cuda and w.dim() == 2 and w.is_contiguous() and w.dtype in DTYPE_CODE and w.shape[0] == n):
+            raise KernelError("gemm_slices_folded w must be [N, K] contiguous")
+        if not (partials.is_cuda and partials.dtype == torch.float32 and partials.is_contiguous()
+                and slices == self.gemm_slices_count(k)):
+            raise KernelError(f"gemm_slices_folded partials must be float32 [{self.gemm_slices_count(k)}, M, N]")
+        if not self.gemm_slices_folded_ok(w.dtype, m, n, k, head_dim, splits):
+            raise KernelError(f"gemm_slices_folded does not take M={m} N={n} K={k} head_dim={head_dim} splits={splits}")
+        rows = m * (k // head_dim) * splits
+        for name, t, width in (("part_acc", part_acc, head_dim), ("part_ml", part_ml, 2)):
+            if not (t.is_cuda and t.dtype == torch.float32 and t.is_contiguous() and t.dim() == 2
+                    and t.shape[1] == width and t.shape[0] >= rows):
+                raise KernelError(f"gemm_slices_folded {name} must be float32 [>= {rows}, {width}]")
+        self._launch(self.core, self.core.ls_gemm_slices_folded, (
+            c_int(DTYPE_CODE[w.dtype]), _ptr(part_acc), _ptr(part_ml), c_int(splits), c_int(head_dim), _ptr(w),
+            _ptr(partials), c_int(m), c_int(n), c_int(k), _stream()))
 
     def add_rmsnorm(self, h: torch.Tensor, partials: torch.Tensor, weight, out, eps: float = 0.0,
                     rows: torch.Tensor | None = None) -> None:
@@ -501,13 +533,15 @@ class Kernels:
 
     def attention(self, q: torch.Tensor, nq: int, nkv: int, d: int, k_pages, v_pages, page_size: int, table,
                   seqs, items, n_items: int, out: torch.Tensor, part_acc, part_ml, scale: float,
-                  window: int, variant: int = 0, max_rows: int = 0, spans: bool = False) -> None:
+                  window: int, variant: int = 0, max_rows: int = 0, spans: bool = False,
+                  single_tile: bool = False) -> None:
         """Launch the attention kernel over ``n_items`` work items (see attention.hip).
         ``variant``: 0 staged through LDS where it fits, 1 direct from global memory, 2 staged or
         error, 3 cooperative (every item has at most 16 rows; ``max_rows`` states the largest),
         4 wide (prompt portions; items count row blocks of ``attention_block_rows``), 5 the same
         with half the rows a block (for steps with few rows).  ``spans`` (cooperative only): items
-        that leave partial results may hold several splits each."""
+        that leave partial results may hold several splits each.  ``single_tile`` (cooperative only): every
+        item holds one key tile (a hint: such a launch needs one tile buffer a workgroup, not two)."""
         lib = self.attention_lib(d)
         _rows_ok(q, "attention q"); _rows_ok(out, "attention out")
         if not (q.dtype in DTYPE_CODE and out.dtype == q.dtype):
@@ -530,12 +564,13 @@ class Kernels:
             c_int(DTYPE_CODE[q.dtype]), _ptr(q), c_long(q.stride(0)), _ptr(k_pages), _ptr(v_pages), c_int(nkv),
             c_int(page_size), _ptr(table), c_int(table.shape[1]), _ptr(seqs), _ptr(items), c_int(n_items),
             _ptr(out), c_long(out.stride(0)), _ptr(part_acc), _ptr(part_ml), c_int(nq // nkv), c_float(scale),
-            c_int(window), c_int(variant), c_int(max_rows), c_int(1 if spans else 0), _stream()))
+            c_int(window), c_int(variant), c_int(max_rows), c_int((1 if spans else 0) | (2 if single_tile else 0)),
+            _stream()))
 
     def attention_decode(self, qkv: torch.Tensor, nq: int, nkv: int, d: int, k_pages, v_pages, page_size: int,
                          table, seqs, items, n_items: int, out: torch.Tensor, part_acc, part_ml, scale: float,
                          window: int, q_weight, k_weight, eps: float, cos, sin, rot: int, max_pos: int,
-                         write_kv: bool, spans: bool = False) -> None:
+                         write_kv: bool, spans: bool = False, single_tile: bool = False) -> None:
         """A step of single decoded tokens: what ``qk_rope_kv`` and ``attention`` (cooperative items) do,
         in one launch.  ``qkv`` is the raw fused projection; every request brings exactly one token."""
         lib = self.attention_lib(d)
@@ -572,7 +607,8 @@ class Kernels:
             c_int(nkv), c_int(page_size), _ptr(table), c_int(table.shape[1]), _ptr(seqs), _ptr(items),
             c_int(n_items), _ptr(out), c_long(out.stride(0)), _ptr(part_acc), _ptr(part_ml), c_float(scale),
             c_int(window), _ptr(q_weight), _ptr(k_weight), c_float(eps), _ptr(cos), _ptr(sin), c_int(rot),
-            c_int(positions), c_int(max_pos), c_int(1 if write_kv else 0), c_int(1 if spans else 0), _stream()))
+            c_int(positions), c_int(max_pos), c_int(1 if write_kv else 0),
+            c_int((1 if spans else 0) | (2 if single_tile else 0)), _stream()))
 
     def attention_combine(self, d: int, seqs, items, n_items: int, nq: int, nkv: int, part_acc, part_ml,
                           out: torch.Tensor, max_rows: int = 0) -> None:

@@ -33,11 +33,18 @@ FUSE_DECODE = os.environ.get("LOCKSTEP_FUSE_DECODE", "1") not in ("", "0")
 # into many items repeats only the query's part of the prologue in each, and one launch less still pays
 # (eight requests of 16,384 tokens: 4.23 -> 4.13 ms a step).
 FUSE_DECODE_BELOW = int(os.environ.get("LOCKSTEP_FUSE_DECODE_BELOW", "512"))
-# The most splits (of 256 keys) one cooperative workgroup walks when a request is cut over several.
-MAX_SPAN = 4               # splits of a work item where requests of a ragged batch are cut
+# The most splits one cooperative workgroup walks when a request is cut over several.
+MAX_SPAN = 8               # splits of a work item where requests of a ragged batch are cut
 WORKGROUPS_A_CU = 2         # work items (times kv heads) a CU that a decode step is cut for
 RAGGED_RATIO = 2.0         # a batch is ragged when its longest request has more than this many times the mean splits
 PART_ROWS_STEP = 4096      # rows of partial results are taken in steps of this many (sizes of replayed steps)
+# A step of few decoded tokens whose requests have few splits each leaves the fold of the splits to the output
+# product (``gemm_slices_folded``: one launch and one round trip less a layer); every request is then laid out
+# with the same number of splits.  Each column block of the product repeats the fold, so this is for few rows
+# times splits only.  "0" switches it off.
+FOLD_IN_PRODUCT = os.environ.get("LOCKSTEP_FOLD_IN_PRODUCT", "1") not in ("", "0")
+FOLD_MAX_SPLITS = int(os.environ.get("LOCKSTEP_FOLD_MAX_SPLITS", "8"))
+FOLD_MAX_ROW_SPLITS = int(os.environ.get("LOCKSTEP_FOLD_MAX_ROW_SPLITS", "128"))   # requests times splits
 
 
 # ---------------------------------------------------------------------------
@@ -60,6 +67,10 @@ class AttentionPlan:
     decode_fused: bool        # every request brings one token and the fused decode kernel can take the step
     wide_variant: int = 4     # 4: row blocks of 128 rows, 5: of 64
     spans: bool = False       # cooperative items that leave partial results hold several splits each
+    #: > 0: single decoded tokens only, every request laid out with this many splits, partial row of
+    #: (request i, head h, split s) = (i * heads + h) * fold_splits + s: the output product may fold them itself
+    fold_splits: int = 0
+    single_tile: bool = False  # every cooperative item holds one key tile (one tile buffer a workgroup is enough)
 
     ITEM, COMBINE = 16, 8
 
@@ -72,7 +83,7 @@ class AttentionPlan:
 
     def signature(self):
         return (self.n_items, self.n_combine, self.n_coop, self.n_wide, self.part_rows, self.decode_fused,
-                self.wide_variant, self.spans)
+                self.wide_variant, self.spans, self.fold_splits, self.single_tile)
 
 
 def _round_up(n: int, buckets=(1, 2, 4, 8, 12, 16, 24, 32, 40, 48, 56, 64), step: int = 16) -> int:
@@ -137,9 +148,26 @@ def plan_attention(ctx, group_size: int, nkv: int, head_dim: int, window: int):
             if int(mine.max()) > RAGGED_RATIO * float(mine.mean()):
                 span = min(span, MAX_SPAN)
 
+    fold_splits = 0
+    if (FOLD_IN_PRODUCT and span == 1 and window == 0 and ctx.n_seqs <= 16 and bool(to_coop.all())
+            and bool((ctx.q_len == 1).all())):
+        most = int(counts.max())
+        # (with one split everywhere nothing is folded anyway: the workgroups write the output themselves)
+        if 2 <= most <= FOLD_MAX_SPLITS and most * ctx.n_seqs <= FOLD_MAX_ROW_SPLITS:
+            fold_splits = most
+
     items, coop, wide, combine = [], [], [], []
     coop_max_rows = part_rows = 0
     for i in range(ctx.n_seqs):
+        if fold_splits:
+            # the same number of splits for every request (those beyond a request's end leave empty sums), the
+            # partial rows of a request one after the other in the order of its heads
+            base = i * nkv * group_size * fold_splits
+            coop_max_rows = max(coop_max_rows, group_size)
+            coop += [(i, 0, int(lo[i]) + s, int(lo[i]) + s + 1, base, fold_splits, int(lo[i]), 0) for s in range(fold_splits)]
+            combine.append((i, 0, base, fold_splits))
+            part_rows = base + nkv * group_size * fold_splits
+            continue
         q_len, q_start = int(ctx.q_len[i]), int(ctx.q_start[i])
         rows = int(rows_of[i])
         split_lo, n_splits = int(lo[i]), int(counts[i])
@@ -181,8 +209,9 @@ def plan_attention(ctx, group_size: int, nkv: int, head_dim: int, window: int):
     # the longest row blocks first: they decide when the launch ends
     wide.sort(key=lambda it: it[2] - it[3])
     spans = any(it[4] >= 0 and it[3] - it[2] > 1 for it in coop)
+    single_tile = bool(coop) and all((it[3] - it[2]) * split <= tile for it in coop)
     plan = AttentionPlan(len(items), len(combine), len(coop), coop_max_rows, len(wide), part_rows, decode_fused,
-                         wide_variant, spans)
+                         wide_variant, spans, fold_splits, single_tile)
     return plan, np.concatenate([pack_attention_items(items, ctx.seq_rows), pack_combine_items(combine, ctx.seq_rows),
                                  pack_attention_items(coop, ctx.seq_rows), pack_attention_items(wide, ctx.seq_rows)])
 
@@ -370,11 +399,13 @@ class Attention(Mixer):
             k.attention_decode(qkv, nq, nkv, d, key_pages, value_pages, group.page_size, group.table, ctx.seqs,
                                coop_items, plan.n_coop, attn, part_acc, part_ml, self.scale, window,
                                self.q_norm, self.k_norm, self.norm_eps, self.position.cos, self.position.sin,
-                               self.position.rotary_dim, ctx.max_position, run.writes_cache, plan.spans)
-            if plan.n_combine:
+                               self.position.rotary_dim, ctx.max_position, run.writes_cache, plan.spans,
+                               plan.single_tile)
+            folded = self._folded_operand(ctx, plan, part_acc, part_ml, out, accumulate, defer)
+            if plan.n_combine and folded is None:
                 k.attention_combine(d, ctx.seqs, combine_items, plan.n_combine, nq, nkv, part_acc, part_ml, attn,
                                     max_rows=plan.coop_max_rows if not plan.n_items else 0)
-            return self._project_out(ctx, attn, out, accumulate, defer)
+            return self._project_out(ctx, attn, out, accumulate, defer, folded)
         k.qk_rope_kv(qkv, t, nq, nkv, d, self.q_norm, self.k_norm, self.norm_eps, self.position.cos,
                      self.position.sin, self.position.rotary_dim, ctx.tok_seq, ctx.tok_pos, ctx.seqs,
                      ctx.max_position, group.table, key_pages, value_pages, group.page_size, run.writes_cache)
@@ -384,18 +415,38 @@ class Attention(Mixer):
         if plan.n_coop:
             k.attention(qkv, nq, nkv, d, key_pages, value_pages, group.page_size, group.table, ctx.seqs,
                         coop_items, plan.n_coop, attn, part_acc, part_ml, self.scale, window,
-                        variant=3, max_rows=plan.coop_max_rows, spans=plan.spans)
+                        variant=3, max_rows=plan.coop_max_rows, spans=plan.spans, single_tile=plan.single_tile)
         if plan.n_wide:
             k.attention(qkv, nq, nkv, d, key_pages, value_pages, group.page_size, group.table, ctx.seqs,
                         wide_items, plan.n_wide, attn, part_acc, part_ml, self.scale, window,
                         variant=plan.wide_variant)
-        if plan.n_combine:
+        folded = self._folded_operand(ctx, plan, part_acc, part_ml, out, accumulate, defer)
+        if plan.n_combine and folded is None:
             k.attention_combine(d, ctx.seqs, combine_items, plan.n_combine, nq, nkv, part_acc, part_ml, attn,
                                     max_rows=plan.coop_max_rows if not plan.n_items else 0)
-        return self._project_out(ctx, attn, out, accumulate, defer)
+        return self._project_out(ctx, attn, out, accumulate, defer, folded)
 
-    def _project_out(self, ctx, attn, out, accumulate: bool, defer: bool):
+    def _folded_operand(self, ctx, plan, part_acc, part_ml, out, accumulate: bool, defer: bool):
+        """(part_acc, part_ml, splits) if the output product of this step can fold the splits' partial
+        results itself (the plan laid them out for it, the product is left as slice sums, and the kernel
+        takes these sizes), else None: the combine launch folds them into the attention output."""
+        if not plan.fold_splits or not (defer and accumulate) or self.b_o is not None:
+            return None
+        if not 0 < ctx.n_tokens <= deferred_rows(ctx, self.nq * self.d, out.shape[1]):
+            return None
+        if not ctx.rt.kernels.gemm_slices_folded_ok(ctx.rt.dtype, ctx.n_tokens, out.shape[1], self.nq * self.d, self.d,
+                                                    plan.fold_splits):
+            return None
+        return part_acc, part_ml, plan.fold_splits
+
+    def _project_out(self, ctx, attn, out, accumulate: bool, defer: bool, folded=None):
         k = ctx.rt.kernels
+        if folded is not None:
+            slices = k.gemm_slices_count(self.nq * self.d)
+            partials = ctx.buf("attention.out_slices", (slices * ctx.n_tokens, out.shape[1]), torch.float32)
+            partials = partials.view(slices, ctx.n_tokens, out.shape[1])
+            k.gemm_slices_folded(folded[0], folded[1], folded[2], self.d, self.w_o, partials)
+            return PendingAdd(partials)
         if self.b_o is not None:
             # (stream + product) + bias, at once: the order of the additions must not depend on the batch
             k.gemm(attn, self.w_o, out, ADD_F32 if accumulate else STORE_F32)

@@ -127,10 +127,11 @@ def test_a_sampler_whose_cut_depends_on_the_rows_of_a_call_is_caught(control_ker
 
 def test_a_reversed_fold_over_the_splits_is_caught_where_there_are_three_splits(tiny_dirs, control_kernels):
     """A whole prompt (its workgroups walk the splits themselves) against the same tokens with the
-    tail decoded one by one (one split a workgroup, folded by the combine kernel): equal bits.  With
-    the combine kernel folding backwards they differ, and only at positions that have three splits
-    (two partial results give the same sum in either order).  On the 32-bit path: the bfloat16
-    path rounds the attention output to eight bits, which hides a reordered 32-bit sum almost always."""
+    tail in steps of one and of two tokens (one split a workgroup; the sums of a single token are
+    folded by the output product, those of two tokens by the combine kernel): equal bits.  With the
+    folds running backwards they differ, and only at positions that have three splits of 128 keys and more
+    (two partial results give the same sum in either order).  On the 32-bit path: the bfloat16 path rounds the
+    attention output to eight bits, which hides a reordered 32-bit sum almost always."""
     from lockstep_amd.engine.model import load_model
 
     model = load_model(tiny_dirs[("B", "sharp")], dtype="float32")
@@ -141,19 +142,26 @@ def test_a_reversed_fold_over_the_splits_is_caught_where_there_are_three_splits(
     def both_ways():
         cache = model.make_cache(num_pages=160, page_size=8, max_requests=2)
         whole = feed(model, cache, "w", tokens, [])
-        tail = feed(model, cache, "t", tokens, [head] + [1] * (len(tokens) - head))
+        tail = feed(model, cache, "t", tokens, [head] + [1, 2] * ((len(tokens) - head) // 3 + 1))
         return whole, tail
 
     def same_bits():
         whole, tail = both_ways()
         return torch.equal(whole, tail)
 
-    holds_breaks_holds(same_bits, lambda: mutant(control_kernels, attention=control_kernels.MUTANT_REVERSED_FOLD))
-    with mutant(control_kernels, attention=control_kernels.MUTANT_REVERSED_FOLD):
+    # (decoded tokens with few splits are folded by the output product, longer ones by the combine launch:
+    # both folds are reversed)
+    reversed_folds = dict(core=control_kernels.MUTANT_REVERSED_FOLD_IN_PRODUCT,
+                          attention=control_kernels.MUTANT_REVERSED_FOLD)
+    holds_breaks_holds(same_bits, lambda: mutant(control_kernels, **reversed_folds))
+    for one in ({"core": reversed_folds["core"]}, {"attention": reversed_folds["attention"]}):
+        with mutant(control_kernels, **one):          # each of the two alone is noticed too: both folds are in use
+            assert not same_bits(), one
+    with mutant(control_kernels, **reversed_folds):
         whole, tail = both_ways()
         differs = (whole != tail).any(dim=1)
-        assert not differs[:512].any(), "a position with one or two splits changed: the control fails for the wrong reason"
-        assert differs[512:].any() and float((whole - tail).abs().max()) < 1e-3 * float(whole.abs().max())
+        assert not differs[:256].any(), "a position with one or two splits changed: the control fails for the wrong reason"
+        assert differs[256:].any() and float((whole - tail).abs().max()) < 1e-3 * float(whole.abs().max())
 
 
 def test_batch_dependent_k_blocking_is_caught_by_the_decode_test(tmp_path_factory, control_kernels):

@@ -816,6 +816,8 @@ def test_the_fold_for_few_rows_is_right_when_it_is_handed_more_rows_than_it_was_
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("nq,nkv,d,ps,rot,normed,window", [
     (16, 8, 128, 16, 128, True, 0), (64, 8, 128, 16, 128, True, 0), (8, 1, 64, 32, 64, True, 0), (4, 4, 16, 8, 16, True, 0),
+    # sixteen query heads a kv head: with the new key and value more heads than a workgroup has groups of sixteen lanes
+    (16, 1, 64, 16, 64, True, 0), (30, 2, 32, 8, 16, True, 0),
     (6, 2, 48, 16, 32, False, 0), (4, 2, 32, 8, 0, True, 0), (4, 2, 64, 16, 64, True, 200)])
 def test_fused_decode_attention_equals_the_separate_kernels(dtype, nq, nkv, d, ps, rot, normed, window):
     """A decoded token through qk_rope_kv + cooperative attention, and through the one fused launch:
@@ -987,3 +989,51 @@ def test_slice_sums_and_fused_add_norm_equal_the_separate_kernels(dtype, m, n, k
     K().add_rmsnorm(h, partials, weight, y, eps, rows)
     assert torch.equal(y, y_ref[rows.long()])
     assert torch.equal(h[rows.long()], h_ref[rows.long()])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("m,nq,nkv,d,n,splits", [(1, 16, 8, 128, 1024, 3), (8, 16, 8, 128, 1024, 4), (16, 4, 2, 64, 520, 2),
+                                                 (5, 32, 8, 128, 4096, 8), (3, 6, 3, 32, 96, 5), (2, 64, 8, 128, 5120, 2),
+                                                 (7, 2, 1, 256, 300, 3)])
+def test_the_product_that_folds_the_splits_itself_equals_fold_then_product(dtype, m, nq, nkv, d, n, splits):
+    """The per-split sums of m decoded tokens (some splits empty, with NaN where nothing may be read; one
+    token with nothing but empty splits) through the combine launch and ``gemm_slices``, and through
+    ``gemm_slices_folded`` alone: the same slice sums, bit for bit."""
+    from lockstep_amd.ops import pack_combine_items
+
+    k = nq * d
+    if not K().gemm_slices_folded_ok(dtype, m, n, k, d, splits):
+        assert dtype is torch.float32 or n * k * 2 >= 64 << 20, "refused although the plain slice kernel would run"
+        pytest.skip("the folded product does not take these sizes")
+    g = torch.Generator().manual_seed(m * 100 + nq + d + splits)
+    rows = m * nq * splits
+    acc = torch.randn(rows, d, generator=g) * 3
+    ml = torch.stack([torch.randn(rows, generator=g) * 4, torch.rand(rows, generator=g) * 50 + 0.01], dim=1)
+    empty = torch.rand(rows, generator=g) < 0.25
+    empty.view(m, nq, splits)[m - 1] = True                     # the last token saw no key at all
+    ml[empty, 0], ml[empty, 1] = -1e30, 0.0
+    acc[empty] = float("nan")
+    acc, ml = acc.cuda(), ml.cuda()
+    w = (torch.randn(n, k, generator=g) * 0.1).to(dtype).cuda()
+    seqs = torch.tensor([[i, 1, 700 + i, 701 + i, i, 0, 0, 0] for i in range(m)], dtype=torch.int32)
+    items = torch.from_numpy(pack_combine_items([(i, 0, i * nq * splits, splits) for i in range(m)], seqs.numpy())).to(torch.int32)
+    attn = torch.full((m, k), float("nan"), dtype=dtype, device="cuda")
+    K().attention_combine(d, seqs.cuda(), items.cuda(), m, nq, nkv, acc, ml, attn, max_rows=nq // nkv)
+    assert not torch.isnan(attn).any() and (attn[m - 1] == 0).all()
+    slices = K().gemm_slices_count(k)
+    want = torch.full((slices, m, n), float("nan"), device="cuda")
+    K().gemm_slices(attn, w, want)
+    got = torch.full((slices, m, n), float("nan"), device="cuda")
+    K().gemm_slices_folded(acc, ml, splits, d, w, got)
+    assert not torch.isnan(got).any()
+    assert torch.equal(got, want)
+    # and right: against the fold in float64
+    a, b = acc.cpu().double().view(m, nq, splits, d), ml.cpu().double().view(m, nq, splits, 2)
+    a[b[..., 1] <= 0] = 0
+    top = b[..., 0].max(dim=2, keepdim=True).values
+    scale = torch.where(b[..., 1] > 0, (b[..., 0] - top).exp(), torch.zeros_like(top))
+    total = (b[..., 1] * scale).sum(2)
+    x = (a * scale[..., None]).sum(2) / total.clamp_min(1e-300)[..., None]
+    x[total <= 0] = 0
+    product = x.reshape(m, k) @ w.cpu().double().T
+    assert rel_err(got.sum(0), product) < (1e-4 if dtype is torch.float32 else 2e-2)
