@@ -62,6 +62,9 @@ constexpr int kRing = LS_ATTN_RING;  // LDS operand reads kept in flight ahead o
 constexpr int kPageWindow = 32;      // tiles whose page ids a workgroup of the streaming kernels holds in LDS at a time
 #ifdef LS_ATTN_PROBE
 #define PROBE(i) { long long now_ = clock64(); pr_t[i] += now_ - pr_last; pr_last = now_; }
+#ifndef LS_ATTN_PROBE_KVH
+#define LS_ATTN_PROBE_KVH 0  // the workgroups of this kv head report
+#endif
 #else
 #define PROBE(i)
 #endif
@@ -73,16 +76,18 @@ struct SeqMeta {
 };
 // An item of all zeros stands for no work (lists of graph-replayed steps are rounded up with them): a request
 // of no rows has no row to load for and none to write, and the kernels need no test of their own for it.
-struct AttnItem {  // one workgroup column of the attention launch (16 ints)
+struct AttnItem {  // one workgroup column of the attention launch (32 ints)
   int seq;         // index into SeqMeta
   int row_block;   // row block of the sequence's rows
   int split_begin, split_end;
   int part_base;   // first partial row of the sequence, or -1: direct
   int n_splits;    // splits of the sequence that have a partial
   int split_lo;    // first of them (splits below lie behind the window)
-  int reserved;
+  int pages_here;  // 1: `pages` holds the page ids of the item's one tile (cooperative items of one tile)
   SeqMeta sm;      // a copy of seqs[seq], so that the kernel needs one load to know its work
+  int pages[16];   // the block table's entries for the tile split_begin, so that the tile's loads need no second one
 };
+static_assert(sizeof(AttnItem) == 128, "the host packs 32 ints an item");
 
 // A masked score is minus infinity, so its probability exp(-inf - m) is an
 // exact zero without a select; running maxima start at the finite -1e30, so
@@ -99,6 +104,24 @@ constexpr float kMasked = -__builtin_huge_valf();
 __device__ __forceinline__ void load_to_lds16(const void* src, __attribute__((address_space(3))) void* lds_wave_base) {
   const unsigned base = __builtin_amdgcn_readfirstlane((unsigned)(unsigned long)lds_wave_base);
   __asm__ volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(base) : "memory", "m0");
+}
+
+// Sixteen bytes into registers by an instruction the compiler does not know to be a load: it places no wait for
+// it, so the kernel can keep it in flight across other loads and wait with a count of its own (wait_for_loads,
+// which also ties the registers, so that no use moves above the wait).
+__device__ __forceinline__ f32x4 load16_unwaited(const void* src) {
+  f32x4 r;
+  __asm__ volatile("global_load_dwordx4 %0, %1, off" : "=&v"(r) : "v"(src) : "memory");
+  return r;
+}
+template <int YOUNGER>  // loads issued after those that are waited for (loads complete in the order of their issue)
+__device__ __forceinline__ void wait_for_loads(f32x4& a, f32x4& b, f32x4& c, f32x4& d, f32x4& e, f32x4& f, f32x4& g,
+                                               f32x4& h) {
+  static_assert(YOUNGER >= 0 && YOUNGER <= 63, "the count of a wait has six bits");
+  __asm__ volatile("s_waitcnt vmcnt(%8)"
+                   : "+v"(a), "+v"(b), "+v"(c), "+v"(d), "+v"(e), "+v"(f), "+v"(g), "+v"(h)
+                   : "n"(YOUNGER)
+                   : "memory");
 }
 
 // A workgroup barrier that makes the waves' own LDS writes visible and nothing else.  __syncthreads() also
@@ -1074,10 +1097,18 @@ struct DecodeFuse {
 
 template <typename T, int NBUF, bool FUSE, bool SPANS>
 __global__ __launch_bounds__(256) void attention_coop_kernel(
-    const T* __restrict__ q, long ldq, const T* __restrict__ k_pages, const T* __restrict__ v_pages, int nkv,
-    int page_size, int page_shift, const int* __restrict__ table, int table_stride,
-    const SeqMeta* __restrict__ seqs, const AttnItem* __restrict__ items, T* __restrict__ out, long ldo,
-    float* __restrict__ part_acc, float* __restrict__ part_ml, int G, float scale, int window, DecodeFuse<T> fz) {
+    // (the first sixteen words of the arguments are in registers when a wave starts: the ones that the first
+    // loads of the kernel need come first; `fz` is `fz_rest` with its four tables taken from here)
+    const AttnItem* __restrict__ items, const T* __restrict__ q, long ldq, const float* __restrict__ head_q_weight,
+    const float* __restrict__ head_k_weight, const float* __restrict__ cos_table, const float* __restrict__ sin_table,
+    int G, int nkv, const T* __restrict__ k_pages, const T* __restrict__ v_pages, int page_size, int page_shift,
+    const int* __restrict__ table, int table_stride, const SeqMeta* __restrict__ seqs, T* __restrict__ out, long ldo,
+    float* __restrict__ part_acc, float* __restrict__ part_ml, float scale, int window, DecodeFuse<T> fz_rest) {
+  DecodeFuse<T> fz = fz_rest;
+  fz.q_weight = head_q_weight;
+  fz.k_weight = head_k_weight;
+  fz.cos_table = cos_table;
+  fz.sin_table = sin_table;
   typedef Atom<T> A;
   typedef typename A::vec_t vec_t;
   constexpr int SZ = sizeof(T);
@@ -1104,14 +1135,31 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
   T* vnew = knew + D;
 
 #ifdef LS_ATTN_PROBE
-  long long pr_t[16];
-  for (int i = 0; i < 16; ++i) pr_t[i] = 0;
+  long long pr_t[24];
+  for (int i = 0; i < 24; ++i) pr_t[i] = 0;
   long long pr_last = clock64();
   const long long pr_begin = pr_last;
 #endif
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
-  const AttnItem item = items[blockIdx.x];
+  // The item is the same for every lane: its fields go to scalar registers, so that what follows from them
+  // (tile range, addresses, branch conditions) is scalar work too.
+  AttnItem item;
+  {
+    const int* src = reinterpret_cast<const int*>(items + blockIdx.x);
+    int* dst = reinterpret_cast<int*>(&item);
+#pragma unroll
+    for (int i = 0; i < 16; ++i) dst[i] = __builtin_amdgcn_readfirstlane(src[i]);
+  }
+  // the page ids an item of one tile brings, one a thread, requested together with the item itself
+  const int own_page = FUSE ? items[blockIdx.x].pages[threadIdx.x & 15] : 0;
+  if (FUSE) {
+    // every other argument is requested now, while the item is on its way: left to themselves their loads
+    // stand where each is first used, each with a wait of its own for memory that no cache holds yet
+    __asm__ volatile("" ::"s"(k_pages), "s"(v_pages), "s"(page_size), "s"(page_shift), "s"(part_acc), "s"(part_ml),
+                     "s"(scale), "s"(window), "s"(fz.eps), "s"(fz.rot), "s"(fz.nq), "s"(fz.write_kv), "s"(fz.k_out),
+                     "s"(fz.v_out), "s"(out), "s"(ldo), "s"(table), "s"(table_stride));
+  }
   const SeqMeta sm = item.sm;
   const int kvh = blockIdx.y;
   const int rows_total = sm.q_len * G;  // <= 16, checked on the host
@@ -1159,6 +1207,7 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
   auto pages_of = [&](int ti) -> const int* { return tile_pages + ((ti - ti_lo) % kPageWindow) * 16; };
   auto window_start = [&](int ti) -> bool { return (ti - ti_lo) % kPageWindow == 0; };  // tile ti opens a window of ids
   const long page_stride = (long)nkv * page_size * D;  // elements of one page, K or V
+  PROBE(16)
   int k_off[PER], v_off[PER];
 #pragma unroll
   for (int i = 0; i < PER; ++i) {
@@ -1171,6 +1220,11 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
     const int d = p % D;
     v_off[i] = ((kvh * D + d) << page_shift) + ((c * VEC) & (page_size - 1));
   }
+#ifdef LS_ATTN_PROBE
+#pragma unroll
+  for (int i = 0; i < PER; ++i) __asm__ volatile("" ::"v"(k_off[i]), "v"(v_off[i]));
+#endif
+  PROBE(17)
   auto issue = [&](int ti) {
     const int* pages = pages_of(ti);
     unsigned char* k_buf = lds + (NBUF == 2 ? (ti & 1) : 0) * BUF_BYTES;
@@ -1302,28 +1356,21 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
       }
     }
   };
-  if (FUSE) {
-    if (owner) page_new = tbl[p_new >> page_shift];
-    if (grp < n_vec) head_fetch(grp);
-  }
-  if (ti_lo < ti_hi) fill_pages(ti_lo);
-  __syncthreads();
-  if (FUSE) {
-    // The head's operands are awaited here, before the tile loads go out: a wait placed after them would also
-    // wait for the tiles (loads complete in the order of their issue, and the compiler does not count the tile
-    // loads), and the norm, the rotation and the cache write below would start only when the tiles are in.
-#pragma unroll
-    for (int i = 0; i < 8 * PASSES; ++i) __asm__ volatile("" ::"v"(hx[i]), "v"(hf.w[i]), "v"(hf.c[i]), "v"(hf.s[i]));
-    __asm__ volatile("" ::"v"((int)page_new));
-    if (n_vec > 16) {  // more heads than groups of sixteen lanes (fifteen query heads a kv head and more): all of
-      finish_head(grp);  // them now, so that no load of a head stands behind the tile loads
-      if (grp + 16 < n_vec) {
-        head_fetch(grp + 16);
-        finish_head(grp + 16);
-      }
-    }
-  }
-  PROBE(1)
+  // An item of one tile may bring the tile's page ids itself (embedded): the tile loads then wait for no second
+  // round trip.  The head's operands are then requested by loads the compiler does not count (unwaited), ahead
+  // of the tile loads, and awaited with a count that leaves the tile loads in flight, so that norm, rotation and
+  // cache write run while the tile is on its way.
+  PROBE(18)
+  const bool embedded = FUSE && item.pages_here != 0;
+  // (the ids go to their place in LDS before any unwaited load is issued: the compiler's wait for `own_page`
+  // would wait for those as well)
+  if (embedded && threadIdx.x < 16) tile_pages[threadIdx.x] = own_page;
+  PROBE(19)
+  const bool aligned_turn = !rotated || (((fz.rot / 2) & 7) == 0);
+  const bool unwaited = embedded && PASSES == 1 && aligned_turn && n_vec <= 16 && 2 * PER <= 63;
+  const int e0_head = 8 * gl;                    // the lane's eight elements of a head (PASSES == 1)
+  const bool lane_in_head = e0_head < D;
+  const bool lane_turns = rotated && e0_head < fz.rot;
   auto issue_tile = [&](int ti) {
     if (NBUF == 2) {
       issue(ti);
@@ -1332,16 +1379,103 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
       issue_v(ti);
     }
   };
-  if (ti_lo < ti_hi) issue_tile(ti_lo);
-  // two buffers: both are free now, so the second tile is requested at once as well and its wait overlaps the
-  // first one's (a workgroup of a decode step mostly has two tiles, and a miss takes longer than a tile's work)
   constexpr bool CAN_PRIME = NBUF == 2 && 2 * PER <= 63;  // (the wait names the loads of one tile: a 6-bit count)
-  const bool primed = CAN_PRIME && ti_lo + 1 < ti_hi && !window_start(ti_lo + 1);
-  if (primed) issue(ti_lo + 1);
+  bool primed = false;
+  if (FUSE && unwaited) {
+    if constexpr (PASSES == 1 && 2 * PER <= 63) {  // (what `unwaited` asks for, said to the compiler)
+      // Straight-line code from the loads to their wait, every load unconditional: a register that such a load
+      // writes must not be copied or merged with another value before the wait (the compiler takes it to be
+      // written when the instruction is issued).  Lanes and groups that need no operand load a spare address
+      // and drop the result.
+      const int vi = min(grp, n_vec - 1);
+      const float* spare = reinterpret_cast<const float*>(items + blockIdx.x);  // 128 readable bytes
+      const T* src = head_src(vi) + (lane_in_head ? e0_head : 0);
+      const float* weight = vi < G ? fz.q_weight : vi == G ? fz.k_weight : nullptr;
+      const bool weighted = weight != nullptr && lane_in_head && grp < n_vec;
+      const float* w_at = weighted ? weight + e0_head : spare;
+      const int half = fz.rot / 2;
+      const bool turns = lane_turns && vi <= G;
+      const float* c_at = turns ? fz.cos_table + (long)p_new * half + (e0_head < half ? e0_head : e0_head - half) : spare;
+      const float* s_at = turns ? fz.sin_table + (long)p_new * half + (e0_head < half ? e0_head : e0_head - half) : spare;
+      PROBE(12)
+      f32x4 raw_x0 = load16_unwaited(src);
+      f32x4 raw_x1 = load16_unwaited(sizeof(T) == 4 ? reinterpret_cast<const float*>(src) + 4 : spare);
+      f32x4 raw_w0 = load16_unwaited(w_at);
+      f32x4 raw_w1 = load16_unwaited(w_at + 4);
+      f32x4 raw_c0 = load16_unwaited(c_at);
+      f32x4 raw_c1 = load16_unwaited(c_at + 4);
+      f32x4 raw_s0 = load16_unwaited(s_at);
+      f32x4 raw_s1 = load16_unwaited(s_at + 4);
+      PROBE(13)
+      __syncthreads();  // the page ids are in LDS
+      if (owner) page_new = tile_pages[(p_new & (kTileKeys - 1)) >> page_shift];
+      PROBE(1)
+      // the head's operands: everything but the tile's 2 * PER loads (if the item has a tile at all) has arrived
+      // (one wait statement for both cases, so that the registers reach it by one way only and are not moved on
+      // the way; without a tile everything is awaited first, and the counted wait finds nothing left)
+      if (ti_lo < ti_hi)
+        issue_tile(ti_lo);
+      else
+        __asm__ volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      wait_for_loads<2 * PER>(raw_x0, raw_x1, raw_w0, raw_w1, raw_c0, raw_c1, raw_s0, raw_s1);
+      PROBE(2)
+      if (sizeof(T) == 2) {
+        const bf16x8 v = __builtin_bit_cast(bf16x8, raw_x0);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) hx[j] = lane_in_head ? to_f32(v[j]) : 0.f;
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          hx[j] = lane_in_head ? raw_x0[j] : 0.f;
+          hx[4 + j] = lane_in_head ? raw_x1[j] : 0.f;
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        hf.w[j] = weighted ? raw_w0[j] : 1.f;
+        hf.w[4 + j] = weighted ? raw_w1[j] : 1.f;
+        hf.c[j] = turns ? raw_c0[j] : 1.f;
+        hf.c[4 + j] = turns ? raw_c1[j] : 1.f;
+        hf.s[j] = turns ? raw_s0[j] : 0.f;
+        hf.s[4 + j] = turns ? raw_s1[j] : 0.f;
+      }
+    }
+  } else {
+    if (FUSE) {
+      if (owner && !embedded) page_new = tbl[p_new >> page_shift];
+      if (grp < n_vec) head_fetch(grp);
+    }
+    if (!embedded && ti_lo < ti_hi) fill_pages(ti_lo);
+    __syncthreads();
+    if (embedded && owner) page_new = tile_pages[(p_new & (kTileKeys - 1)) >> page_shift];
+    if (FUSE) {
+      // The head's operands are awaited here, before the tile loads go out: a wait placed after them would also
+      // wait for the tiles (loads complete in the order of their issue, and the compiler does not count the tile
+      // loads), and the norm, the rotation and the cache write below would start only when the tiles are in.
+#pragma unroll
+      for (int i = 0; i < 8 * PASSES; ++i) __asm__ volatile("" ::"v"(hx[i]), "v"(hf.w[i]), "v"(hf.c[i]), "v"(hf.s[i]));
+      __asm__ volatile("" ::"v"((int)page_new));
+      if (n_vec > 16) {  // more heads than groups of sixteen lanes (fifteen query heads a kv head and more): all of
+        finish_head(grp);  // them now, so that no load of a head stands behind the tile loads
+        if (grp + 16 < n_vec) {
+          head_fetch(grp + 16);
+          finish_head(grp + 16);
+        }
+      }
+    }
+    PROBE(1)
+    if (ti_lo < ti_hi) issue_tile(ti_lo);
+    // two buffers: both are free now, so the second tile is requested at once as well and its wait overlaps the
+    // first one's (a workgroup of a decode step mostly has two tiles, and a miss takes longer than a tile's work)
+    primed = CAN_PRIME && !embedded && ti_lo + 1 < ti_hi && !window_start(ti_lo + 1);
+    if (primed) issue(ti_lo + 1);
+  }
   PROBE(2)
   if (FUSE) {
     if (n_vec <= 16 && grp < n_vec) finish_head(grp);  // (more heads than groups: done above, before the tile loads)
+    PROBE(14)
     lds_barrier();
+    PROBE(15)
 #pragma unroll
     for (int c = 0; c < NC; ++c) {
       const int col = c * A::KCHUNK + g * VEC;
@@ -1580,11 +1714,12 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
   }
 
 #ifdef LS_ATTN_PROBE
-  if (threadIdx.x == 0 && kvh == 0 && part_ml != nullptr) {
-    long long* dst = reinterpret_cast<long long*>(part_ml + (1 << 20)) + blockIdx.x * 16;
+  if (threadIdx.x == 0 && kvh == LS_ATTN_PROBE_KVH && part_ml != nullptr) {
+    long long* dst = reinterpret_cast<long long*>(part_ml + (1 << 20)) + blockIdx.x * 32;
     for (int i = 0; i < 12; ++i) dst[i] = pr_t[i];
     dst[12] = clock64() - pr_begin;
     dst[13] = ti_hi - ti_lo;
+    for (int i = 12; i < 24; ++i) dst[i + 4] = pr_t[i];
   }
 #endif
   if (!row_ok) return;
@@ -1933,9 +2068,9 @@ static int launch_coop_as(dim3 grid, hipStream_t s, const void* q, long ldq, con
   const bool crowded = (long)grid.x * grid.y >= LS_COOP_CROWDED_FROM || single_tile;
 #define LS_COOP(NBUF_)                                                                                              \
   hipLaunchKernelGGL((attention_coop_kernel<T, NBUF_, FUSE, SPANS>), grid, dim3(256), (coop_kernel_lds<T, NBUF_>()), s, \
-                     (const T*)q, ldq, (const T*)k_pages, (const T*)v_pages, nkv, page_size, page_shift, table,        \
-                     table_stride, (const SeqMeta*)seqs, (const AttnItem*)items, (T*)out, ldo, part_acc, part_ml, G,   \
-                     scale, window, fz)
+                     (const AttnItem*)items, (const T*)q, ldq, fz.q_weight, fz.k_weight, fz.cos_table, fz.sin_table, G, \
+                     nkv, (const T*)k_pages, (const T*)v_pages, page_size, page_shift, table, table_stride,            \
+                     (const SeqMeta*)seqs, (T*)out, ldo, part_acc, part_ml, scale, window, fz)
   if (BUFS == 2 && !(crowded && coop_kernel_ready<T, 1, FUSE, SPANS>())) {
     if (!coop_kernel_ready<T, 2, FUSE, SPANS>()) return fail("attention: the cooperative kernel does not fit into LDS");
     LS_COOP(2);

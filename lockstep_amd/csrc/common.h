@@ -238,6 +238,14 @@ __device__ __forceinline__ void head16_load_values(float (&x)[8 * PASSES], const
   }
 }
 
+// The value `v` of the lane K places on in the caller's row of sixteen lanes, the row taken as a ring (a
+// data-parallel move inside the row: no trip through LDS as a fetch from an arbitrary lane takes).
+template <int K>
+__device__ __forceinline__ float row16_rotated(float v) {
+  static_assert(K >= 1 && K <= 15, "a rotation inside a row of sixteen");
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x120 + K, 0xf, 0xf, false));
+}
+
 // Value of `v` in lane `from` (0..15) of the caller's group.
 __device__ __forceinline__ float group16_get(float v, int from) {
   return __shfl(v, (threadIdx.x & 48) | from, kWave);
@@ -252,8 +260,13 @@ __device__ __forceinline__ void head16_finish(const float (&x)[8 * PASSES], cons
 #pragma unroll
   for (int i = 0; i < 8 * PASSES; ++i) part = part + x[i] * x[i];  // elements past d are zeros
   if (normed) {
-#pragma unroll
-    for (int k = 8; k > 0; k >>= 1) part = part + group16_get(part, (gl + k) & 15);
+    // part_i + part_(i+8), then + the sum four lanes on, two, one: after each step the sums repeat with the
+    // step's period, so the lane k on and the lane k back hold the same value and a rotation of the row of
+    // sixteen lanes in either direction gives the same bits as a fetch from lane (gl + k) & 15
+    part = part + row16_rotated<8>(part);
+    part = part + row16_rotated<4>(part);
+    part = part + row16_rotated<2>(part);
+    part = part + row16_rotated<1>(part);
     const float scale = 1.0f / sqrtf(part / (float)d + eps);
 #pragma unroll
     for (int i = 0; i < 8 * PASSES; ++i) y[i] = (x[i] * scale) * f.w[i];
@@ -263,6 +276,25 @@ __device__ __forceinline__ void head16_finish(const float (&x)[8 * PASSES], cons
   }
   const int half = rot / 2;
   const bool run_aligned = (half & 7) == 0;  // uniform
+  if (PASSES == 1 && rotated && run_aligned) {  // uniform: a lane's eight partners are the eight of one other lane
+    const int e0 = 8 * gl;
+    const bool lower = e0 < half, turns = e0 < rot;
+    const int lanes_apart = half >> 3;
+    const int from = (((threadIdx.x & 63 & ~15) | ((gl + (lower ? lanes_apart : 16 - lanes_apart)) & 15))) << 2;
+    float other[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) other[j] = __int_as_float(__builtin_amdgcn_ds_bpermute(from, __float_as_int(y[j])));
+    T out[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      // lower half: y c - other s; upper half: y c + other s (a - b and a + (-b) are the same bits)
+      const float s = lower ? -f.s[j] : f.s[j];
+      const float turned = y[j] * f.c[j] + other[j] * s;
+      out[j] = from_f32<T>(turns ? turned : y[j]);
+    }
+    if (e0 < d) dst(e0, out);
+    return;
+  }
 #pragma unroll
   for (int p = 0; p < PASSES; ++p) {
     const int e0 = 128 * p + 8 * gl;

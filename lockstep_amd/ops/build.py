@@ -34,6 +34,7 @@ ARCH = "gfx950"
 FLAGS = [
     f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-ffp-contract=off", "-Wno-pass-failed",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-mllvm", "-amdgpu-kernarg-preload-count=16",
     "-shared", "-fPIC",
 ]
 CORE_SOURCES = ("core.hip", "gemm.hip", "sample.hip")

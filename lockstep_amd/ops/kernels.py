@@ -557,7 +557,7 @@ class Kernels:
         if not (table.dtype == torch.int32 and table.dim() == 2 and table.is_contiguous()):
             raise KernelError("attention block table")
         if not (items.dtype == torch.int32 and items.is_contiguous() and items.numel() >= ATTENTION_ITEM_INTS * n_items):
-            raise KernelError("attention items must hold 16 int32 each (see pack_attention_items)")
+            raise KernelError("attention items must hold 32 int32 each (see pack_attention_items)")
         if n_items == 0:
             return
         self._launch(lib, lib.ls_attention, (
@@ -589,7 +589,7 @@ class Kernels:
         if not (table.dtype == torch.int32 and table.dim() == 2 and table.is_contiguous()):
             raise KernelError("attention block table")
         if not (items.dtype == torch.int32 and items.is_contiguous() and items.numel() >= ATTENTION_ITEM_INTS * n_items):
-            raise KernelError("attention items must hold 16 int32 each (see pack_attention_items)")
+            raise KernelError("attention items must hold 32 int32 each (see pack_attention_items)")
         for w in (q_weight, k_weight):
             if not (w is None or (w.dtype == torch.float32 and w.is_contiguous() and w.numel() == d)):
                 raise KernelError("per-head norm weights must be float32 [head_dim]")
@@ -628,16 +628,18 @@ class Kernels:
             _ptr(part_ml), _ptr(out), c_long(out.stride(0)), c_int(nq // nkv), c_int(max_rows), _stream()))
 
 
-ATTENTION_ITEM_INTS = 16
+ATTENTION_ITEM_INTS = 32
 COMBINE_ITEM_INTS = 8
 
 
-def pack_attention_items(items, seqs) -> "np.ndarray":
+def pack_attention_items(items, seqs, pages=None) -> "np.ndarray":
     """Work items of the attention kernels as the device wants them.  ``items``:
     rows of (seq, row_block, split_begin, split_end, part_base, n_splits,
     split_lo, 0), seq -1 for an item that stands for no work; ``seqs``: the step's rows of (q_off, q_len, q_start, kv_len,
     table_row, 0, 0, 0).  Each item gets a copy of its request's row appended, so
-    that a workgroup learns its work from one load."""
+    that a workgroup learns its work from one load, and sixteen more ints: with ``pages`` (an int array
+    ``[items, 16]``, or None) the block-table entries of the item's one key tile, which the fused decode kernel
+    then takes from the item instead of the block table (the eighth int of the item says so)."""
     import numpy as np
 
     items = np.asarray(items, dtype=np.int64).reshape(-1, 8)
@@ -648,7 +650,14 @@ def pack_attention_items(items, seqs) -> "np.ndarray":
     rows = seqs[np.maximum(items[:, 0], 0)]
     rows[null] = 0                               # a null item is all zeros: a request of no rows, no splits
     items = np.where(null[:, None], 0, items)
-    return np.concatenate([items, rows], axis=1).reshape(-1)
+    if pages is None:
+        ids = np.zeros((len(items), 16), dtype=np.int64)
+    else:
+        ids = np.asarray(pages, dtype=np.int64).reshape(len(items), 16)
+        ids = np.where(null[:, None], 0, ids)
+        items = items.copy()
+        items[:, 7] = np.where(null, 0, 1)
+    return np.concatenate([items, rows, ids], axis=1).reshape(-1)
 
 
 def pack_combine_items(items, seqs) -> "np.ndarray":

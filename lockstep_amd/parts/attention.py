@@ -43,6 +43,9 @@ PART_ROWS_STEP = 4096      # rows of partial results are taken in steps of this 
 # with the same number of splits.  Each column block of the product repeats the fold, so this is for few rows
 # times splits only.  "0" switches it off.
 FOLD_IN_PRODUCT = os.environ.get("LOCKSTEP_FOLD_IN_PRODUCT", "1") not in ("", "0")
+# Items of one key tile of a fused decode step bring the tile's page ids along, so that the kernel's tile loads
+# need no look-up in the block table first; "0" switches it off.
+EMBED_PAGES = os.environ.get("LOCKSTEP_EMBED_PAGES", "1") not in ("", "0")
 FOLD_MAX_SPLITS = int(os.environ.get("LOCKSTEP_FOLD_MAX_SPLITS", "8"))
 FOLD_MAX_ROW_SPLITS = int(os.environ.get("LOCKSTEP_FOLD_MAX_ROW_SPLITS", "128"))   # requests times splits
 
@@ -58,7 +61,7 @@ class AttentionPlan:
     """Where the lists of one set of attention constants lie inside their block, and what the
     launches need to know about them."""
 
-    n_items: int              # staged / direct items (16 ints each), first in the block
+    n_items: int              # staged / direct items (32 ints each), first in the block
     n_combine: int            # combine items (8 ints each)
     n_coop: int               # cooperative items (decoded tokens)
     coop_max_rows: int
@@ -72,7 +75,7 @@ class AttentionPlan:
     fold_splits: int = 0
     single_tile: bool = False  # every cooperative item holds one key tile (one tile buffer a workgroup is enough)
 
-    ITEM, COMBINE = 16, 8
+    ITEM, COMBINE = 32, 8
 
     def offsets(self):
         items = 0
@@ -212,8 +215,34 @@ def plan_attention(ctx, group_size: int, nkv: int, head_dim: int, window: int):
     single_tile = bool(coop) and all((it[3] - it[2]) * split <= tile for it in coop)
     plan = AttentionPlan(len(items), len(combine), len(coop), coop_max_rows, len(wide), part_rows, decode_fused,
                          wide_variant, spans, fold_splits, single_tile)
+    coop_pages = None
+    if EMBED_PAGES and decode_fused and single_tile and split == tile and tile // page_size <= 16:
+        coop_pages = tile_page_ids(ctx, coop, nkv, head_dim, window, tile)
     return plan, np.concatenate([pack_attention_items(items, ctx.seq_rows), pack_combine_items(combine, ctx.seq_rows),
-                                 pack_attention_items(coop, ctx.seq_rows), pack_attention_items(wide, ctx.seq_rows)])
+                                 pack_attention_items(coop, ctx.seq_rows, coop_pages),
+                                 pack_attention_items(wide, ctx.seq_rows)])
+
+
+def tile_page_ids(ctx, coop, nkv: int, head_dim: int, window: int, tile: int):
+    """The block-table entries of the one key tile of every cooperative item (``[items, 16]``, -1 where the
+    request holds no page), read from the host's copy of the table of the cache group with these constants;
+    None if no group has them."""
+    cache, page_size = ctx.cache, ctx.cache.page_size
+    group = next((g for g in cache.groups if (g.spec.num_kv_heads, g.spec.head_dim, g.spec.window or 0)
+                  == (nkv, head_dim, window)), None)
+    if group is None:
+        return None
+    per_tile = tile // page_size
+    work = np.asarray(coop, dtype=np.int64).reshape(-1, 8)
+    live = work[:, 0] >= 0
+    slots = ctx.slots[np.maximum(work[:, 0], 0)]
+    first = work[:, 2] * per_tile                                        # first logical page of the item's tile
+    columns = first[:, None] + np.arange(per_tile)[None, :]
+    inside = columns < group.table_host.shape[1]
+    ids = np.where(inside, group.table_host[slots[:, None], np.minimum(columns, group.table_host.shape[1] - 1)], -1)
+    out = np.full((len(work), 16), -1, dtype=np.int64)
+    out[:, :per_tile] = np.where(live[:, None], ids, -1)
+    return out
 
 
 def advancing_fields(plan: AttentionPlan):
@@ -222,7 +251,7 @@ def advancing_fields(plan: AttentionPlan):
     items, _, coop, wide, _ = plan.offsets()
     runs = []
     for first, count in ((items, plan.n_items), (coop, plan.n_coop), (wide, plan.n_wide)):
-        runs += [(first + 10, 16, count), (first + 11, 16, count)]
+        runs += [(first + 10, AttentionPlan.ITEM, count), (first + 11, AttentionPlan.ITEM, count)]
     return [r for r in runs if r[2]]
 
 

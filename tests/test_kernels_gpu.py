@@ -3,6 +3,7 @@ operation, at sizes other than the engine's, in float32 and in bfloat16."""
 
 from __future__ import annotations
 
+import numpy as np
 import pytest
 import torch
 
@@ -868,18 +869,31 @@ def test_fused_decode_attention_equals_the_separate_kernels(dtype, nq, nkv, d, p
             from lockstep_amd.ops import pack_attention_items, pack_combine_items
 
             seq_row = base.seqs(p, 1).cpu().numpy()
-            items_t = torch.from_numpy(pack_attention_items(items, seq_row)).to(torch.int32).cuda()
-            raw = qkv[p:p + 1].clone()
-            K().attention_decode(raw, nq, nkv, d, base.k_pages, base.v_pages, ps, base.table, base.seqs(p, 1), items_t,
-                                 len(items) // 8, out, part_acc, part_ml, d ** -0.5, window, qw, kw, eps, cos, sin, rot,
-                                 p, True)
-            if combine:
-                comb = torch.from_numpy(pack_combine_items(combine, seq_row)).to(torch.int32).cuda()
-                K().attention_combine(d, base.seqs(p, 1), comb, 1, nq, nkv, part_acc, part_ml, out)
-            assert torch.equal(out.view(1, nq, d), want), f"position {p}, split={use_split}"
-            same_k = (base.k_pages == k_want) | ((base.k_pages != base.k_pages) & (k_want != k_want))
-            same_v = (base.v_pages == v_want) | ((base.v_pages != base.v_pages) & (v_want != v_want))
-            assert bool(same_k.all()) and bool(same_v.all()), f"cache after position {p}, split={use_split}"
+            # the items of one tile once as they are and once with the tile's page ids inside them
+            one_tile = split == tile and all(items[i + 3] - items[i + 2] == 1 for i in range(0, len(items), 8))
+            for with_pages in (False, True) if one_tile and tile // ps <= 16 else (False,):
+                base.k_pages.copy_(k0); base.v_pages.copy_(v0)
+                part_acc.fill_(float("nan")); part_ml.fill_(float("nan")); out.fill_(float("nan"))
+                ids = None
+                if with_pages:
+                    row_of_table = base.table[int(seq_row.reshape(-1, 8)[0, 4])].cpu().numpy()
+                    ids = np.full((len(items) // 8, 16), -1, dtype=np.int64)
+                    for i in range(len(items) // 8):
+                        held = row_of_table[items[8 * i + 2] * (tile // ps):][: tile // ps]
+                        ids[i, : len(held)] = held
+                items_t = torch.from_numpy(pack_attention_items(items, seq_row, ids)).to(torch.int32).cuda()
+                raw = qkv[p:p + 1].clone()
+                K().attention_decode(raw, nq, nkv, d, base.k_pages, base.v_pages, ps, base.table, base.seqs(p, 1),
+                                     items_t, len(items) // 8, out, part_acc, part_ml, d ** -0.5, window, qw, kw, eps,
+                                     cos, sin, rot, p, True, single_tile=one_tile)
+                if combine:
+                    comb = torch.from_numpy(pack_combine_items(combine, seq_row)).to(torch.int32).cuda()
+                    K().attention_combine(d, base.seqs(p, 1), comb, 1, nq, nkv, part_acc, part_ml, out)
+                what = f"position {p}, split={use_split}, page ids in the items: {with_pages}"
+                assert torch.equal(out.view(1, nq, d), want), what
+                same_k = (base.k_pages == k_want) | ((base.k_pages != base.k_pages) & (k_want != k_want))
+                same_v = (base.v_pages == v_want) | ((base.v_pages != base.v_pages) & (v_want != v_want))
+                assert bool(same_k.all()) and bool(same_v.all()), f"cache after {what}"
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
