@@ -1204,27 +1204,29 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
       }
     }
   };
-  auto pages_of = [&](int ti) -> const int* { return tile_pages + ((ti - ti_lo) % kPageWindow) * 16; };
+  // (an item that brings its one tile's ids: every wave keeps a copy of its own, so that none waits for another)
+  const bool embedded = FUSE && item.pages_here != 0;
+  auto pages_of = [&](int ti) -> const int* {
+    return tile_pages + (embedded ? wave : (ti - ti_lo) % kPageWindow) * 16;
+  };
   auto window_start = [&](int ti) -> bool { return (ti - ti_lo) % kPageWindow == 0; };  // tile ti opens a window of ids
   const long page_stride = (long)nkv * page_size * D;  // elements of one page, K or V
   PROBE(16)
+  // where a thread's pieces of a tile lie inside their pages (the same for every tile)
   int k_off[PER], v_off[PER];
+  auto piece_offsets = [&]() {
 #pragma unroll
-  for (int i = 0; i < PER; ++i) {
-    const int p = i * NT + (int)threadIdx.x;
-    const int row = p / KPIECES;
-    const int slot = p % KPIECES;
-    const int piece = (slot - row_rotation<T>(row) % KPIECES + KPIECES) % KPIECES;
-    k_off[i] = (kvh * page_size + (row & (page_size - 1))) * D + piece * VEC;
-    const int c = p / D;
-    const int d = p % D;
-    v_off[i] = ((kvh * D + d) << page_shift) + ((c * VEC) & (page_size - 1));
-  }
-#ifdef LS_ATTN_PROBE
-#pragma unroll
-  for (int i = 0; i < PER; ++i) __asm__ volatile("" ::"v"(k_off[i]), "v"(v_off[i]));
-#endif
-  PROBE(17)
+    for (int i = 0; i < PER; ++i) {
+      const int p = i * NT + (int)threadIdx.x;
+      const int row = p / KPIECES;
+      const int slot = p % KPIECES;
+      const int piece = (slot - row_rotation<T>(row) % KPIECES + KPIECES) % KPIECES;
+      k_off[i] = (kvh * page_size + (row & (page_size - 1))) * D + piece * VEC;
+      const int c = p / D;
+      const int d = p % D;
+      v_off[i] = ((kvh * D + d) << page_shift) + ((c * VEC) & (page_size - 1));
+    }
+  };
   auto issue = [&](int ti) {
     const int* pages = pages_of(ti);
     unsigned char* k_buf = lds + (NBUF == 2 ? (ti & 1) : 0) * BUF_BYTES;
@@ -1330,41 +1332,46 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
   T* qrot = reinterpret_cast<T*>(prob);  // FUSE: [16][D] rotated query heads; the exchange buffers are free until the loop
   // norm and rotation of head vi from hx / hf: a query head to qrot, the new key and value to LDS and to the cache
   auto finish_head = [&](int vi) {
-    const int slot_new = p_new & (page_size - 1);
     if (vi < G) {
       head16_finish<T, PASSES>(hx, hf, D, fz.q_weight != nullptr, fz.eps, rotated, fz.rot, gl,
                                [&](int e0, const T (&v)[8]) { store8<T>(qrot + vi * D + e0, v); });
     } else if (vi == G) {
-      T* dst = fz.k_out + ((max(page_new, 0L) * nkv + kvh) * page_size + slot_new) * D;
       head16_finish<T, PASSES>(hx, hf, D, fz.k_weight != nullptr, fz.eps, rotated, fz.rot, gl,
-                               [&](int e0, const T (&v)[8]) {
-                                 store8<T>(knew + e0, v);
-                                 if (page_new >= 0) store8<T>(dst + e0, v);
-                               });
+                               [&](int e0, const T (&v)[8]) { store8<T>(knew + e0, v); });
     } else {
-      T* dst = fz.v_out + ((max(page_new, 0L) * nkv + kvh) * D) * page_size + slot_new;
 #pragma unroll
       for (int p = 0; p < PASSES; ++p) {
         const int e0 = 128 * p + 8 * gl;
         if (e0 >= D) continue;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          const T v = from_f32<T>(hx[8 * p + j]);
-          vnew[e0 + j] = v;
-          if (page_new >= 0) dst[(long)(e0 + j) * page_size] = v;
-        }
+        for (int j = 0; j < 8; ++j) vnew[e0 + j] = from_f32<T>(hx[8 * p + j]);
       }
     }
+  };
+  // The new key and value go from LDS to the cache when the workgroup's tiles are done: a store issued while
+  // the tile loads are queued waits behind them, and its wave reaches the next barrier that much later.
+  auto write_new_to_cache = [&]() {
+    if (page_new < 0) return;
+    const int slot_new = p_new & (page_size - 1);
+    T* k_dst = fz.k_out + ((page_new * nkv + kvh) * page_size + slot_new) * D;
+    T* v_dst = fz.v_out + ((page_new * nkv + kvh) * D) * page_size + slot_new;
+    const int t = (int)threadIdx.x - (NT - 64);  // the key by the last wave, the value by the first ones
+    if (t >= 0 && 8 * t < D) {
+      T piece[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) piece[j] = knew[8 * t + j];
+      store8<T>(k_dst + 8 * t, piece);
+    }
+    for (int e = threadIdx.x; e < D; e += NT) v_dst[(long)e * page_size] = vnew[e];
   };
   // An item of one tile may bring the tile's page ids itself (embedded): the tile loads then wait for no second
   // round trip.  The head's operands are then requested by loads the compiler does not count (unwaited), ahead
   // of the tile loads, and awaited with a count that leaves the tile loads in flight, so that norm, rotation and
   // cache write run while the tile is on its way.
   PROBE(18)
-  const bool embedded = FUSE && item.pages_here != 0;
   // (the ids go to their place in LDS before any unwaited load is issued: the compiler's wait for `own_page`
   // would wait for those as well)
-  if (embedded && threadIdx.x < 16) tile_pages[threadIdx.x] = own_page;
+  if (embedded && lane < 16) tile_pages[wave * 16 + lane] = own_page;
   PROBE(19)
   const bool aligned_turn = !rotated || (((fz.rot / 2) & 7) == 0);
   const bool unwaited = embedded && PASSES == 1 && aligned_turn && n_vec <= 16 && 2 * PER <= 63;
@@ -1407,8 +1414,8 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
       f32x4 raw_s0 = load16_unwaited(s_at);
       f32x4 raw_s1 = load16_unwaited(s_at + 4);
       PROBE(13)
-      __syncthreads();  // the page ids are in LDS
-      if (owner) page_new = tile_pages[(p_new & (kTileKeys - 1)) >> page_shift];
+      piece_offsets();  // (while the loads are on their way)
+      if (owner) page_new = tile_pages[wave * 16 + ((p_new & (kTileKeys - 1)) >> page_shift)];
       PROBE(1)
       // the head's operands: everything but the tile's 2 * PER loads (if the item has a tile at all) has arrived
       // (one wait statement for both cases, so that the registers reach it by one way only and are not moved on
@@ -1441,13 +1448,14 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
       }
     }
   } else {
+    piece_offsets();
     if (FUSE) {
       if (owner && !embedded) page_new = tbl[p_new >> page_shift];
       if (grp < n_vec) head_fetch(grp);
     }
     if (!embedded && ti_lo < ti_hi) fill_pages(ti_lo);
     __syncthreads();
-    if (embedded && owner) page_new = tile_pages[(p_new & (kTileKeys - 1)) >> page_shift];
+    if (embedded && owner) page_new = tile_pages[wave * 16 + ((p_new & (kTileKeys - 1)) >> page_shift)];
     if (FUSE) {
       // The head's operands are awaited here, before the tile loads go out: a wait placed after them would also
       // wait for the tiles (loads complete in the order of their issue, and the compiler does not count the tile
@@ -1619,8 +1627,14 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
       for (int kp = 0; kp < NPAIR; ++kp) {
         const int key0 = t0 + key_of_row<T>(kp * KB16, 4 * g);
         const int n_lo = lo_valid - key0, n_hi = sm.kv_len - key0;
-        if (t0 + kp * (16 * KB16) + 16 * KB16 <= sm.kv_len && t0 + kp * (16 * KB16) >= lo_valid && !(FUSE && patch))
-          continue;  // uniform: every key of this pair of blocks is held
+        const int first_key = t0 + kp * (16 * KB16), end_key = first_key + 16 * KB16;  // of all lanes together
+        const bool has_new = FUSE && patch && p_new >= first_key && p_new < end_key;
+        if (end_key <= sm.kv_len && first_key >= lo_valid && !has_new) continue;  // uniform: every key is held
+        if ((first_key >= sm.kv_len || end_key <= lo_valid) && !has_new) {        // uniform: none is
+#pragma unroll
+          for (int j = 0; j < MYDB; ++j) vop[kp][j] = A::zero();
+          continue;
+        }
         if (n_lo > 0 || n_hi < VEC) {
           // one mask for the lane's VEC keys, used for all of its columns
           const vec_t keep = mask_keys(ones_vec<T>(), n_lo, n_hi);
@@ -1713,6 +1727,7 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
     }
   }
 
+  if (FUSE && owner) write_new_to_cache();
 #ifdef LS_ATTN_PROBE
   if (threadIdx.x == 0 && kvh == LS_ATTN_PROBE_KVH && part_ml != nullptr) {
     long long* dst = reinterpret_cast<long long*>(part_ml + (1 << 20)) + blockIdx.x * 32;
