@@ -12,11 +12,10 @@ from pathlib import Path
 import numpy as np
 import pytest
 
-from helpers import BF16_STORED_TOL, FP32_TOL, make_mixed_trace, max_live_tokens, random_tokens, rel_err
+from helpers import make_mixed_trace, max_live_tokens, random_tokens, rel_err, tol_for
 
 pytestmark = pytest.mark.gpu
 ROOT = Path(__file__).resolve().parent.parent
-TOL = {"float32": FP32_TOL, "bfloat16": BF16_STORED_TOL}
 
 
 def run_trace(model_dir, dtype, steps, out_dir, vocab, max_tokens):
@@ -123,7 +122,7 @@ def test_replay_under_four_cuttings(tiny_dirs, tmp_path, dtype, name):
         results[label] = run_trace(folder, dtype, steps, out, vocab, max_live_tokens(steps))
         for rid in requests:
             err = rel_err(results[label][rid], want[rid])
-            assert err < TOL[dtype], f"{label} {rid}: rel err {err:.3e}"
+            assert err < tol_for(dtype, name), f"{label} {rid}: rel err {err:.3e}"
     for label in ("tail", "portions", "mixed"):
         for rid in requests:
             assert np.array_equal(results[label][rid], results["whole"][rid]), f"{label} {rid} differs from whole"
