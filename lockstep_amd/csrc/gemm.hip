@@ -74,12 +74,6 @@ namespace ls {
 #ifndef LS_GEMM_PD_SMALL
 #define LS_GEMM_PD_SMALL 4    // ... and of the 64 x 64 kernel (measured 1 to 4: 4 is 2 to 10 % ahead of 2)
 #endif
-#ifndef LS_GEMM_TALL
-#define LS_GEMM_TALL 1        // 0: never 128 x 64 tiles (many rows over few columns: O and down of a long prompt)
-#endif
-#ifndef LS_GEMM_PD_TALL
-#define LS_GEMM_PD_TALL 2     // their register prefetch depth
-#endif
 
 enum Epilogue : int {
   kStore = 0,     // C[m][n] = total, in the compute dtype
@@ -1207,10 +1201,6 @@ int launch_gemm(const void* X, const void* W, void* C, int M, int N, int K, long
       if constexpr (sizeof(T) == 2) LS_TILED_WAVES(128, 256, LS_GEMM_PD_WIDE, true, 2, 4)
     }
     else if (big_tiles >= (LS_GEMM_BIG ? LS_GEMM_BIG : cus) && M > LS_GEMM_BIG_ROWS) LS_TILED(128, 128, LS_GEMM_PD_BIG, true)
-    // too few columns for that, but tiles of 128 rows by 64 columns still give every CU a workgroup: they load
-    // three quarters of the operand bytes per MFMA that 64 x 64 tiles load
-    else if (LS_GEMM_TALL && M > LS_GEMM_BIG_ROWS && (long)((M + 127) / 128) * ((N + 63) / 64) >= cus)
-      LS_TILED(128, 64, LS_GEMM_PD_TALL, true)
     // up to 64 rows over so many columns that tiles of 128 columns still give every CU a workgroup (the
     // logits head, gate and up of 32B sizes): every workgroup reads all rows of X, so half as many
     // workgroups halve that traffic (gate and up of 32B sizes at 64 rows 135 -> 112 us, the head 82 -> 77 us)
