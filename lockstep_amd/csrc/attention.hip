@@ -2332,3 +2332,7 @@ extern "C" int ls_attention_combine(int dtype, const void* seqs, const void* ite
 #undef LS_COMBINE
   return check_launch("combine");
 }
+
+// The entry points that a list of launches may name (see ls_run_list of the core library).
+#define LS_ATTENTION_LISTED(X) X(ls_attention) X(ls_attention_decode) X(ls_attention_combine)
+LS_DEFINE_LISTED_CALLS(LS_ATTENTION_LISTED)

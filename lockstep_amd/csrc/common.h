@@ -372,6 +372,58 @@ inline int check_launch(const char* what) {
   if (e != hipSuccess) return fail("%s: %s", what, hipGetErrorString(e));
   return 0;
 }
+}  // namespace ls
+
+// Entry points called from a list of 8-byte words, one word an argument (an integer, a pointer, or a float's
+// bits in the low half): a caller that repeats many launches hands the whole list over in one call instead of
+// crossing into the library once a launch.  A library names its listed entry points once,
+//   #define MY_LISTED(X) X(ls_gemm) X(ls_rmsnorm) ...
+//   LS_DEFINE_LISTED_CALLS(MY_LISTED)
+// which defines ls_listed_index(name) (-1: not listed) and ls_call_listed(index, words, n).
+#include <string.h>
+
+#include <type_traits>
+#include <utility>
+namespace ls {
+template <typename T>
+inline T word_as(long long w) {
+  if constexpr (std::is_pointer_v<T>) {
+    return reinterpret_cast<T>(static_cast<uintptr_t>(w));
+  } else if constexpr (std::is_same_v<T, float>) {
+    const unsigned int bits = static_cast<unsigned int>(w);
+    float f;
+    memcpy(&f, &bits, sizeof(f));
+    return f;
+  } else {
+    static_assert(std::is_integral_v<T>, "listed entry points take integers, pointers and floats");
+    return static_cast<T>(w);
+  }
+}
+template <typename... A, size_t... I>
+inline int call_words(int (*fn)(A...), const long long* w, std::index_sequence<I...>) {
+  return fn(word_as<A>(w[I])...);
+}
+template <typename... A>
+inline int call_words(const char* name, int (*fn)(A...), const long long* w, int n) {
+  if (n != (int)sizeof...(A)) return fail("%s takes %d arguments, the list brings %d", name, (int)sizeof...(A), n);
+  return call_words(fn, w, std::index_sequence_for<A...>{});
+}
+#define LS_LISTED_NAME(f) \
+  if (strcmp(name, #f) == 0) return at; \
+  ++at;
+#define LS_LISTED_CALL(f) \
+  if (index == at++) return ls::call_words(#f, &f, words, n);
+#define LS_DEFINE_LISTED_CALLS(ENTRIES)                                             \
+  extern "C" int ls_listed_index(const char* name) {                                \
+    int at = 0;                                                                     \
+    ENTRIES(LS_LISTED_NAME)                                                         \
+    return -1;                                                                      \
+  }                                                                                 \
+  extern "C" int ls_call_listed(int index, const long long* words, int n) {         \
+    int at = 0;                                                                     \
+    ENTRIES(LS_LISTED_CALL)                                                         \
+    return ls::fail("there is no listed entry point %d", index);                    \
+  }
 
 // Compute units of the current device (asked once per device).
 inline int compute_units() {

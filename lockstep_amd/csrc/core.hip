@@ -488,6 +488,32 @@ __global__ __launch_bounds__(256) void advance_decode_kernel(int* __restrict__ m
 }  // namespace ls
 
 LS_DEFINE_ERROR_API
+
+// The entry points that a list of launches may name (the kernels of a layer).
+#define LS_CORE_LISTED(X)                                                                                        \
+  X(ls_gemm) X(ls_gemm_slices) X(ls_gemm_slices_folded) X(ls_add_rmsnorm) X(ls_rmsnorm) X(ls_qk_rope_kv) X(ls_swiglu) \
+  X(ls_bias_act) X(ls_embed)
+LS_DEFINE_LISTED_CALLS(LS_CORE_LISTED)
+
+extern "C" int ls_run_list(const long long* words, long n_words, long* failed_at) {
+  typedef int (*callee_t)(int, const long long*, int);
+  long at = 0;
+  while (at < n_words) {
+    if (at + 3 > n_words || words[at + 2] < 0 || at + 3 + words[at + 2] > n_words) {
+      if (failed_at) *failed_at = at;
+      return ls::fail("run_list: the record at word %ld runs past the end of the list", at);
+    }
+    const callee_t callee = reinterpret_cast<callee_t>(static_cast<uintptr_t>(words[at]));
+    const int n = (int)words[at + 2];
+    const int code = callee((int)words[at + 1], words + at + 3, n);
+    if (code != 0) {
+      if (failed_at) *failed_at = at;
+      return code;
+    }
+    at += 3 + n;
+  }
+  return 0;
+}
 LS_DEFINE_MUTANT_API
 
 using namespace ls;

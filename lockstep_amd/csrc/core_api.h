@@ -73,6 +73,18 @@ int ls_gemm_kslice(int K);
 int ls_gemm_slices_count(int K);
 int ls_gemm_slices_max_rows(int dtype, int K);
 int ls_gemm_slices(int dtype, const void* X, const void* W, float* P, int M, int N, int K, long ldx, void* stream);
+int ls_gemm_slices_folded_ok(int dtype, int M, int N, int K, int head_dim, int splits);
+int ls_gemm_slices_folded(int dtype, const float* part_acc, const float* part_ml, int splits, int head_dim,
+                          const void* W, float* P, int M, int N, int K, void* stream);
+
+// A list of launches in one call.  `words` holds records of 8-byte words one after the other:
+//   [the address of a library's ls_call_listed, the entry point's ls_listed_index there, n, n argument words]
+// (an integer, a pointer, or a float's bits in the low half of its word).  The calls are made in order on the
+// calling thread; the first that fails ends the run: its code is returned, `failed_at` (if not null) gets the
+// offset of its record, and the message is with the library that the record names.
+int ls_listed_index(const char* name);
+int ls_call_listed(int index, const long long* words, int n);
+int ls_run_list(const long long* words, long n_words, long* failed_at);
 
 #ifdef __cplusplus
 }

@@ -88,6 +88,8 @@ class Model:
         # layers alike repeat the launches of the second of them (engine/tape.py)
         self.use_tapes = os.environ.get("LOCKSTEP_NO_TAPES", "") in ("", "0")
         self.verify_tapes = os.environ.get("LOCKSTEP_VERIFY_TAPE", "") not in ("", "0")
+        # the launches of repeated layers handed to the library as one list ("0": one call a launch, from Python)
+        self.list_launches = os.environ.get("LOCKSTEP_LIST_LAUNCHES", "1") not in ("", "0")
         self._run_kinds = weakref.WeakKeyDictionary()      # cache manager -> (device epoch, RunKinds)
         self.layers_repeated = 0
         self.tapes_refused = 0
@@ -196,7 +198,10 @@ class Model:
         kernels = self.rt.kernels
         kinds = self._kinds_for(ctx.cache) if self.use_tapes else None
         met: dict = {}          # kind of run -> None after its first run, then (tape, situation, what it left)
-        for index, run in enumerate(self.schedule):
+        index = -1
+        while index + 1 < len(self.schedule):
+            index += 1
+            run = self.schedule[index]
             kind = kinds.kind[index] if kinds is not None else None
             situation = None
             if kind is not None:
@@ -204,9 +209,22 @@ class Model:
                              None if pending is None else (pending.partials.data_ptr(), tuple(pending.partials.shape)))
                 held = met.get(kind)
                 if held is not None and held[1] == situation and kind in kinds.verified and not self.verify_tapes:
-                    held[0].repeat(kinds.addresses[index])
+                    if held[0].words is not None:
+                        # this layer and the ones like it that follow at once (a repeated layer leaves the
+                        # situation it found): their launches go to the library as one list
+                        left = held[2]
+                        follows = held[1] == (self.workspace.version, None if left is None else (
+                            left.partials.data_ptr(), tuple(left.partials.shape)))
+                        last = index
+                        while follows and last + 1 < len(self.schedule) and kinds.kind[last + 1] == kind:
+                            last += 1
+                        held[0].repeat_many(kernels, [kinds.addresses[i] for i in range(index, last + 1)])
+                        self.layers_repeated += last + 1 - index
+                        index = last
+                    else:
+                        held[0].repeat(kinds.addresses[index])
+                        self.layers_repeated += 1
                     pending = held[2]
-                    self.layers_repeated += 1
                     continue
             noting = kind is not None and kind in met
             if noting:
@@ -245,7 +263,10 @@ class Model:
                     continue
             if situation[0] == self.workspace.version:             # the run did not move the workspace
                 try:
-                    met[kind] = (LayerTape(launches, kinds.addresses[index], kinds.foreign[index]), situation, pending)
+                    tape = LayerTape(launches, kinds.addresses[index], kinds.foreign[index])
+                    if self.list_launches:
+                        tape.as_words(kernels)
+                    met[kind] = (tape, situation, pending)
                 except TapeRefused:
                     kinds.refuse(kind)
                     self.tapes_refused += 1

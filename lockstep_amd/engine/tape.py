@@ -30,7 +30,7 @@ from __future__ import annotations
 
 import bisect
 import dataclasses
-from ctypes import c_void_p
+from ctypes import c_float, c_int, c_long, c_void_p
 
 import torch
 
@@ -154,6 +154,64 @@ class LayerTape:
                                 f"argument {i} of {getattr(entry, '__name__', entry)} points into a tensor of "
                                 "another layer that this layer's parts do not list among their own")
             self.calls.append((lib, entry, args, tuple(marks)))
+        self.names = sorted({name for _, _, _, marks in self.calls for _, name, _ in marks})
+        self._bases: dict = {}       # id of an addresses mapping -> its base addresses in the order of names
+        self.words = None            # the launches as one list for Kernels.run_list, if every entry point is listed
+
+    def as_words(self, kernels) -> bool:
+        """Lay the launches out as the list of words that the core library runs in one call
+        (``Kernels.run_list``); False if a launch names an entry point that cannot be listed."""
+        import struct
+
+        import numpy as np
+
+        words, at_word, name_at, offset, libs = [], [], [], [], []
+        for lib, entry, args, marks in self.calls:
+            listed = kernels.listed(lib, entry)
+            if listed is None:
+                return False
+            libs.append((len(words), listed[2]))
+            words += [listed[0], listed[1], len(args)]
+            first = len(words)
+            for a in args:
+                if isinstance(a, c_float):
+                    words.append(struct.unpack("<I", struct.pack("<f", a.value))[0])
+                elif isinstance(a, (c_void_p, c_int, c_long)):
+                    words.append(a.value or 0)
+                else:
+                    return False
+            for i, name, off in marks:
+                at_word.append(first + i)
+                name_at.append(self.names.index(name))
+                offset.append(off)
+        self.words = np.asarray(words, dtype=np.int64)
+        self._at_word = np.asarray(at_word, dtype=np.int64)
+        self._name_at = np.asarray(name_at, dtype=np.int64)
+        self._offset = np.asarray(offset, dtype=np.int64)
+        self._libs = libs
+        return True
+
+    def _bases_of(self, addresses: dict):
+        import numpy as np
+
+        held = self._bases.get(id(addresses))
+        if held is None:
+            held = np.asarray([addresses[name][0] for name in self.names], dtype=np.int64)
+            self._bases[id(addresses)] = held
+        return held
+
+    def repeat_many(self, kernels, layers) -> None:
+        """The launches for every mapping of addresses in ``layers``, one layer after the other, in one call."""
+        import numpy as np
+
+        n, size = len(layers), self.words.size
+        words = np.tile(self.words, n)
+        if self._at_word.size:
+            bases = np.stack([self._bases_of(a) for a in layers])                       # [layers, names]
+            values = bases[:, self._name_at] + self._offset[None, :]                    # [layers, marks]
+            places = self._at_word[None, :] + (np.arange(n, dtype=np.int64) * size)[:, None]
+            words[places.reshape(-1)] = values.reshape(-1)
+        kernels.run_list(words, self._libs, size)
 
     def arguments(self, addresses: dict):
         """(library, entry point, arguments) of every launch, for the layer with these addresses."""

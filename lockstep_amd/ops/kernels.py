@@ -86,6 +86,7 @@ class Kernels:
         #: while this is a list, every launch is noted on it as (library, entry point, arguments):
         #: the engine repeats the launches of one layer for the next layers that are alike
         self.tape: list | None = None
+        self._listed: dict = {}
 
     # -- helpers ------------------------------------------------------------
     @staticmethod
@@ -98,6 +99,32 @@ class Kernels:
             raise KernelError(lib.ls_last_error().decode())
         if self.tape is not None:
             self.tape.append((lib, entry, args))
+
+    # -- launches handed over as one list ----------------------------------------
+    def listed(self, lib, entry):
+        """(address of the library's ``ls_call_listed``, the entry point's index there) for an entry point
+        that ``run_list`` may name, or None."""
+        key = (id(lib), entry.__name__)
+        found = self._listed.get(key, False)
+        if found is False:
+            found = None
+            if hasattr(lib, "ls_listed_index"):
+                index = lib.ls_listed_index(entry.__name__.encode())
+                if index >= 0:
+                    found = (ctypes.cast(lib.ls_call_listed, c_void_p).value, index, lib)
+            self._listed[key] = found
+        return found
+
+    def run_list(self, words, libs=(), period: int = 0) -> None:
+        """Make the calls that ``words`` (a contiguous int64 array of records, see ``ls_run_list`` in
+        csrc/core_api.h) lists, in order.  ``libs``: (word offset of a record, its library) pairs, for the
+        message of a call that fails; with ``period`` the offsets repeat with that many words."""
+        failed_at = ctypes.c_long(-1)
+        code = self.core.ls_run_list(c_void_p(words.ctypes.data), c_long(words.size), ctypes.byref(failed_at))
+        if code != 0:
+            at = failed_at.value % period if period else failed_at.value
+            lib = dict(libs).get(at, self.core)
+            raise KernelError(lib.ls_last_error().decode())
 
     def attention_lib(self, head_dim: int):
         lib = self._attention.get(head_dim)
