@@ -182,7 +182,10 @@ def build(kind: str, sources, defines=(), force: bool = False) -> Path:
 
 
 def build_core(force: bool = False) -> Path:
-    return build("core", CORE_SOURCES, (), force)
+    # LOCKSTEP_CORE_DEFINES: further -D switches for the core library (the tuning macros at the top of the
+    # sources), for measurements; the file name carries them in its hash like every other flag
+    extra = tuple(os.environ.get("LOCKSTEP_CORE_DEFINES", "").split())
+    return build("core", CORE_SOURCES, extra, force)
 
 
 def build_attention(head_dim: int, force: bool = False) -> Path:
