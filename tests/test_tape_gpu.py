@@ -132,3 +132,47 @@ def test_a_tensor_that_the_walk_does_not_find_switches_the_repetition_off(deep_d
 
     with pytest.raises(RuntimeError, match="layer run 2: launch 0 .* differs from the tape"):
         checked.step(cache, [StepEntry("r", random_tokens(20, 1000, seed=1), [19])])
+
+
+def test_launches_from_a_list_give_the_bits_of_launches_one_by_one(deep_dirs):
+    """Repeated layers go to the library as one list of words (``ls_run_list``) or launch by launch
+    from Python: the same logits, bit for bit, and the list really is what ran."""
+    folder = deep_dirs["A"]
+    listed = load(folder, "bfloat16", use_tapes=True, verify_tapes=False, list_launches=True)
+    one_by_one = load(folder, "bfloat16", use_tapes=True, verify_tapes=False, list_launches=False)
+    requests, steps = trace_for(listed.spec.vocab_size)
+    calls = []
+    kernels = listed.rt.kernels
+    run_list = kernels.run_list
+    kernels.run_list = lambda words, *a, **k: (calls.append(int(words.size)), run_list(words, *a, **k))[1]
+    try:
+        results = []
+        for model in (listed, one_by_one):
+            cache = model.make_cache(num_pages=60, page_size=16, max_requests=4, poison_on_free=True)
+            results.append(replay_in_process(model, cache, steps))
+    finally:
+        kernels.run_list = run_list
+    assert calls and listed.layers_repeated == one_by_one.layers_repeated > 0
+    for rid in requests:
+        assert torch.equal(results[0][rid], results[1][rid]), rid
+
+
+def test_a_list_of_launches_that_is_wrong_is_refused_with_its_reason():
+    """The runner checks a record before it calls: a record that runs past the list's end, an entry point
+    that is not listed, and a call with the wrong number of arguments each end the run with a message."""
+    import ctypes
+
+    import numpy as np
+
+    from lockstep_amd.ops import KernelError, kernels
+
+    k = kernels()
+    callee, index, lib = k.listed(k.core, k.core.ls_rmsnorm)
+    assert k.listed(k.core, k.core.ls_argmax) is None                      # not among the listed entry points
+    with pytest.raises(KernelError, match="runs past the end"):
+        k.run_list(np.asarray([callee, index, 40, 1, 2], dtype=np.int64))
+    with pytest.raises(KernelError, match="ls_rmsnorm takes 11 arguments, the list brings 2"):
+        k.run_list(np.asarray([callee, index, 2, 0, 0], dtype=np.int64))
+    with pytest.raises(KernelError, match="no listed entry point 99"):
+        k.run_list(np.asarray([callee, 99, 0], dtype=np.int64))
+    assert ctypes.cast(lib.ls_call_listed, ctypes.c_void_p).value == callee
