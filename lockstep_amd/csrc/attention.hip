@@ -1983,8 +1983,35 @@ __global__ __launch_bounds__(256) void combine_few_rows_kernel(const SeqMeta* __
         if (q * 256 + (int)threadIdx.x >= owned) continue;
         const float* mine = &stage_acc[buf][row_of[q] * row_stride + quad_of[q] * 4];
         const float* ml = &stage_ml[buf][2 * row_of[q] * batch];
-        for (int u = 0; u < count; ++u)
-          fold(q, *reinterpret_cast<const f32x4*>(mine + u * D), ml[2 * u], ml[2 * u + 1]);
+        // Four splits' sums are read before the first of them is folded (the reads of one split take as long
+        // as its fold), and a split of no weight is passed over by selects, not by a branch, so that nothing
+        // stands between the reads and the chain of folds: fold_split's operations, the same bits.
+        for (int u0 = 0; u0 < count; u0 += 4) {
+          f32x4 acc4[4];
+          float m4[4], l4[4];
+#pragma unroll
+          for (int k = 0; k < 4; ++k) {
+            const int u = min(u0 + k, count - 1);
+            acc4[k] = *reinterpret_cast<const f32x4*>(mine + u * D);
+            m4[k] = ml[2 * u];
+            l4[k] = u0 + k < count ? ml[2 * u + 1] : 0.f;
+          }
+#pragma unroll
+          for (int k = 0; k < 4; ++k) {
+            const bool take = l4[k] > 0.f;
+            const float m_new = fmaxf(run_m[q], m4[k]);
+            const float a = softmax_exp<T>(run_m[q] - m_new);
+            const float b = softmax_exp<T>(m4[k] - m_new);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const float folded = run_acc[q][e] * a + acc4[k][e] * b;
+              run_acc[q][e] = take ? folded : run_acc[q][e];
+            }
+            const float l_new = run_l[q] * a + l4[k] * b;
+            run_l[q] = take ? l_new : run_l[q];
+            run_m[q] = take ? m_new : run_m[q];
+          }
+        }
       }
     }
   }
