@@ -1902,6 +1902,9 @@ __global__ __launch_bounds__(256) void combine_few_rows_kernel(const SeqMeta* __
     row_of[q] = it / QUADS;
     quad_of[q] = it - row_of[q] * QUADS;
   }
+  // (not under the reversed-fold mutant, whose loop folds by groups of four columns)
+  const bool narrow = rows_total * D <= 256 && !LS_MUTANT_DEVICE(kMutantReversedFold);
+  const int one_row = min((int)threadIdx.x / D, rows_total - 1), one_col = (int)threadIdx.x % D;
   auto fold = [&](int q, const f32x4& acc, float m, float l) {  // fold_split on these four columns
     if (!(l > 0.f)) return;
     const float m_new = fmaxf(run_m[q], m);
@@ -1978,6 +1981,37 @@ __global__ __launch_bounds__(256) void combine_few_rows_kernel(const SeqMeta* __
       __syncthreads();  // the batch is in its buffer; the other buffer has been folded by every wave
       if (s0 + batch < n_splits) request(s0 + batch);
       const int count = min(batch, n_splits - s0);
+      if (narrow) {
+        // so few rows that every thread can have one column of one row: a quarter of the multiplications in
+        // each thread's chain, and no wave stands by (the same operations on every element: the same bits)
+        if ((int)threadIdx.x < rows_total * D) {
+          const float* mine = &stage_acc[buf][one_row * row_stride + one_col];
+          const float* ml = &stage_ml[buf][2 * one_row * batch];
+          for (int u0 = 0; u0 < count; u0 += 4) {
+            float acc4[4], m4[4], l4[4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+              const int u = min(u0 + k, count - 1);
+              acc4[k] = mine[u * D];
+              m4[k] = ml[2 * u];
+              l4[k] = u0 + k < count ? ml[2 * u + 1] : 0.f;
+            }
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+              const bool take = l4[k] > 0.f;
+              const float m_new = fmaxf(run_m[0], m4[k]);
+              const float a = softmax_exp<T>(run_m[0] - m_new);
+              const float b = softmax_exp<T>(m4[k] - m_new);
+              const float folded = run_acc[0][0] * a + acc4[k] * b;
+              const float l_new = run_l[0] * a + l4[k] * b;
+              run_acc[0][0] = take ? folded : run_acc[0][0];
+              run_l[0] = take ? l_new : run_l[0];
+              run_m[0] = take ? m_new : run_m[0];
+            }
+          }
+        }
+        continue;
+      }
 #pragma unroll
       for (int q = 0; q < MAXQ; ++q) {
         if (q * 256 + (int)threadIdx.x >= owned) continue;
@@ -2014,6 +2048,13 @@ __global__ __launch_bounds__(256) void combine_few_rows_kernel(const SeqMeta* __
         }
       }
     }
+  }
+  if (narrow) {
+    if ((int)threadIdx.x < rows_total * D) {
+      const float o = run_l[0] > 0.f ? run_acc[0][0] / run_l[0] : 0.f;
+      out[(long)(item.q_off + one_row / G) * ldo + (long)(kvh * G + one_row % G) * D + one_col] = from_f32<T>(o);
+    }
+    return;
   }
 #pragma unroll
   for (int q = 0; q < MAXQ; ++q) {
