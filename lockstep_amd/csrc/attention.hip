@@ -124,6 +124,11 @@ __device__ __forceinline__ void wait_for_loads(f32x4& a, f32x4& b, f32x4& c, f32
                    : "memory");
 }
 
+// Every lambda of a kernel is part of the kernel's body: one that the compiler leaves as a function of its own
+// is called through the stack, with everything it captures kept in scratch memory (seen in the float instances
+// of the fused decode kernel: 75 us a launch instead of 13).
+#define LS_INLINED __attribute__((always_inline))
+
 // A workgroup barrier that makes the waves' own LDS writes visible and nothing else.  __syncthreads() also
 // waits for every load that is still writing into LDS (global_load_lds), which would end the overlap of the
 // next tile's loads with the work on this one; where a tile has to be complete, the kernel waits for its own
@@ -487,7 +492,7 @@ __global__ __launch_bounds__(256, LS_STAGED_MIN_BLOCKS) void attention_staged_ke
   // Page ids are looked up one tile ahead of the data they address, so the
   // two dependent loads of a tile do not wait for each other.
   int kpage[PER], vpage[PER];
-  auto lookup = [&](int ti) {
+  auto lookup = [&](int ti) LS_INLINED {
     const int t0 = ti * kTileKeys;
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
@@ -503,7 +508,7 @@ __global__ __launch_bounds__(256, LS_STAGED_MIN_BLOCKS) void attention_staged_ke
   // of a tile's loads are in flight together; stash() zeroes what is not a
   // held key and writes to LDS.
   vec_t kreg[GROUP], vreg[GROUP];
-  auto fetch = [&](int ti, int i0) {
+  auto fetch = [&](int ti, int i0) LS_INLINED {
     const int t0 = ti * kTileKeys;
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -530,14 +535,14 @@ __global__ __launch_bounds__(256, LS_STAGED_MIN_BLOCKS) void attention_staged_ke
   };
   // page ids of the tile whose data is in kreg/vreg (fetch() ran with them)
   int kpage_held[PER], vpage_held[PER];
-  auto hold_pages = [&]() {
+  auto hold_pages = [&]() LS_INLINED {
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
       kpage_held[i] = kpage[i];
       vpage_held[i] = vpage[i];
     }
   };
-  auto stash = [&](int ti, int i0) {
+  auto stash = [&](int ti, int i0) LS_INLINED {
     const int t0 = ti * kTileKeys;
 #pragma unroll
     for (int j = 0; j < GROUP; ++j) {
@@ -612,7 +617,7 @@ __global__ __launch_bounds__(256, LS_STAGED_MIN_BLOCKS) void attention_staged_ke
       {
         constexpr int NS = NB * NC;
         constexpr int RING = NS < kRing ? NS : kRing;
-        auto k_read = [&](int idx) -> vec_t {
+        auto k_read = [&](int idx) LS_INLINED -> vec_t {
           const int row = key_of_row<T>(idx / NC, row16);
           const int piece = (idx % NC) * 4 + g;
           const int pc = (4 * NC == KPIECES) ? piece : min(piece, KPIECES - 1);
@@ -678,7 +683,7 @@ __global__ __launch_bounds__(256, LS_STAGED_MIN_BLOCKS) void attention_staged_ke
       {
         constexpr int NP = (NB / KB16) * DB;
         constexpr int RING = NP < kRing ? NP : kRing;
-        auto v_read = [&](int idx) -> vec_t {
+        auto v_read = [&](int idx) LS_INLINED -> vec_t {
           const int kb = (idx / DB) * KB16;
           const int d = (idx % DB) * 16 + row16;
           vec_t vv;
@@ -824,7 +829,7 @@ __global__ __launch_bounds__(64 * NW) void attention_wide_kernel(
 
   // The page ids of kPageWindow tiles at a time go into LDS, by ordinary loads, while no tile load is in
   // flight (the compiler's waits for ordinary loads do not know of the tile loads and would wait for them too).
-  auto fill_pages = [&](int first_tile) {
+  auto fill_pages = [&](int first_tile) LS_INLINED {
     for (int idx = threadIdx.x; idx < kPageWindow * 16; idx += NT) {
       const int t = first_tile + idx / 16;
       const int pg = idx % 16;
@@ -834,7 +839,7 @@ __global__ __launch_bounds__(64 * NW) void attention_wide_kernel(
       }
     }
   };
-  auto window_start = [&](int ti) -> bool { return (ti - ti_lo) % kPageWindow == 0; };  // tile ti opens a window of ids
+  auto window_start = [&](int ti) LS_INLINED -> bool { return (ti - ti_lo) % kPageWindow == 0; };  // tile ti opens a window of ids
   // Start the loads of a tile into its buffer.  What does not depend on the
   // tile is computed once: the offset of each of the thread's pieces inside
   // its page.  Keys past the request's end need no clamp of their own: the
@@ -853,7 +858,7 @@ __global__ __launch_bounds__(64 * NW) void attention_wide_kernel(
     const int d = p % D;
     v_off[i] = ((kvh * D + d) << page_shift) + ((c * VEC) & (page_size - 1));
   }
-  auto issue = [&](int ti) {
+  auto issue = [&](int ti) LS_INLINED {
     const int* pages = tile_pages + ((ti - ti_lo) % kPageWindow) * 16;
     unsigned char* k_buf = lds + (ti & 1) * BUF_BYTES;
     unsigned char* v_buf = k_buf + TILE_BYTES;
@@ -926,7 +931,7 @@ __global__ __launch_bounds__(64 * NW) void attention_wide_kernel(
       {
         constexpr int NS = NB * NC;
         constexpr int RING = NS < kRing ? NS : kRing;
-        auto k_read = [&](int idx) -> vec_t {
+        auto k_read = [&](int idx) LS_INLINED -> vec_t {
           const int row = key_of_row<T>(idx / NC, row16);
           const int piece = (idx % NC) * 4 + g;
           const int pc = (4 * NC == KPIECES) ? piece : min(piece, KPIECES - 1);
@@ -991,7 +996,7 @@ __global__ __launch_bounds__(64 * NW) void attention_wide_kernel(
       {
         constexpr int NP = (NB / KB16) * DB;
         constexpr int RING = NP < kRing ? NP : kRing;
-        auto v_read = [&](int idx) -> vec_t {
+        auto v_read = [&](int idx) LS_INLINED -> vec_t {
           const int kb = (idx / DB) * KB16;
           const int d = (idx % DB) * 16 + row16;
           vec_t vv;
@@ -1194,7 +1199,7 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
 
   // The page ids of kPageWindow tiles at a time go into LDS, by ordinary loads, while no tile load is in
   // flight (the compiler's waits for ordinary loads do not know of the tile loads and would wait for them too).
-  auto fill_pages = [&](int first_tile) {
+  auto fill_pages = [&](int first_tile) LS_INLINED {
     for (int idx = threadIdx.x; idx < kPageWindow * 16; idx += NT) {
       const int t = first_tile + idx / 16;
       const int pg = idx % 16;
@@ -1206,15 +1211,15 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
   };
   // (an item that brings its one tile's ids: every wave keeps a copy of its own, so that none waits for another)
   const bool embedded = FUSE && item.pages_here != 0;
-  auto pages_of = [&](int ti) -> const int* {
+  auto pages_of = [&](int ti) LS_INLINED -> const int* {
     return tile_pages + (embedded ? wave : (ti - ti_lo) % kPageWindow) * 16;
   };
-  auto window_start = [&](int ti) -> bool { return (ti - ti_lo) % kPageWindow == 0; };  // tile ti opens a window of ids
+  auto window_start = [&](int ti) LS_INLINED -> bool { return (ti - ti_lo) % kPageWindow == 0; };  // tile ti opens a window of ids
   const long page_stride = (long)nkv * page_size * D;  // elements of one page, K or V
   PROBE(16)
   // where a thread's pieces of a tile lie inside their pages (the same for every tile)
   int k_off[PER], v_off[PER];
-  auto piece_offsets = [&]() {
+  auto piece_offsets = [&]() LS_INLINED {
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
       const int p = i * NT + (int)threadIdx.x;
@@ -1227,7 +1232,7 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
       v_off[i] = ((kvh * D + d) << page_shift) + ((c * VEC) & (page_size - 1));
     }
   };
-  auto issue = [&](int ti) {
+  auto issue = [&](int ti) LS_INLINED {
     const int* pages = pages_of(ti);
     unsigned char* k_buf = lds + (NBUF == 2 ? (ti & 1) : 0) * BUF_BYTES;
     unsigned char* v_buf = k_buf + TILE_BYTES;
@@ -1252,7 +1257,7 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
   // Each thread issues exactly PER loads for a K tile and PER for a V tile, in this order for a given tile,
   // which is what the waits below count on (loads complete in the order of their issue).
   static_assert(NBUF == 2 || PER * NT == TOTAL, "the split loads assume whole rounds");
-  auto issue_k = [&](int ti) {
+  auto issue_k = [&](int ti) LS_INLINED {
     const int* pages = pages_of(ti);
     int k_page[PER];
 #pragma unroll
@@ -1263,7 +1268,7 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
       load_to_lds16(k_src, (lptr_t)(lds + (i * NT + wave * 64) * 16));
     }
   };
-  auto issue_v = [&](int ti) {
+  auto issue_v = [&](int ti) LS_INLINED {
     const int* pages = pages_of(ti);
     int v_page[PER];
 #pragma unroll
@@ -1286,7 +1291,7 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
   }
 
   // The sums of one split to their place among the partial results (an item may hold several splits).
-  auto write_partial = [&](int split, const f32x4 (&acc)[MYDB], float m, float l) {
+  auto write_partial = [&](int split, const f32x4 (&acc)[MYDB], float m, float l) LS_INLINED {
     if (!row_ok) return;
     const long pr = item.part_base + ((long)kvh * rows_total + r) * item.n_splits + (split - item.split_lo);
     float* pa = part_acc + pr * D;
@@ -1320,10 +1325,10 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
   long page_new = -1;
   float hx[8 * PASSES] = {};
   HeadFactors<PASSES> hf = {};
-  auto head_src = [&](int vi) -> const T* {
+  auto head_src = [&](int vi) LS_INLINED -> const T* {
     return new_row + (long)(vi < G ? kvh * G + vi : vi == G ? fz.nq + kvh : fz.nq + nkv + kvh) * D;
   };
-  auto head_fetch = [&](int vi) {
+  auto head_fetch = [&](int vi) LS_INLINED {
     head16_load_values<T, PASSES>(hx, head_src(vi), D, gl);
     if (vi <= G)
       head16_load_factors<PASSES>(hf, D, vi < G ? fz.q_weight : fz.k_weight, fz.cos_table, fz.sin_table, p_new,
@@ -1331,13 +1336,13 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
   };
   T* qrot = reinterpret_cast<T*>(prob);  // FUSE: [16][D] rotated query heads; the exchange buffers are free until the loop
   // norm and rotation of head vi from hx / hf: a query head to qrot, the new key and value to LDS and to the cache
-  auto finish_head = [&](int vi) {
+  auto finish_head = [&](int vi) LS_INLINED {
     if (vi < G) {
       head16_finish<T, PASSES>(hx, hf, D, fz.q_weight != nullptr, fz.eps, rotated, fz.rot, gl,
-                               [&](int e0, const T (&v)[8]) { store8<T>(qrot + vi * D + e0, v); });
+                               [&](int e0, const T (&v)[8]) LS_INLINED { store8<T>(qrot + vi * D + e0, v); });
     } else if (vi == G) {
       head16_finish<T, PASSES>(hx, hf, D, fz.k_weight != nullptr, fz.eps, rotated, fz.rot, gl,
-                               [&](int e0, const T (&v)[8]) { store8<T>(knew + e0, v); });
+                               [&](int e0, const T (&v)[8]) LS_INLINED { store8<T>(knew + e0, v); });
     } else {
 #pragma unroll
       for (int p = 0; p < PASSES; ++p) {
@@ -1350,7 +1355,7 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
   };
   // The new key and value go from LDS to the cache when the workgroup's tiles are done: a store issued while
   // the tile loads are queued waits behind them, and its wave reaches the next barrier that much later.
-  auto write_new_to_cache = [&]() {
+  auto write_new_to_cache = [&]() LS_INLINED {
     if (page_new < 0) return;
     const int slot_new = p_new & (page_size - 1);
     T* k_dst = fz.k_out + ((page_new * nkv + kvh) * page_size + slot_new) * D;
@@ -1378,7 +1383,7 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
   const int e0_head = 8 * gl;                    // the lane's eight elements of a head (PASSES == 1)
   const bool lane_in_head = e0_head < D;
   const bool lane_turns = rotated && e0_head < fz.rot;
-  auto issue_tile = [&](int ti) {
+  auto issue_tile = [&](int ti) LS_INLINED {
     if (NBUF == 2) {
       issue(ti);
     } else {
@@ -1595,7 +1600,7 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
     constexpr int KB16 = VEC / 4;
     constexpr int NPAIR = NB / KB16;
     vec_t vop[NPAIR][MYDB];
-    auto read_values = [&]() {
+    auto read_values = [&]() LS_INLINED {
 #pragma unroll
     for (int kp = 0; kp < NPAIR; ++kp)
 #pragma unroll
@@ -1622,7 +1627,7 @@ __global__ __launch_bounds__(256) void attention_coop_kernel(
     };
     // The values of keys that are not held become zeros and the new token's value takes its place: in the
     // operands as they were read (a lane's VEC values of a column belong to VEC consecutive keys), not in LDS.
-    auto fix_values = [&]() {
+    auto fix_values = [&]() LS_INLINED {
 #pragma unroll
       for (int kp = 0; kp < NPAIR; ++kp) {
         const int key0 = t0 + key_of_row<T>(kp * KB16, 4 * g);
@@ -1905,7 +1910,7 @@ __global__ __launch_bounds__(256) void combine_few_rows_kernel(const SeqMeta* __
   // (not under the reversed-fold mutant, whose loop folds by groups of four columns)
   const bool narrow = rows_total * D <= 256 && !LS_MUTANT_DEVICE(kMutantReversedFold);
   const int one_row = min((int)threadIdx.x / D, rows_total - 1), one_col = (int)threadIdx.x % D;
-  auto fold = [&](int q, const f32x4& acc, float m, float l) {  // fold_split on these four columns
+  auto fold = [&](int q, const f32x4& acc, float m, float l) LS_INLINED {  // fold_split on these four columns
     if (!(l > 0.f)) return;
     const float m_new = fmaxf(run_m[q], m);
     const float a = softmax_exp<T>(run_m[q] - m_new);
@@ -1934,7 +1939,7 @@ __global__ __launch_bounds__(256) void combine_few_rows_kernel(const SeqMeta* __
     const int total = rows_total * per_row;          // <= STAGE / 4
     f32x4 moved[PIECES];
     float2 moved_ml[2] = {float2{0.f, 0.f}, float2{0.f, 0.f}};  // up to 16 rows x 32 splits over 256 threads
-    auto request = [&](int s0) {  // the loads of the batch that starts at split s0, into registers
+    auto request = [&](int s0) LS_INLINED {  // the loads of the batch that starts at split s0, into registers
 #pragma unroll
       for (int i = 0; i < PIECES; ++i) {
         const int idx = i * 256 + (int)threadIdx.x;
@@ -1956,7 +1961,7 @@ __global__ __launch_bounds__(256) void combine_few_rows_kernel(const SeqMeta* __
         }
       }
     };
-    auto put = [&](int buf) {  // ... and from the registers to their place in LDS
+    auto put = [&](int buf) LS_INLINED {  // ... and from the registers to their place in LDS
 #pragma unroll
       for (int i = 0; i < PIECES; ++i) {
         const int idx = i * 256 + (int)threadIdx.x;
