@@ -124,11 +124,6 @@ __device__ __forceinline__ void wait_for_loads(f32x4& a, f32x4& b, f32x4& c, f32
                    : "memory");
 }
 
-// Every lambda of a kernel is part of the kernel's body: one that the compiler leaves as a function of its own
-// is called through the stack, with everything it captures kept in scratch memory (seen in the float instances
-// of the fused decode kernel: 75 us a launch instead of 13).
-#define LS_INLINED __attribute__((always_inline))
-
 // A workgroup barrier that makes the waves' own LDS writes visible and nothing else.  __syncthreads() also
 // waits for every load that is still writing into LDS (global_load_lds), which would end the overlap of the
 // next tile's loads with the work on this one; where a tile has to be complete, the kernel waits for its own

@@ -184,7 +184,7 @@ __global__ __launch_bounds__(256) void qk_rope_kv_kernel(
   HeadFactors<PASSES> f;
   head16_load_values<T, PASSES>(x, src, d, gl);
   head16_load_factors<PASSES>(f, d, weight, cos_table, sin_table, pos, rot, gl);
-  head16_finish<T, PASSES>(x, f, d, weight != nullptr, eps, cos_table != nullptr, rot, gl, [&](int e0, const T (&v)[8]) {
+  head16_finish<T, PASSES>(x, f, d, weight != nullptr, eps, cos_table != nullptr, rot, gl, [&](int e0, const T (&v)[8]) LS_INLINED {
     if (held) store8<T>(dst + e0, v);
   });
 }

@@ -204,7 +204,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const void* __rest
   // needs one, so a wave keeps several kilobytes in flight.
   // as many chunks as the registers of a wave allow (512 / (NW / 4) a lane), so that a slice of 256 elements is one round
   constexpr int UNR = ((NT + MT) * 8 * 4 + NT * MT * 4 + 32 <= 2048 / NW && !NORM) ? 8 : 4;
-  auto load_w = [&](int k0, int k_end, vec_t (&w)[NT][UNR]) {
+  auto load_w = [&](int k0, int k_end, vec_t (&w)[NT][UNR]) LS_INLINED {
 #pragma unroll
     for (int u = 0; u < UNR; ++u) {
       const int k = k0 + u * A::KCHUNK + g * A::VEC;
@@ -370,7 +370,7 @@ __global__ __launch_bounds__(1024) void gemm_stream_kernel(const T* __restrict__
   const int walkers = gridDim.x / row_groups;
   const int m_base = row_group * MT * 16;
 
-  auto fetch = [&](int b, int t, int q, vec_t (&dst)[UC]) {
+  auto fetch = [&](int b, int t, int q, vec_t (&dst)[UC]) LS_INLINED {
     const int n = (b * NT + t) * 16 + row16;
 #pragma unroll
     for (int c = 0; c < UC; ++c) {
@@ -402,7 +402,7 @@ __global__ __launch_bounds__(1024) void gemm_stream_kernel(const T* __restrict__
   // One column block; `par` is the buffer that holds the block's first unit (static, so that the
   // register buffers are addressed statically).
   static_assert(UNITS % RING == 0 || (2 * UNITS) % RING == 0, "the buffer of a block's first unit has period two");
-  auto block_step = [&](auto par, int it) {
+  auto block_step = [&](auto par, int it) LS_INLINED {
     constexpr int P = decltype(par)::value;
     float* mine = part + (it & 1) * (nw * NT * MT * 256);
     f32x4 acc[MT];  // of the tile in work; a finished tile's sums go to LDS at once
@@ -777,7 +777,7 @@ __global__ __launch_bounds__(256) void gemm_slices_stream_kernel(const T* __rest
   const int walkers = gridDim.x;
   const int m_base = blockIdx.z * MT * 16;  // more than 16 * MT rows: groups of rows, each with workgroups of its own
 
-  auto fetch = [&](int b, int q, vec_t (&dst)[UC]) {
+  auto fetch = [&](int b, int q, vec_t (&dst)[UC]) LS_INLINED {
     const int n = b * 16 + row16;
 #pragma unroll
     for (int c = 0; c < UC; ++c) {
@@ -802,7 +802,7 @@ __global__ __launch_bounds__(256) void gemm_slices_stream_kernel(const T* __rest
                              m_base + j * 16 + row16 < M && kc < k_end, aligned);
     }
 
-  auto block_step = [&](auto par) {
+  auto block_step = [&](auto par) LS_INLINED {
     constexpr int P0 = decltype(par)::value;
     f32x4 acc[MT];
 #pragma unroll
@@ -934,7 +934,7 @@ __global__ __launch_bounds__(64 * NWM * NWN) void gemm_tiled_kernel(const T* __r
 #pragma unroll
     for (int p = 0; p < XP; ++p) x_src[p] = X + (long)min(m_base + st_row + PASS * p, M - 1) * ldx;
   }
-  auto fetch = [&](int slot, int k0) {
+  auto fetch = [&](int slot, int k0) LS_INLINED {
     if (AL) {
       const int k = min(k0 + st_col, K - A::VEC);
 #pragma unroll
@@ -954,7 +954,7 @@ __global__ __launch_bounds__(64 * NWM * NWN) void gemm_tiled_kernel(const T* __r
       xv[slot][p] = load_vec<T>(X, m_base + r, k0 + st_col, K, ldx, m_base + r < M, false);
     }
   };
-  auto stash = [&](int slot, int buf, int k0) {
+  auto stash = [&](int slot, int buf, int k0) LS_INLINED {
     unsigned char* w_lds = lds + buf * STAGE_BYTES;
     unsigned char* x_lds = w_lds + BN * kRowStride;
 #pragma unroll
@@ -980,8 +980,8 @@ __global__ __launch_bounds__(64 * NWM * NWN) void gemm_tiled_kernel(const T* __r
   const int all_stages = (K + BK - 1) / BK;
   const int first_stage = SLICES ? (int)blockIdx.y * out_cols * (kslice / BK) : 0;
   const int stages = SLICES ? min(all_stages - first_stage, out_cols * (kslice / BK)) : all_stages;
-  auto k_of = [&](int st) { return (first_stage + st) * BK; };
-  auto store_slice = [&](int slice) {  // the sums of one slice to their place among the slice sums
+  auto k_of = [&](int st) LS_INLINED { return (first_stage + st) * BK; };
+  auto store_slice = [&](int slice) LS_INLINED {  // the sums of one slice to their place among the slice sums
     float* sums = reinterpret_cast<float*>(C) + (long)slice * M * N;
 #pragma unroll
     for (int i = 0; i < TI; ++i)
@@ -1025,7 +1025,7 @@ __global__ __launch_bounds__(64 * NWM * NWN) void gemm_tiled_kernel(const T* __r
       const unsigned char* x_lds = w_lds + BN * kRowStride;
       // the fragments of the second chunk are read while the first is multiplied
       vec_t a[2][TI], b[2][TJ];
-      auto fragments = [&](int c) {
+      auto fragments = [&](int c) LS_INLINED {
 #pragma unroll
         for (int i = 0; i < TI; ++i)
           a[c][i] = *reinterpret_cast<const vec_t*>(&w_lds[(wn + i * 16 + row16) * kRowStride + c * 64 + g * 16]);
@@ -1311,7 +1311,7 @@ extern "C" int ls_gemm_slices(int dtype, const void* X, const void* W, float* P,
     const int stages_a_slice = kslice / (128 / (dtype == kF32 ? 4 : 2));
     int per = std::min(nslices, std::max(1, (8 + stages_a_slice - 1) / stages_a_slice));
     const int tiles_m = (M + 63) / 64, tiles_n = (N + 63) / 64;
-    auto workgroups = [&](int p) { return (long)tiles_m * tiles_n * ((nslices + p - 1) / p); };
+    auto workgroups = [&](int p) LS_INLINED { return (long)tiles_m * tiles_n * ((nslices + p - 1) / p); };
     while (per > 1 && workgroups(per) < compute_units()) per = (per + 1) / 2;
     if (workgroups(per) >= compute_units()) {
       const int groups_y = (nslices + per - 1) / per;

@@ -460,7 +460,7 @@ extern "C" int ls_sample_top_p(const float* logits, long ld, const void* request
              scratch_bytes, ls_sample_scratch_bytes(n, vocab));
   SampleScratch sc;
   char* at = reinterpret_cast<char*>(scratch);
-  auto take = [&](size_t bytes) { char* here = at; at += align_up(bytes); return here; };
+  auto take = [&](size_t bytes) LS_INLINED { char* here = at; at += align_up(bytes); return here; };
   sc.weights = reinterpret_cast<double*>(take((size_t)n * vocab * sizeof(double)));
   sc.keys = reinterpret_cast<unsigned int*>(take((size_t)n * vocab * sizeof(unsigned int)));
   sc.part_max = reinterpret_cast<float*>(take((size_t)n * kChunks * sizeof(float)));
