@@ -48,6 +48,10 @@ FOLD_IN_PRODUCT = os.environ.get("LOCKSTEP_FOLD_IN_PRODUCT", "1") not in ("", "0
 EMBED_PAGES = os.environ.get("LOCKSTEP_EMBED_PAGES", "1") not in ("", "0")
 FOLD_MAX_SPLITS = int(os.environ.get("LOCKSTEP_FOLD_MAX_SPLITS", "8"))
 FOLD_MAX_ROW_SPLITS = int(os.environ.get("LOCKSTEP_FOLD_MAX_ROW_SPLITS", "128"))   # requests times splits
+# ... and for output products of at most this many columns: every block of 64 columns repeats the fold (measured at
+# 4,096 columns, Qwen3-8B sizes: 1 % slower at 8 requests and 8 % at 16 than the combine launch; at 1,024 columns
+# the fold is ahead at every batch it takes)
+FOLD_MAX_COLUMNS = int(os.environ.get("LOCKSTEP_FOLD_MAX_COLUMNS", "2048"))
 
 
 # ---------------------------------------------------------------------------
@@ -98,7 +102,7 @@ def _round_up(n: int, buckets=(1, 2, 4, 8, 12, 16, 24, 32, 40, 48, 56, 64), step
     return -(-n // step) * step
 
 
-def plan_attention(ctx, group_size: int, nkv: int, head_dim: int, window: int):
+def plan_attention(ctx, group_size: int, nkv: int, head_dim: int, window: int, out_columns: int = 0):
     """Work items of one set of attention constants for this step: (plan, ints of the block).
 
     Requests are cut at the kernels' own, position-anchored splits; which kernel takes a request
@@ -152,7 +156,8 @@ def plan_attention(ctx, group_size: int, nkv: int, head_dim: int, window: int):
                 span = min(span, MAX_SPAN)
 
     fold_splits = 0
-    if (FOLD_IN_PRODUCT and span == 1 and window == 0 and ctx.n_seqs <= 16 and bool(to_coop.all())
+    if (FOLD_IN_PRODUCT and 0 < out_columns <= FOLD_MAX_COLUMNS and span == 1 and window == 0 and ctx.n_seqs <= 16
+            and bool(to_coop.all())
             and bool((ctx.q_len == 1).all())):
         most = int(counts.max())
         # (with one split everywhere nothing is folded anyway: the workgroups write the output themselves)
@@ -374,7 +379,8 @@ class Attention(Mixer):
 
     def _block_key(self):
         window = int(self.window) if self.window is not None else 0
-        return ("attention", self.nq // self.nkv, self.nkv, self.d, window)
+        # (the width of the output product is part of the plan: the fold of the splits may be left to it)
+        return ("attention", self.nq // self.nkv, self.nkv, self.d, window, self.hidden)
 
     def prepare(self, ctx) -> None:
         self.position.ensure(ctx.max_position + 1, ctx.rt)
