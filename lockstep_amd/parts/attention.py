@@ -28,11 +28,11 @@ from .base import Mixer, PagedKVSpec, PendingAdd, WeightSpec, build_part, deferr
 # Steps of single decoded tokens run norm, rotation and cache write inside the
 # attention kernel (one launch less per layer); "0" keeps the separate kernel.
 FUSE_DECODE = os.environ.get("LOCKSTEP_FUSE_DECODE", "1") not in ("", "0")
-# From this many (request, kv head) pairs on, the prologue of the fused kernel costs more than the separate
-# norm/rotation launch (measured +2 % at batch 64, 8 kv heads).  Pairs, not workgroups: a request that is cut
-# into many items repeats only the query's part of the prologue in each, and one launch less still pays
-# (eight requests of 16,384 tokens: 4.23 -> 4.13 ms a step).
-FUSE_DECODE_BELOW = int(os.environ.get("LOCKSTEP_FUSE_DECODE_BELOW", "512"))
+# A bound on the (request, kv head) pairs of a step that is fused, for measurements: with the prologue as it
+# is now (operands requested ahead of the tile, norm and rotation by row rotations) one launch less pays at every
+# batch measured (batch 64: 2.36 -> 2.32 ms a step at 0.6B sizes, 3.35 -> 3.32 at 8B, 3.43 -> 3.41 at 32B; batch
+# 128: 3.30 -> 3.25); with the earlier prologue it cost 2 % from 512 pairs on.
+FUSE_DECODE_BELOW = int(os.environ.get("LOCKSTEP_FUSE_DECODE_BELOW", str(1 << 30)))
 # The most splits one cooperative workgroup walks when a request is cut over several.
 MAX_SPAN = 8               # splits of a work item where requests of a ragged batch are cut
 WORKGROUPS_A_CU = 2         # work items (times kv heads) a CU that a decode step is cut for
