@@ -2148,7 +2148,9 @@ static int launch_coop_as(dim3 grid, hipStream_t s, const void* q, long ldq, con
   constexpr int BUFS = coop_bufs(sizeof(T));
   // one tile buffer (two workgroups a CU) where a second one could not be used: many workgroups, or items of
   // one tile each, which have no next tile to request ahead
-  const bool crowded = (long)grid.x * grid.y >= LS_COOP_CROWDED_FROM || single_tile;
+  // (more workgroups than CUs but fewer than two a CU would be two rounds of one a CU with two buffers; with one
+  // buffer they all run together: 48 requests of 8 kv heads 2.37 -> see the measurements in the planner)
+  const bool crowded = (long)grid.x * grid.y >= LS_COOP_CROWDED_FROM || (long)grid.x * grid.y > compute_units() || single_tile;
 #define LS_COOP(NBUF_)                                                                                              \
   hipLaunchKernelGGL((attention_coop_kernel<T, NBUF_, FUSE, SPANS>), grid, dim3(256), (coop_kernel_lds<T, NBUF_>()), s, \
                      (const AttnItem*)items, (const T*)q, ldq, fz.q_weight, fz.k_weight, fz.cos_table, fz.sin_table, G, \

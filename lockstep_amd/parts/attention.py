@@ -35,7 +35,11 @@ FUSE_DECODE = os.environ.get("LOCKSTEP_FUSE_DECODE", "1") not in ("", "0")
 FUSE_DECODE_BELOW = int(os.environ.get("LOCKSTEP_FUSE_DECODE_BELOW", str(1 << 30)))
 # The most splits one cooperative workgroup walks when a request is cut over several.
 MAX_SPAN = 8               # splits of a work item where requests of a ragged batch are cut
-WORKGROUPS_A_CU = 2         # work items (times kv heads) a CU that a decode step is cut for
+# Work items (times kv heads) a CU that a decode step of few long requests is cut for.  Measured at 0.6B sizes
+# (ms a step, whole requests / this rule / every split an item): 8 requests of 2,048 tokens 2.23 / 1.50 / 1.50,
+# 8 of 4,096 - / 1.94 / 1.94 (2.12 with two items a CU), 24 of 512 - / 1.56 / 1.56 (1.65), 16 of 8,192 5.82 / - / 4.34;
+# from a workgroup for every CU on, whole requests win (32 of 2,048: 2.70 against 2.87; 32 of 8,192: 6.29 against 7.46).
+WORKGROUPS_A_CU = int(os.environ.get("LOCKSTEP_WORKGROUPS_A_CU", "8"))
 RAGGED_RATIO = 2.0         # a batch is ragged when its longest request has more than this many times the mean splits
 PART_ROWS_STEP = 4096      # rows of partial results are taken in steps of this many (sizes of replayed steps)
 # A step of few decoded tokens whose requests have few splits each leaves the fold of the splits to the output
@@ -140,11 +144,15 @@ def plan_attention(ctx, group_size: int, nkv: int, head_dim: int, window: int, o
     span = 1
     if to_coop.any():
         mine = counts[to_coop]
-        enough = WORKGROUPS_A_CU * kernels.compute_units()
-        if int(mine.sum()) * nkv >= enough:
-            span = int(mine.max())                              # every request is walked whole ...
-            if len(mine) * nkv < kernels.compute_units():       # ... unless that leaves CUs without work: the
-                low, high = 1, span                             # longest items that still give every CU two
+        cus = kernels.compute_units()
+        if len(mine) * nkv >= cus:
+            span = int(mine.max())                              # a workgroup for every CU: requests are walked whole
+        else:
+            # fewer: items of one split (one tile, the kernel's shortest chain) while their number stays moderate,
+            # else the longest items that still give every CU WORKGROUPS_A_CU of them
+            enough = WORKGROUPS_A_CU * cus
+            if int(mine.sum()) * nkv >= enough:
+                low, high = 1, int(mine.max())
                 while low < high:
                     middle = (low + high + 1) // 2
                     if int((-(-mine // middle)).sum()) * nkv >= enough:
@@ -152,8 +160,8 @@ def plan_attention(ctx, group_size: int, nkv: int, head_dim: int, window: int, o
                     else:
                         high = middle - 1
                 span = low
-            if int(mine.max()) > RAGGED_RATIO * float(mine.mean()):
-                span = min(span, MAX_SPAN)
+        if span > 1 and int(mine.max()) > RAGGED_RATIO * float(mine.mean()):
+            span = min(span, MAX_SPAN)
 
     fold_splits = 0
     if (FOLD_IN_PRODUCT and 0 < out_columns <= FOLD_MAX_COLUMNS and span == 1 and window == 0 and ctx.n_seqs <= 16

@@ -166,11 +166,12 @@ def test_requests_of_very_different_lengths_decode_with_the_bits_of_one(models):
         assert torch.equal(torch.stack([t[i] for t in together]), want), f"request {i} (context {lengths[i]})"
 
 
-def test_few_long_requests_are_cut_so_that_every_cu_has_work(tmp_path):
+def test_few_long_requests_are_cut_so_that_every_cu_has_work(tmp_path, monkeypatch):
     """Three requests of some 12,300 tokens in one decode step: walked whole they would be 24 workgroups;
-    the planner cuts them into the longest items that still give every CU two (here two splits an
-    item), the decode loop lays the same out for the lengths to come, and each request has the bits
-    it has alone."""
+    the planner cuts them into the longest items that still give every CU a set number (the test asks for
+    two a CU, which makes items of two splits and so runs the kernel instance that leaves a partial result
+    for each split of an item; the default of eight a CU makes items of one split here), the decode loop
+    lays the same out for the lengths to come, and each request has the bits it has alone."""
     import lockstep_amd.parts.attention as attention_module
     from lockstep_amd.config import Qwen3Config
     from lockstep_amd.engine.batch import StepEntry
@@ -202,12 +203,28 @@ def test_few_long_requests_are_cut_so_that_every_cu_has_work(tmp_path):
         return plan, ints
 
     attention_module.plan_attention = watching
+    a_cu = attention_module.WORKGROUPS_A_CU
+    monkeypatch.setattr(attention_module, "WORKGROUPS_A_CU", 2)
     try:
         together = [model.step(cache, [StepEntry(f"r{i}", [prompts[i][lengths[i] + k]], [0]) for i in range(3)]).cpu()
                     for k in range(n_decode)]
+        assert seen and all(p.spans and p.n_combine >= 3 and 8 * p.n_coop >= 512 for p in seen), seen
+        # ... and with the default, items of one split: the same bits
+        monkeypatch.setattr(attention_module, "WORKGROUPS_A_CU", a_cu)
+        cache_b = model.make_cache(num_pages=4 * 780, page_size=16, max_requests=4)
+        for i, m in enumerate(lengths):
+            cache_b.open(f"r{i}")
+            for lo in range(0, m, 4096):
+                model.step(cache_b, [StepEntry(f"r{i}", prompts[i][lo:min(lo + 4096, m)], [])])
+        del seen[:]
+        again = [model.step(cache_b, [StepEntry(f"r{i}", [prompts[i][lengths[i] + k]], [0]) for i in range(3)]).cpu()
+                 for k in range(n_decode)]
+        assert seen and all(not p.spans and p.single_tile for p in seen), seen
+        assert all(torch.equal(a, b) for a, b in zip(together, again))
+        del cache_b
+        monkeypatch.setattr(attention_module, "WORKGROUPS_A_CU", 2)
     finally:
         attention_module.plan_attention = original
-    assert seen and all(p.spans and p.n_combine >= 3 and 8 * p.n_coop >= 512 for p in seen), seen
     prefill("alone", prompts[1][:lengths[1]])
     for k in range(n_decode):
         want = model.step(cache, [StepEntry("alone", [prompts[1][lengths[1] + k]], [0])]).cpu()
