@@ -34,7 +34,7 @@ FUSE_DECODE = os.environ.get("LOCKSTEP_FUSE_DECODE", "1") not in ("", "0")
 # 128: 3.30 -> 3.25); with the earlier prologue it cost 2 % from 512 pairs on.
 FUSE_DECODE_BELOW = int(os.environ.get("LOCKSTEP_FUSE_DECODE_BELOW", str(1 << 30)))
 # The most splits one cooperative workgroup walks when a request is cut over several.
-MAX_SPAN = 8               # splits of a work item where requests of a ragged batch are cut
+MAX_SPAN = int(os.environ.get("LOCKSTEP_MAX_SPAN", "8"))   # splits of a work item where requests of a ragged batch are cut
 # Work items (times kv heads) a CU that a decode step of few long requests is cut for.  Measured at 0.6B sizes
 # (ms a step, whole requests / this rule / every split an item): 8 requests of 2,048 tokens 2.23 / 1.50 / 1.50,
 # 8 of 4,096 - / 1.94 / 1.94 (2.12 with two items a CU), 24 of 512 - / 1.56 / 1.56 (1.65), 16 of 8,192 5.82 / - / 4.34;
