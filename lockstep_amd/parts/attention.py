@@ -38,7 +38,8 @@ MAX_SPAN = int(os.environ.get("LOCKSTEP_MAX_SPAN", "8"))   # splits of a work it
 # Work items (times kv heads) a CU that a decode step of few long requests is cut for.  Measured at 0.6B sizes
 # (ms a step, whole requests / this rule / every split an item): 8 requests of 2,048 tokens 2.23 / 1.50 / 1.50,
 # 8 of 4,096 - / 1.94 / 1.94 (2.12 with two items a CU), 24 of 512 - / 1.56 / 1.56 (1.65), 16 of 8,192 5.82 / - / 4.34;
-# from a workgroup for every CU on, whole requests win (32 of 2,048: 2.70 against 2.87; 32 of 8,192: 6.29 against 7.46).
+# from a workgroup for every CU on, whole requests win (32 of 2,048: 2.70 against 2.87; 32 of 8,192: 6.29 against 7.46;
+# 64 of 512 cut in items of three and two splits 2.46 to 2.57 against 2.32, 64 of 4,096 in four to six items 7.5 against 6.9).
 WORKGROUPS_A_CU = int(os.environ.get("LOCKSTEP_WORKGROUPS_A_CU", "8"))
 RAGGED_RATIO = 2.0         # a batch is ragged when its longest request has more than this many times the mean splits
 PART_ROWS_STEP = 4096      # rows of partial results are taken in steps of this many (sizes of replayed steps)
