@@ -136,15 +136,18 @@ __global__ __launch_bounds__(256) void qk_rope_kv_kernel(
   const int head_blocks = (int)(((long)n_tokens * (write_kv ? nq + nkv : nq) + 15) / 16);
   if ((int)blockIdx.x >= head_blocks) {
     // Values: a workgroup copies 16 consecutive tokens of the batch.  Sixteen neighbouring lanes
-    // hold the same column of 16 tokens, so where the tokens are neighbours in a page their
-    // 2-byte elements leave as whole 32-byte runs of the transposed page.
-    // A workgroup takes 64 columns of its 16 tokens: four loads a thread, all in flight together.
+    // hold the same columns of 16 tokens, so where the tokens are neighbours in a page their
+    // elements leave as whole runs of 16 slots of the transposed page.  A thread loads one 16-byte run of
+    // its token's row (a workgroup takes 16 such runs of its 16 tokens) and stores its elements one by one.
+    constexpr int RUN = 16 / (int)sizeof(T);
     const int width = nkv * d;  // the value heads of a token are contiguous; so are the rows of a page
-    const int col_blocks = (width + 63) / 64;
+    const int col_blocks = (width + 16 * RUN - 1) / (16 * RUN);
     const int vb = (int)blockIdx.x - head_blocks;
     const int j = threadIdx.x & 15;
     const int t = (vb / col_blocks) * 16 + j;
     if (t >= n_tokens) return;
+    const int c0 = (vb % col_blocks) * 16 * RUN + (threadIdx.x >> 4) * RUN;
+    if (c0 >= width) return;  // (d is a multiple of RUN: a run lies inside the row or outside)
     const int pos = tok_pos[t];
     const SeqMeta sm = seqs[tok_seq[t]];
     const long page = table[(long)sm.table_row * table_stride + pos / page_size];
@@ -152,13 +155,18 @@ __global__ __launch_bounds__(256) void qk_rope_kv_kernel(
     const int slot = pos % page_size;
     const T* src = qkv + (long)t * ld + (long)(nq + nkv) * d;
     T* dst = v_pages + page * nkv * d * page_size + slot;
-    const int c0 = (vb % col_blocks) * 64 + (threadIdx.x >> 4);
-    T v[4];
+    T v[RUN];
+    if (sizeof(T) == 2) {
+      const bf16x8 run = *reinterpret_cast<const bf16x8*>(src + c0);
 #pragma unroll
-    for (int u = 0; u < 4; ++u) v[u] = src[min(c0 + 16 * u, width - 1)];
+      for (int u = 0; u < RUN; ++u) v[u] = run[u];
+    } else {
+      const f32x4 run = *reinterpret_cast<const f32x4*>(src + c0);
 #pragma unroll
-    for (int u = 0; u < 4; ++u)
-      if (c0 + 16 * u < width) dst[(long)(c0 + 16 * u) * page_size] = v[u];
+      for (int u = 0; u < RUN; ++u) v[u] = run[u];
+    }
+#pragma unroll
+    for (int u = 0; u < RUN; ++u) dst[(long)(c0 + u) * page_size] = v[u];
     return;
   }
   // Query and key heads: sixteen lanes a head (see head16_finish), sixteen heads a workgroup.
@@ -608,7 +616,8 @@ extern "C" int ls_qk_rope_kv(int dtype, void* qkv, long ld, int n_tokens, int nq
                                  reinterpret_cast<uintptr_t>(sin_table) % 16 == 0)),
              "qk_rope_kv: norm weights and rotation tables must be 16-byte aligned");
   const long head_blocks = ((long)n_tokens * (write_kv ? nq + nkv : nq) + 15) / 16;
-  const long value_blocks = write_kv ? (long)((n_tokens + 15) / 16) * (((long)nkv * d + 63) / 64) : 0;
+  const long run = 16 / (long)elem;  // elements of a 16-byte run: a workgroup of the value copy takes 16 runs of 16 tokens
+  const long value_blocks = write_kv ? (long)((n_tokens + 15) / 16) * (((long)nkv * d + 16 * run - 1) / (16 * run)) : 0;
   dim3 grid((unsigned)(head_blocks + value_blocks));
 #define LS_ROPE(T_, P_)                                                                                            \
   hipLaunchKernelGGL((qk_rope_kv_kernel<T_, P_>), grid, dim3(256), 0, s, (T_*)qkv, ld, nq, nkv, d, q_weight, k_weight, \
